@@ -1,0 +1,12 @@
+"""gesso_amd: a small, whole inference engine for one MI355X (gfx950).
+
+From a request's tokens to its next token: typed configuration and architecture registry,
+weights by tensor name, layers composed of parts, a paged cache with per-request state slots,
+one step function over mixed batches, a scheduler with sampling, and hand-written HIP kernels.
+"""
+from . import parts as _parts  # noqa: F401  registers part kinds
+from .models import lfm2 as _lfm2  # noqa: F401  registers the architecture
+from .errors import (ConfigError, GessoError, InvalidPlan, KernelError, NumericalInstability, OutOfPages,
+                     OutOfSlots, ResourceLimit, WeightError)
+
+__version__ = "0.1.0"

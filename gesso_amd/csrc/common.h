@@ -1,0 +1,100 @@
+// Shared helpers of the gfx950 kernels: storage types, conversions, reductions, error reporting.
+//
+// Every entry point is extern "C", takes raw device pointers, sizes and a stream, checks
+// what it assumes about sizes on the host, and returns 0 or a negative code after recording
+// a message that gs_last_error() returns.  dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define GS_F32 0
+#define GS_BF16 1
+
+#define GS_WAVE 64
+
+extern "C" const char* gs_last_error();
+void gs_set_error(const char* fmt, ...);
+
+#define GS_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      gs_set_error(__VA_ARGS__);         \
+      return -1;                         \
+    }                                    \
+  } while (0)
+
+#define GS_LAUNCH_CHECK(name)                                                 \
+  do {                                                                        \
+    hipError_t e_ = hipGetLastError();                                        \
+    if (e_ != hipSuccess) {                                                   \
+      gs_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));     \
+      return -2;                                                              \
+    }                                                                         \
+  } while (0)
+
+// bfloat16 as bits; conversions are explicit so that every rounding is visible in the code.
+struct bf16 {
+  uint16_t x;
+};
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16 v) { return __uint_as_float(((uint32_t)v.x) << 16); }
+
+// round to nearest, ties to even; NaN stays NaN
+__device__ __forceinline__ bf16 f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  bf16 r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r.x = (uint16_t)((u >> 16) | 0x40);
+    return r;
+  }
+  u += 0x7fffu + ((u >> 16) & 1u);
+  r.x = (uint16_t)(u >> 16);
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) {
+  return v;
+}
+template <>
+__device__ __forceinline__ bf16 from_f32<bf16>(float v) {
+  return f32_to_bf16(v);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, GS_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, GS_WAVE));
+  return v;
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, GS_WAVE);
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.  `red` holds 17 floats.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (int i = 0; i < nw; ++i) s += red[i];
+    red[16] = s;
+  }
+  __syncthreads();
+  return red[16];
+}
+
+static inline int gs_ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -1,0 +1,191 @@
+// Embedding gather, residual add + RMSNorm, SwiGLU activation, small fills.
+//
+// The residual stream is float32 in both precisions; the rows that feed matrix products
+// are written in the activation type.  Sums of squares are float32 in a fixed order per row,
+// so a row's result does not depend on which other rows share the launch.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+static thread_local char g_err[512] = "";
+
+void gs_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* gs_last_error() { return g_err; }
+
+extern "C" int gs_abi_version() { return 1; }
+
+// ------------------------------------------------------------------ embedding
+
+// out[t, :] = table[ids[t], :] as float32; an id outside the table gives a NaN row.
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
+                             int H, int V) {
+  int t = blockIdx.x;
+  int id = ids[t];
+  float* o = out + (size_t)t * H;
+  if (id < 0 || id >= V) {
+    for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  const T* row = table + (size_t)id * H;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = to_f32(row[j]);
+}
+
+extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, float* out, int T, int H, int V,
+                        hipStream_t stream) {
+  GS_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+  if (T == 0) return 0;
+  if (table_dtype == GS_F32)
+    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, H, V);
+  else if (table_dtype == GS_BF16)
+    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, H, V);
+  else
+    GS_REQUIRE(false, "embed: unknown dtype %d", table_dtype);
+  GS_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ------------------------------------------------------------------ add + RMSNorm
+
+// One block per output row r.  Source row s = rows ? rows[r] : r.
+//   x = res[s] (+ delta[s]);  out[r] = x / sqrt(mean(x^2) + eps) * w
+// Without `rows` the sum is written back to res (the stream moves on); with `rows` (a gather
+// at the model's end) res is left as it is, so a row may be asked for twice.
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict__ delta, const float* __restrict__ w,
+                                   float eps, TO* __restrict__ out, const int* __restrict__ rows, int H) {
+  __shared__ float red[17];
+  int r = blockIdx.x;
+  int s = rows ? rows[r] : r;
+  float* x = res + (size_t)s * H;
+  const TD* dl = delta ? delta + (size_t)s * H : nullptr;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    float v = x[j];
+    if (dl) {
+      v += to_f32(dl[j]);
+      if (!rows) x[j] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)r * H;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    float v = x[j];
+    if (dl && rows) v += to_f32(dl[j]);
+    o[j] = from_f32<TO>(v * inv * w[j]);
+  }
+}
+
+extern "C" int gs_add_rmsnorm(float* res, const void* delta, int delta_dtype, const float* w, float eps, void* out,
+                              int out_dtype, const int* rows, int n_out, int H, hipStream_t stream) {
+  GS_REQUIRE(n_out >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_out, H);
+  GS_REQUIRE(eps > 0.f, "add_rmsnorm: eps must be positive");
+  if (n_out == 0) return 0;
+  int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+#define GS_RUN(TD, TO)                                                                                          \
+  add_rmsnorm_kernel<TD, TO><<<n_out, threads, 0, stream>>>(res, (const TD*)delta, w, eps, (TO*)out, rows, H)
+  if (delta_dtype == GS_F32 && out_dtype == GS_F32)
+    GS_RUN(float, float);
+  else if (delta_dtype == GS_BF16 && out_dtype == GS_BF16)
+    GS_RUN(bf16, bf16);
+  else if (delta_dtype == GS_F32 && out_dtype == GS_BF16)
+    GS_RUN(float, bf16);
+  else if (delta_dtype == GS_BF16 && out_dtype == GS_F32)
+    GS_RUN(bf16, float);
+  else
+    GS_REQUIRE(false, "add_rmsnorm: unknown dtypes %d %d", delta_dtype, out_dtype);
+#undef GS_RUN
+  GS_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+// res[t, :] += delta[t, :]   (the last sub-layer's output, when no norm follows it)
+template <typename TD>
+__global__ void add_kernel(float* __restrict__ res, const TD* __restrict__ delta, long n) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) res[i] += to_f32(delta[i]);
+}
+
+extern "C" int gs_residual_add(float* res, const void* delta, int delta_dtype, long n, hipStream_t stream) {
+  GS_REQUIRE(n >= 0, "residual_add: bad size");
+  if (n == 0) return 0;
+  int blocks = gs_ceil_div(n, 256);
+  if (delta_dtype == GS_F32)
+    add_kernel<float><<<blocks, 256, 0, stream>>>(res, (const float*)delta, n);
+  else if (delta_dtype == GS_BF16)
+    add_kernel<bf16><<<blocks, 256, 0, stream>>>(res, (const bf16*)delta, n);
+  else
+    GS_REQUIRE(false, "residual_add: unknown dtype %d", delta_dtype);
+  GS_LAUNCH_CHECK("residual_add");
+  return 0;
+}
+
+// ------------------------------------------------------------------ SwiGLU
+
+// in (T, 2F): gate in columns [0, F), up in [F, 2F).  out[t, j] = silu(gate) * up, silu(g) = g / (1 + exp(-g)).
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ in, T* __restrict__ out, int F, long n) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  long t = i / F;
+  int j = (int)(i - t * F);
+  float g = to_f32(in[t * 2 * F + j]);
+  float u = to_f32(in[t * 2 * F + F + j]);
+  out[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int gs_swiglu(const void* in, void* out, int dtype, int T, int F, hipStream_t stream) {
+  GS_REQUIRE(T >= 0 && F > 0, "swiglu: bad sizes T=%d F=%d", T, F);
+  long n = (long)T * F;
+  if (n == 0) return 0;
+  int blocks = gs_ceil_div(n, 256);
+  if (dtype == GS_F32)
+    swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, F, n);
+  else if (dtype == GS_BF16)
+    swiglu_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)in, (bf16*)out, F, n);
+  else
+    GS_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+  GS_LAUNCH_CHECK("swiglu");
+  return 0;
+}
+
+// ------------------------------------------------------------------ fills
+
+__global__ void fill_f32_kernel(float* p, float v, long n) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// A fill that is an ordinary kernel, so that it may be recorded into a HIP graph.
+extern "C" int gs_fill_f32(float* p, float v, long n, hipStream_t stream) {
+  GS_REQUIRE(n >= 0, "fill: bad size");
+  if (n == 0) return 0;
+  fill_f32_kernel<<<gs_ceil_div(n, 256), 256, 0, stream>>>(p, v, n);
+  GS_LAUNCH_CHECK("fill_f32");
+  return 0;
+}
+
+// Zero the state rows of given slots: state (num_slots, row) float32; slots (n).
+__global__ void zero_slots_kernel(float* state, const int* slots, long row) {
+  int s = slots[blockIdx.y];
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= 0 && i < row) state[(size_t)s * row + i] = 0.f;
+}
+
+extern "C" int gs_zero_slots(float* state, const int* slots, int n, long row, hipStream_t stream) {
+  GS_REQUIRE(n >= 0 && row >= 0, "zero_slots: bad sizes");
+  if (n == 0 || row == 0) return 0;
+  dim3 grid(gs_ceil_div(row, 256), n);
+  zero_slots_kernel<<<grid, 256, 0, stream>>>(state, slots, row);
+  GS_LAUNCH_CHECK("zero_slots");
+  return 0;
+}

@@ -1,0 +1,109 @@
+// Gated short convolution over a batch of sequence segments, with per-request history.
+//
+// bcx (T, 3H) holds B, C, X side by side.  Per channel c and token t of a segment:
+//   u[t]  = B[t,c] * X[t,c]
+//   y[t]  = sum_{p=0}^{W-1} taps[c,p] * u[t-(W-1)+p]      (taps oldest to newest, current input last)
+//   out   = C[t,c] * (y[t] + bias[c])
+// where u before the segment's first token comes from the request's history
+// state[slot, c, 0..W-2] (oldest to newest).  After the segment the history holds the last
+// W-1 values of u (older history shifts out).  Products and sums are float32; the history is
+// float32 in both precisions.
+//
+// Two kernels: outputs (one thread per token and channel, all reading the old history), then
+// the history update (one thread per sequence and channel).  When every segment is a single
+// token the first kernel also updates the history, since no other thread reads it.
+#include "common.h"
+
+#define GS_CONV_MAX_W 16
+
+template <typename T>
+__global__ void short_conv_kernel(const T* __restrict__ bcx, const float* __restrict__ taps,
+                                  const float* __restrict__ bias, float* __restrict__ state,
+                                  const int* __restrict__ seq_of_token, const int* __restrict__ q_start,
+                                  const int* __restrict__ slots, T* __restrict__ out, int ntok, int H, int W,
+                                  int update_state) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= H) return;
+  const float* wt = taps + (size_t)c * W;
+  for (int t = blockIdx.y; t < ntok; t += gridDim.y) {
+    int s = seq_of_token[t];
+    int t0 = q_start[s];
+    float* hist = state + ((size_t)slots[s] * H + c) * (W - 1);
+    float y = 0.f;
+    float u_now = 0.f;
+    for (int p = 0; p < W; ++p) {
+      int j = t - (W - 1) + p;  // token index of this tap
+      float u;
+      if (j >= t0) {
+        const T* row = bcx + (size_t)j * 3 * H;
+        u = to_f32(row[c]) * to_f32(row[2 * H + c]);
+      } else {
+        // k = t0 - j tokens before the segment: history entry W-1-k
+        u = hist[(W - 1) - (t0 - j)];
+      }
+      y += wt[p] * u;
+      u_now = u;
+    }
+    if (bias) y += bias[c];
+    out[(size_t)t * H + c] = from_f32<T>(to_f32(bcx[(size_t)t * 3 * H + H + c]) * y);
+    if (update_state) {
+      // single-token segment: shift by one, newest last
+      for (int p = 0; p < W - 2; ++p) hist[p] = hist[p + 1];
+      hist[W - 2] = u_now;
+    }
+  }
+}
+
+template <typename T>
+__global__ void short_conv_state_kernel(const T* __restrict__ bcx, float* __restrict__ state,
+                                        const int* __restrict__ q_start, const int* __restrict__ slots, int H,
+                                        int W) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x;
+  int s = blockIdx.y;
+  if (c >= H) return;
+  int t0 = q_start[s], t1 = q_start[s + 1];
+  int n = t1 - t0;
+  if (n <= 0) return;
+  float* hist = state + ((size_t)slots[s] * H + c) * (W - 1);
+  float nh[GS_CONV_MAX_W];
+  for (int p = 0; p < W - 1; ++p) {
+    int j = t1 - (W - 1) + p;  // token whose u lands in entry p
+    if (j >= t0) {
+      const T* row = bcx + (size_t)j * 3 * H;
+      nh[p] = to_f32(row[c]) * to_f32(row[2 * H + c]);
+    } else {
+      nh[p] = hist[p + n];  // old entries move n places towards "older"
+    }
+  }
+  for (int p = 0; p < W - 1; ++p) hist[p] = nh[p];
+}
+
+extern "C" int gs_short_conv(const void* bcx, int dtype, const float* taps, const float* bias, float* state,
+                             const int* seq_of_token, const int* q_start, const int* slots, void* out, int ntok,
+                             int nseq, int H, int W, int all_single, hipStream_t stream) {
+  GS_REQUIRE(ntok >= 0 && nseq >= 0 && H > 0, "short_conv: bad sizes T=%d nseq=%d H=%d", ntok, nseq, H);
+  GS_REQUIRE(W >= 2 && W <= GS_CONV_MAX_W, "short_conv: width %d outside [2, %d]", W, GS_CONV_MAX_W);
+  if (ntok == 0) return 0;
+  int threads = H >= 256 ? 256 : 64;
+  int cx = gs_ceil_div(H, threads);
+  dim3 grid(cx, ntok < 65535 ? ntok : 65535);  // the kernel strides over tokens beyond gridDim.y
+  if (dtype == GS_F32)
+    short_conv_kernel<float><<<grid, threads, 0, stream>>>((const float*)bcx, taps, bias, state, seq_of_token,
+                                                            q_start, slots, (float*)out, ntok, H, W, all_single);
+  else if (dtype == GS_BF16)
+    short_conv_kernel<bf16><<<grid, threads, 0, stream>>>((const bf16*)bcx, taps, bias, state, seq_of_token,
+                                                           q_start, slots, (bf16*)out, ntok, H, W, all_single);
+  else
+    GS_REQUIRE(false, "short_conv: unknown dtype %d", dtype);
+  GS_LAUNCH_CHECK("short_conv");
+  if (!all_single) {
+    GS_REQUIRE(nseq <= 65535, "short_conv: more than 65535 sequences in one call");
+    dim3 grid(cx, nseq);
+    if (dtype == GS_F32)
+      short_conv_state_kernel<float><<<grid, threads, 0, stream>>>((const float*)bcx, state, q_start, slots, H, W);
+    else
+      short_conv_state_kernel<bf16><<<grid, threads, 0, stream>>>((const bf16*)bcx, state, q_start, slots, H, W);
+    GS_LAUNCH_CHECK("short_conv_state");
+  }
+  return 0;
+}

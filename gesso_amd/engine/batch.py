@@ -1,0 +1,105 @@
+"""One step's batch: entries as the caller gives them, and the flattened form the kernels read.
+
+An entry is a request's next tokens (a portion of its prompt, or one decoded token) and the
+places among them whose logits are wanted.  All entries of a step are flattened into one row of
+tokens; per token its position and its sequence, per sequence its start among the rows, its
+length after the step, its slot and its block tables.  Everything the device needs travels in
+one int32 buffer, one copy per step.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Sequence
+
+import numpy as np
+import torch
+
+from ..errors import InvalidPlan
+
+
+@dataclass
+class StepEntry:
+    rid: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)   # indices into ``tokens``
+
+
+def check_entries(entries: List[StepEntry], manager, vocab: int) -> None:
+    """Refuse a step that cannot run, before anything is reserved or written."""
+    seen = set()
+    for e in entries:
+        manager.get(e.rid)
+        if e.rid in seen:
+            raise InvalidPlan(f"request {e.rid!r} occurs twice in one step")
+        seen.add(e.rid)
+        n = len(e.tokens)
+        if n < 1:
+            raise InvalidPlan(f"request {e.rid!r} brings no tokens to this step")
+        for t in e.tokens:
+            if not 0 <= int(t) < vocab:
+                raise InvalidPlan(f"token id {int(t)} outside the vocabulary of {vocab}", token=int(t), vocab=vocab)
+        for w in e.want:
+            if not 0 <= int(w) < n:
+                raise InvalidPlan(f"request {e.rid!r} wants logits at place {w} of {n} tokens")
+
+
+class StepContext:
+    """The flattened batch on the device, plus the host-side facts kernels are chosen by."""
+
+    def __init__(self, entries: List[StepEntry], manager, storage, vocab: int, device, pad_to: int = 0):
+        ps = manager.page_size
+        nseq = len(entries)
+        lens = []
+        for e in entries:
+            lens.append(len(e.tokens))
+        T = sum(lens)
+        self.T, self.nseq = T, nseq
+        self.q_lens = lens
+        self.all_single = all(n == 1 for n in lens)
+        self.max_q_len = max(lens)
+
+        rcs = [manager.get(e.rid) for e in entries]
+        starts = np.zeros(nseq + 1, dtype=np.int32)
+        starts[1:] = np.cumsum(lens)
+        tokens = np.empty(T, dtype=np.int64)
+        positions = np.empty(T, dtype=np.int32)
+        seq_of = np.empty(T, dtype=np.int32)
+        want_rows: List[int] = []
+        for i, (e, rc) in enumerate(zip(entries, rcs)):
+            a, b = starts[i], starts[i + 1]
+            tokens[a:b] = np.asarray(e.tokens, dtype=np.int64)
+            positions[a:b] = np.arange(rc.length, rc.length + lens[i], dtype=np.int32)
+            seq_of[a:b] = i
+            want_rows.extend(int(a) + int(w) for w in e.want)
+        kv_len = np.asarray([rc.length + n for rc, n in zip(rcs, lens)], dtype=np.int32)
+        self.max_kv_len = int(kv_len.max()) if nseq else 0
+        slots = np.asarray([storage.scratch_slot if rc.slot is None else rc.slot for rc in rcs], dtype=np.int32)
+        self.n_want = len(want_rows)
+
+        n_groups = len(manager.pools)
+        max_blocks = max(1, -(-self.max_kv_len // ps))
+        tables = np.empty((n_groups, nseq, max_blocks), dtype=np.int32)
+        for g in range(n_groups):
+            tables[g, :, :] = storage.num_pages[g]            # the scratch page: never read
+            for i, rc in enumerate(rcs):
+                t = rc.tables[g]
+                n = min(len(t), max_blocks)
+                row = np.asarray(t[:n], dtype=np.int32)
+                row[row < 0] = storage.num_pages[g]
+                tables[g, i, :n] = row
+        self.max_blocks = max_blocks
+
+        parts = [tokens.astype(np.int32), positions, seq_of, starts, kv_len, slots,
+                 np.asarray(want_rows, dtype=np.int32), tables.reshape(-1)]
+        sizes = [p.size for p in parts]
+        host = torch.from_numpy(np.concatenate(parts)).pin_memory() if device.type == "cuda" else torch.from_numpy(np.concatenate(parts))
+        dev = host.to(device, non_blocking=True)
+        views = torch.split(dev, sizes)
+        (self.token_ids, self.positions, self.seq_of_token, self.q_start, self.kv_len, self.slots,
+         self.want_rows, flat_tables) = views
+        self.block_tables = [flat_tables.view(n_groups, nseq, max_blocks)[g] for g in range(n_groups)] if n_groups else []
+        self._host = host          # keeps the pinned buffer alive until the copy has run
+        self._storage = storage
+
+    def cache_view(self, call: int):
+        return self._storage.view(call, self.block_tables)

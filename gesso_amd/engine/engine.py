@@ -1,0 +1,127 @@
+"""The engine: a model, its cache, and the one step function.
+
+``step(entries)`` runs exactly the tokens it is given, as one batch, from the cache that earlier
+steps left, and returns float32 logits at the wanted places, in the order of the entries and of
+their ``want`` lists.  Portions of prompts may stand beside single decoded tokens, cut anywhere.
+The reference runs one sequence per pass (a prefill pass of n rows, ``src/Inference/Inference.jl:2272-2530``,
+or one decode row, ``:3270-3383``); a mixed batch over several requests has no counterpart there.
+
+What happens when a pool is exhausted: ``step`` raises :class:`~gesso_amd.errors.OutOfPages`
+before it has changed anything; the scheduler decides what to do then.
+"""
+from __future__ import annotations
+
+from typing import Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheLayout, CacheManager
+from ..cache.storage import CacheStorage
+from ..config.registry import load_config
+from ..config.spec import ModelSpec
+from ..errors import InvalidPlan
+from ..models.model import Model, tensor_table, tied_aliases
+from ..parts.runtime import Runtime
+from ..weights.loader import load_tensors, random_tensors
+from .batch import StepContext, StepEntry, check_entries
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise InvalidPlan(f"dtype must be bfloat16 or float32, got {dtype!r}") from None
+
+
+class Engine:
+    def __init__(self, spec: ModelSpec, tensors, dtype, device="cuda:0", page_size: int = 16,
+                 num_pages: Optional[int] = None, max_tokens: Optional[int] = None, num_slots: int = 8,
+                 max_context: Optional[int] = None):
+        """``tensors``: ``file name -> tensor`` on the device, in the widths the loader chose.
+
+        The page pool holds ``num_pages`` pages per group, or enough for ``max_tokens`` tokens.
+        """
+        self.spec = spec
+        self.dtype = parse_dtype(dtype)
+        self.device = torch.device(device)
+        self.rt = Runtime(self.device, self.dtype)
+        self.model = Model(spec, self.rt)
+        self.model.bind(tensors)
+        self.page_size = int(page_size)
+        self.max_context = min(spec.max_position, max_context or spec.max_position)
+        if num_pages is None:
+            if max_tokens is None:
+                raise InvalidPlan("give the cache a size: num_pages or max_tokens")
+            num_pages = -(-int(max_tokens) // self.page_size)
+        needs = self.model.cache_needs()
+        layout = CacheLayout.plan(needs, [c.cache for c in spec.schedule])
+        self.manager = CacheManager(layout, self.page_size, int(num_pages), int(num_slots), self.max_context)
+        self.storage = CacheStorage(layout, self.page_size, int(num_pages), int(num_slots), self.dtype, self.device)
+        self.steps = 0
+
+    # ------------------------------------------------------------------ construction
+
+    @classmethod
+    def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        arch, cfg = load_config(model_dir)
+        spec = arch.to_spec(cfg)
+        mode = parse_dtype(dtype)
+        tensors = load_tensors(model_dir, tensor_table(spec), mode, device, aliases=tied_aliases(spec),
+                               ignored_suffixes=spec.ignored_tensors)
+        return cls(spec, tensors, mode, device, **kw)
+
+    @classmethod
+    def from_config(cls, config, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02, **kw) -> "Engine":
+        """Random weights drawn on the device (for measurements; a folder is written by ``write_model_folder``)."""
+        from ..config.registry import architecture_of
+        from ..weights.loader import held_dtype
+
+        spec = architecture_of(config.to_json()).to_spec(config)
+        mode = parse_dtype(dtype)
+        table = tensor_table(spec)
+        drawn = random_tensors(table, seed, torch.float32 if mode == torch.float32 else torch.bfloat16, device, std)
+        tensors = {name: t.to(held_dtype(t.dtype, table[name].role, mode)) for name, t in drawn.items()}
+        return cls(spec, tensors, mode, device, **kw)
+
+    # ------------------------------------------------------------------ requests
+
+    def add_request(self, rid: Hashable) -> None:
+        self.manager.admit(rid)
+
+    def finish_request(self, rid: Hashable) -> None:
+        self.manager.release(rid)
+
+    def has_request(self, rid: Hashable) -> bool:
+        return rid in self.manager.requests
+
+    def length(self, rid: Hashable) -> int:
+        return self.manager.get(rid).length
+
+    # ------------------------------------------------------------------ the step
+
+    def _zero_fresh_slots(self) -> None:
+        fresh = self.manager.fresh_slots
+        if not fresh:
+            return
+        slots = torch.tensor(fresh, dtype=torch.int32, device=self.device)
+        for states in self.storage.state.values():
+            for t in states.values():
+                self.rt.ops.zero_slots(t, slots)
+        fresh.clear()
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        if not entries:
+            return None
+        check_entries(entries, self.manager, self.spec.vocab)
+        self.manager.reserve_many([(e.rid, len(e.tokens)) for e in entries])
+        self._zero_fresh_slots()
+        ctx = StepContext(entries, self.manager, self.storage, self.spec.vocab, self.device)
+        logits = self.model.forward(ctx)
+        for e in entries:
+            self.manager.commit(e.rid, len(e.tokens))
+        self.steps += 1
+        return logits

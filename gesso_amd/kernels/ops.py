@@ -1,0 +1,261 @@
+"""Python faces of the HIP kernels: they check shapes and types on the host, then launch.
+
+Every function takes torch tensors that live on the GPU, launches on torch's current stream
+and returns its output tensor.  There is no other implementation behind these functions: a
+missing library or a refused size raises :class:`~gesso_amd.errors.KernelError`.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_double, c_float, c_int, c_long, c_void_p
+
+import torch
+
+from ..errors import KernelError
+from . import build as _build
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = _build.load()
+    return _lib
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, got {t.dtype}") from None
+
+
+def _p(t):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise KernelError(lib().gs_last_error().decode())
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must live on the GPU")
+            _need(t.is_contiguous(), "kernel operands must be contiguous")
+
+
+def _i32(t, n=None, what="index"):
+    _need(t.dtype == torch.int32, f"{what} must be int32, got {t.dtype}")
+    if n is not None:
+        _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} needed")
+
+
+# ---------------------------------------------------------------------- elementwise
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """``out[t] = table[ids[t]]`` as float32 ``(T, H)``."""
+    _dev(ids, table, out)
+    _i32(ids, what="token ids")
+    V, H = table.shape
+    T = ids.numel()
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.shape == (T, H), "embed: out must be float32 (T, H)")
+    _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), c_int(T), c_int(H), c_int(V), _stream()))
+    return out
+
+
+def add_rmsnorm(res: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_dtype, rows=None,
+                out: torch.Tensor = None) -> torch.Tensor:
+    """``res += delta`` (when given and no ``rows``), then ``out = rmsnorm(res) * weight``.
+
+    ``rows`` (int32) picks source rows; then ``res`` is not written.
+    """
+    _dev(res, delta, weight, rows, out)
+    _need(res.dtype == torch.float32 and res.dim() == 2, "add_rmsnorm: the residual stream is float32 (T, H)")
+    T, H = res.shape
+    _need(weight.dtype == torch.float32 and weight.shape == (H,), "add_rmsnorm: weight must be float32 (H,)")
+    if delta is not None:
+        _need(delta.shape == res.shape, "add_rmsnorm: delta must have the stream's shape")
+    n_out = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, what="rows")
+    if out is None:
+        out = torch.empty((n_out, H), dtype=out_dtype, device=res.device)
+    _need(out.shape == (n_out, H) and out.dtype == out_dtype, "add_rmsnorm: out has the wrong shape or type")
+    _check(lib().gs_add_rmsnorm(_p(res), _p(delta), c_int(_dt(delta) if delta is not None else _dt(out)),
+                                _p(weight), c_float(eps), _p(out), c_int(_dt(out)), _p(rows), c_int(n_out),
+                                c_int(H), _stream()))
+    return out
+
+
+def residual_add(res: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _dev(res, delta)
+    _need(res.dtype == torch.float32 and delta.shape == res.shape, "residual_add: shapes or types differ")
+    _check(lib().gs_residual_add(_p(res), _p(delta), c_int(_dt(delta)), c_long(res.numel()), _stream()))
+    return res
+
+
+def swiglu(x: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """``x (T, 2F)`` = gate | up  ->  ``silu(gate) * up (T, F)``."""
+    _dev(x, out)
+    T, F2 = x.shape
+    _need(F2 % 2 == 0, "swiglu: the input holds gate and up side by side")
+    F = F2 // 2
+    if out is None:
+        out = torch.empty((T, F), dtype=x.dtype, device=x.device)
+    _need(out.shape == (T, F) and out.dtype == x.dtype, "swiglu: out has the wrong shape or type")
+    _check(lib().gs_swiglu(_p(x), _p(out), c_int(_dt(x)), c_int(T), c_int(F), _stream()))
+    return out
+
+
+def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
+    _dev(t)
+    _need(t.dtype == torch.float32, "fill_f32 takes float32")
+    _check(lib().gs_fill_f32(_p(t), c_float(value), c_long(t.numel()), _stream()))
+    return t
+
+
+def zero_slots(state: torch.Tensor, slots: torch.Tensor) -> None:
+    """Zero ``state[slot]`` for each slot in ``slots`` (int32); ``state (num_slots, ...)`` float32."""
+    _dev(state, slots)
+    _i32(slots, what="slots")
+    _need(state.dtype == torch.float32, "state is float32")
+    row = state[0].numel()
+    _check(lib().gs_zero_slots(_p(state), _p(slots), c_int(slots.numel()), c_long(row), _stream()))
+
+
+# ---------------------------------------------------------------------- short convolution
+
+def short_conv(bcx, taps, bias, state, seq_of_token, q_start, slots, nseq: int, all_single: bool,
+               out: torch.Tensor = None) -> torch.Tensor:
+    """Gated short convolution over segments; ``state (num_slots, H, W-1)`` is read and advanced."""
+    _dev(bcx, taps, bias, state, seq_of_token, q_start, slots, out)
+    T, H3 = bcx.shape
+    _need(H3 % 3 == 0, "short_conv: bcx holds B, C, X side by side")
+    H = H3 // 3
+    W = taps.shape[1]
+    _need(taps.dtype == torch.float32 and taps.shape == (H, W), "short_conv: taps must be float32 (H, W)")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (H,)), "short_conv: bias must be float32 (H,)")
+    _need(state.dtype == torch.float32 and state.dim() == 3 and state.shape[1:] == (H, W - 1),
+          "short_conv: state must be float32 (slots, H, W-1)")
+    _i32(seq_of_token, T, "seq_of_token")
+    _i32(q_start, nseq + 1, "q_start")
+    _i32(slots, nseq, "slots")
+    if out is None:
+        out = torch.empty((T, H), dtype=bcx.dtype, device=bcx.device)
+    _need(out.shape == (T, H) and out.dtype == bcx.dtype, "short_conv: out has the wrong shape or type")
+    _check(lib().gs_short_conv(_p(bcx), c_int(_dt(bcx)), _p(taps), _p(bias), _p(state), _p(seq_of_token),
+                               _p(q_start), _p(slots), _p(out), c_int(T), c_int(nseq), c_int(H), c_int(W),
+                               c_int(1 if all_single else 0), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- attention
+
+def qknorm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, positions, seq_of_token, block_table,
+                   page_size, kcache, vcache, nh, nkv, d, write_kv=True) -> None:
+    """Head norm and rotation of q (in place) and k; k and v written into the pages."""
+    _dev(qkv, q_weight, k_weight, cos, sin, positions, seq_of_token, block_table, kcache, vcache)
+    T = qkv.shape[0]
+    _need(qkv.shape == (T, (nh + 2 * nkv) * d), "qknorm_rope_kv: qkv must be (T, (nh + 2 nkv) d)")
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "qknorm_rope_kv: head norm weight must be float32 (d,)")
+    max_pos = 0
+    if rotary_dim:
+        _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+              and cos.dim() == 2 and cos.shape[1] == rotary_dim // 2, "qknorm_rope_kv: tables must be float32 (P, rotary_dim/2)")
+        max_pos = cos.shape[0]
+    _i32(positions, T, "positions")
+    _i32(seq_of_token, T, "seq_of_token")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
+    _need(kcache.dtype == qkv.dtype and vcache.dtype == qkv.dtype, "cache and activations differ in type")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
+          "cache must be (pages, nkv, page_size, d)")
+    _check(lib().gs_qknorm_rope_kv(_p(qkv), c_int(_dt(qkv)), _p(q_weight), _p(k_weight), c_float(eps), _p(cos),
+                                   _p(sin), c_int(rotary_dim), c_int(max_pos), _p(positions), _p(seq_of_token),
+                                   _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
+                                   _p(vcache), c_int(T), c_int(nh), c_int(nkv), c_int(d),
+                                   c_int(1 if write_kv else 0), _stream()))
+
+
+def attention_generic(q, q_stride, kcache, vcache, positions, seq_of_token, block_table, page_size, window, scale,
+                      nh, nkv, d, ntok, out: torch.Tensor = None) -> torch.Tensor:
+    """Causal GQA over the paged cache, any sizes; ``q`` rows are ``q_stride`` apart."""
+    _dev(q, kcache, vcache, positions, seq_of_token, block_table, out)
+    _need(q.numel() >= (ntok - 1) * q_stride + nh * d if ntok else True, "attention: q is too small")
+    _need(kcache.dtype == q.dtype and vcache.dtype == q.dtype, "cache and activations differ in type")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
+          "cache must be (pages, nkv, page_size, d)")
+    _i32(positions, ntok, "positions")
+    _i32(seq_of_token, ntok, "seq_of_token")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
+    if out is None:
+        out = torch.empty((ntok, nh * d), dtype=q.dtype, device=q.device)
+    _need(out.shape == (ntok, nh * d) and out.dtype == q.dtype, "attention: out has the wrong shape or type")
+    _check(lib().gs_attention_generic(_p(q), c_int(q_stride), _p(kcache), _p(vcache), c_int(_dt(q)), _p(positions),
+                                      _p(seq_of_token), _p(block_table), c_int(block_table.shape[1]),
+                                      c_int(page_size), c_int(window or 0), c_float(scale), _p(out), c_int(ntok),
+                                      c_int(nh), c_int(nkv), c_int(d), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- matrix products
+
+def gemm_tiled(x: torch.Tensor, w: torch.Tensor, bias=None, out_dtype=None, out: torch.Tensor = None) -> torch.Tensor:
+    """``y = x @ w.T (+ bias)`` by float32 FMAs; any sizes, any mix of float32/bfloat16 storage."""
+    _dev(w, bias, out)
+    _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1, "gemm: x must be (M, K) with unit column stride")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape == (N, K), f"gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (N,)), "gemm: bias must be float32 (N,)")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or x.dtype, device=x.device)
+    _need(out.shape == (M, N) and out.stride(1) == 1, "gemm: out has the wrong shape")
+    _check(lib().gs_gemm_tiled(_p(x), c_int(_dt(x)), c_int(x.stride(0) if M > 1 else K), _p(w), c_int(_dt(w)),
+                               _p(bias), _p(out), c_int(_dt(out)), c_int(out.stride(0) if M > 1 else N), c_int(M),
+                               c_int(N), c_int(K), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- sampling
+
+def argmax_rows(logits: torch.Tensor):
+    """``(ids int32 (rows,), bad int32 (rows,))``: first maximum per row; bad = a non-finite logit."""
+    _dev(logits)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "argmax: logits are float32 (rows, V)")
+    rows, V = logits.shape
+    ids = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    bad = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    _check(lib().gs_argmax_rows(_p(logits), c_int(rows), c_int(V), _p(ids), _p(bad), _stream()))
+    return ids, bad
+
+
+def sample_temperature(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor):
+    """One id per row from ``softmax(logits / temperature)`` by inverse CDF at ``u`` (float64 each)."""
+    _dev(logits, temperature, u)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits are float32 (rows, V)")
+    rows, V = logits.shape
+    _need(temperature.dtype == torch.float64 and temperature.numel() == rows, "sample: temperature is float64 (rows,)")
+    _need(u.dtype == torch.float64 and u.numel() == rows, "sample: u is float64 (rows,)")
+    ids = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    bad = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    _check(lib().gs_sample_temperature(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(u), _p(ids), _p(bad),
+                                       _stream()))
+    return ids, bad

@@ -1,0 +1,87 @@
+"""The model: an embedding table, blocks run in the order the schedule gives, a final norm, a head.
+
+Built from a :class:`~gesso_amd.config.spec.ModelSpec` alone; which architecture the spec came
+from plays no part here.  ``tensor_table`` lists every tensor the model reads, by its name in
+the weight file, with the shape the spec implies (the reference's shape law,
+``src/Inference/materialize_architecture.jl:31-121``).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config.spec import ModelSpec
+from ..errors import ConfigError
+from ..parts.base import MATRIX, TABLE, TensorSpec, sub_tensors
+from ..parts.registry import build, part_class
+from ..parts.rmsnorm import ResidualStream
+
+
+def tensor_table(spec: ModelSpec) -> Dict[str, TensorSpec]:
+    """``file name -> TensorSpec`` of every tensor the model must find."""
+    out: Dict[str, TensorSpec] = {}
+
+    def put(name, ts):
+        if name in out and out[name] != ts:
+            raise ConfigError(f"tensor {name!r} is claimed twice with different shapes")
+        out[name] = ts
+
+    put(spec.names["embed"], TensorSpec((spec.vocab, spec.hidden), TABLE))
+    for local, ts in part_class("norm", spec.final_norm).tensor_specs(spec.final_norm).items():
+        put(spec.names["final_norm." + local], ts)
+    if not spec.tie_embeddings:
+        put(spec.names["head"], TensorSpec((spec.vocab, spec.hidden), MATRIX))
+    for i, b in enumerate(spec.blocks):
+        for local, ts in part_class("block", b).tensor_specs(b).items():
+            if local not in b.names:
+                raise ConfigError(f"block {i} has no file name for its tensor {local!r}")
+            put(b.names[local], ts)
+    return out
+
+
+def tied_aliases(spec: ModelSpec) -> Dict[str, str]:
+    """Tensors a file may hold though nobody reads them, if they equal another: a tied head."""
+    if spec.tie_embeddings and "head" in spec.names:
+        return {spec.names["head"]: spec.names["embed"]}
+    return {}
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, rt):
+        self.spec = spec
+        self.rt = rt
+        self.blocks = [build("block", b, rt) for b in spec.blocks]
+        self.final_norm = build("norm", spec.final_norm, rt)
+        self.embed = None
+        self.head = None
+
+    def cache_needs(self) -> List[Optional[object]]:
+        """For each entry of the schedule: what its own cache must hold (None: none, or it reads another's)."""
+        out = []
+        for call in self.spec.schedule:
+            b = self.spec.blocks[call.layer]
+            need = part_class("block", b).cache_need(b)
+            out.append(None if call.cache is not None else need)
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        s = self.spec
+        self.embed = tensors[s.names["embed"]]
+        self.head = self.embed if s.tie_embeddings else tensors[s.names["head"]]
+        self.final_norm.bind({k: tensors[s.names["final_norm." + k]]
+                              for k in part_class("norm", s.final_norm).tensor_specs(s.final_norm)})
+        for b, block in zip(s.blocks, self.blocks):
+            local = {k: tensors[b.names[k]] for k in part_class("block", b).tensor_specs(b)}
+            block.bind(local)
+
+    def forward(self, ctx) -> Optional[torch.Tensor]:
+        """Run the tokens of ``ctx`` through every scheduled block; float32 logits at ``ctx.want_rows``."""
+        ops = self.rt.ops
+        stream = ResidualStream(ops.embed(ctx.token_ids, self.embed))
+        for i, call in enumerate(self.spec.schedule):
+            self.blocks[call.layer].forward(stream, ctx, ctx.cache_view(i))
+        if ctx.n_want == 0:
+            return None
+        normed = self.final_norm.add_norm(stream, rows=ctx.want_rows)
+        return self.rt.linear(normed, self.head, out_dtype=torch.float32)

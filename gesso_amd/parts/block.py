@@ -1,0 +1,55 @@
+"""A block: how a mixer, a feed-forward and their norms are arranged around the residual stream.
+
+``prenorm``: ``h += mixer(norm_a(h)); h += ffn(norm_b(h))`` (reference
+``src/Inference/Inference.jl:270-363``).  Each add is folded into the norm that follows it;
+the model adds what is still pending after the last block.  Another arrangement (post-norms on
+sub-layer outputs, a parallel block) is another class registered under another kind.
+"""
+from __future__ import annotations
+
+from .base import Part, sub_tensors
+from .registry import build, part_class, register
+
+
+class PreNormBlock(Part):
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer_norm = build("norm", spec.mixer_norm, rt)
+        self.mixer = build("mixer", spec.mixer, rt)
+        self.ffn = self.ffn_norm = None
+        if spec.ffn is not None:
+            self.ffn_norm = build("norm", spec.ffn_norm, rt)
+            self.ffn = build("ffn", spec.ffn, rt)
+
+    @staticmethod
+    def tensor_specs(spec):
+        out = {}
+        roles = [("mixer_norm", "norm", spec.mixer_norm), ("mixer", "mixer", spec.mixer)]
+        if spec.ffn is not None:
+            roles += [("ffn_norm", "norm", spec.ffn_norm), ("ffn", "ffn", spec.ffn)]
+        for role, category, sub in roles:
+            for name, ts in part_class(category, sub).tensor_specs(sub).items():
+                out[f"{role}.{name}"] = ts
+        return out
+
+    @staticmethod
+    def cache_need(spec):
+        cls = part_class("mixer", spec.mixer)
+        return cls.cache_need(spec.mixer) if hasattr(cls, "cache_need") else None
+
+    def bind(self, tensors):
+        self.mixer_norm.bind(sub_tensors(tensors, "mixer_norm"))
+        self.mixer.bind(sub_tensors(tensors, "mixer"))
+        if self.ffn is not None:
+            self.ffn_norm.bind(sub_tensors(tensors, "ffn_norm"))
+            self.ffn.bind(sub_tensors(tensors, "ffn"))
+
+    def forward(self, stream, ctx, cache):
+        x = self.mixer_norm.add_norm(stream)
+        stream.pending = self.mixer.forward(x, ctx, cache)
+        if self.ffn is not None:
+            x = self.ffn_norm.add_norm(stream)
+            stream.pending = self.ffn.forward(x, ctx)
+
+
+register("block", "prenorm", PreNormBlock)

@@ -1,0 +1,56 @@
+"""What parts share at run time: device, activation type, kernels, matrix products.
+
+``Runtime.linear`` is the one place where a matrix product is chosen:
+
+* float32 anywhere (activations, weight or wanted output) -> the tiled FMA kernel, which is the
+  true 32-bit product and also takes mixed storage (a weight stored in 32-bit stays so);
+* bfloat16 x bfloat16 -> bfloat16: the hand-written skinny kernel for few rows, the vendor
+  library (through ``torch``) for many.  The reference hands every matrix product to the
+  vendor library as well (``ext/amdgpu_ops.jl:453-465``).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..errors import KernelError
+
+
+class Runtime:
+    def __init__(self, device, dtype: torch.dtype):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise KernelError(f"the engine runs in float32 or bfloat16, not {dtype}")
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise KernelError("the engine runs on the GPU only; there is no CPU path")
+        from ..kernels import ops
+        ops.lib()                      # fail here, loudly, if the extension is missing
+        self.ops = ops
+        self.dtype = dtype
+        self._shared = {}
+        # rows up to which the skinny bf16 kernel beats the library product (set by measurement)
+        self.skinny_rows = 0
+
+    def shared(self, key, make):
+        """One object per key for all parts (rotary tables and the like)."""
+        if key not in self._shared:
+            self._shared[key] = make()
+        return self._shared[key]
+
+    def linear(self, x: torch.Tensor, w: torch.Tensor, bias=None, out_dtype=None, out=None) -> torch.Tensor:
+        """``x @ w.T (+ bias)``; ``w (out, in)``."""
+        out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
+            if x.shape[0] <= self.skinny_rows:
+                return self.ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out)
+            if out_dtype == torch.bfloat16:
+                return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
+        return self.ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
+
+    def attention(self, q, q_stride, cache, ctx, window, scale, nh, nkv, d) -> torch.Tensor:
+        """Causal attention of this step's queries over the paged cache; ``(T, nh * d)``.
+
+        The generic kernel takes every size; faster kernels take over for the sizes and batch
+        shapes they are written for.
+        """
+        return self.ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
+                                          cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)
