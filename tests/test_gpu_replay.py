@@ -1,0 +1,68 @@
+"""bin/trace_run against the plain implementation, in the four ways of cutting the work.
+
+One process of trace_run per (configuration, precision) replays: each request alone and whole;
+most of it in one step and the last 32 tokens one by one; portions of changing size down to two
+tokens; and a mix of up to four live requests with a pool so small that pages are used again.
+Every fed position's logits are compared with the plain implementation's whole-sequence logits.
+
+Tolerances, set before the first run and never widened: float32 ``1e-4 * max(1, max|ref|)``
+(the reference's own device bound, ``test/test_amdgpu_lfm2.jl:34``); bfloat16 ``3e-2 * max(1, max|ref|)``:
+the matrix products round their inputs and outputs to 8 bits of mantissa (2^-9 relative per
+rounding) over up to six blocks of about ten roundings each.
+"""
+import numpy as np
+import pytest
+import torch
+
+import replay as R
+from tiny import CONFIGS, random_ids, write_tiny
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 1e-4, "bfloat16": 3e-2}
+
+# sequence lengths: the benchmark description's prompts plus generated tokens
+LENGTHS = {"A": (5 + 16, 17 + 16, 32 + 16, 70), "B": (1 + 24, 9 + 24, 40 + 24, 100 + 24), "C": (3, 50, 97)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return str(tmp_path_factory.mktemp("models"))
+
+
+def sequences(name):
+    cfg, seed = CONFIGS[name]
+    return {f"s{i}": random_ids(n, cfg.vocab_size, 100 * seed + i) for i, n in enumerate(LENGTHS[name])}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_replay_four_ways(name, dtype, folders, tmp_path):
+    cfg, _ = CONFIGS[name]
+    model_dir = write_tiny(folders, name, torch.float32 if dtype == "float32" else torch.bfloat16)
+    seqs = sequences(name)
+    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
+    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    tol = TOL[dtype] * scale
+
+    # the four ways in one process: names differ per way so that all requests are distinct
+    ways = {"whole": R.trace_whole, "tail": R.trace_tail, "portions": R.trace_portions,
+            "mixed": lambda s: R.trace_mixed(s, seed=7)}
+    big = R.Trace()
+    owner = []
+    for way, make in ways.items():
+        t = make({f"{way}.{k}": v for k, v in seqs.items()})
+        for rec, rows in zip(t.steps, t.rows):
+            rec = dict(rec, step=len(big.steps))
+            big.steps.append(rec)
+            big.rows.append(rows)
+            owner.append(way)
+        big.max_tokens = max(big.max_tokens, t.max_tokens)
+    got, rc = R.run_trace(model_dir, dtype, str(tmp_path / "out"), big, cfg.vocab_size)
+    assert rc == 0
+    for way in ways:
+        mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
+        assert {k: len(v) for k, v in mine.items()} == {k: len(v) for k, v in seqs.items()}, way
+        w, where = R.worst(mine, ref)
+        print(f"{name} {dtype} {way}: worst |diff| {w:.3e} at {where} (tolerance {tol:.3e}, scale {scale:.2f})")
+        assert w <= tol, f"{way}: first look at {where}"
