@@ -9,4 +9,10 @@ from .models import lfm2 as _lfm2  # noqa: F401  registers the architecture
 from .errors import (ConfigError, GessoError, InvalidPlan, KernelError, NumericalInstability, OutOfPages,
                      OutOfSlots, ResourceLimit, WeightError)
 
+from .engine.batch import StepEntry
+from .engine.engine import Engine
+from .engine.scheduler import Request, Scheduler
+from .engine.session import BatchRequest, BatchResult, Session, cancel, generate, run_batch
+from .sampling.sampler import Sampler
+
 __version__ = "0.1.0"

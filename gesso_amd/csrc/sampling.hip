@@ -142,3 +142,186 @@ extern "C" int gs_sample_temperature(const float* logits, int rows, int V, const
   GS_LAUNCH_CHECK("sample_temperature");
   return 0;
 }
+
+// ------------------------------------------------------------------ nucleus (top-p) sampling
+//
+// The reference orders ids by weight, descending and stable (ties keep id order), keeps the
+// shortest prefix whose mass reaches top_p * total, draws r = u * (mass kept) and returns the
+// first id of that order whose running sum exceeds r (src/Inference/sampling.jl:62-73).  No sort
+// is needed for that: positive float64 bit patterns order like their values, so a radix descent
+// over the pattern (eight passes of one byte, each a histogram of masses) finds the weight at
+// which a running sum in that order crosses a target, and the mass above it; ties at that weight
+// are then counted off in id order.  Done twice: for the nucleus' edge, and for the draw.
+// Sums run in another order than a sequential walk, so results differ from it by rounding only.
+//
+// wbuf (rows, V) float64 is scratch for the weights.
+
+struct Crossing {
+  unsigned long long bits;  // pattern of the weight at which the running sum crosses the target
+  double above;             // mass of all weights greater than it
+};
+
+// strict = 0: first running sum >= target; strict = 1: first running sum > target.
+__device__ Crossing radix_descend(const double* __restrict__ w, int V, double target, int strict, double* hmass,
+                                  int* hcount, Crossing* shared_out) {
+  unsigned long long prefix = 0;
+  double above = 0.0;
+  for (int pass = 0; pass < 8; ++pass) {
+    int shift = 56 - 8 * pass;
+    for (int b = threadIdx.x; b < 256; b += blockDim.x) {
+      hmass[b] = 0.0;
+      hcount[b] = 0;
+    }
+    __syncthreads();
+    unsigned long long himask = pass == 0 ? 0ull : (~0ull) << (shift + 8);
+    for (int j = threadIdx.x; j < V; j += blockDim.x) {
+      unsigned long long bits = (unsigned long long)__double_as_longlong(w[j]);
+      if ((bits & himask) == prefix) {
+        int b = (int)((bits >> shift) & 0xff);
+        atomicAdd(&hmass[b], w[j]);
+        atomicAdd(&hcount[b], 1);
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double acc = above;
+      int pick = -1, lowest = -1;
+      for (int b = 255; b >= 0; --b) {
+        if (hcount[b] == 0) continue;
+        lowest = b;
+        double next = acc + hmass[b];
+        if (strict ? (target < next) : (next >= target)) {
+          pick = b;
+          break;
+        }
+        acc = next;
+      }
+      if (pick < 0) {  // rounding left the target just above the whole mass: the last weight it is
+        pick = lowest;
+        acc -= hmass[lowest];
+      }
+      shared_out->bits = prefix | ((unsigned long long)pick << shift);
+      shared_out->above = acc;
+    }
+    __syncthreads();
+    prefix = shared_out->bits;
+    above = shared_out->above;
+    __syncthreads();
+  }
+  Crossing c;
+  c.bits = prefix;
+  c.above = above;
+  return c;
+}
+
+__global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
+                                    const double* __restrict__ top_p, const double* __restrict__ u,
+                                    double* __restrict__ wbuf, int* __restrict__ ids, int* __restrict__ bad) {
+  __shared__ double hmass[256];
+  __shared__ int hcount[256];
+  __shared__ Crossing cross;
+  __shared__ float redf[SAMP_THREADS / 64];
+  __shared__ double redd[SAMP_THREADS / 64];
+  __shared__ int bbad;
+  __shared__ int tie_before[SAMP_THREADS];
+  int row = blockIdx.x;
+  const float* x = logits + (size_t)row * V;
+  double* w = wbuf + (size_t)row * V;
+  int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+  if (tid == 0) bbad = 0;
+  __syncthreads();
+  float mx = -INFINITY;
+  int notfinite = 0;
+  for (int j = tid; j < V; j += blockDim.x) {
+    float v = x[j];
+    if (!(fabsf(v) <= 3.402823466e38f)) notfinite = 1;
+    mx = fmaxf(mx, v);
+  }
+  if (notfinite) atomicOr(&bbad, 1);
+  mx = wave_max(mx);
+  if (lane == 0) redf[wave] = mx;
+  __syncthreads();
+  mx = redf[0];
+  for (int i = 1; i < nw; ++i) mx = fmaxf(mx, redf[i]);
+  if (bbad) {
+    if (tid == 0) {
+      ids[row] = 0;
+      bad[row] = 1;
+    }
+    return;
+  }
+  double hi = (double)mx, T = temperature[row];
+  double s = 0.0;
+  for (int j = tid; j < V; j += blockDim.x) {
+    double wj = exp(((double)x[j] - hi) / T);
+    w[j] = wj;
+    s += wj;
+  }
+  s = wave_sum_f64(s);
+  if (lane == 0) redd[wave] = s;
+  __syncthreads();
+  double total = 0.0;
+  for (int i = 0; i < nw; ++i) total += redd[i];
+  __syncthreads();
+
+  // the nucleus' edge: weight tau at which the sorted running sum reaches top_p * total
+  double target = top_p[row] * total;
+  Crossing edge = radix_descend(w, V, target, 0, hmass, hcount, &cross);
+  double tau = __longlong_as_double((long long)edge.bits);
+  // ties at tau that belong to the nucleus: added one by one until the sum reaches the target
+  double need = target - edge.above;
+  long long ties_kept = tau > 0.0 ? (long long)ceil(need / tau) : 1;
+  if (ties_kept < 1) ties_kept = 1;
+  double cut = edge.above + (double)ties_kept * tau;
+
+  // the draw: first running sum above r = u * cut, in the same order
+  double r = u[row] * cut;
+  Crossing hit = radix_descend(w, V, r, 1, hmass, hcount, &cross);
+  double wv = __longlong_as_double((long long)hit.bits);
+  long long k = wv > 0.0 ? (long long)floor((r - hit.above) / wv) : 0;  // 0-based tie in id order
+  if (k < 0) k = 0;
+  // the k-th id, in id order, whose weight has exactly this pattern (the last such, if k overshoots)
+  int per = (V + blockDim.x - 1) / blockDim.x;
+  int j0 = tid * per, j1 = j0 + per < V ? j0 + per : V;
+  int cnt = 0;
+  for (int j = j0; j < j1; ++j) cnt += ((unsigned long long)__double_as_longlong(w[j]) == hit.bits);
+  tie_before[tid] = cnt;
+  __syncthreads();
+  if (tid == 0) {
+    long long seen = 0;
+    int pick = -1, last = -1;
+    for (int i = 0; i < (int)blockDim.x && pick < 0; ++i) {
+      if (tie_before[i] == 0) continue;
+      int a = i * per, b = a + per < V ? a + per : V;
+      if (seen + tie_before[i] <= k) {
+        seen += tie_before[i];
+        for (int j = b - 1; j >= a; --j)
+          if ((unsigned long long)__double_as_longlong(w[j]) == hit.bits) {
+            last = j;
+            break;
+          }
+        continue;
+      }
+      for (int j = a; j < b; ++j)
+        if ((unsigned long long)__double_as_longlong(w[j]) == hit.bits) {
+          last = j;
+          if (seen == k) {
+            pick = j;
+            break;
+          }
+          ++seen;
+        }
+    }
+    ids[row] = pick >= 0 ? pick : (last >= 0 ? last : 0);
+    bad[row] = 0;
+  }
+}
+
+extern "C" int gs_sample_top_p(const float* logits, int rows, int V, const double* temperature, const double* top_p,
+                               const double* u, double* wbuf, int* ids, int* bad, hipStream_t stream) {
+  GS_REQUIRE(rows >= 0 && V > 0, "sample_top_p: bad sizes rows=%d V=%d", rows, V);
+  if (rows == 0) return 0;
+  sample_top_p_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, u, wbuf, ids, bad);
+  GS_LAUNCH_CHECK("sample_top_p");
+  return 0;
+}

@@ -1,0 +1,269 @@
+"""The scheduler: which requests run in the next step, with which tokens.
+
+It admits requests in arrival order, cuts prompts into portions under a token budget, lets every
+request whose prompt is consumed decode one token per step, finishes requests and frees what
+they hold at once.  The reference has no counterpart above one sequence: its ``run_batch``
+prefills each request whole and then decodes them round-robin (``src/Runtime/Runtime.jl:98-182``),
+with passes bounded by ``GESSO_PREFILL_CHUNK`` (``src/Inference/Inference.jl:1765-1773``); the
+statuses a request ends with are the reference's (``Runtime.jl:167-178``): ``eos``, ``complete``,
+``cancelled``, ``failed``.
+
+Decisions, all tested without a GPU:
+
+* Order within a step: decoding requests first (one token each), then portions of prompts,
+  oldest request first, each at most ``chunk_size`` and together at most the step's budget of
+  ``max_num_batched_tokens``.
+* Admission: while fewer than ``max_num_seqs`` requests run, a slot is free and pages for the
+  first portion are free.
+* Out of pages: the request admitted last is preempted: everything it holds is given back, and
+  it returns to the front of the waiting line to be computed again from its prompt and the
+  tokens it has generated (its sampler state is kept, so a sampled request draws on where it
+  stopped).  This repeats until the step fits.  A request that does not fit into the empty pool
+  on its own ends as ``failed`` with :class:`~gesso_amd.errors.ResourceLimit`; nothing else stops.
+* The token that ends a request (an id in ``eos_ids``/``stop_ids``) is returned and never fed.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Callable, Deque, Hashable, List, Optional, Sequence, Tuple
+
+from ..errors import GessoError, InvalidPlan, OutOfPages, OutOfSlots, ResourceLimit
+from ..sampling.sampler import Sampler
+from .batch import StepEntry
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class Request:
+    rid: Hashable
+    prompt: List[int]
+    max_new_tokens: int = 8
+    sampler: Optional[Sampler] = None               # None = greedy
+    eos_ids: Tuple[int, ...] = ()
+    stop_ids: Tuple[int, ...] = ()
+    on_token: Optional[Callable[[int], Optional[bool]]] = None
+    # ---- state
+    output: List[int] = field(default_factory=list)
+    computed: int = 0                                # tokens whose state is in the cache
+    status: str = WAITING
+    finish_reason: Optional[str] = None              # eos | complete | cancelled | failed
+    error: Optional[Exception] = None
+    cancelled: bool = False
+    preemptions: int = 0
+
+    def __post_init__(self):
+        self.prompt = [int(t) for t in self.prompt]
+        if not self.prompt:
+            raise InvalidPlan("a request needs a prompt of at least one token")
+        if self.max_new_tokens < 0:
+            raise InvalidPlan("the token budget must be nonnegative")
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def pending(self) -> int:
+        """Tokens known and not yet in the cache."""
+        return len(self.prompt) + len(self.output) - self.computed
+
+
+@dataclass
+class Scheduled:
+    request: Request
+    start: int          # first token (index into request.tokens) fed in this step
+    count: int
+    samples: bool       # the portion reaches the last known token: its logits choose the next
+
+
+class Scheduler:
+    def __init__(self, executor, choose: Callable, max_num_seqs: int = 64, max_num_batched_tokens: int = 2048,
+                 chunk_size: int = 1024):
+        """``executor``: ``add_request``, ``finish_request``, ``step(entries) -> logits`` and ``manager``.
+
+        ``choose(logits, samplers) -> ids or exceptions``, one per row.
+        """
+        if max_num_seqs < 1 or max_num_batched_tokens < 1 or chunk_size < 1:
+            raise InvalidPlan("max_num_seqs, max_num_batched_tokens and chunk_size must be positive")
+        self.executor = executor
+        self.manager = executor.manager
+        self.choose = choose
+        self.max_num_seqs = max_num_seqs
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.chunk_size = chunk_size
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []          # in admission order
+        self.finished: List[Request] = []
+        self.stats = {"steps": 0, "preemptions": 0, "prompt_tokens": 0, "decode_tokens": 0}
+
+    # ------------------------------------------------------------------ requests
+
+    def add(self, request: Request) -> Request:
+        if request.max_new_tokens == 0:
+            self._finish(request, "complete", live=False)
+            return request
+        self.waiting.append(request)
+        return request
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def _finish(self, r: Request, reason: str, live: bool = True, error: Exception = None) -> None:
+        if live:
+            self.executor.finish_request(r.rid)
+            self.running.remove(r)
+        r.status, r.finish_reason, r.error = FINISHED, reason, error
+        self.finished.append(r)
+
+    def _preempt(self, r: Request) -> None:
+        self.executor.finish_request(r.rid)
+        self.running.remove(r)
+        r.status, r.computed = WAITING, 0
+        r.preemptions += 1
+        self.stats["preemptions"] += 1
+        self.waiting.appendleft(r)
+
+    # ------------------------------------------------------------------ one step's plan
+
+    def _portion(self, r: Request, budget: int) -> int:
+        return min(r.pending, self.chunk_size, budget)
+
+    def _pages_short(self, plan: List[Scheduled]) -> bool:
+        need = [0] * len(self.manager.pools)
+        for s in plan:
+            for g, n in enumerate(self.manager.pages_needed(s.request.rid, s.count)):
+                need[g] += n
+        return any(n > pool.n_free for n, pool in zip(need, self.manager.pools))
+
+    def schedule(self) -> List[Scheduled]:
+        """Decide the next step.  Admits, and preempts if pages run out; returns the plan (may be empty)."""
+        # requests cancelled from outside leave first
+        for r in [r for r in self.running if r.cancelled]:
+            self._finish(r, "cancelled")
+        for r in [r for r in self.waiting if r.cancelled]:
+            self.waiting.remove(r)
+            self._finish(r, "cancelled", live=False)
+
+        while True:
+            budget = self.max_num_batched_tokens
+            plan: List[Scheduled] = []
+            decoding = [r for r in self.running if r.pending == 1 and r.computed >= len(r.prompt)]
+            prefilling = [r for r in self.running if r not in decoding]
+            for r in decoding:
+                if budget < 1:
+                    break
+                plan.append(Scheduled(r, r.computed, 1, True))
+                budget -= 1
+            for r in prefilling:
+                n = self._portion(r, budget)
+                if n < 1:
+                    continue
+                plan.append(Scheduled(r, r.computed, n, n == r.pending))
+                budget -= n
+            if self._pages_short(plan):
+                victim = self.running[-1]
+                if len(self.running) == 1:
+                    # alone in the pool and still too large: nothing can be given back for it
+                    err = ResourceLimit(f"request {victim.rid!r} does not fit into the cache on its own",
+                                        tokens=victim.computed + victim.pending)
+                    self._finish(victim, "failed", error=err)
+                else:
+                    self._preempt(victim)
+                continue
+            # admission, oldest first, while the step has room
+            while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
+                r = self.waiting[0]
+                n = self._portion(r, budget)
+                if n < 1:
+                    break
+                if self.manager.needs_slot and self.manager.slot_pool.n_free < 1:
+                    break
+                try:
+                    self.executor.add_request(r.rid)
+                except OutOfSlots:
+                    break
+                trial = plan + [Scheduled(r, 0, n, n == r.pending)]
+                if self._pages_short(trial):
+                    self.executor.finish_request(r.rid)
+                    if not self.running:
+                        # the pool is empty and the first portion still does not fit: try a smaller one
+                        fit = self._largest_fit(r, n)
+                        if fit < 1:
+                            self.waiting.popleft()
+                            err = ResourceLimit(f"request {r.rid!r} does not fit into the cache on its own",
+                                                tokens=r.pending)
+                            self._finish(r, "failed", live=False, error=err)
+                            continue
+                        self.executor.add_request(r.rid)
+                        n = fit
+                        trial = plan + [Scheduled(r, 0, n, n == r.pending)]
+                    else:
+                        break
+                self.waiting.popleft()
+                r.status = RUNNING
+                self.running.append(r)
+                plan = trial
+                budget -= n
+            return plan
+
+    def _largest_fit(self, r: Request, n: int) -> int:
+        """Largest first portion of a request that the empty pool can hold."""
+        ps = self.manager.page_size
+        free = min((p.n_free for p in self.manager.pools), default=1 << 40)
+        return min(n, free * ps)
+
+    # ------------------------------------------------------------------ run
+
+    def step(self) -> Optional[List[Tuple[Request, int]]]:
+        """Plan, run and account one step; returns the (request, token) pairs it emitted, None if nothing ran."""
+        plan = self.schedule()
+        if not plan:
+            return None
+        entries = []
+        for s in plan:
+            toks = s.request.tokens[s.start:s.start + s.count]
+            entries.append(StepEntry(s.request.rid, toks, [s.count - 1] if s.samples else []))
+        try:
+            logits = self.executor.step(entries)
+        except OutOfPages:
+            raise AssertionError("the plan was checked against the pools and still ran out of pages")
+        self.stats["steps"] += 1
+        emitted: List[Tuple[Request, int]] = []
+        sampling = [s for s in plan if s.samples]
+        for s in plan:
+            r = s.request
+            r.computed += s.count
+            if s.start < len(r.prompt):
+                self.stats["prompt_tokens"] += min(s.count, len(r.prompt) - s.start)
+        if sampling:
+            picks = self.choose(logits, [s.request.sampler for s in sampling])
+            for s, tok in zip(sampling, picks):
+                r = s.request
+                if isinstance(tok, Exception):
+                    self._finish(r, "failed", error=tok)
+                    continue
+                r.output.append(int(tok))
+                self.stats["decode_tokens"] += 1
+                emitted.append((r, int(tok)))
+                keep = True
+                if r.on_token is not None:
+                    try:
+                        keep = r.on_token(int(tok)) is not False
+                    except Exception as err:    # a failing callback ends its own request only
+                        self._finish(r, "failed", error=err)
+                        continue
+                if tok in r.eos_ids or tok in r.stop_ids:
+                    self._finish(r, "eos")
+                elif len(r.output) >= r.max_new_tokens:
+                    self._finish(r, "complete")
+                elif not keep or r.cancelled:
+                    self._finish(r, "cancelled")
+        return emitted
+
+    def run(self) -> None:
+        while self.has_work():
+            if self.step() is None and self.has_work():
+                raise GessoError("the scheduler found nothing to run though requests are left",
+                                 waiting=len(self.waiting), running=len(self.running))

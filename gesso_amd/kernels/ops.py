@@ -259,3 +259,18 @@ def sample_temperature(logits: torch.Tensor, temperature: torch.Tensor, u: torch
     _check(lib().gs_sample_temperature(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(u), _p(ids), _p(bad),
                                        _stream()))
     return ids, bad
+
+
+def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, u: torch.Tensor):
+    """Nucleus sampling: one id per row from the shortest descending-weight prefix whose mass reaches ``top_p``."""
+    _dev(logits, temperature, top_p, u)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits are float32 (rows, V)")
+    rows, V = logits.shape
+    for name, t in (("temperature", temperature), ("top_p", top_p), ("u", u)):
+        _need(t.dtype == torch.float64 and t.numel() == rows, f"sample: {name} is float64 (rows,)")
+    wbuf = torch.empty((rows, V), dtype=torch.float64, device=logits.device)
+    ids = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    bad = torch.empty(rows, dtype=torch.int32, device=logits.device)
+    _check(lib().gs_sample_top_p(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(u), _p(wbuf),
+                                 _p(ids), _p(bad), _stream()))
+    return ids, bad

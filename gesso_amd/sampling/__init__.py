@@ -1,0 +1,1 @@
+from .sampler import Sampler, choose

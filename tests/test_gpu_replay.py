@@ -6,7 +6,7 @@ tokens; and a mix of up to four live requests with a pool so small that pages ar
 Every fed position's logits are compared with the plain implementation's whole-sequence logits.
 
 Tolerances, set before the first run and never widened: float32 ``1e-4 * max(1, max|ref|)``
-(the reference's own device bound, ``test/test_amdgpu_lfm2.jl:34``); bfloat16 ``3e-2 * max(1, max|ref|)``:
+(the reference's own device bound, ``test/test_amdgpu_lfm2.jl:34``); bfloat16 ``1.5e-2 * max(1, max|ref|)``:
 the matrix products round their inputs and outputs to 8 bits of mantissa (2^-9 relative per
 rounding) over up to six blocks of about ten roundings each.
 """
@@ -19,7 +19,7 @@ from tiny import CONFIGS, random_ids, write_tiny
 
 pytestmark = pytest.mark.gpu
 
-TOL = {"float32": 1e-4, "bfloat16": 3e-2}
+TOL = {"float32": 1e-4, "bfloat16": 1.5e-2}
 
 # sequence lengths: the benchmark description's prompts plus generated tokens
 LENGTHS = {"A": (5 + 16, 17 + 16, 32 + 16, 70), "B": (1 + 24, 9 + 24, 40 + 24, 100 + 24), "C": (3, 50, 97)}

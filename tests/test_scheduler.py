@@ -1,0 +1,237 @@
+"""The scheduler's decisions, on a host-only stand-in for the engine.
+
+The stand-in keeps the real cache manager, checks that every request's tokens arrive in order
+and exactly once since its (re)admission, and answers with logits that depend on all tokens a
+request has been fed, so that a request computed again after a preemption must come out the same.
+"""
+import numpy as np
+import pytest
+
+from gesso_amd.cache import CacheLayout, CacheManager
+from gesso_amd.engine.scheduler import Request, Scheduler
+from gesso_amd.errors import InvalidPlan, NumericalInstability, ResourceLimit
+from gesso_amd.parts.base import PagedKV, SlotState
+from gesso_amd.sampling.sampler import Sampler
+
+V = 50
+
+
+def next_token(tokens):
+    h = 7
+    for t in tokens:
+        h = (h * 31 + t + 1) % 1000003
+    return h % V
+
+
+class FakeEngine:
+    def __init__(self, num_pages=64, page_size=4, num_slots=8, max_length=256):
+        lay = CacheLayout.plan([SlotState((("history", (4, 2), "float32"),)), PagedKV(1, 16, None)], [None, None])
+        self.manager = CacheManager(lay, page_size, num_pages, num_slots, max_length)
+        self.fed = {}
+        self.batches = []
+
+    def add_request(self, rid):
+        self.manager.admit(rid)
+        self.fed[rid] = []
+
+    def finish_request(self, rid):
+        self.manager.release(rid)
+        del self.fed[rid]
+
+    def step(self, entries):
+        self.manager.reserve_many([(e.rid, len(e.tokens)) for e in entries])
+        rows = []
+        self.batches.append([(e.rid, len(e.tokens), list(e.want)) for e in entries])
+        for e in entries:
+            assert self.manager.get(e.rid).length == len(self.fed[e.rid])
+            for i, t in enumerate(e.tokens):
+                self.fed[e.rid].append(t)
+                if i in e.want:
+                    row = np.zeros(V, dtype=np.float32)
+                    row[next_token(self.fed[e.rid])] = 1.0
+                    rows.append(row)
+            self.manager.commit(e.rid, len(e.tokens))
+        self.manager.check()
+        return np.stack(rows) if rows else None
+
+
+def choose(logits, samplers):
+    out = []
+    for row, s in zip(logits, samplers):
+        if not np.isfinite(row).all():
+            out.append(NumericalInstability("non-finite logits"))
+        elif s is None:
+            out.append(int(np.argmax(row)))
+        else:
+            s.unit()
+            out.append(int(np.argmax(row)))
+    return out
+
+
+def expected(prompt, n, eos=()):
+    ids = list(prompt)
+    for _ in range(n):
+        t = next_token(ids)
+        ids.append(t)
+        if t in eos:
+            break
+    return ids
+
+
+def make(engine=None, **kw):
+    engine = engine or FakeEngine()
+    return engine, Scheduler(engine, choose, **kw)
+
+
+def test_single_request_chunks_then_decodes():
+    eng, s = make(chunk_size=5, max_num_batched_tokens=16)
+    r = s.add(Request("a", list(range(12)), max_new_tokens=3))
+    s.run()
+    assert r.tokens == expected(range(12), 3) and r.finish_reason == "complete"
+    # portions of at most 5; only the last portion of the prompt asks for logits; then single tokens
+    assert eng.batches == [[("a", 5, [])], [("a", 5, [])], [("a", 2, [1])], [("a", 1, [0])], [("a", 1, [0])]]
+    assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+    assert s.stats["prompt_tokens"] == 12 and s.stats["decode_tokens"] == 3
+
+
+def test_decodes_go_first_and_prompts_share_the_budget():
+    eng, s = make(chunk_size=8, max_num_batched_tokens=10)
+    a = s.add(Request("a", [1, 2, 3], max_new_tokens=6))
+    s.step()                                            # a's whole prompt
+    b = s.add(Request("b", list(range(20)), max_new_tokens=2))
+    c = s.add(Request("c", list(range(5)), max_new_tokens=2))
+    s.step()
+    # a decodes (1 token), b gets a portion of 8, c the one token the budget has left
+    assert eng.batches[-1] == [("a", 1, [0]), ("b", 8, []), ("c", 1, [])]
+    s.step()
+    assert eng.batches[-1] == [("a", 1, [0]), ("b", 8, []), ("c", 1, [])]
+    s.run()
+    for r, p in ((a, [1, 2, 3]), (b, range(20)), (c, range(5))):
+        assert r.tokens == expected(p, r.max_new_tokens)
+    assert sum(n for batch in eng.batches for _, n, _ in batch) == sum(len(r.tokens) - 1 for r in (a, b, c))
+    assert all(sum(n for _, n, _ in batch) <= 10 for batch in eng.batches)
+
+
+def test_max_num_seqs_and_slots_bound_admission():
+    eng, s = make(FakeEngine(num_slots=2), max_num_seqs=3)
+    rs = [s.add(Request(i, [i, i + 1], max_new_tokens=4)) for i in range(5)]
+    s.step()
+    assert len(s.running) == 2 and len(s.waiting) == 3           # two slots
+    s.run()
+    assert all(r.tokens == expected([i, i + 1], 4) for i, r in enumerate(rs))
+    eng2, s2 = make(FakeEngine(num_slots=8), max_num_seqs=3)
+    for i in range(5):
+        s2.add(Request(i, [i], max_new_tokens=2))
+    s2.step()
+    assert len(s2.running) == 3
+
+
+def test_eos_is_returned_and_not_fed():
+    prompt = [3, 4, 5]
+    full = expected(prompt, 6)
+    eos = full[5]                                          # the third new token
+    eng, s = make()
+    r = s.add(Request("a", prompt, max_new_tokens=6, eos_ids=(eos,)))
+    s.run()
+    assert r.tokens == full[:6] and r.finish_reason == "eos"
+    assert sum(n for b in eng.batches for _, n, _ in b) == 5   # 3 prompt tokens + 2 generated ones; the eos never
+    r2 = s.add(Request("b", prompt, max_new_tokens=6, stop_ids=(eos,)))
+    s.run()
+    assert r2.tokens == full[:6] and r2.finish_reason == "eos"
+
+
+def test_zero_budget_returns_the_prompt():
+    eng, s = make()
+    r = s.add(Request("a", [1, 2], max_new_tokens=0))
+    assert r.finish_reason == "complete" and r.tokens == [1, 2] and not s.has_work() and eng.batches == []
+    with pytest.raises(InvalidPlan):
+        Request("b", [], max_new_tokens=1)
+    with pytest.raises(InvalidPlan):
+        Request("b", [1], max_new_tokens=-1)
+
+
+def test_on_token_and_cancel():
+    eng, s = make()
+    seen = []
+    a = s.add(Request("a", [1], max_new_tokens=10, on_token=lambda t: (seen.append(t), len(seen) < 3)[1]))
+    b = s.add(Request("b", [2], max_new_tokens=10))
+    c = s.add(Request("c", [3], max_new_tokens=10))
+    c.cancelled = True                                     # cancelled before it ever ran
+    s.step(); s.step()
+    b.cancelled = True                                     # cancelled between tokens
+    s.run()
+    assert a.finish_reason == "cancelled" and len(a.output) == 3 and seen == a.output
+    assert b.finish_reason == "cancelled" and len(b.output) == 2
+    assert c.finish_reason == "cancelled" and c.output == []
+    assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+
+    def boom(t):
+        raise RuntimeError("callback failed")
+
+    d = s.add(Request("d", [4], max_new_tokens=5, on_token=boom))
+    e = s.add(Request("e", [5], max_new_tokens=5))
+    s.run()
+    assert d.finish_reason == "failed" and isinstance(d.error, RuntimeError)
+    assert e.finish_reason == "complete" and e.tokens == expected([5], 5)   # one request's failure is its own
+
+
+def test_out_of_pages_preempts_the_youngest_and_recomputes_it():
+    # 6 pages of 4 = 24 tokens; two requests that grow to 16 each cannot both stay
+    eng, s = make(FakeEngine(num_pages=6, page_size=4), chunk_size=8, max_num_batched_tokens=16)
+    a = s.add(Request("a", list(range(8)), max_new_tokens=8, sampler=Sampler(0.7, 1.0, 1)))
+    b = s.add(Request("b", list(range(10, 18)), max_new_tokens=8, sampler=Sampler(0.7, 1.0, 2)))
+    s.run()
+    assert s.stats["preemptions"] >= 1 and b.preemptions >= 1 and a.preemptions == 0
+    assert a.tokens == expected(range(8), 8) and b.tokens == expected(range(10, 18), 8)
+    # each sampler drew exactly once per token it emitted, preemption or not
+    ref = Sampler(0.7, 1.0, 2)
+    for _ in range(8):
+        ref.unit()
+    assert b.sampler.state == ref.state
+    assert eng.manager.stats()["pages_free"] == [6]
+    # the recomputation fed prompt and generated tokens again, from position 0
+    fed_b = [n for batch in eng.batches for rid, n, _ in batch if rid == "b"]
+    assert sum(fed_b) > len(b.tokens) - 1
+
+
+def test_a_request_larger_than_the_pool_fails_alone():
+    eng, s = make(FakeEngine(num_pages=3, page_size=4), chunk_size=8)
+    big = s.add(Request("big", list(range(20)), max_new_tokens=2))
+    ok = s.add(Request("ok", [1, 2, 3], max_new_tokens=2))
+    s.run()
+    assert big.finish_reason == "failed" and isinstance(big.error, ResourceLimit)
+    assert ok.finish_reason == "complete" and ok.tokens == expected([1, 2, 3], 2)
+    assert eng.manager.stats()["pages_free"] == [3] and eng.manager.stats()["slots_free"] == 8
+
+
+def test_a_bad_row_fails_its_request_only():
+    class Poisoned(FakeEngine):
+        def step(self, entries):
+            logits = super().step(entries)
+            if logits is not None and entries[0].rid == "bad":
+                logits[0, 3] = np.nan
+            return logits
+
+    eng, s = make(Poisoned())
+    bad = s.add(Request("bad", [1, 2], max_new_tokens=3))
+    good = s.add(Request("good", [5, 6], max_new_tokens=3))
+    s.run()
+    assert bad.finish_reason == "failed" and isinstance(bad.error, NumericalInstability) and bad.output == []
+    assert good.tokens == expected([5, 6], 3)
+    assert eng.manager.stats()["slots_free"] == 8
+
+
+def test_many_requests_under_pressure_all_come_out_right():
+    import random
+    rng = random.Random(3)
+    eng, s = make(FakeEngine(num_pages=20, page_size=4, num_slots=4), chunk_size=7, max_num_batched_tokens=12,
+                  max_num_seqs=4)
+    reqs = []
+    for i in range(25):
+        p = [rng.randrange(V) for _ in range(rng.randint(1, 30))]
+        reqs.append((p, s.add(Request(i, p, max_new_tokens=rng.randint(1, 12)))))
+    s.run()
+    for p, r in reqs:
+        assert r.finish_reason == "complete" and r.tokens == expected(p, r.max_new_tokens), r.rid
+    assert eng.manager.stats()["pages_free"] == [20] and eng.manager.stats()["slots_free"] == 4
+    assert s.stats["preemptions"] > 0
