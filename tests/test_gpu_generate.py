@@ -1,0 +1,222 @@
+"""Generation through the entry points, against the plain implementation's whole re-forwards."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_lfm2 as P
+from tiny import CONFIGS, STD, TINY_B, random_ids, write_tiny
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# the benchmark description's workloads for the two tiny configurations
+PROMPTS = {"A": (5, 17, 32), "B": (1, 9, 40, 100)}
+NEW = {"A": 16, "B": 24}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return str(tmp_path_factory.mktemp("gen"))
+
+
+@pytest.fixture(scope="module")
+def plain(folders):
+    out = {}
+    for name in ("A", "B"):
+        d = write_tiny(folders, name, torch.float32)
+        out[name] = (d, P.read_config(d), P.read_weights(d))
+    return out
+
+
+def prompts_of(name):
+    cfg, seed = CONFIGS[name]
+    return [random_ids(n, cfg.vocab_size, 1000 * seed + n) for n in PROMPTS[name]]
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_float32_equals_plain_greedy(plain, name):
+    from gesso_amd import Session
+    d, cfg, w = plain[name]
+    s = Session(d, dtype="float32", context_length=160, page_size=8 if name == "B" else 16, chunk_size=13 if name == "B" else 7)
+    prompts = prompts_of(name)
+    got = s.generate(prompts, max_new_tokens=NEW[name], eos_ids=())
+    for p, g in zip(prompts, got):
+        assert g == P.greedy(cfg, w, p, NEW[name])
+    # one prompt alone gives what it gave in the batch; nothing new returns the prompt
+    assert s.generate(prompts[1], max_new_tokens=NEW[name], eos_ids=()) == got[1]
+    assert s.generate(prompts[0], max_new_tokens=0) == prompts[0]
+    # the first new token is the argmax of the prompt's last row (test/test_reference_generate.jl:24-46)
+    lg = s.prefill(prompts[2])
+    assert lg.shape == (len(prompts[2]), cfg["V"]) and int(lg[-1].argmax()) == got[2][len(prompts[2])]
+    st = s.engine.manager.stats()
+    assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_bfloat16_picks_tokens_the_plain_logits_support(folders, name):
+    from gesso_amd import Session
+    d = write_tiny(folders, name, torch.bfloat16)
+    cfg, w = P.read_config(d), P.read_weights(d)
+    s = Session(d, dtype="bfloat16", context_length=160)
+    prompts = prompts_of(name)
+    got = s.generate(prompts, max_new_tokens=NEW[name], eos_ids=())
+    for p, g in zip(prompts, got):
+        ref = P.forward(cfg, w, g[:-1])
+        for i in range(len(p), len(g)):
+            row = ref[i - 1]
+            # the token chosen is the plain argmax, or as good as it within the bfloat16 tolerance of the logits
+            assert float(row.max() - row[g[i]]) <= 1.5e-2 * max(1.0, float(row.abs().max())), (i, g[i])
+
+
+def test_temperature_sampling_follows_the_plain_sampler(plain):
+    from gesso_amd import Sampler, Session
+    d, cfg, w = plain["B"]
+    s = Session(d, dtype="float32", context_length=160, page_size=8, chunk_size=13)
+    prompts = prompts_of("B")[:3]
+    got = s.generate(prompts, max_new_tokens=12, sampler=Sampler(temperature=0.8, seed=7), eos_ids=())
+    for i, (p, g) in enumerate(zip(prompts, got)):
+        ids, state = list(p), 7 + i
+        for _ in range(12):
+            tok, state = P.sample_id(P.forward(cfg, w, ids)[-1].tolist(), 0.8, 1.0, state)
+            ids.append(tok)
+        assert g == ids
+    # the same seed gives the same ids again; top_p narrows the choice and stays reproducible
+    again = s.generate(prompts, max_new_tokens=12, temperature=0.8, seed=7, eos_ids=())
+    assert again == got
+    one = s.generate(prompts[2], max_new_tokens=8, temperature=0.8, top_p=0.5, seed=3, eos_ids=())
+    ids, state = list(prompts[2]), 3
+    for _ in range(8):
+        tok, state = P.sample_id(P.forward(cfg, w, ids)[-1].tolist(), 0.8, 0.5, state)
+        ids.append(tok)
+    assert one == ids
+
+
+def test_long_decoding_and_first_tokens(plain):
+    """One token a step for 150 steps after a prompt of one token: every row against the plain model."""
+    from gesso_amd import Engine, StepEntry
+    d, cfg, w = plain["B"]
+    ids = random_ids(151, cfg["V"], 77)
+    ref = P.forward(cfg, w, ids).numpy()
+    eng = Engine.from_folder(d, dtype="float32", page_size=8, max_tokens=192)
+    eng.add_request("r")
+    rows = [eng.step([StepEntry("r", [t], [0])])[0].cpu().numpy() for t in ids]
+    got = np.stack(rows)
+    d_first = np.abs(got[:2] - ref[:2]).max()
+    assert d_first <= 1e-4 * max(1.0, np.abs(ref).max())            # the first tokens of a sequence
+    assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+    assert eng.length("r") == 151
+
+
+def test_a_far_token_decides(plain):
+    """The logits at the end depend on the first token through hundreds of cached keys."""
+    from gesso_amd import Engine, StepEntry
+    d, cfg, w = plain["A"]
+    ids = random_ids(240, cfg["V"], 5)
+    other = [(ids[0] + 1) % cfg["V"]] + ids[1:]
+    ref_a, ref_b = P.forward(cfg, w, ids)[-1].numpy(), P.forward(cfg, w, other)[-1].numpy()
+    assert np.abs(ref_a - ref_b).max() > 1e-3                        # it matters in the plain model ...
+    eng = Engine.from_folder(d, dtype="float32", page_size=16, max_tokens=512)
+    out = []
+    for name, seq in (("a", ids), ("b", other)):
+        eng.add_request(name)
+        eng.step([StepEntry(name, seq[:200], [])])
+        for t in seq[200:-1]:
+            eng.step([StepEntry(name, [t], [])])
+        out.append(eng.step([StepEntry(name, [seq[-1]], [0])])[0].cpu().numpy())
+    scale = max(1.0, np.abs(ref_a).max())
+    assert np.abs(out[0] - ref_a).max() <= 1e-4 * scale and np.abs(out[1] - ref_b).max() <= 1e-4 * scale
+
+
+def test_preemption_on_the_gpu_changes_no_output(plain):
+    from gesso_amd import Session
+    d, cfg, w = plain["A"]
+    prompts = [random_ids(n, cfg["V"], 50 + n) for n in (20, 33, 9, 41, 15)]
+    roomy = Session(d, dtype="float32", context_length=128, max_tokens=1024)
+    want = roomy.generate(prompts, max_new_tokens=20, eos_ids=())
+    tight = Session(d, dtype="float32", context_length=128, num_pages=7, page_size=16, chunk_size=16, max_num_seqs=3)
+    got = tight.generate(prompts, max_new_tokens=20, eos_ids=())
+    assert got == want
+    assert tight.last_stats["preemptions"] > 0
+    st = tight.engine.manager.stats()
+    assert st["pages_free"] == [7] and st["slots_free"] == st["slots_total"]
+
+
+def test_run_batch_statuses_and_cancel(plain):
+    from gesso_amd import BatchRequest, Session, cancel, run_batch
+    d, cfg, w = plain["B"]       # the untied model: its greedy tokens vary, so one of them can serve as the end
+    s = Session(d, dtype="float32", context_length=64)
+    p = random_ids(6, cfg["V"], 9)
+    full = P.greedy(cfg, w, p, 8)
+    new = full[6:]
+    # an id that ends a request: the first new token that has not occurred before among the new ones, after the first
+    k = next(i for i in range(1, 8) if new[i] not in new[:i])
+    s.eos_ids = (new[k],)
+
+    def until_eos(n):
+        out = []
+        for t in new[:n]:
+            out.append(t)
+            if t == new[k]:
+                break
+        return p + out
+
+    reqs = [BatchRequest(s, p, max_new_tokens=8), BatchRequest(s, p, max_new_tokens=1),
+            BatchRequest(s, p, max_new_tokens=8), BatchRequest(s, p[:3], max_new_tokens=0)]
+    seen = []
+
+    def on_token(i, tok):
+        seen.append((i, tok))
+        if i == 2:
+            cancel(reqs[2])
+
+    res = run_batch(reqs, on_token=on_token)
+    assert [r.status for r in res] == ["eos", "complete", "cancelled", "complete"]
+    assert res[0].ids == until_eos(8) and res[1].ids == p + new[:1] and res[2].ids == p + new[:1] and res[3].ids == p[:3]
+    assert [t for i, t in seen if i == 0] == res[0].ids[6:]
+    with pytest.raises(Exception):
+        BatchRequest(s, p, max_new_tokens=-1)
+
+
+def test_non_finite_logits_fail_their_request(folders):
+    from gesso_amd import BatchRequest, Session, run_batch
+    from gesso_amd.errors import InvalidPlan, NumericalInstability
+    d = write_tiny(folders, "A", torch.float32)
+    s = Session(d, dtype="float32", context_length=64)
+    s.engine.model.final_norm.weight[3] = float("nan")               # a planted NaN
+    res = run_batch([BatchRequest(s, [1, 2, 3], max_new_tokens=4)])
+    assert res[0].status == "failed" and isinstance(res[0].error, NumericalInstability) and res[0].ids == [1, 2, 3]
+    with pytest.raises(NumericalInstability):
+        s.generate([1, 2, 3], max_new_tokens=2)
+    with pytest.raises(InvalidPlan, match="outside the vocabulary"):
+        s.generate([1, 999999], max_new_tokens=2)
+    with pytest.raises(InvalidPlan, match="exceed the context"):
+        s.generate(list(range(60)), max_new_tokens=10)
+    st = s.engine.manager.stats()
+    assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+
+
+def test_random_weights_session_and_cli(tmp_path):
+    from gesso_amd import Session
+    s = Session(TINY_B, random_weights_seed=4, random_weights_std=STD, dtype="bfloat16", context_length=64)
+    a = s.generate([5, 6, 7], max_new_tokens=5, eos_ids=())
+    assert len(a) == 8 and a == s.generate([5, 6, 7], max_new_tokens=5, eos_ids=())
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    r = subprocess.run([sys.executable, "-m", "gesso_amd", "--check"], capture_output=True, text=True, env=env, cwd=ROOT)
+    assert r.returncode == 0 and "check ok" in r.stdout, r.stderr[-2000:]
+    d = write_tiny(str(tmp_path), "A", torch.float32)
+    r = subprocess.run([sys.executable, "-m", "gesso_amd", "--model", d, "--dtype", "float32", "--prompt-ids", "1,2,3",
+                        "--prompt-ids", "9 8", "--max-new-tokens", "4", "--n-ctx", "32", "--model-id", "tiny-a"],
+                       capture_output=True, text=True, env=env, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-2000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    cfg, w = P.read_config(d), P.read_weights(d)
+    assert out["model"] == "tiny-a" and out["ids"][0][:3] == [1, 2, 3] and len(out["ids"][1]) <= 6
+    assert out["ids"][0] == P.greedy(cfg, w, [1, 2, 3], 4)[:len(out["ids"][0])]
+    r = subprocess.run([sys.executable, "-m", "gesso_amd", "--model", d, "--gguf", "x"], capture_output=True, text=True,
+                       env=env, cwd=ROOT)
+    assert r.returncode != 0 and "unrecognized" in r.stderr

@@ -1,0 +1,363 @@
+"""Each HIP kernel alone against the plain implementation's function, at other sizes than the models'.
+
+Sizes are chosen off the kernels' tiles: widths below a wavefront, no multiples of the tile,
+one token, partially filled pages, head widths in steps of 16.  float32 results must agree to
+rounding of float32 sums; bfloat16 results to the rounding of their stored outputs.
+"""
+import math
+
+import pytest
+import torch
+
+import plain_lfm2 as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from gesso_amd.kernels import ops
+    ops.lib()
+    return ops
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def close(got, want, dtype, scale=1.0):
+    got = got.detach().double().cpu()
+    tol = (2e-6 if dtype == torch.float32 else 1e-2) * max(1.0, float(want.abs().max())) * scale
+    d = float((got - want).abs().max())
+    assert d <= tol, f"max |diff| {d:.3e} above {tol:.3e}"
+
+
+# ------------------------------------------------------------------ elementwise
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(ops, dtype):
+    table = torch.randn(37, 24, generator=gen(0)).to(dtype)
+    ids = torch.tensor([36, 0, 5, 5, 36], dtype=torch.int32)
+    out = ops.embed(ids.to(DEV), table.to(DEV))
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), P.embedding(table.float(), ids.tolist()))
+    bad = ops.embed(torch.tensor([1, 37, -1], dtype=torch.int32, device=DEV), table.to(DEV)).cpu()
+    assert torch.isfinite(bad[0]).all() and torch.isnan(bad[1]).all() and torch.isnan(bad[2]).all()
+
+
+@pytest.mark.parametrize("H", [24, 80, 2048, 3000])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm(ops, H, dtype):
+    g = gen(H)
+    T, eps = 5, 1e-4
+    res = torch.randn(T, H, generator=g) * 3
+    delta = torch.randn(T, H, generator=g).to(dtype)
+    w = 1 + 0.1 * torch.randn(H, generator=g)
+    r = res.clone().to(DEV)
+    out = ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, dtype)
+    summed = res.double() + delta.double()
+    close(r, summed, torch.float32)                       # the stream moved on, in float32
+    close(out, P.rmsnorm(summed, w.double(), eps), dtype)
+    # no delta: the stream stays
+    r2 = res.clone().to(DEV)
+    close(ops.add_rmsnorm(r2, None, w.to(DEV), eps, dtype), P.rmsnorm(res.double(), w.double(), eps), dtype)
+    assert torch.equal(r2.cpu(), res)
+    # gathered rows (one of them twice): the stream is left alone
+    rows = torch.tensor([4, 1, 4], dtype=torch.int32, device=DEV)
+    r3 = res.clone().to(DEV)
+    got = ops.add_rmsnorm(r3, delta.to(DEV), w.to(DEV), eps, dtype, rows=rows)
+    close(got, P.rmsnorm(summed, w.double(), eps)[[4, 1, 4]], dtype)
+    assert torch.equal(r3.cpu(), res)
+
+
+def test_rmsnorm_does_not_depend_on_the_batch(ops):
+    g = gen(1)
+    res = torch.randn(9, 200, generator=g)
+    w = torch.randn(200, generator=g)
+    whole = ops.add_rmsnorm(res.clone().to(DEV), None, w.to(DEV), 1e-5, torch.float32).cpu()
+    one = ops.add_rmsnorm(res[4:5].clone().to(DEV), None, w.to(DEV), 1e-5, torch.float32).cpu()
+    assert torch.equal(whole[4:5], one)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(ops, dtype):
+    x = (torch.randn(7, 200, generator=gen(2)) * 3).to(dtype)
+    got = ops.swiglu(x.to(DEV))
+    close(got, P.swiglu(x[:, :100].double(), x[:, 100:].double()), dtype)
+
+
+def test_residual_add_and_zero_slots(ops):
+    res = torch.randn(3, 10, generator=gen(3))
+    d = torch.randn(3, 10, generator=gen(4)).bfloat16()
+    assert torch.equal(ops.residual_add(res.clone().to(DEV), d.to(DEV)).cpu(), res + d.float())
+    state = torch.ones(5, 4, 2, device=DEV)
+    ops.zero_slots(state, torch.tensor([3, 1], dtype=torch.int32, device=DEV))
+    assert state.sum(dim=(1, 2)).tolist() == [8, 0, 8, 0, 8]
+
+
+# ------------------------------------------------------------------ short convolution
+
+@pytest.mark.parametrize("H,W,bias", [(13, 3, False), (200, 4, True), (64, 2, False), (1, 3, True)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_short_conv_segments_and_history(ops, H, W, bias, dtype):
+    g = gen(10 * H + W)
+    taps = torch.randn(H, W, generator=g)
+    b = torch.randn(H, generator=g) if bias else None
+    # three requests in slots 2, 0, 3 of a pool of 5; they advance in steps cut differently
+    lens = {2: [5, 1, 1, 4], 0: [1, 1, 7, 2], 3: [11]}
+    total = {s: sum(v) for s, v in lens.items()}
+    data = {s: torch.randn(total[s], 3 * H, generator=g).to(dtype) for s in lens}
+    want = {s: P.short_conv(data[s].double(), taps.double(), None if b is None else b.double()) for s in lens}
+    state = torch.full((5, H, W - 1), 7.0, device=DEV)
+    ops.zero_slots(state, torch.tensor(list(lens), dtype=torch.int32, device=DEV))
+    at = {s: 0 for s in lens}
+    got = {s: [] for s in lens}
+    for step in range(4):
+        live = [s for s in lens if step < len(lens[s])]
+        n = [lens[s][step] for s in live]
+        bcx = torch.cat([data[s][at[s]:at[s] + k] for s, k in zip(live, n)]).to(DEV)
+        q_start = torch.tensor([0] + list(torch.tensor(n).cumsum(0)), dtype=torch.int32, device=DEV)
+        seq_of = torch.cat([torch.full((k,), i, dtype=torch.int32) for i, k in enumerate(n)]).to(DEV)
+        slots = torch.tensor(live, dtype=torch.int32, device=DEV)
+        out = ops.short_conv(bcx, taps.to(DEV), None if b is None else b.to(DEV), state, seq_of, q_start, slots,
+                             len(live), all(k == 1 for k in n)).cpu()
+        o = 0
+        for s, k in zip(live, n):
+            got[s].append(out[o:o + k])
+            o += k
+            at[s] += k
+    for s in lens:
+        close(torch.cat(got[s]), want[s][0], dtype)
+        close(state[s], want[s][1], torch.float32)        # the history is float32 in both precisions
+    assert torch.equal(state[1].cpu(), torch.full((H, W - 1), 7.0)) and torch.equal(state[4].cpu(), torch.full((H, W - 1), 7.0))
+
+
+def test_short_conv_refuses_a_width_it_cannot_take(ops):
+    from gesso_amd.errors import KernelError
+    H, W = 4, 17
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelError, match="width 17"):
+        ops.short_conv(torch.zeros(1, 3 * H, device=DEV), torch.zeros(H, W, device=DEV), None,
+                       torch.zeros(1, H, W - 1, device=DEV), z, torch.tensor([0, 1], dtype=torch.int32, device=DEV), z, 1, True)
+
+
+# ------------------------------------------------------------------ head norm, rotation, cache write
+
+def rope_tables(rd, theta, n):
+    from gesso_amd.parts.rope import rope_tables as rt
+    cos, sin = rt(rd, theta, n)
+    return cos.to(DEV), sin.to(DEV)
+
+
+@pytest.mark.parametrize("nh,nkv,d,rd,norm", [(4, 2, 16, 16, True), (3, 1, 48, 48, True), (2, 2, 128, 64, False),
+                                               (5, 5, 80, 80, True), (8, 2, 256, 256, True)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_qknorm_rope_kv(ops, nh, nkv, d, rd, norm, dtype):
+    g = gen(nh * 100 + d)
+    ps, theta, eps = 8, 1e4, 1e-5
+    # two sequences: one continues at position 13 with 5 tokens (crossing a page edge at 16), one starts with 3
+    pos = [13, 14, 15, 16, 17, 0, 1, 2]
+    seq = [0] * 5 + [1] * 3
+    T = len(pos)
+    qkv = torch.randn(T, (nh + 2 * nkv) * d, generator=g).to(dtype)
+    qw = (1 + 0.1 * torch.randn(d, generator=g)) if norm else None
+    kw = (1 + 0.1 * torch.randn(d, generator=g)) if norm else None
+    table = torch.tensor([[5, 2, 7], [4, 0, 0]], dtype=torch.int32)     # pages out of order
+    kc = torch.zeros(9, nkv, ps, d, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    cos, sin = rope_tables(rd, theta, 64)
+    x = qkv.clone().to(DEV)
+    ops.qknorm_rope_kv(x, None if qw is None else qw.to(DEV), None if kw is None else kw.to(DEV), eps, cos, sin, rd,
+                       torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(seq, dtype=torch.int32, device=DEV),
+                       table.to(DEV), ps, kc, vc, nh, nkv, d)
+    src = qkv.double()
+    q = src[:, :nh * d].reshape(T, nh, d)
+    k = src[:, nh * d:(nh + nkv) * d].reshape(T, nkv, d)
+    v = src[:, (nh + nkv) * d:].reshape(T, nkv, d)
+    if norm:
+        q, k = P.rmsnorm(q, qw.double(), eps), P.rmsnorm(k, kw.double(), eps)
+
+    def rot(t):
+        out = t.clone()
+        out[..., :rd] = P.rope(t[..., :rd], pos, theta)
+        return out
+
+    q, k = rot(q), rot(k)
+    close(x[:, :nh * d].reshape(T, nh, d), q, dtype)
+    for t in range(T):
+        page = int(table[seq[t], pos[t] // ps])
+        close(kc[page, :, pos[t] % ps, :], k[t], dtype)
+        assert torch.equal(vc[page, :, pos[t] % ps, :].cpu(), qkv[t, (nh + nkv) * d:].reshape(nkv, d))
+    # nothing else was written: 8 rows of the cache are filled
+    assert int((kc.float().abs().sum(dim=(1, 3)) > 0).sum()) == T
+
+
+# ------------------------------------------------------------------ attention over pages
+
+def paged_case(ops, dtype, nh, nkv, d, ps, prefix, new, window, seed, boost=None):
+    """One sequence with `prefix` cached tokens and `new` queries, another short one beside it."""
+    g = gen(seed)
+    K = prefix + new
+    k = torch.randn(K, nkv, d, generator=g)
+    v = torch.randn(K, nkv, d, generator=g)
+    q = torch.randn(new, nh, d, generator=g)
+    if boost is not None:                       # make one far key stand out for the last query
+        far, amount = boost
+        q[-1] *= amount
+        k[far] = q[-1, ::nh // nkv][:nkv] / amount * 2.0
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    nblk = -(-K // ps)
+    pages = torch.randperm(nblk + 3, generator=g)[:nblk] + 1
+    kc = torch.randn(nblk + 5, nkv, ps, d, generator=g).to(dtype)      # garbage wherever nothing is written
+    vc = torch.randn(nblk + 5, nkv, ps, d, generator=g).to(dtype)
+    for u in range(K):
+        kc[pages[u // ps], :, u % ps] = k[u]
+        vc[pages[u // ps], :, u % ps] = v[u]
+    # the second sequence: 3 tokens on page 0
+    k2, v2, q2 = (torch.randn(3, n, d, generator=g).to(dtype) for n in (nkv, nkv, nh))
+    kc[0, :, :3] = k2.transpose(0, 1)
+    vc[0, :, :3] = v2.transpose(0, 1)
+    table = torch.zeros(2, nblk, dtype=torch.int32)
+    table[0] = pages.to(torch.int32)
+    qall = torch.cat([q.reshape(new, -1), q2.reshape(3, -1)])
+    positions = torch.tensor(list(range(prefix, K)) + [0, 1, 2], dtype=torch.int32)
+    seq = torch.tensor([0] * new + [1] * 3, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    got = ops.attention_generic(qall.to(DEV), nh * d, kc.to(DEV), vc.to(DEV), positions.to(DEV), seq.to(DEV),
+                                table.to(DEV), ps, window, scale, nh, nkv, d, new + 3)
+    want = torch.cat([P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(new, -1),
+                      P.causal_attention(q2.double(), k2.double(), v2.double(), window or 0).reshape(3, -1)])
+    return got, want
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 16, 8), (3, 1, 32, 16), (5, 5, 80, 4), (8, 2, 64, 16), (2, 1, 256, 16),
+                                         (6, 3, 48, 32)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_generic_chunk_over_prefix(ops, nh, nkv, d, ps, dtype):
+    got, want = paged_case(ops, dtype, nh, nkv, d, ps, prefix=37, new=9, window=None, seed=d + nh)
+    close(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_generic_decode_far_key_among_hundreds(ops, dtype):
+    # 700 cached keys, one query; key 3 (on the first page) carries most of the weight
+    got, want = paged_case(ops, dtype, 4, 2, 64, 16, prefix=700, new=1, window=None, seed=5, boost=(3, 4.0))
+    close(got, want, dtype)
+    got2, want2 = paged_case(ops, dtype, 4, 2, 64, 16, prefix=700, new=1, window=None, seed=5)
+    assert float((want - want2).abs().max()) > 0.1        # the far key did matter
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 64, 200])
+def test_attention_generic_window_edge(ops, window):
+    # a key just outside the window stands out: it must have no weight at all
+    prefix, new = 90, 4
+    far = prefix + new - 1 - window                        # first key the last query does not see
+    boost = (far, 4.0) if far >= 0 else None
+    got, want = paged_case(ops, torch.float32, 2, 1, 32, 16, prefix, new, window, seed=window, boost=boost)
+    close(got, want, torch.float32)
+
+
+def test_attention_refuses_what_it_cannot_take(ops):
+    from gesso_amd.errors import KernelError
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    kc = torch.zeros(1, 1, 16, 272, device=DEV)
+    with pytest.raises(KernelError, match="head width 272"):
+        ops.attention_generic(torch.zeros(1, 272, device=DEV), 272, kc, kc, z, z, z.reshape(1, 1), 16, None, 1.0, 1, 1, 272, 1)
+    kc = torch.zeros(1, 2, 16, 16, device=DEV)
+    with pytest.raises(KernelError, match="no multiple"):
+        ops.attention_generic(torch.zeros(1, 48, device=DEV), 48, kc, kc, z, z, z.reshape(1, 1), 16, None, 1.0, 3, 2, 16, 1)
+
+
+# ------------------------------------------------------------------ matrix products
+
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (70, 130, 100), (3, 301, 144), (64, 64, 16), (129, 65, 33)])
+@pytest.mark.parametrize("xd,wd,yd", [(torch.float32,) * 3, (torch.bfloat16,) * 3, (torch.bfloat16, torch.bfloat16, torch.float32),
+                                      (torch.bfloat16, torch.float32, torch.bfloat16)])
+def test_gemm_tiled(ops, M, N, K, xd, wd, yd):
+    g = gen(M + N + K)
+    x = torch.randn(M, K, generator=g).to(xd)
+    w = torch.randn(N, K, generator=g).to(wd)
+    b = torch.randn(N, generator=g)
+    want = x.double() @ w.double().T
+    close(ops.gemm_tiled(x.to(DEV), w.to(DEV), out_dtype=yd), want, yd, scale=math.sqrt(K) / 4 if yd == torch.float32 else 1)
+    close(ops.gemm_tiled(x.to(DEV), w.to(DEV), b.to(DEV), out_dtype=yd), want + b.double(), yd,
+          scale=math.sqrt(K) / 4 if yd == torch.float32 else 1)
+
+
+def test_gemm_rows_do_not_depend_on_the_batch(ops):
+    g = gen(9)
+    x = torch.randn(70, 100, generator=g).to(DEV)
+    w = torch.randn(130, 100, generator=g).to(DEV)
+    whole = ops.gemm_tiled(x, w)
+    assert torch.equal(whole[69:70], ops.gemm_tiled(x[69:70].contiguous(), w))
+    # a view with a row stride
+    wide = torch.randn(6, 250, generator=g).to(DEV)
+    assert torch.equal(ops.gemm_tiled(wide[:, 50:150], w), ops.gemm_tiled(wide[:, 50:150].contiguous(), w))
+
+
+# ------------------------------------------------------------------ choosing tokens
+
+def test_argmax_rows(ops):
+    x = torch.randn(6, 301, generator=gen(11))
+    x[1, 17] = x[1, 200] = 50.0                     # a tie: the lowest id wins
+    x[2, 300] = 60.0
+    x[3, 5] = float("nan")
+    x[4, 7] = float("inf")
+    x[5] = -1e30
+    ids, bad = ops.argmax_rows(x.to(DEV))
+    ids, bad = ids.tolist(), bad.tolist()
+    assert bad == [0, 0, 0, 1, 1, 0]
+    assert ids[0] == int(x[0].argmax()) and ids[1] == 17 and ids[2] == 300 and ids[5] == 0
+    big = torch.randn(3, 65536, generator=gen(12))
+    ids, bad = ops.argmax_rows(big.to(DEV))
+    assert ids.tolist() == big.argmax(1).tolist() and bad.tolist() == [0, 0, 0]
+
+
+@pytest.mark.parametrize("V,temp", [(301, 0.8), (512, 1.5), (5000, 0.3)])
+def test_sample_temperature_follows_the_plain_sampler(ops, V, temp):
+    rows = 24
+    logits = torch.randn(rows, V, generator=gen(V)) * 2
+    states = list(range(100, 100 + rows))
+    want, us = [], []
+    for r in range(rows):
+        i, _ = P.sample_id(logits[r].tolist(), temp, 1.0, states[r])
+        want.append(i)
+        us.append(P.splitmix64_unit(states[r])[1])
+    ids, bad = ops.sample_temperature(logits.to(DEV), torch.full((rows,), temp, dtype=torch.float64, device=DEV),
+                                      torch.tensor(us, dtype=torch.float64, device=DEV))
+    assert ids.tolist() == want and not any(bad.tolist())
+
+
+def test_sample_edges(ops):
+    x = torch.tensor([[0.0, 1.0, 2.0, 1.0]])
+    t = torch.tensor([1.0], dtype=torch.float64, device=DEV)
+    w = torch.exp(x[0].double() - 2.0)
+    cdf = (w.cumsum(0) / w.sum()).tolist()
+    for u, want in ((0.0, 0), (cdf[0] - 1e-9, 0), (cdf[0] + 1e-9, 1), (cdf[2] + 1e-9, 3), (1 - 1e-12, 3)):
+        ids, _ = ops.sample_temperature(x.to(DEV), t, torch.tensor([u], dtype=torch.float64, device=DEV))
+        assert ids.tolist() == [want], u
+    # a very low temperature is the argmax; a NaN row is flagged and emits nothing
+    ids, _ = ops.sample_temperature(x.to(DEV), t * 1e-3, torch.tensor([0.999], dtype=torch.float64, device=DEV))
+    assert ids.tolist() == [2]
+    x[0, 1] = float("nan")
+    _, bad = ops.sample_temperature(x.to(DEV), t, torch.tensor([0.5], dtype=torch.float64, device=DEV))
+    assert bad.tolist() == [1]
+
+
+@pytest.mark.parametrize("V,temp,top_p", [(301, 0.8, 0.9), (512, 1.0, 0.5), (5000, 1.2, 0.95), (64, 1.0, 0.1)])
+def test_sample_top_p_follows_the_plain_sampler(ops, V, temp, top_p):
+    rows = 24
+    logits = torch.randn(rows, V, generator=gen(V + 1)) * 2
+    logits[3, 10] = logits[3, 20] = logits[3, 5] = 6.0          # ties inside the nucleus keep id order
+    logits[4] = 0.0                                             # all equal: the nucleus is a prefix of the ids
+    want, us = [], []
+    for r in range(rows):
+        i, _ = P.sample_id(logits[r].tolist(), temp, top_p, 500 + r)
+        want.append(i)
+        us.append(P.splitmix64_unit(500 + r)[1])
+    ids, bad = ops.sample_top_p(logits.to(DEV), torch.full((rows,), temp, dtype=torch.float64, device=DEV),
+                                torch.full((rows,), top_p, dtype=torch.float64, device=DEV),
+                                torch.tensor(us, dtype=torch.float64, device=DEV))
+    assert ids.tolist() == want and not any(bad.tolist())

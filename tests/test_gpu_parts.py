@@ -1,0 +1,372 @@
+"""Each part alone against the plain implementation, and parts that the framework has never seen.
+
+A harness builds one part from its spec with random tensors, a cache for it and step contexts,
+and runs it whole and in portions.  The toy parts at the end (a mixer with a running state of
+its own, a position encoding with another table, a schedule that runs a block twice and lets a
+layer read another layer's cache) are defined here, registered here and stepped through the
+unchanged engine.
+"""
+import dataclasses
+import math
+
+import pytest
+import torch
+
+import plain_lfm2 as P
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def fw():
+    import gesso_amd
+    from gesso_amd.kernels import ops
+    ops.lib()
+    return gesso_amd
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+class Harness:
+    """One mixer (or any part with tensors) with its own cache, stepped like the engine steps it."""
+
+    def __init__(self, category, spec, dtype, seed=0, page_size=8, num_pages=32, std=0.2):
+        from gesso_amd.cache.manager import CacheLayout, CacheManager
+        from gesso_amd.cache.storage import CacheStorage
+        from gesso_amd.parts import Runtime, build, part_class
+        from gesso_amd.weights import random_tensors
+        from gesso_amd.weights.loader import held_dtype
+
+        self.rt = Runtime(DEV, dtype)
+        self.part = build(category, spec, self.rt)
+        cls = part_class(category, spec)
+        table = cls.tensor_specs(spec)
+        cpu = random_tensors(table, seed, dtype, std=std)
+        self.tensors = {k: v.double() for k, v in cpu.items()}
+        self.part.bind({k: v.to(DEV, held_dtype(v.dtype, table[k].role, dtype)) for k, v in cpu.items()})
+        need = cls.cache_need(spec) if hasattr(cls, "cache_need") else None
+        layout = CacheLayout.plan([need], [None])
+        self.manager = CacheManager(layout, page_size, num_pages, 4, 4096)
+        self.storage = CacheStorage(layout, page_size, num_pages, 4, dtype, DEV)
+        self.dtype = dtype
+
+    def ctx(self, entries):
+        from gesso_amd.engine.batch import StepContext, StepEntry
+        es = [StepEntry(rid, [0] * n, []) for rid, n in entries]
+        for e in es:
+            if e.rid not in self.manager.requests:
+                self.manager.admit(e.rid)
+        if self.manager.fresh_slots:
+            slots = torch.tensor(self.manager.fresh_slots, dtype=torch.int32, device=DEV)
+            for states in self.storage.state.values():
+                for t in states.values():
+                    self.rt.ops.zero_slots(t, slots)
+            self.manager.fresh_slots.clear()
+        self.manager.reserve_many([(e.rid, len(e.tokens)) for e in es])
+        c = StepContext(es, self.manager, self.storage, 1, DEV)
+        for e in es:
+            self.manager.commit(e.rid, len(e.tokens))
+        return c
+
+    def mixer(self, x, entries):
+        c = self.ctx(entries)
+        return self.part.forward(x.to(DEV, self.dtype), c, c.cache_view(0)).double().cpu()
+
+
+def tol(dtype, ref):
+    return (2e-5 if dtype == torch.float32 else 2e-2) * max(1.0, float(ref.abs().max()))
+
+
+# ------------------------------------------------------------------ norm, position, feed-forward
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(fw, dtype):
+    from gesso_amd.config import RMSNormSpec
+    from gesso_amd.parts import ResidualStream
+    h = Harness("norm", RMSNormSpec(size=144, eps=1e-4), dtype)
+    res = torch.randn(6, 144, generator=gen(0))
+    delta = torch.randn(6, 144, generator=gen(1)).to(dtype)
+    stream = ResidualStream(res.clone().to(DEV), delta.to(DEV))
+    out = h.part.add_norm(stream).double().cpu()
+    want = P.rmsnorm(res.double() + delta.double(), h.tensors["weight"], 1e-4)
+    assert float((out - want).abs().max()) <= tol(dtype, want)
+    assert stream.pending is None and torch.allclose(stream.res.cpu().double(), res.double() + delta.double(), atol=1e-6)
+
+
+def test_rope_part_tables(fw):
+    from gesso_amd.config import RopeSpec
+    from gesso_amd.parts import Runtime, build
+    rt = Runtime(DEV, torch.float32)
+    r = build("position", RopeSpec(head_dim=48, rotary_dim=32, theta=5e5, max_position=300), rt)
+    assert r.cos.shape == (300, 16) and r.rotary_dim == 32
+    for pos, i in ((0, 0), (1, 0), (299, 15), (77, 9)):
+        ang = pos * 5e5 ** (-2 * i / 32)
+        assert float(r.cos[pos, i]) == pytest.approx(math.cos(ang), abs=1e-7)
+        assert float(r.sin[pos, i]) == pytest.approx(math.sin(ang), abs=1e-7)
+    assert build("position", RopeSpec(head_dim=48, rotary_dim=32, theta=5e5, max_position=300), rt).cos is r.cos
+    with pytest.raises(ValueError):
+        build("position", RopeSpec(head_dim=16, rotary_dim=18, theta=1e4, max_position=8), rt)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_part(fw, dtype):
+    from gesso_amd.config import SwiGLUSpec
+    h = Harness("ffn", SwiGLUSpec(hidden=80, intermediate=100), dtype)
+    x = torch.randn(7, 80, generator=gen(2)).to(dtype)
+    got = h.part.forward(x.to(DEV), None).double().cpu()
+    w = h.tensors
+    want = P.linear(P.swiglu(P.linear(x.double(), w["w1.weight"]), P.linear(x.double(), w["w3.weight"])), w["w2.weight"])
+    assert float((got - want).abs().max()) <= tol(dtype, want)
+
+
+# ------------------------------------------------------------------ mixers
+
+@pytest.mark.parametrize("bias,W", [(False, 3), (True, 4), (False, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_short_conv_mixer_whole_and_in_portions(fw, dtype, bias, W):
+    from gesso_amd.config import ShortConvSpec
+    H = 48
+    h = Harness("mixer", ShortConvSpec(hidden=H, width=W, bias=bias), dtype, seed=W)
+    x = torch.randn(19, H, generator=gen(3)).to(dtype)
+    w = h.tensors
+    bcx = P.linear(x.double(), w["in_proj.weight"], w.get("in_proj.bias"))
+    mixed, _ = P.short_conv(bcx, w["conv.weight"].reshape(H, W), w.get("conv.bias"))
+    want = P.linear(mixed, w["out_proj.weight"], w.get("out_proj.bias"))
+    whole = h.mixer(x, [("a", 19)])
+    assert float((whole - want).abs().max()) <= tol(dtype, want)
+    parts, at = [], 0
+    for n in (5, 1, 1, 4, 2, 6):
+        parts.append(h.mixer(x[at:at + n], [("b", n)]))
+        at += n
+    cut = torch.cat(parts)
+    assert float((cut - want).abs().max()) <= tol(dtype, want)
+    if dtype == torch.float32:
+        assert torch.equal(cut, whole)             # the cut changes nothing at all
+
+
+@pytest.mark.parametrize("nh,nkv,d,window,qk", [(4, 2, 16, None, True), (3, 1, 32, None, True), (3, 3, 48, 7, False),
+                                                (8, 2, 64, None, True)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_mixer_whole_and_in_portions(fw, dtype, nh, nkv, d, window, qk):
+    from gesso_amd.config import AttentionSpec, RMSNormSpec, RopeSpec
+    H, eps, theta = nh * d, 1e-5, 1e4
+    spec = AttentionSpec(hidden=H, n_heads=nh, n_kv_heads=nkv, head_dim=d, window=window,
+                         position=RopeSpec(head_dim=d, rotary_dim=d, theta=theta, max_position=128),
+                         qk_norm=RMSNormSpec(size=d, eps=eps) if qk else None)
+    h = Harness("mixer", spec, dtype, seed=d, std=1.0 / math.sqrt(H))
+    T = 29
+    x = torch.randn(T, H, generator=gen(4)).to(dtype)
+    w = h.tensors
+    q = P.linear(x.double(), w["q_proj.weight"]).reshape(T, nh, d)
+    k = P.linear(x.double(), w["k_proj.weight"]).reshape(T, nkv, d)
+    v = P.linear(x.double(), w["v_proj.weight"]).reshape(T, nkv, d)
+    if qk:
+        q, k = P.rmsnorm(q, w["q_norm.weight"], eps), P.rmsnorm(k, w["k_norm.weight"], eps)
+    q, k = P.rope(q, range(T), theta), P.rope(k, range(T), theta)
+    want = P.linear(P.causal_attention(q, k, v, window or 0).reshape(T, H), w["out_proj.weight"])
+    whole = h.mixer(x, [("a", T)])
+    assert float((whole - want).abs().max()) <= tol(dtype, want)
+    parts, at = [], 0
+    for n in (7, 1, 9, 2, 1, 1, 8):
+        parts.append(h.mixer(x[at:at + n], [("b", n)]))
+        at += n
+    cut = torch.cat(parts)
+    assert float((cut - want).abs().max()) <= tol(dtype, want)
+    if dtype == torch.float32:
+        assert torch.equal(cut, whole)
+    if window:
+        # the windowed group gave pages back as it went: 29 tokens, window 7, pages of 8
+        held = [p for p in h.manager.get("b").tables[0] if p >= 0]
+        assert len(held) <= 2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_alone(fw, dtype):
+    from gesso_amd.config import BlockSpec, RMSNormSpec, ShortConvSpec, SwiGLUSpec
+    from gesso_amd.parts import ResidualStream
+    H = 32
+    spec = BlockSpec(mixer=ShortConvSpec(hidden=H, width=3), mixer_norm=RMSNormSpec(H, 1e-5),
+                     ffn=SwiGLUSpec(hidden=H, intermediate=40), ffn_norm=RMSNormSpec(H, 1e-5))
+    h = Harness("block", spec, dtype, std=0.2)
+    x = torch.randn(9, H, generator=gen(5))
+    w = {"p." + {"mixer_norm.weight": "operator_norm.weight", "ffn_norm.weight": "ffn_norm.weight"}.get(k, k)
+         .replace("mixer.", "conv.").replace("ffn.w", "feed_forward.w"): v for k, v in h.tensors.items()}
+    hh, _ = P.conv_block(x.double(), w, "p.", 1e-5)
+    want = P.feed_forward_block(hh, w, "p.", 1e-5)
+    c = h.ctx([("a", 9)])
+    stream = ResidualStream(x.clone().to(DEV))
+    h.part.forward(stream, c, c.cache_view(0))
+    got = stream.res.double().cpu() + stream.pending.double().cpu()
+    assert float((got - want).abs().max()) <= tol(dtype, want)
+
+
+# ------------------------------------------------------------------ parts the framework has never seen
+
+@dataclasses.dataclass(frozen=True)
+class DecaySpec:
+    hidden: int
+    decay: float
+    kind: str = "toy_decay"
+
+
+def register_toys():
+    from gesso_amd.parts import MATRIX, Part, SlotState, TensorSpec, register
+
+    class DecayMixer(Part):
+        """s_t = decay * s_{t-1} + x_t W^T, output s_t: a running state per request, of fixed size."""
+
+        @staticmethod
+        def tensor_specs(spec):
+            return {"proj.weight": TensorSpec((spec.hidden, spec.hidden), MATRIX)}
+
+        @staticmethod
+        def cache_need(spec):
+            return SlotState((("running", (spec.hidden,), "float32"),))
+
+        def bind(self, tensors):
+            self.w = tensors["proj.weight"]
+
+        def forward(self, x, ctx, cache):
+            y = self.rt.linear(x, self.w).float()
+            state = cache.state["running"]
+            out = torch.empty_like(y)
+            slots = ctx.slots.tolist()
+            at = 0
+            for slot, n in zip(slots, ctx.q_lens):
+                s = state[slot]
+                for t in range(at, at + n):
+                    s = self.spec.decay * s + y[t]
+                    out[t] = s
+                state[slot] = s
+                at += n
+            return out.to(x.dtype)
+
+    class ScaledRope(Part):
+        """Another position encoding: angles divided by a factor; the same three attributes."""
+
+        def __init__(self, spec, rt):
+            super().__init__(spec, rt)
+            from gesso_amd.parts.rope import rope_tables
+            cos, sin = rope_tables(spec.rotary_dim, spec.theta, spec.max_position * 4)
+            self.rotary_dim = spec.rotary_dim
+            self.cos = cos[::4].contiguous().to(rt.device)      # position p rotates by the angle of p / ... 4 p
+            self.sin = sin[::4].contiguous().to(rt.device)
+
+    register("mixer", "toy_decay", DecayMixer, replace=True)
+    register("position", "toy_scaled_rope", ScaledRope, replace=True)
+
+
+def toy_spec():
+    from gesso_amd.config import AttentionSpec, BlockSpec, LayerCall, ModelSpec, RMSNormSpec, RopeSpec, SwiGLUSpec
+    H, V = 32, 40
+    norm = RMSNormSpec(H, 1e-5)
+    pos = dataclasses.replace(RopeSpec(head_dim=16, rotary_dim=16, theta=1e4, max_position=64), kind="toy_scaled_rope")
+    attn = AttentionSpec(hidden=H, n_heads=2, n_kv_heads=1, head_dim=16, position=pos, qk_norm=None)
+    ffn = SwiGLUSpec(hidden=H, intermediate=24)
+
+    def names(i, mixer_names):
+        n = {"mixer_norm.weight": f"L{i}.n1", "ffn_norm.weight": f"L{i}.n2", "ffn.w1.weight": f"L{i}.w1",
+             "ffn.w3.weight": f"L{i}.w3", "ffn.w2.weight": f"L{i}.w2"}
+        n.update({f"mixer.{k}": f"L{i}.{k}" for k in mixer_names})
+        return n
+
+    attn_names = ["q_proj.weight", "k_proj.weight", "v_proj.weight", "out_proj.weight"]
+    blocks = (BlockSpec(DecaySpec(H, 0.5), norm, ffn, norm, names(0, ["proj.weight"])),
+              BlockSpec(attn, norm, ffn, norm, names(1, attn_names)),
+              BlockSpec(attn, norm, None, None, {k: v for k, v in names(2, attn_names).items() if not k.startswith("ffn")}))
+    # block 0 runs twice (two states of its own); the last call reads the cache that call 1 wrote
+    schedule = (LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(2, cache=1))
+    return ModelSpec(architecture="ToyForTests", hidden=H, vocab=V, blocks=blocks, schedule=schedule, final_norm=norm,
+                     tie_embeddings=True, max_position=64, names={"embed": "emb", "final_norm.weight": "fn", "head": "head"})
+
+
+def toy_plain(w, ids):
+    """The toy model by hand, whole sequence, float64."""
+    T = len(ids)
+    h = P.embedding(w["emb"], ids)
+    eps = 1e-5
+
+    def decay_block(h, i):
+        y = P.linear(P.rmsnorm(h, w[f"L{i}.n1"], eps), w[f"L{i}.proj.weight"])
+        s, out = torch.zeros(h.shape[1], dtype=h.dtype), []
+        for t in range(T):
+            s = 0.5 * s + y[t]
+            out.append(s)
+        return h + torch.stack(out)
+
+    def ffn(h, i):
+        n = P.rmsnorm(h, w[f"L{i}.n2"], eps)
+        return h + P.linear(P.swiglu(P.linear(n, w[f"L{i}.w1"]), P.linear(n, w[f"L{i}.w3"])), w[f"L{i}.w2"])
+
+    def qkv(h, i):
+        n = P.rmsnorm(h, w[f"L{i}.n1"], eps)
+        q = P.linear(n, w[f"L{i}.q_proj.weight"]).reshape(T, 2, 16)
+        k = P.linear(n, w[f"L{i}.k_proj.weight"]).reshape(T, 1, 16)
+        v = P.linear(n, w[f"L{i}.v_proj.weight"]).reshape(T, 1, 16)
+        pos = [4 * t for t in range(T)]                      # the scaled encoding: table row p is angle of 4 p
+        return P.rope(q, pos, 1e4), P.rope(k, pos, 1e4), v
+
+    h = ffn(decay_block(h, 0), 0)
+    q1, k1, v1 = qkv(h, 1)
+    h = ffn(h + P.linear(P.causal_attention(q1, k1, v1).reshape(T, 32), w["L1.out_proj.weight"]), 1)
+    h = ffn(decay_block(h, 0), 0)
+    q2, _, _ = qkv(h, 2)                                     # its own queries over layer 1's keys and values
+    h = h + P.linear(P.causal_attention(q2, k1, v1).reshape(T, 32), w["L2.out_proj.weight"])
+    return P.linear(P.rmsnorm(h, w["fn"], eps), w["emb"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_parts_register_build_and_step(fw, dtype):
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.models.model import tensor_table
+    from gesso_amd.parts import unregister
+    from gesso_amd.weights import random_tensors
+    from gesso_amd.weights.loader import held_dtype
+
+    register_toys()
+    try:
+        spec = toy_spec()
+        table = tensor_table(spec)
+        assert "L0.proj.weight" in table and "L2.w1" not in table
+        cpu = random_tensors(table, 3, dtype, std=0.2)
+        eng = Engine(spec, {k: v.to(DEV, held_dtype(v.dtype, table[k].role, dtype)) for k, v in cpu.items()}, dtype,
+                     DEV, page_size=4, num_pages=24, num_slots=3)
+        lay = eng.manager.layout
+        assert len(lay.paged) == 1 and lay.paged[0].members == (1,) and [m.call for m in lay.slots] == [0, 2]
+        assert lay.source_of_call[3] == 1
+        ids = {"a": [3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7], "b": [2, 7, 1, 8, 2, 8, 1, 8, 2, 8, 4]}
+        w64 = {k: v.double() for k, v in cpu.items()}
+        want = {k: toy_plain(w64, v) for k, v in ids.items()}
+        t = (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, max(float(x.abs().max()) for x in want.values()))
+        # whole
+        for k, v in ids.items():
+            eng.add_request(k)
+            got = eng.step([StepEntry(k, v, list(range(len(v))))]).double().cpu()
+            eng.finish_request(k)
+            assert float((got - want[k]).abs().max()) <= t, k
+        # mixed and cut: a in portions 5, 1, 1, 7 beside b in 3, 6, 1, 1
+        eng.add_request("a"); eng.add_request("b")
+        got = {"a": [], "b": []}
+        cuts = {"a": [5, 1, 1, 7], "b": [3, 6, 1, 1]}
+        at = {"a": 0, "b": 0}
+        for s in range(4):
+            entries = []
+            for k in ("a", "b"):
+                n = cuts[k][s]
+                entries.append(StepEntry(k, ids[k][at[k]:at[k] + n], list(range(n))))
+                at[k] += n
+            lg = eng.step(entries).double().cpu()
+            o = 0
+            for e in entries:
+                got[e.rid].append(lg[o:o + len(e.tokens)])
+                o += len(e.tokens)
+        for k in ids:
+            assert float((torch.cat(got[k]) - want[k]).abs().max()) <= t, k
+        eng.finish_request("a"); eng.finish_request("b")
+        assert eng.manager.stats()["pages_free"] == [24] and eng.manager.stats()["slots_free"] == 3
+    finally:
+        unregister("mixer", "toy_decay")
+        unregister("position", "toy_scaled_rope")

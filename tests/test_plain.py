@@ -14,7 +14,15 @@ import torch.nn.functional as F
 import plain_lfm2 as P
 from tiny import CONFIGS, random_ids, write_tiny
 
-torch.set_default_dtype(torch.float64)
+
+
+@pytest.fixture(autouse=True)
+def float64_by_default():
+    """The plain implementation is exercised in float64; the default is put back after each test."""
+    before = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float64)
+    yield
+    torch.set_default_dtype(before)
 
 
 # ------------------------------------------------------------------ vectors of the reference's tests
