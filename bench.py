@@ -1,0 +1,190 @@
+"""Decode and prefill throughput of LFM2-1.2B sizes on one MI355X, with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch: every live request gets its next token (the
+model's forward from the cache, the head, and greedy choice of the token that is fed back).
+The default run: 16 layers of the 1.2B sizes, bfloat16, batch 8, 512-token random prompts,
+context 4,096 with 16-token pages.  Prints one JSON line; for more than one GPU it prints
+one line that says so and exits with 2 (this engine runs on one GPU).
+
+Roofline of the decode step: the bytes it has to read (every weight it uses once, the keys and
+values of the live requests, their convolution state) over its time, against 8 TB/s.  Prefill:
+2,048 tokens of one prompt; its flops over its time against 2.5 PFLOP/s (bfloat16 dense).
+"""
+import argparse
+import json
+import sys
+import time
+
+import torch
+
+HBM_GBPS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def model_config():
+    from gesso_amd.config import Lfm2Config
+    return Lfm2Config.from_dict({
+        "architectures": ["Lfm2ForCausalLM"], "vocab_size": 65536, "hidden_size": 2048, "num_hidden_layers": 16,
+        "num_attention_heads": 32, "num_key_value_heads": 8, "full_attn_idxs": [2, 5, 8, 10, 12, 14],
+        "conv_L_cache": 3, "conv_bias": False, "block_ff_dim": 12288, "block_auto_adjust_ff_dim": True,
+        "block_multiple_of": 256, "block_ffn_dim_multiplier": 1.0, "norm_eps": 1e-5, "rope_theta": 1000000.0,
+        "tie_word_embeddings": True, "max_position_embeddings": 4096})
+
+
+def weight_bytes(engine) -> int:
+    """Bytes of every weight a decode step reads once (the tied table counts once: it is the head)."""
+    seen, n = set(), 0
+    m = engine.model
+    tensors = [m.head, m.final_norm.weight]
+    for b in m.blocks:
+        for part in (b.mixer_norm, b.mixer, b.ffn_norm, b.ffn):
+            tensors += [v for v in vars(part).values() if isinstance(v, torch.Tensor)]
+    for t in tensors:
+        if t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            n += t.numel() * t.element_size()
+    return n
+
+
+def step_flops(cfg, tokens: int, attn_pairs: int, rows_out: int) -> float:
+    """Multiply-adds x 2 of one step: projections over `tokens`, attention over visible (query, key) pairs."""
+    H, F, d = cfg.hidden_size, cfg.intermediate_size, cfg.head_dim
+    nh, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
+    n_attn = sum(t == "full_attention" for t in cfg.layer_types)
+    n_conv = cfg.num_hidden_layers - n_attn
+    per_tok = n_conv * (3 * H * H + H * H) + n_attn * ((nh + 2 * nkv) * d * H + nh * d * H) \
+        + cfg.num_hidden_layers * 3 * H * F
+    return 2.0 * (per_tok * tokens + n_attn * 2 * nh * d * attn_pairs + rows_out * H * cfg.vocab_size)
+
+
+def kv_bytes(cfg, engine, lengths) -> int:
+    n_attn = sum(t == "full_attention" for t in cfg.layer_types)
+    n_conv = cfg.num_hidden_layers - n_attn
+    el = 2 if engine.dtype == torch.bfloat16 else 4
+    kv = sum(lengths) * n_attn * 2 * cfg.num_key_value_heads * cfg.head_dim * el
+    conv = len(lengths) * n_conv * cfg.hidden_size * (cfg.conv_L_cache - 1) * 4 * 2      # read and written
+    return kv + conv
+
+
+def decode_run(engine, cfg, batch: int, prompt_len: int, steps: int, warmup: int, seed: int):
+    """Prefill `batch` random prompts, then time `steps` decode steps.  Returns (seconds, mean context)."""
+    from gesso_amd.engine.decode import DecodeLoop
+    g = torch.Generator().manual_seed(seed)
+    rids = [("bench", seed, i) for i in range(batch)]
+    first = []
+    for rid in rids:
+        engine.add_request(rid)
+    from gesso_amd import StepEntry
+    prompts = [torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist() for _ in rids]
+    at = 0
+    while at < batch:                                   # prompts in steps of at most 8,192 tokens
+        n = max(1, min(batch - at, 8192 // prompt_len))
+        logits = engine.step([StepEntry(r, p, [prompt_len - 1]) for r, p in zip(rids[at:at + n], prompts[at:at + n])])
+        first += logits.argmax(1).tolist()
+        at += n
+    loop = DecodeLoop(engine, rids, first)
+    loop.run(warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    loop.run(steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lengths = [engine.length(r) for r in rids]
+    mean_ctx = sum(lengths) / batch - steps / 2.0
+    loop.close()
+    for rid in rids:
+        engine.finish_request(rid)
+    return dt, mean_ctx
+
+
+def prefill_run(engine, cfg, tokens: int, reps: int = 5):
+    from gesso_amd import StepEntry
+    g = torch.Generator().manual_seed(99)
+    ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
+    times = []
+    for i in range(reps + 2):
+        rid = ("prefill", i)
+        engine.add_request(rid)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry(rid, ids, [tokens - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.finish_request(rid)
+    times = sorted(times[2:])
+    return times[len(times) // 2]
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
+    ap.add_argument("--only-prefill", action="store_true", help="measure the 2,048-token prefill alone (for profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
+        return 2
+
+    from gesso_amd import Engine
+
+    cfg = model_config()
+    layers_full = cfg.num_hidden_layers
+    if args.layers is not None and args.layers < layers_full:
+        import dataclasses
+        cfg = dataclasses.replace(cfg, num_hidden_layers=args.layers, layer_types=cfg.layer_types[:args.layers])
+    prompt_len, context = 512, 4096
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    engine = Engine.from_config(cfg, seed=0, dtype=dtype, page_size=16, max_context=context,
+                                max_tokens=max_batch * (prompt_len + args.steps + args.warmup + 32) + 4096,
+                                num_slots=max_batch + 1)
+    wbytes = weight_bytes(engine)
+    if args.only_prefill:
+        sec = prefill_run(engine, cfg, 2048)
+        print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tok_s": round(2048 / sec, 1)}))
+        return 0
+
+    dt, mean_ctx = decode_run(engine, cfg, args.batch, prompt_len, args.steps, args.warmup, seed=1)
+    ms = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    bytes_step = wbytes + kv_bytes(cfg, engine, [mean_ctx] * args.batch)
+    achieved = bytes_step / (ms * 1e-3) / 1e9
+    out = {
+        "metric": "decode tok/s at batch 8 (LFM2-1.2B sizes, 512-token prompts)", "value": round(value, 1),
+        "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "config": {"model": "LFM2-1.2B sizes", "layers": cfg.num_hidden_layers, "layers_full": layers_full,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "ff": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "conv_L_cache": cfg.conv_L_cache, "attn_layers": sum(t == "full_attention" for t in cfg.layer_types),
+                   "global_batch": args.batch, "prompt_len": prompt_len, "seq_len": context, "page_size": 16,
+                   "parallelism": "single GPU", "weights_gb": round(wbytes / 1e9, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+    }
+    if not args.no_points:
+        points = {}
+        for b, name in ((1, "decode_b1"), (64, "decode_b64")):
+            steps = min(args.steps, 128)
+            dtb, _ = decode_run(engine, cfg, b, prompt_len, steps, min(args.warmup, 8), seed=10 + b)
+            points[name] = round(b * steps / dtb, 1)
+        out["points"] = points
+        T = 2048
+        sec = prefill_run(engine, cfg, T)
+        flops = step_flops(cfg, T, T * (T + 1) // 2, 1)
+        out["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
+                          "frac": round(flops / sec / PEAK_FLOPS[args.dtype], 4)}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
