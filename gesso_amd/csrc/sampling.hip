@@ -10,13 +10,11 @@
 
 #define SAMP_THREADS 1024
 
-__global__ void argmax_rows_kernel(const float* __restrict__ logits, int V, int* __restrict__ ids,
-                                   int* __restrict__ bad) {
+// First maximum of one row by the whole block; thread 0 returns (id, bad) through the pointers.
+__device__ void row_argmax(const float* __restrict__ x, int V, int* id_out, int* bad_out) {
   __shared__ float bv[SAMP_THREADS / 64];
   __shared__ int bi[SAMP_THREADS / 64];
   __shared__ int bbad;
-  int row = blockIdx.x;
-  const float* x = logits + (size_t)row * V;
   if (threadIdx.x == 0) bbad = 0;
   __syncthreads();
   float best = -INFINITY;
@@ -51,9 +49,15 @@ __global__ void argmax_rows_kernel(const float* __restrict__ logits, int V, int*
         best = bv[w];
         idx = bi[w];
       }
-    ids[row] = idx == 0x7fffffff ? 0 : idx;
-    bad[row] = bbad;
+    *id_out = idx == 0x7fffffff ? 0 : idx;
+    *bad_out = bbad;
   }
+}
+
+__global__ void argmax_rows_kernel(const float* __restrict__ logits, int V, int* __restrict__ ids,
+                                   int* __restrict__ bad) {
+  int row = blockIdx.x;
+  row_argmax(logits + (size_t)row * V, V, ids + row, bad + row);
 }
 
 extern "C" int gs_argmax_rows(const float* logits, int rows, int V, int* ids, int* bad, hipStream_t stream) {
@@ -64,15 +68,11 @@ extern "C" int gs_argmax_rows(const float* logits, int rows, int V, int* ids, in
   return 0;
 }
 
-// One block per row.  temperature[row] > 0, u[row] in [0, 1).
-__global__ void sample_temperature_kernel(const float* __restrict__ logits, int V,
-                                          const double* __restrict__ temperature, const double* __restrict__ u,
-                                          int* __restrict__ ids, int* __restrict__ bad) {
+// One row by the whole block: T > 0, u in [0, 1); thread 0 returns (id, bad) through the pointers.
+__device__ void row_sample(const float* __restrict__ x, int V, double T, double uu, int* id_out, int* bad_out) {
   __shared__ double part[SAMP_THREADS];
   __shared__ float redf[SAMP_THREADS / 64];
   __shared__ int bbad;
-  int row = blockIdx.x;
-  const float* x = logits + (size_t)row * V;
   int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
   if (tid == 0) bbad = 0;
   __syncthreads();
@@ -95,12 +95,12 @@ __global__ void sample_temperature_kernel(const float* __restrict__ logits, int 
   for (int w = 1; w < nw; ++w) mx = fmaxf(mx, redf[w]);
   if (bbad) {
     if (tid == 0) {
-      ids[row] = 0;
-      bad[row] = 1;
+      *id_out = 0;
+      *bad_out = 1;
     }
     return;
   }
-  double hi = (double)mx, T = temperature[row];
+  double hi = (double)mx;
   double s = 0.0;
   for (int j = j0; j < j1; ++j) s += exp(((double)x[j] - hi) / T);
   part[tid] = s;
@@ -110,7 +110,7 @@ __global__ void sample_temperature_kernel(const float* __restrict__ logits, int 
   if (tid == 0) {
     double total = 0.0;
     for (int i = 0; i < (int)blockDim.x; ++i) total += part[i];
-    double r = u[row] * total;
+    double r = uu * total;
     double acc = 0.0;
     int pick = V - 1;
     bool found = false;
@@ -129,10 +129,68 @@ __global__ void sample_temperature_kernel(const float* __restrict__ logits, int 
         acc += part[i];
       }
     }
-    ids[row] = pick;
-    bad[row] = 0;
+    *id_out = pick;
+    *bad_out = 0;
   }
 }
+
+__global__ void sample_temperature_kernel(const float* __restrict__ logits, int V,
+                                          const double* __restrict__ temperature, const double* __restrict__ u,
+                                          int* __restrict__ ids, int* __restrict__ bad) {
+  int row = blockIdx.x;
+  row_sample(logits + (size_t)row * V, V, temperature[row], u[row], ids + row, bad + row);
+}
+
+// The decode loop's choice, made to be recorded into a HIP graph: everything that changes from step to
+// step is read from device memory.  Row r: temperature[r] <= 0 means greedy, else a draw with
+// u[step * rows + r], step = *counter.  The chosen id goes to next_ids[r] (the token fed back) and,
+// with the row's flag, to ring[step * rows + r] and bad_ring[...], which the host reads once per run.
+__global__ void decode_choose_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
+                                     const double* __restrict__ u, const int* __restrict__ counter,
+                                     int* __restrict__ next_ids, int* __restrict__ ring, int* __restrict__ bad_ring) {
+  __shared__ int sid, sbad;
+  int row = blockIdx.x, rows = gridDim.x;
+  int step = *counter;
+  double T = temperature[row];
+  const float* x = logits + (size_t)row * V;
+  if (T > 0.0)
+    row_sample(x, V, T, u[(size_t)step * rows + row], &sid, &sbad);
+  else
+    row_argmax(x, V, &sid, &sbad);
+  if (threadIdx.x == 0) {
+    next_ids[row] = sid;
+    ring[(size_t)step * rows + row] = sid;
+    bad_ring[(size_t)step * rows + row] = sbad;
+  }
+}
+
+// After a decode step: live rows move one position on; the step counter counts up.  One block.
+__global__ void decode_advance_kernel(int* __restrict__ positions, int* __restrict__ kv_len,
+                                      const int* __restrict__ live, int* __restrict__ counter, int rows) {
+  int r = threadIdx.x;
+  if (r < rows && live[r]) {
+    positions[r] += 1;
+    kv_len[r] += 1;
+  }
+  if (r == 0) *counter += 1;
+}
+
+extern "C" int gs_decode_choose(const float* logits, int rows, int V, const double* temperature, const double* u,
+                                const int* counter, int* next_ids, int* ring, int* bad_ring, hipStream_t stream) {
+  GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
+  decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, counter, next_ids, ring, bad_ring);
+  GS_LAUNCH_CHECK("decode_choose");
+  return 0;
+}
+
+extern "C" int gs_decode_advance(int* positions, int* kv_len, const int* live, int* counter, int rows,
+                                 hipStream_t stream) {
+  GS_REQUIRE(rows > 0 && rows <= 1024, "decode_advance: %d rows; at most 1024", rows);
+  decode_advance_kernel<<<1, 1024, 0, stream>>>(positions, kv_len, live, counter, rows);
+  GS_LAUNCH_CHECK("decode_advance");
+  return 0;
+}
+
 
 extern "C" int gs_sample_temperature(const float* logits, int rows, int V, const double* temperature,
                                      const double* u, int* ids, int* bad, hipStream_t stream) {

@@ -1,32 +1,189 @@
-"""The decode loop: every live request gets one token per step, the token chosen is fed back.
+"""The decode fast path: steps in which every request brings one token, recorded once as a HIP graph.
 
-``DecodeLoop(engine, rids, first_tokens)`` continues requests whose prompts are in the cache;
-``run(n)`` makes ``n`` steps and returns the tokens ``(n, batch)`` it chose.  Greedy choice
-runs on the device; the tokens come to the host once per call, not once per step.
+A decode step of a small batch is bound by launch overhead, not by arithmetic: more than a
+hundred kernels of a few microseconds each.  So the step (embedding, all blocks, head, the choice
+of the next token, the advance of positions) is recorded into a graph per batch capacity and
+replayed; everything that changes between steps lives in device buffers the kernels read
+(tokens, positions, block tables, slots, the step counter).  The token a step chooses is written
+where the next step's embedding reads it, so ``n`` steps run back to back without the host; the
+host reads the chosen tokens once per call.  The reference decodes one row per call with one
+host round trip per token (``src/Inference/Inference.jl:2547-2712``).
+
+Rows beyond the live batch (the capacity is the batch rounded up to a power of two) point at the
+scratch page and the scratch slot, so they compute and write garbage that nobody reads.
+
+Graph hygiene: nothing in the graph clears memory with a memset node; the step counter is reset by
+an ordinary fill before the replays.
 """
 from __future__ import annotations
 
-from typing import Hashable, List, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
-from .batch import StepEntry
+from ..errors import InvalidPlan
+from ..sampling.sampler import Sampler
+
+
+def _capacity(n: int) -> int:
+    c = 1
+    while c < n:
+        c *= 2
+    return c
+
+
+class _DecodeContext:
+    """What the parts read of a step, all of it static device buffers (see StepContext for the fields)."""
+
+    def __init__(self, runner):
+        r = runner
+        self.T = self.nseq = self.n_want = r.cap
+        self.q_lens = [1] * r.cap
+        self.all_single = True
+        self.max_q_len = 1
+        self.max_kv_len = None            # not known on the host: kernels read kv_len on the device
+        self.decode_only = True
+        self.token_ids, self.positions, self.kv_len, self.slots = r.tok, r.pos, r.kv_len, r.slots
+        self.seq_of_token, self.q_start, self.want_rows = r.seq_of_token, r.q_start, r.seq_of_token
+        self.block_tables = r.block_tables
+        self._storage = r.engine.storage
+
+    def cache_view(self, call: int):
+        return self._storage.view(call, self.block_tables)
+
+
+class DecodeRunner:
+    """Static buffers and the recorded graph for one batch capacity."""
+
+    MAX_STEPS = 32
+
+    def __init__(self, engine, cap: int):
+        self.engine, self.cap = engine, cap
+        dev = engine.device
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.max_blocks = -(-engine.max_context // engine.page_size)
+        st = engine.storage
+        self.tok = torch.zeros(cap, **i32)
+        self.pos = torch.zeros(cap, **i32)
+        self.kv_len = torch.ones(cap, **i32)
+        self.slots = torch.full((cap,), st.scratch_slot, **i32)
+        self.live = torch.zeros(cap, **i32)
+        self.seq_of_token = torch.arange(cap, **i32)
+        self.q_start = torch.arange(cap + 1, **i32)
+        self.block_tables = [torch.full((cap, self.max_blocks), n, **i32) for n in st.num_pages]
+        self.temperature = torch.zeros(cap, dtype=torch.float64, device=dev)
+        self.u = torch.zeros((self.MAX_STEPS, cap), dtype=torch.float64, device=dev)
+        self.counter = torch.zeros(1, **i32)
+        self.ring = torch.zeros((self.MAX_STEPS, cap), **i32)
+        self.bad_ring = torch.zeros((self.MAX_STEPS, cap), **i32)
+        self.ctx = _DecodeContext(self)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+
+    def _body(self) -> None:
+        ops = self.engine.rt.ops
+        self.engine.rt.no_library = True
+        try:
+            logits = self.engine.model.forward(self.ctx)
+        finally:
+            self.engine.rt.no_library = False
+        ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring)
+        ops.decode_advance(self.pos, self.kv_len, self.live, self.counter)
+
+    def _record(self) -> None:
+        """One eager run on scratch rows (everything lazily initialised gets initialised), then the capture."""
+        side = torch.cuda.Stream(device=self.engine.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._body()
+        torch.cuda.current_stream().wait_stream(side)
+        self.counter.zero_()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self._body()
+        self.graph = graph
+
+    def run(self, rids: Sequence[Hashable], tokens: Sequence[int], n: int, samplers=None
+            ) -> Tuple[np.ndarray, np.ndarray]:
+        """``n`` steps for the requests ``rids`` whose next input tokens are ``tokens``.
+
+        Returns ``(ids (n, batch), bad (n, batch))``.  Pages for ``n`` more tokens are reserved first;
+        :class:`~gesso_amd.errors.OutOfPages` leaves everything as it was.
+        """
+        eng, cap, B = self.engine, self.cap, len(rids)
+        if not 1 <= n <= self.MAX_STEPS:
+            raise InvalidPlan(f"a decode run takes 1 to {self.MAX_STEPS} steps, not {n}")
+        if self.graph is None:
+            self._record()                       # before any live row is set: the eager run sees scratch rows only
+        mgr, st = eng.manager, eng.storage
+        rcs = [mgr.get(r) for r in rids]
+        for t in tokens:
+            if not 0 <= int(t) < eng.spec.vocab:
+                raise InvalidPlan(f"token id {int(t)} outside the vocabulary of {eng.spec.vocab}")
+        mgr.reserve_many([(r, n) for r in rids])
+        eng._zero_fresh_slots()
+        # one int32 buffer for the per-row facts, one copy
+        host = np.zeros((5, cap), dtype=np.int32)
+        host[0, :B] = tokens
+        host[1, :B] = [rc.length for rc in rcs]
+        host[2] = 1
+        host[2, :B] = [rc.length + 1 for rc in rcs]
+        host[3] = st.scratch_slot
+        host[3, :B] = [st.scratch_slot if rc.slot is None else rc.slot for rc in rcs]
+        host[4, :B] = 1
+        dev = torch.from_numpy(host).pin_memory().to(eng.device, non_blocking=True)
+        self.tok.copy_(dev[0]); self.pos.copy_(dev[1]); self.kv_len.copy_(dev[2])
+        self.slots.copy_(dev[3]); self.live.copy_(dev[4])
+        width = max(1, max(-(-(rc.length + n) // eng.page_size) for rc in rcs))
+        for g, bt in enumerate(self.block_tables):
+            tab = np.full((cap, width), st.num_pages[g], dtype=np.int32)
+            for i, rc in enumerate(rcs):
+                row = np.asarray(rc.tables[g][:width], dtype=np.int32)
+                row[row < 0] = st.num_pages[g]
+                tab[i, :len(row)] = row
+            bt[:, :width].copy_(torch.from_numpy(tab).pin_memory().to(eng.device, non_blocking=True))
+        temp = np.zeros(cap, dtype=np.float64)
+        if samplers is not None and any(s is not None for s in samplers):
+            u = np.zeros((n, cap), dtype=np.float64)
+            for i, s in enumerate(samplers):
+                if s is not None:
+                    if s.top_p < 1:
+                        raise InvalidPlan("nucleus sampling does not run in the recorded decode loop")
+                    temp[i] = s.temperature
+                    u[:, i] = [s.unit() for _ in range(n)]
+            self.u[:n].copy_(torch.from_numpy(u).pin_memory().to(eng.device, non_blocking=True))
+        self.temperature.copy_(torch.from_numpy(temp).pin_memory().to(eng.device, non_blocking=True))
+        self.counter.zero_()
+        for _ in range(n):
+            self.graph.replay()
+        ids = self.ring[:n, :B].cpu().numpy()
+        bad = self.bad_ring[:n, :B].cpu().numpy()
+        for r in rids:
+            mgr.commit(r, n)
+        eng.steps += n
+        return ids, bad
 
 
 class DecodeLoop:
-    def __init__(self, engine, rids: Sequence[Hashable], first_tokens: Sequence[int]):
+    """Continue requests whose prompts are in the cache: ``run(n)`` makes ``n`` greedy steps for all of them."""
+
+    def __init__(self, engine, rids: Sequence[Hashable], first_tokens: Sequence[int], samplers=None):
         self.engine = engine
         self.rids = list(rids)
         self.tokens = [int(t) for t in first_tokens]
+        self.samplers = samplers
 
     def run(self, n: int) -> List[List[int]]:
-        out = []
-        ops = self.engine.rt.ops
-        for _ in range(n):
-            logits = self.engine.step([StepEntry(r, [t], [0]) for r, t in zip(self.rids, self.tokens)])
-            ids, _ = ops.argmax_rows(logits)
-            self.tokens = ids.tolist()
-            out.append(self.tokens)
+        out: List[List[int]] = []
+        while n > 0:
+            k = min(n, DecodeRunner.MAX_STEPS)
+            ids, bad = self.engine.decode(self.rids, self.tokens, k, self.samplers)
+            if bad.any():
+                from ..errors import NumericalInstability
+                raise NumericalInstability("non-finite logits in the decode loop")
+            out += ids.tolist()
+            self.tokens = ids[-1].tolist()
+            n -= k
         return out
 
     def close(self) -> None:

@@ -61,6 +61,7 @@ class Engine:
         self.manager = CacheManager(layout, self.page_size, int(num_pages), int(num_slots), self.max_context)
         self.storage = CacheStorage(layout, self.page_size, int(num_pages), int(num_slots), self.dtype, self.device)
         self.steps = 0
+        self._runners = {}
 
     # ------------------------------------------------------------------ construction
 
@@ -125,3 +126,26 @@ class Engine:
             self.manager.commit(e.rid, len(e.tokens))
         self.steps += 1
         return logits
+
+    # ------------------------------------------------------------------ decoding, recorded
+
+    DECODE_MAX_BATCH = 64
+
+    def decode(self, rids: Sequence[Hashable], tokens: Sequence[int], n: int, samplers=None):
+        """``n`` decode steps for requests that each bring one token, as replays of a recorded graph.
+
+        ``tokens``: each request's next input token; the tokens chosen are fed back on the device.
+        ``samplers``: per request None (greedy) or a :class:`~gesso_amd.sampling.sampler.Sampler`
+        without nucleus.  Returns ``(ids, bad)`` as ``(n, batch)`` arrays; a row of ``bad`` marks a step
+        whose logits were not finite.  Raises :class:`~gesso_amd.errors.OutOfPages` before changing anything.
+        """
+        from .decode import DecodeRunner, _capacity
+        if not 1 <= len(rids) <= self.DECODE_MAX_BATCH:
+            raise InvalidPlan(f"the recorded decode loop takes 1 to {self.DECODE_MAX_BATCH} requests, not {len(rids)}")
+        if len(set(rids)) != len(rids) or len(tokens) != len(rids):
+            raise InvalidPlan("one token per request, each request once")
+        cap = _capacity(len(rids))
+        runner = self._runners.get(cap)
+        if runner is None:
+            runner = self._runners[cap] = DecodeRunner(self, cap)
+        return runner.run(rids, tokens, n, samplers)

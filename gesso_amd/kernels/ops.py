@@ -274,3 +274,58 @@ def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.T
     _check(lib().gs_sample_top_p(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(u), _p(wbuf),
                                  _p(ids), _p(bad), _stream()))
     return ids, bad
+
+
+# ---------------------------------------------------------------------- decoding
+
+SKINNY_MAX_ROWS = 64
+
+
+def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the weight-streaming kernel takes this product (few rows, bfloat16, aligned rows)."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[0] <= SKINNY_MAX_ROWS
+            and x.shape[1] % 8 == 0 and x.stride(1) == 1 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0)
+            and x.data_ptr() % 16 == 0 and w.is_contiguous() and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, swiglu: bool = False):
+    """``x @ w.T`` for at most 64 rows, streaming the weights once; optionally ``silu(gate) * up`` of the result.
+
+    With ``swiglu`` the weight holds gate rows then up rows and the output is half as wide.
+    """
+    _dev(w, out)
+    _need(skinny_ok(x, w), "gemm_skinny: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape == (N, K), f"gemm_skinny: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    cols = N // 2 if swiglu else N
+    if out is None:
+        out = torch.empty((M, cols), dtype=out_dtype or x.dtype, device=x.device)
+    _need(out.shape == (M, cols) and out.stride(1) == 1, "gemm_skinny: out has the wrong shape")
+    _check(lib().gs_gemm_skinny(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(out), c_int(_dt(out)),
+                                c_int(out.stride(0) if M > 1 else cols), c_int(M), c_int(N), c_int(K),
+                                c_int(1 if swiglu else 0), _stream()))
+    return out
+
+
+def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring) -> None:
+    """Per row: greedy (temperature <= 0) or a draw with ``u[counter, row]``; results into the loop's buffers."""
+    _dev(logits, temperature, u, counter, next_ids, ring, bad_ring)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "decode_choose: logits are float32 (rows, V)")
+    rows, V = logits.shape
+    _need(temperature.dtype == torch.float64 and temperature.numel() == rows, "decode_choose: temperature float64 (rows,)")
+    _need(u.dtype == torch.float64 and u.dim() == 2 and u.shape[1] == rows, "decode_choose: u is float64 (steps, rows)")
+    for t in (counter, next_ids, ring, bad_ring):
+        _i32(t)
+    _need(ring.shape == u.shape and bad_ring.shape == u.shape and next_ids.numel() == rows, "decode_choose: buffer shapes")
+    _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(u), _p(counter), _p(next_ids),
+                                  _p(ring), _p(bad_ring), _stream()))
+
+
+def decode_advance(positions, kv_len, live, counter) -> None:
+    _dev(positions, kv_len, live, counter)
+    rows = positions.numel()
+    for t in (positions, kv_len, live, counter):
+        _i32(t)
+    _need(kv_len.numel() == rows and live.numel() == rows, "decode_advance: buffer shapes")
+    _check(lib().gs_decode_advance(_p(positions), _p(kv_len), _p(live), _p(counter), c_int(rows), _stream()))

@@ -27,8 +27,7 @@ class Runtime:
         self.ops = ops
         self.dtype = dtype
         self._shared = {}
-        # rows up to which the skinny bf16 kernel beats the library product (set by measurement)
-        self.skinny_rows = 0
+        self.no_library = False        # set while a HIP graph is recorded: only our own kernels go into it
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""
@@ -40,11 +39,17 @@ class Runtime:
         """``x @ w.T (+ bias)``; ``w (out, in)``."""
         out_dtype = out_dtype or x.dtype
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
-            if x.shape[0] <= self.skinny_rows:
+            if self.ops.skinny_ok(x, w):
                 return self.ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out)
-            if out_dtype == torch.bfloat16:
+            if out_dtype == torch.bfloat16 and not self.no_library:
                 return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
         return self.ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
+
+    def linear_swiglu(self, x: torch.Tensor, w13: torch.Tensor) -> torch.Tensor:
+        """``silu(x @ w1.T) * (x @ w3.T)`` with ``w13`` holding w1's rows, then w3's."""
+        if self.ops.skinny_ok(x, w13):
+            return self.ops.gemm_skinny(x, w13, swiglu=True)
+        return self.ops.swiglu(self.linear(x, w13))
 
     def attention(self, q, q_stride, cache, ctx, window, scale, nh, nkv, d) -> torch.Tensor:
         """Causal attention of this step's queries over the paged cache; ``(T, nh * d)``.

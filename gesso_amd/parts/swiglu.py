@@ -27,8 +27,7 @@ class SwiGLU(Part):
         self.w2 = tensors["w2.weight"]
 
     def forward(self, x, ctx):
-        gu = self.rt.linear(x, self.w13)
-        a = self.rt.ops.swiglu(gu)
+        a = self.rt.linear_swiglu(x, self.w13)
         return self.rt.linear(a, self.w2)
 
 

@@ -220,3 +220,49 @@ def test_random_weights_session_and_cli(tmp_path):
     r = subprocess.run([sys.executable, "-m", "gesso_amd", "--model", d, "--gguf", "x"], capture_output=True, text=True,
                        env=env, cwd=ROOT)
     assert r.returncode != 0 and "unrecognized" in r.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_recorded_decode_loop_equals_single_steps(folders, name, dtype):
+    """Replays of the recorded step, several runs with other work between them, against step-by-step decoding."""
+    from gesso_amd import Engine, Sampler, StepEntry
+    d = write_tiny(folders, name, torch.float32 if dtype == "float32" else torch.bfloat16)
+    cfg, _ = CONFIGS[name]
+    prompts = [random_ids(n, cfg.vocab_size, 300 + n) for n in (7, 19, 33)]
+    samplers = lambda: [None, Sampler(0.8, 1.0, 5), None]
+
+    def prefill(eng):
+        firsts = []
+        for i, p in enumerate(prompts):
+            eng.add_request(i)
+            firsts.append(int(eng.step([StepEntry(i, p, [len(p) - 1])]).argmax()))
+        return firsts
+
+    # step by step through the plain step function
+    eng = Engine.from_folder(d, dtype=dtype, page_size=8, max_tokens=512)
+    toks, sm, ref = prefill(eng), samplers(), []
+    from gesso_amd.sampling import choose
+    for _ in range(21):
+        logits = eng.step([StepEntry(i, [t], [0]) for i, t in enumerate(toks)])
+        toks = choose(eng.rt.ops, logits, sm)
+        ref.append(list(toks))
+    # the recorded loop: runs of 1, 8, 5 and 7 steps, with unrelated work between the runs
+    eng2 = Engine.from_folder(d, dtype=dtype, page_size=8, max_tokens=512)
+    toks, sm, got = prefill(eng2), samplers(), []
+    for n in (1, 8, 5, 7):
+        ids, bad = eng2.decode([0, 1, 2], toks, n, sm)
+        assert not bad.any()
+        got += ids.tolist()
+        toks = ids[-1].tolist()
+        eng2.add_request("other")                        # eager work and a synchronisation between replays
+        eng2.step([StepEntry("other", prompts[0], [0])])
+        eng2.finish_request("other")
+        torch.cuda.synchronize()
+    if dtype == "float32":
+        assert got == ref
+    else:
+        # bfloat16: the recorded loop uses the weight-streaming products throughout; near-ties may fall the other way
+        agree = sum(a == b for ra, rb in zip(got, ref) for a, b in zip(ra, rb))
+        assert agree >= 0.9 * 21 * 3
+    assert [eng2.length(i) for i in range(3)] == [len(p) + 21 for p in prompts]

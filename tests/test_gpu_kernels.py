@@ -361,3 +361,42 @@ def test_sample_top_p_follows_the_plain_sampler(ops, V, temp, top_p):
                                 torch.full((rows,), top_p, dtype=torch.float64, device=DEV),
                                 torch.tensor(us, dtype=torch.float64, device=DEV))
     assert ids.tolist() == want and not any(bad.tolist())
+
+
+# ------------------------------------------------------------------ the weight-streaming product
+
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(48, 64), (100, 200), (2048, 2048), (6144, 2048), (2048, 8192), (301, 144)])
+def test_gemm_skinny(ops, M, N, K):
+    g = gen(M * 7 + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    want = x.double() @ w.double().T
+    got32 = ops.gemm_skinny(x.to(DEV), w.to(DEV), out_dtype=torch.float32)
+    assert float((got32.double().cpu() - want).abs().max()) <= 2e-5 * max(1.0, float(want.abs().max())) * math.sqrt(K)
+    close(ops.gemm_skinny(x.to(DEV), w.to(DEV)), want, torch.bfloat16)
+    # a view with a row stride, as the attention output and portions of a buffer are
+    wide = torch.randn(M, K + 16, generator=g).bfloat16().to(DEV)
+    close(ops.gemm_skinny(wide[:, 8:8 + K], w.to(DEV)), wide[:, 8:8 + K].double().cpu() @ w.double().T, torch.bfloat16) \
+        if ops.skinny_ok(wide[:, 8:8 + K], w.to(DEV)) else None
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 24, 64), (8, 100, 96), (40, 8192, 2048), (64, 50, 144)])
+def test_gemm_skinny_swiglu(ops, M, F, K):
+    g = gen(M + F + K)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(2 * F, K, generator=g) / math.sqrt(K) * 2).bfloat16()
+    y = x.double() @ w.double().T
+    want = P.swiglu(y[:, :F], y[:, F:])
+    got = ops.gemm_skinny(x.to(DEV), w.to(DEV), swiglu=True)
+    assert got.shape == (M, F)
+    close(got, want, torch.bfloat16)
+
+
+def test_gemm_skinny_refuses(ops):
+    from gesso_amd.errors import KernelError
+    x = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(16, 64, dtype=torch.bfloat16, device=DEV)
+    assert not ops.skinny_ok(x, w) and not ops.skinny_ok(x[:4, :60], w[:, :60])
+    with pytest.raises(KernelError):
+        ops.gemm_skinny(x, w)
