@@ -329,3 +329,40 @@ def decode_advance(positions, kv_len, live, counter) -> None:
         _i32(t)
     _need(kv_len.numel() == rows and live.numel() == rows, "decode_advance: buffer shapes")
     _check(lib().gs_decode_advance(_p(positions), _p(kv_len), _p(live), _p(counter), c_int(rows), _stream()))
+
+
+def attention_decode_supports(nh: int, nkv: int, d: int) -> bool:
+    return bool(lib().gs_attention_decode_supports(c_int(nh), c_int(nkv), c_int(d)))
+
+
+_decode_ws = {}
+
+
+def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_size, window, scale, nh, nkv, d, nseq,
+                     nsplit: int, out: torch.Tensor = None) -> torch.Tensor:
+    """One query per sequence over its paged keys (bfloat16), keys split over ``nsplit`` blocks per key head."""
+    _dev(q, kcache, vcache, positions, block_table, out)
+    _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
+          "attention_decode takes bfloat16")
+    _need(q.numel() >= (nseq - 1) * q_stride + nh * d if nseq else True, "attention_decode: q is too small")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
+          "cache must be (pages, nkv, page_size, d)")
+    _i32(positions, nseq, "positions")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= nseq,
+          "block_table must be int32 (nseq, max_blocks)")
+    key = (q.device, nseq, nh, nkv, d, nsplit)
+    ws = _decode_ws.get(key)
+    if ws is None:
+        n = lib().gs_attention_decode_workspace
+        n.restype = c_long
+        floats = n(c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit))
+        ws = _decode_ws[key] = (torch.empty(floats, dtype=torch.float32, device=q.device),
+                                torch.zeros(nseq * nkv, dtype=torch.int32, device=q.device))
+    if out is None:
+        out = torch.empty((nseq, nh * d), dtype=q.dtype, device=q.device)
+    _need(out.shape == (nseq, nh * d) and out.dtype == q.dtype, "attention_decode: out has the wrong shape or type")
+    _check(lib().gs_attention_decode(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
+                                     c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
+                                     _p(out), _p(ws[0]), _p(ws[1]), c_int(nseq), c_int(nh), c_int(nkv), c_int(d),
+                                     c_int(nsplit), _stream()))
+    return out

@@ -57,5 +57,11 @@ class Runtime:
         The generic kernel takes every size; faster kernels take over for the sizes and batch
         shapes they are written for.
         """
-        return self.ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
-                                          cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)
+        ops = self.ops
+        if ctx.all_single and q.dtype == torch.bfloat16 and ops.attention_decode_supports(nh, nkv, d):
+            # one query per sequence: the key stream is split so that the whole chip reads it
+            nsplit = max(1, min(16, 512 // max(1, ctx.nseq * nkv)))
+            return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
+                                        cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
+        return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
+                                     cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)

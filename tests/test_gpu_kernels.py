@@ -400,3 +400,47 @@ def test_gemm_skinny_refuses(ops):
     assert not ops.skinny_ok(x, w) and not ops.skinny_ok(x[:4, :60], w[:, :60])
     with pytest.raises(KernelError):
         ops.gemm_skinny(x, w)
+
+
+# ------------------------------------------------------------------ decode attention (one query per sequence)
+
+@pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 16, 8), (3, 1, 32, 16), (32, 8, 64, 16), (8, 1, 128, 16), (5, 5, 64, 4)])
+@pytest.mark.parametrize("nsplit", [1, 3, 16])
+@pytest.mark.parametrize("window", [None, 70])
+def test_attention_decode(ops, nh, nkv, d, ps, nsplit, window):
+    g = gen(nh + d + nsplit)
+    lens = [1, 2, 63, 64, 65, 300, 700, 129]            # keys per sequence, the query's own included
+    nseq = len(lens)
+    nblk = [-(-n // ps) for n in lens]
+    total = sum(nblk)
+    perm = torch.randperm(total + 2, generator=g)[:total] + 1
+    kc = torch.randn(total + 3, nkv, ps, d, generator=g).bfloat16()
+    vc = torch.randn(total + 3, nkv, ps, d, generator=g).bfloat16()
+    table = torch.zeros(nseq, max(nblk), dtype=torch.int32)
+    q = torch.randn(nseq, nh * d, generator=g)
+    q[5] *= 3.0                                           # sharper weights on one sequence
+    q = q.bfloat16()
+    want, at = [], 0
+    for i, n in enumerate(lens):
+        pages = perm[at:at + nblk[i]]
+        at += nblk[i]
+        table[i, :nblk[i]] = pages.to(torch.int32)
+        k = kc[pages].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:n]
+        v = vc[pages].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:n]
+        want.append(P.causal_attention(q[i].double().reshape(1, nh, d), k.double(), v.double(), window or 0).reshape(-1))
+    want = torch.stack(want)
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    for _ in range(2):                                    # twice: the counters must be back at zero
+        got = ops.attention_decode(q.to(DEV), nh * d, kc.to(DEV), vc.to(DEV), positions.to(DEV), table.to(DEV), ps,
+                                   window, scale, nh, nkv, d, nseq, nsplit)
+        close(got, want, torch.bfloat16)
+    same = ops.attention_generic(q.to(DEV), nh * d, kc.to(DEV), vc.to(DEV), positions.to(DEV),
+                                 torch.arange(nseq, dtype=torch.int32, device=DEV), table.to(DEV), ps, window, scale,
+                                 nh, nkv, d, nseq)
+    close(got, same.double().cpu(), torch.bfloat16)
+
+
+def test_attention_decode_supports(ops):
+    assert ops.attention_decode_supports(32, 8, 64) and ops.attention_decode_supports(3, 1, 32)
+    assert not ops.attention_decode_supports(3, 3, 48) and not ops.attention_decode_supports(18, 2, 64)
