@@ -8,10 +8,12 @@
 // (D bfloat16, 16-byte loads) and dots it with the G queries held in LDS as float32.  Softmax
 // runs online per head across the wavefront (running maximum and sum).  Values: lane = (key
 // group of 8, chunk of 8 features); 16-byte loads of V rows, probabilities broadcast from LDS.
-// Wavefronts, then splits, are merged by the usual (max, sum, accumulator) rule in a fixed order:
-// the last block of a (sequence, key head) to finish, found by a counter, merges the splits and
-// writes the output, so no second launch is needed and the order of arrival does not change the
-// result.  Scores, maxima, sums and accumulators are float32.
+// Wavefronts, then splits, are merged by the usual (max, sum, accumulator) rule in a fixed order.
+// With one split the block writes the output itself; with more, each block writes its partial
+// (accumulator, max, sum) and a second small kernel merges them in split order.  (Merging in the
+// last block to arrive would save that launch, but the device-wide fence it needs writes back and
+// invalidates the L2 in every block, which costs far more than the launch.)  Scores, maxima, sums
+// and accumulators are float32.
 //
 // Everything that changes between steps (positions, block table) is read from device memory, so the
 // launch can be recorded into a graph.  q (T, q_stride), head h at [h D, (h+1) D); caches
@@ -25,8 +27,7 @@ template <int D, int G>
 __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int* __restrict__ positions, const int* __restrict__ block_table, int max_blocks, int page_size, int window,
-    float scale, bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int* __restrict__ counters, int nh, int nkv) {
+    float scale, bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv) {
   constexpr int DC = D / 8;        // 16-byte chunks per row
   constexpr int KG = 64 / DC;      // key groups per wavefront in the value phase
   static_assert(D % 8 == 0 && 64 % DC == 0, "head width must be 8, 16, 32, 64, 128, 256 or 512");
@@ -35,7 +36,6 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
   __shared__ long vrow[DEC_WAVES][64];
   __shared__ float wm[DEC_WAVES][G], wl[DEC_WAVES][G];
   __shared__ float wacc[DEC_WAVES][G][D];
-  __shared__ int is_last;
 
   const int split = blockIdx.x, nsplit = gridDim.x, kvh = blockIdx.y, seq = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -155,33 +155,32 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     int g = i / D, j = i - g * D;
     float M = -INFINITY;
     for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, wm[w][g]);
-    float o = 0.f;
+    float o = 0.f, L = 0.f;
     if (M > -INFINITY)
       for (int w = 0; w < DEC_WAVES; ++w)
-        if (wm[w][g] > -INFINITY) o += wacc[w][g][j] * expf(wm[w][g] - M);
-    part_o[(unit * G + g) * D + j] = o;
-    if (j == 0) {
-      float L = 0.f;
-      if (M > -INFINITY)
-        for (int w = 0; w < DEC_WAVES; ++w)
-          if (wm[w][g] > -INFINITY) L += wl[w][g] * expf(wm[w][g] - M);
-      part_ml[(unit * G + g) * 2] = M;
-      part_ml[(unit * G + g) * 2 + 1] = L;
+        if (wm[w][g] > -INFINITY) {
+          float f = expf(wm[w][g] - M);
+          o += wacc[w][g][j] * f;
+          L += wl[w][g] * f;
+        }
+    if (nsplit == 1) {
+      out[((size_t)seq * nh + kvh * G + g) * D + j] = f32_to_bf16(o / L);
+    } else {
+      part_o[(unit * G + g) * D + j] = o;
+      if (j == 0) {
+        part_ml[(unit * G + g) * 2] = M;
+        part_ml[(unit * G + g) * 2 + 1] = L;
+      }
     }
   }
-  // the last block of this (sequence, key head) merges the splits, in split order
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) {
-    int done = atomicAdd(&counters[seq * nkv + kvh], 1);
-    is_last = (done == nsplit - 1);
-    if (is_last) counters[seq * nkv + kvh] = 0;  // ready for the next launch
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
+}
+
+// Merge the splits of each (sequence, head), in split order.  One block per (sequence, key head).
+__global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                              bf16* __restrict__ out, int nsplit, int nh, int nkv, int G, int D) {
+  const int kvh = blockIdx.x, seq = blockIdx.y;
   const size_t base = ((size_t)seq * nkv + kvh) * nsplit;
-  for (int i = tid; i < G * D; i += blockDim.x) {
+  for (int i = threadIdx.x; i < G * D; i += blockDim.x) {
     int g = i / D, j = i - g * D;
     float M = -INFINITY;
     for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, part_ml[((base + sp) * G + g) * 2]);
@@ -201,12 +200,11 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
 template <int D>
 static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
                          const bf16* vc, const int* positions, const int* bt, int max_blocks, int page_size,
-                         int window, float scale, bf16* out, float* part_o, float* part_ml, int* counters, int nh,
-                         int nkv) {
+                         int window, float scale, bf16* out, float* part_o, float* part_ml, int nh, int nkv) {
 #define GS_RUN(GG)                                                                                                  \
   attention_decode_kernel<D, GG><<<grid, DEC_WAVES * 64, 0, stream>>>(q, q_stride, kc, vc, positions, bt, max_blocks, \
                                                                       page_size, window, scale, out, part_o,       \
-                                                                      part_ml, counters, nh, nkv)
+                                                                      part_ml, nh, nkv)
   switch (G) {
     case 1: GS_RUN(1); break;
     case 2: GS_RUN(2); break;
@@ -229,15 +227,15 @@ extern "C" int gs_attention_decode_supports(int nh, int nkv, int d) {
   return (d == 16 || d == 32 || d == 64 || d == 128) && g >= 1 && g <= DEC_MAXG;
 }
 
-// Floats of workspace for nseq sequences: partial outputs, then (max, sum) pairs; and ints of counters.
+// Floats of workspace for nseq sequences: partial outputs, then (max, sum) pairs.
 extern "C" long gs_attention_decode_workspace(int nseq, int nh, int nkv, int d, int nsplit) {
   return (long)nseq * nh * nsplit * (d + 2);
 }
 
 extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcache, const void* vcache,
                                    const int* positions, const int* block_table, int max_blocks, int page_size,
-                                   int window, float scale, void* out, float* workspace, int* counters, int nseq,
-                                   int nh, int nkv, int d, int nsplit, hipStream_t stream) {
+                                   int window, float scale, void* out, float* workspace, int nseq, int nh, int nkv,
+                                   int d, int nsplit, hipStream_t stream) {
   GS_REQUIRE(gs_attention_decode_supports(nh, nkv, d), "attention_decode: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
   GS_REQUIRE(nseq >= 0 && nseq <= 65535 && nkv <= 65535, "attention_decode: bad batch %d", nseq);
   GS_REQUIRE(nsplit >= 1 && nsplit <= 64, "attention_decode: %d splits outside [1, 64]", nsplit);
@@ -253,7 +251,7 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
   int rc = -1;
 #define GS_ARGS                                                                                                   \
   G, grid, stream, (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions, block_table,    \
-      max_blocks, page_size, window, scale, (bf16*)out, part_o, part_ml, counters, nh, nkv
+      max_blocks, page_size, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
   switch (d) {
     case 16: rc = launch_decode<16>(GS_ARGS); break;
     case 32: rc = launch_decode<32>(GS_ARGS); break;
@@ -263,5 +261,10 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
 #undef GS_ARGS
   GS_REQUIRE(rc == 0, "attention_decode: no kernel for group %d", G);
   GS_LAUNCH_CHECK("attention_decode");
+  if (nsplit > 1) {
+    dim3 mgrid(nkv, nseq);
+    attention_decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, (bf16*)out, nsplit, nh, nkv, G, d);
+    GS_LAUNCH_CHECK("attention_decode_merge");
+  }
   return 0;
 }

@@ -19,33 +19,45 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 1; }
+extern "C" int gs_abi_version() { return 2; }
 
 // ------------------------------------------------------------------ embedding
 
 // out[t, :] = table[ids[t], :] as float32; an id outside the table gives a NaN row.
+// With ssq: ssq[t] = sum of squares of the row (one partial sum per row, for a norm that follows).
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
-                             int H, int V) {
+                             float* __restrict__ ssq, int H, int V) {
+  __shared__ float red[17];
   int t = blockIdx.x;
   int id = ids[t];
   float* o = out + (size_t)t * H;
+  float ss = 0.f;
   if (id < 0 || id >= V) {
     for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = __uint_as_float(0x7fc00000u);
-    return;
+    ss = __uint_as_float(0x7fc00000u);
+  } else {
+    const T* row = table + (size_t)id * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+      float v = to_f32(row[j]);
+      o[j] = v;
+      ss += v * v;
+    }
   }
-  const T* row = table + (size_t)id * H;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = to_f32(row[j]);
+  if (ssq) {
+    ss = block_sum(ss, red);
+    if (threadIdx.x == 0) ssq[t] = ss;
+  }
 }
 
-extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, float* out, int T, int H, int V,
-                        hipStream_t stream) {
+extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, float* out, float* ssq, int T, int H,
+                        int V, hipStream_t stream) {
   GS_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
   if (T == 0) return 0;
   if (table_dtype == GS_F32)
-    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, H, V);
+    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, ssq, H, V);
   else if (table_dtype == GS_BF16)
-    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, H, V);
+    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, ssq, H, V);
   else
     GS_REQUIRE(false, "embed: unknown dtype %d", table_dtype);
   GS_LAUNCH_CHECK("embed");

@@ -82,11 +82,14 @@ class DecodeRunner:
 
     def _body(self) -> None:
         ops = self.engine.rt.ops
-        self.engine.rt.no_library = True
+        rt = self.engine.rt
+        rt.no_library = True
+        rt.fused = rt.dtype == torch.bfloat16
         try:
             logits = self.engine.model.forward(self.ctx)
         finally:
-            self.engine.rt.no_library = False
+            rt.no_library = rt.fused = False
+        self.logits = logits
         ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring)
         ops.decode_advance(self.pos, self.kv_len, self.live, self.counter)
 

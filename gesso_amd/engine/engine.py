@@ -144,8 +144,31 @@ class Engine:
             raise InvalidPlan(f"the recorded decode loop takes 1 to {self.DECODE_MAX_BATCH} requests, not {len(rids)}")
         if len(set(rids)) != len(rids) or len(tokens) != len(rids):
             raise InvalidPlan("one token per request, each request once")
+        if samplers is not None and any(s is not None and s.top_p < 1 for s in samplers):
+            raise InvalidPlan("nucleus sampling does not run in the recorded decode loop")
+        if not self.model.graph_safe:
+            return self._decode_eager(rids, tokens, n, samplers)
         cap = _capacity(len(rids))
         runner = self._runners.get(cap)
         if runner is None:
             runner = self._runners[cap] = DecodeRunner(self, cap)
         return runner.run(rids, tokens, n, samplers)
+
+    def _decode_eager(self, rids, tokens, n, samplers):
+        """The same steps one by one through :meth:`step`, for models with parts that cannot be recorded."""
+        import numpy as np
+        from ..sampling.sampler import choose
+        samplers = list(samplers) if samplers is not None else [None] * len(rids)
+        self.manager.reserve_many([(r, n) for r in rids])
+        ids = np.zeros((n, len(rids)), dtype=np.int32)
+        bad = np.zeros((n, len(rids)), dtype=np.int32)
+        tokens = [int(t) for t in tokens]
+        for s in range(n):
+            logits = self.step([StepEntry(r, [t], [0]) for r, t in zip(rids, tokens)])
+            picks = choose(self.rt.ops, logits, samplers)
+            for i, p in enumerate(picks):
+                if isinstance(p, Exception):
+                    bad[s, i] = 1
+                else:
+                    ids[s, i] = tokens[i] = p
+        return ids, bad

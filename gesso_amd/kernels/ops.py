@@ -67,16 +67,17 @@ def _i32(t, n=None, what="index"):
 
 # ---------------------------------------------------------------------- elementwise
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
-    """``out[t] = table[ids[t]]`` as float32 ``(T, H)``."""
-    _dev(ids, table, out)
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq: torch.Tensor = None) -> torch.Tensor:
+    """``out[t] = table[ids[t]]`` as float32 ``(T, H)``; with ``ssq (T, 1)`` also each row's sum of squares."""
+    _dev(ids, table, out, ssq)
     _i32(ids, what="token ids")
     V, H = table.shape
     T = ids.numel()
     if out is None:
         out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     _need(out.dtype == torch.float32 and out.shape == (T, H), "embed: out must be float32 (T, H)")
-    _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), c_int(T), c_int(H), c_int(V), _stream()))
+    _need(ssq is None or (ssq.dtype == torch.float32 and ssq.numel() == T), "embed: ssq must be float32 (T, 1)")
+    _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), _p(ssq), c_int(T), c_int(H), c_int(V), _stream()))
     return out
 
 
@@ -288,24 +289,119 @@ def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and w.is_contiguous() and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, swiglu: bool = False):
+class LazyNorm:
+    """An RMSNorm not yet applied: the float32 stream, its rows' sums of squares as partial sums, weight and eps.
+
+    The weight-streaming products take it in place of a tensor and norm on the fly; ``materialize``
+    runs the norm kernel for everything else.
+    """
+
+    __slots__ = ("res", "ssq", "weight", "eps", "dtype")
+
+    def __init__(self, res, ssq, weight, eps, dtype):
+        self.res, self.ssq, self.weight, self.eps, self.dtype = res, ssq, weight, eps, dtype
+
+    @property
+    def shape(self):
+        return self.res.shape
+
+    def materialize(self) -> torch.Tensor:
+        return add_rmsnorm(self.res, None, self.weight, self.eps, self.dtype)
+
+
+def lazy_ok(x, w: torch.Tensor) -> bool:
+    return (isinstance(x, LazyNorm) and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and x.res.shape[0] <= SKINNY_MAX_ROWS and x.res.shape[1] % 8 == 0 and x.res.is_contiguous()
+            and w.is_contiguous() and w.data_ptr() % 16 == 0 and x.res.data_ptr() % 16 == 0)
+
+
+def _lazy_args(x):
+    if isinstance(x, LazyNorm):
+        return (None, c_int(x.res.shape[1]), _p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps))
+    M, K = x.shape
+    return (_p(x), c_int(x.stride(0) if M > 1 else K), None, None, c_int(0), None, c_float(0.0))
+
+
+def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, swiglu: bool = False):
     """``x @ w.T`` for at most 64 rows, streaming the weights once; optionally ``silu(gate) * up`` of the result.
 
-    With ``swiglu`` the weight holds gate rows then up rows and the output is half as wide.
+    ``x`` is a bfloat16 tensor or a :class:`LazyNorm`.  With ``swiglu`` the weight holds gate rows then up
+    rows and the output is half as wide.
     """
     _dev(w, out)
-    _need(skinny_ok(x, w), "gemm_skinny: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
+    lazy = isinstance(x, LazyNorm)
+    _need(lazy_ok(x, w) if lazy else skinny_ok(x, w),
+          "gemm_skinny: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
     M, K = x.shape
     N = w.shape[0]
     _need(w.shape == (N, K), f"gemm_skinny: weight is {tuple(w.shape)}, expected ({N}, {K})")
     cols = N // 2 if swiglu else N
     if out is None:
-        out = torch.empty((M, cols), dtype=out_dtype or x.dtype, device=x.device)
+        out = torch.empty((M, cols), dtype=out_dtype or torch.bfloat16, device=w.device)
     _need(out.shape == (M, cols) and out.stride(1) == 1, "gemm_skinny: out has the wrong shape")
-    _check(lib().gs_gemm_skinny(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(out), c_int(_dt(out)),
+    _check(lib().gs_gemm_skinny(*_lazy_args(x), _p(w), _p(out), c_int(_dt(out)),
                                 c_int(out.stride(0) if M > 1 else cols), c_int(M), c_int(N), c_int(K),
                                 c_int(1 if swiglu else 0), _stream()))
     return out
+
+
+def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor) -> torch.Tensor:
+    """``res += x @ w.T`` in place (float32); returns the new rows' sums of squares as partial sums ``(M, nb)``."""
+    _dev(w, res)
+    _need(skinny_ok(x, w), "gemm_skinny_residual: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape == (N, K) and res.shape == (M, N) and res.dtype == torch.float32, "gemm_skinny_residual: shapes")
+    nb = lib().gs_gemm_skinny_residual_blocks(c_int(N))
+    ssq = torch.empty((M, nb), dtype=torch.float32, device=res.device)
+    _check(lib().gs_gemm_skinny_residual(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(res), _p(ssq), c_int(M),
+                                         c_int(N), c_int(K), _stream()))
+    return ssq
+
+
+def gemm_skinny_conv(x: "LazyNorm", w_in, taps, bias, state, slots) -> torch.Tensor:
+    """A decode step's gated short convolution fused into its input product; ``state`` is advanced."""
+    _dev(w_in, taps, bias, state, slots)
+    _need(lazy_ok(x, w_in), "gemm_skinny_conv: needs a lazy norm and a bfloat16 weight")
+    M, K = x.shape
+    H, W = taps.shape
+    _need(w_in.shape == (3 * H, K), "gemm_skinny_conv: the input weight must be (3H, K)")
+    _need(taps.dtype == torch.float32 and state.dtype == torch.float32 and state.shape[1:] == (H, W - 1),
+          "gemm_skinny_conv: taps float32 (H, W), state float32 (slots, H, W-1)")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (H,)), "gemm_skinny_conv: bias float32 (H,)")
+    _i32(slots, M, "slots")
+    out = torch.empty((M, H), dtype=torch.bfloat16, device=w_in.device)
+    _check(lib().gs_gemm_skinny_conv(_p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps),
+                                     _p(w_in), _p(taps), _p(bias), _p(state), _p(slots), c_int(W), _p(out), c_int(M),
+                                     c_int(H), c_int(K), _stream()))
+    return out
+
+
+def gemm_skinny_qkv_supports(d: int, rotary_dim: int) -> bool:
+    return bool(lib().gs_gemm_skinny_qkv_supports(c_int(d), c_int(rotary_dim)))
+
+
+def gemm_skinny_qkv(x: "LazyNorm", wqkv, q_weight, k_weight, head_eps, cos, sin, positions, block_table, page_size,
+                    kcache, vcache, nh, nkv, d, write_kv=True) -> torch.Tensor:
+    """A decode step's q, k, v: product, head norms, rotation and cache write in one kernel; returns q ``(M, nh d)``."""
+    _dev(wqkv, q_weight, k_weight, cos, sin, positions, block_table, kcache, vcache)
+    _need(lazy_ok(x, wqkv), "gemm_skinny_qkv: needs a lazy norm and a bfloat16 weight")
+    M, K = x.shape
+    _need(wqkv.shape == ((nh + 2 * nkv) * d, K), "gemm_skinny_qkv: the weight must be ((nh + 2 nkv) d, K)")
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "gemm_skinny_qkv: head norm weight float32 (d,)")
+    _need(cos.dtype == torch.float32 and cos.shape == sin.shape and cos.shape[1] == d // 2, "gemm_skinny_qkv: tables (P, d/2)")
+    _i32(positions, M, "positions")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= M, "block_table int32 (M, blocks)")
+    _need(kcache.dtype == torch.bfloat16 and kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d)
+          and vcache.shape == kcache.shape, "cache must be bfloat16 (pages, nkv, page_size, d)")
+    q = torch.empty((M, nh * d), dtype=torch.bfloat16, device=wqkv.device)
+    _check(lib().gs_gemm_skinny_qkv(_p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps), _p(wqkv),
+                                    _p(q_weight), _p(k_weight), c_float(head_eps), _p(cos), _p(sin), _p(positions),
+                                    _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
+                                    _p(vcache), c_int(1 if write_kv else 0), _p(q), c_int(M), c_int(nh), c_int(nkv),
+                                    c_int(d), c_int(K), _stream()))
+    return q
 
 
 def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring) -> None:
@@ -356,13 +452,12 @@ def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_s
         n = lib().gs_attention_decode_workspace
         n.restype = c_long
         floats = n(c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit))
-        ws = _decode_ws[key] = (torch.empty(floats, dtype=torch.float32, device=q.device),
-                                torch.zeros(nseq * nkv, dtype=torch.int32, device=q.device))
+        ws = _decode_ws[key] = torch.empty(max(1, floats), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty((nseq, nh * d), dtype=q.dtype, device=q.device)
     _need(out.shape == (nseq, nh * d) and out.dtype == q.dtype, "attention_decode: out has the wrong shape or type")
     _check(lib().gs_attention_decode(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
                                      c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
-                                     _p(out), _p(ws[0]), _p(ws[1]), c_int(nseq), c_int(nh), c_int(nkv), c_int(d),
-                                     c_int(nsplit), _stream()))
+                                     _p(out), _p(ws), c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit),
+                                     _stream()))
     return out

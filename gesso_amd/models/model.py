@@ -75,13 +75,23 @@ class Model:
             local = {k: tensors[b.names[k]] for k in part_class("block", b).tensor_specs(b)}
             block.bind(local)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
+
     def forward(self, ctx) -> Optional[torch.Tensor]:
         """Run the tokens of ``ctx`` through every scheduled block; float32 logits at ``ctx.want_rows``."""
-        ops = self.rt.ops
-        stream = ResidualStream(ops.embed(ctx.token_ids, self.embed))
+        ops, rt = self.rt.ops, self.rt
+        if rt.fused:
+            ssq = torch.empty((ctx.T, 1), dtype=torch.float32, device=rt.device)
+            stream = ResidualStream(ops.embed(ctx.token_ids, self.embed, ssq=ssq), ssq=ssq)
+        else:
+            stream = ResidualStream(ops.embed(ctx.token_ids, self.embed))
         for i, call in enumerate(self.spec.schedule):
             self.blocks[call.layer].forward(stream, ctx, ctx.cache_view(i))
         if ctx.n_want == 0:
             return None
-        normed = self.final_norm.add_norm(stream, rows=ctx.want_rows)
+        # every row wanted, in order (a decode step): no gather, and the norm may stay lazy
+        rows = None if getattr(ctx, "decode_only", False) else ctx.want_rows
+        normed = self.final_norm.add_norm(stream, rows=rows)
         return self.rt.linear(normed, self.head, out_dtype=torch.float32)

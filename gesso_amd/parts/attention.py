@@ -18,6 +18,8 @@ from .registry import build, register
 
 
 class Attention(Part):
+    graph_safe = True
+
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         if spec.n_heads % spec.n_kv_heads:
@@ -56,15 +58,13 @@ class Attention(Part):
         self.k_norm = tensors.get("k_norm.weight")
 
     def forward(self, x, ctx, cache):
-        s, ops = self.spec, self.rt.ops
+        s = self.spec
         nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
-        qkv = self.rt.linear(x, self.wqkv, self.bqkv)
-        pos = self.position
-        ops.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, s.qk_norm.eps if s.qk_norm is not None else 1.0,
-                           pos.cos, pos.sin, pos.rotary_dim, ctx.positions, ctx.seq_of_token, cache.block_table,
-                           cache.page_size, cache.k, cache.v, nh, nkv, d, write_kv=cache.write)
-        o = self.rt.attention(qkv, (nh + 2 * nkv) * d, cache, ctx, s.window, self.scale, nh, nkv, d)
-        return self.rt.linear(o, self.wo, self.bo)
+        q, q_stride = self.rt.attention_in(x, self.wqkv, self.bqkv, self.q_norm, self.k_norm,
+                                           s.qk_norm.eps if s.qk_norm is not None else 1.0, self.position, ctx,
+                                           cache, nh, nkv, d)
+        o = self.rt.attention(q, q_stride, cache, ctx, s.window, self.scale, nh, nkv, d)
+        return self.rt.project(o, self.wo, self.bo)
 
 
 register("mixer", "attention", Attention)

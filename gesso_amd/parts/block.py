@@ -2,7 +2,8 @@
 
 ``prenorm``: ``h += mixer(norm_a(h)); h += ffn(norm_b(h))`` (reference
 ``src/Inference/Inference.jl:270-363``).  Each add is folded into the norm that follows it;
-the model adds what is still pending after the last block.  Another arrangement (post-norms on
+the model adds what is still pending after the last block.  A sub-layer may return a tensor or a
+deferred product (its last projection, computed straight into the stream).  Another arrangement (post-norms on
 sub-layer outputs, a parallel block) is another class registered under another kind.
 """
 from __future__ import annotations
@@ -46,10 +47,16 @@ class PreNormBlock(Part):
 
     def forward(self, stream, ctx, cache):
         x = self.mixer_norm.add_norm(stream)
-        stream.pending = self.mixer.forward(x, ctx, cache)
+        stream.push(self.mixer.forward(x, ctx, cache), self.rt)
         if self.ffn is not None:
             x = self.ffn_norm.add_norm(stream)
-            stream.pending = self.ffn.forward(x, ctx)
+            stream.push(self.ffn.forward(x, ctx), self.rt)
+
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a step through this block may be recorded into a HIP graph (no host round trips inside)."""
+        parts = [self.mixer_norm, self.mixer] + ([self.ffn_norm, self.ffn] if self.ffn is not None else [])
+        return all(getattr(p, "graph_safe", False) for p in parts)
 
 
 register("block", "prenorm", PreNormBlock)

@@ -22,6 +22,8 @@ def rope_tables(rotary_dim: int, theta: float, max_position: int):
 
 
 class Rope(Part):
+    graph_safe = True
+
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         if spec.rotary_dim % 2 or not 0 < spec.rotary_dim <= spec.head_dim:
@@ -36,6 +38,7 @@ class Rope(Part):
 
 
 class NoPosition(Part):
+    graph_safe = True
     rotary_dim = 0
     cos = None
     sin = None

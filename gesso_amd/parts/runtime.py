@@ -15,6 +15,15 @@ import torch
 from ..errors import KernelError
 
 
+class DeferredLinear:
+    """A sub-layer's last product, not yet computed: ``x @ w.T`` to be added to the residual stream."""
+
+    __slots__ = ("x", "w")
+
+    def __init__(self, x, w):
+        self.x, self.w = x, w
+
+
 class Runtime:
     def __init__(self, device, dtype: torch.dtype):
         if dtype not in (torch.float32, torch.bfloat16):
@@ -28,6 +37,7 @@ class Runtime:
         self.dtype = dtype
         self._shared = {}
         self.no_library = False        # set while a HIP graph is recorded: only our own kernels go into it
+        self.fused = False             # set while a decode step is recorded: norms, adds and small ops fold into products
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""
@@ -35,21 +45,74 @@ class Runtime:
             self._shared[key] = make()
         return self._shared[key]
 
-    def linear(self, x: torch.Tensor, w: torch.Tensor, bias=None, out_dtype=None, out=None) -> torch.Tensor:
-        """``x @ w.T (+ bias)``; ``w (out, in)``."""
-        out_dtype = out_dtype or x.dtype
+    # ------------------------------------------------------------------ matrix products
+
+    def _dense(self, x):
+        return x.materialize() if isinstance(x, self.ops.LazyNorm) else x
+
+    def linear(self, x, w: torch.Tensor, bias=None, out_dtype=None, out=None) -> torch.Tensor:
+        """``x @ w.T (+ bias)``; ``w (out, in)``; ``x`` a tensor or a lazy norm."""
+        ops = self.ops
+        out_dtype = out_dtype or self.dtype
+        if isinstance(x, ops.LazyNorm):
+            if bias is None and ops.lazy_ok(x, w):
+                return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out)
+            x = x.materialize()
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
-            if self.ops.skinny_ok(x, w):
-                return self.ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out)
+            if ops.skinny_ok(x, w):
+                return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out)
             if out_dtype == torch.bfloat16 and not self.no_library:
                 return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
-        return self.ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
+        return ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
 
-    def linear_swiglu(self, x: torch.Tensor, w13: torch.Tensor) -> torch.Tensor:
+    def linear_swiglu(self, x, w13: torch.Tensor) -> torch.Tensor:
         """``silu(x @ w1.T) * (x @ w3.T)`` with ``w13`` holding w1's rows, then w3's."""
-        if self.ops.skinny_ok(x, w13):
-            return self.ops.gemm_skinny(x, w13, swiglu=True)
-        return self.ops.swiglu(self.linear(x, w13))
+        ops = self.ops
+        if isinstance(x, ops.LazyNorm):
+            if ops.lazy_ok(x, w13):
+                return ops.gemm_skinny(x, w13, swiglu=True)
+            x = x.materialize()
+        if ops.skinny_ok(x, w13):
+            return ops.gemm_skinny(x, w13, swiglu=True)
+        return ops.swiglu(self.linear(x, w13))
+
+    def project(self, x: torch.Tensor, w: torch.Tensor, bias=None):
+        """A sub-layer's last product.  While fused kernels are on it is deferred, so that the block can
+        compute it straight into the residual stream; else it is computed here."""
+        if self.fused and bias is None and self.ops.skinny_ok(x, w):
+            return DeferredLinear(x, w)
+        return self.linear(x, w, bias)
+
+    # ------------------------------------------------------------------ mixers' inner steps
+
+    def conv_in(self, x, w_in, b_in, taps, b_conv, state, ctx) -> torch.Tensor:
+        """Input product and gated short convolution: ``(T, H)`` mixed rows; ``state`` is advanced."""
+        ops = self.ops
+        if isinstance(x, ops.LazyNorm):
+            if b_in is None and ctx.all_single and ops.lazy_ok(x, w_in) and taps.shape[1] <= 16:
+                return ops.gemm_skinny_conv(x, w_in, taps, b_conv, state, ctx.slots)
+            x = x.materialize()
+        bcx = self.linear(x, w_in, b_in)
+        return ops.short_conv(bcx, taps, b_conv, state, ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq,
+                              ctx.all_single)
+
+    def attention_in(self, x, wqkv, bqkv, q_norm, k_norm, head_eps, position, ctx, cache, nh, nkv, d):
+        """q, k, v products, head norms, position encoding, cache write.  Returns ``(q, q_stride)``:
+        the queries as rows of a buffer, ``q_stride`` apart, head h at ``[h d, (h+1) d)``."""
+        ops = self.ops
+        if isinstance(x, ops.LazyNorm):
+            if (bqkv is None and ctx.all_single and ops.lazy_ok(x, wqkv) and cache.k.dtype == torch.bfloat16
+                    and ops.gemm_skinny_qkv_supports(d, position.rotary_dim)):
+                q = ops.gemm_skinny_qkv(x, wqkv, q_norm, k_norm, head_eps, position.cos, position.sin, ctx.positions,
+                                        cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
+                                        write_kv=cache.write)
+                return q, nh * d
+            x = x.materialize()
+        qkv = self.linear(x, wqkv, bqkv)
+        ops.qknorm_rope_kv(qkv, q_norm, k_norm, head_eps, position.cos, position.sin, position.rotary_dim,
+                           ctx.positions, ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v,
+                           nh, nkv, d, write_kv=cache.write)
+        return qkv, (nh + 2 * nkv) * d
 
     def attention(self, q, q_stride, cache, ctx, window, scale, nh, nkv, d) -> torch.Tensor:
         """Causal attention of this step's queries over the paged cache; ``(T, nh * d)``.
@@ -60,7 +123,7 @@ class Runtime:
         ops = self.ops
         if ctx.all_single and q.dtype == torch.bfloat16 and ops.attention_decode_supports(nh, nkv, d):
             # one query per sequence: the key stream is split so that the whole chip reads it
-            nsplit = max(1, min(16, 512 // max(1, ctx.nseq * nkv)))
+            nsplit = max(1, min(16, 64 // max(1, ctx.nseq * nkv)))
             return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                         cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
         return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,

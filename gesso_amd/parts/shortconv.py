@@ -14,6 +14,8 @@ from .registry import register
 
 
 class ShortConv(Part):
+    graph_safe = True
+
     @staticmethod
     def tensor_specs(spec):
         H, W = spec.hidden, spec.width
@@ -38,10 +40,8 @@ class ShortConv(Part):
         self.b_out = tensors.get("out_proj.bias")
 
     def forward(self, x, ctx, cache):
-        bcx = self.rt.linear(x, self.w_in, self.b_in)
-        mixed = self.rt.ops.short_conv(bcx, self.taps, self.b_conv, cache.state["history"], ctx.seq_of_token,
-                                       ctx.q_start, ctx.slots, ctx.nseq, ctx.all_single)
-        return self.rt.linear(mixed, self.w_out, self.b_out)
+        mixed = self.rt.conv_in(x, self.w_in, self.b_in, self.taps, self.b_conv, cache.state["history"], ctx)
+        return self.rt.project(mixed, self.w_out, self.b_out)
 
 
 register("mixer", "short_conv", ShortConv)

@@ -13,6 +13,8 @@ from .registry import register
 
 
 class SwiGLU(Part):
+    graph_safe = True
+
     @staticmethod
     def tensor_specs(spec):
         H, F = spec.hidden, spec.intermediate
@@ -28,7 +30,7 @@ class SwiGLU(Part):
 
     def forward(self, x, ctx):
         a = self.rt.linear_swiglu(x, self.w13)
-        return self.rt.linear(a, self.w2)
+        return self.rt.project(a, self.w2)
 
 
 register("ffn", "swiglu", SwiGLU)

@@ -444,3 +444,102 @@ def test_attention_decode(ops, nh, nkv, d, ps, nsplit, window):
 def test_attention_decode_supports(ops):
     assert ops.attention_decode_supports(32, 8, 64) and ops.attention_decode_supports(3, 1, 32)
     assert not ops.attention_decode_supports(3, 3, 48) and not ops.attention_decode_supports(18, 2, 64)
+
+
+# ------------------------------------------------------------------ the decode step's fused products
+
+def lazy_case(ops, M, K, seed):
+    g = gen(seed)
+    res = torch.randn(M, K, generator=g)
+    nw = 1 + 0.1 * torch.randn(K, generator=g)
+    nb = 5
+    part = torch.rand(M, nb, generator=g)
+    part = part / part.sum(1, keepdim=True) * (res * res).sum(1, keepdim=True)      # partial sums of the true sums
+    lazy = ops.LazyNorm(res.to(DEV), part.to(DEV), nw.to(DEV), 1e-5, torch.bfloat16)
+    return res, nw, lazy
+
+
+@pytest.mark.parametrize("M", [1, 8, 33, 64])
+@pytest.mark.parametrize("N,K", [(2048, 2048), (100, 96), (6144, 2048)])
+def test_gemm_skinny_with_lazy_norm(ops, M, N, K):
+    res, nw, lazy = lazy_case(ops, M, K, M + N)
+    w = (torch.randn(N, K, generator=gen(N)) / math.sqrt(K)).bfloat16()
+    normed = ops.add_rmsnorm(res.clone().to(DEV), None, nw.to(DEV), 1e-5, torch.bfloat16)
+    want = ops.gemm_skinny(normed, w.to(DEV), out_dtype=torch.float32).double().cpu()
+    got = ops.gemm_skinny(lazy, w.to(DEV), out_dtype=torch.float32).double().cpu()
+    # the same rounded inputs but for the last bit of the inverse root: float32 sums apart by rounding only
+    assert float((got - want).abs().max()) <= 2e-3 * max(1.0, float(want.abs().max()))
+    ref = P.rmsnorm(res.double(), nw.double(), 1e-5) @ w.double().T
+    close(ops.gemm_skinny(lazy, w.to(DEV)), ref, torch.bfloat16)
+    if N % 2 == 0:
+        close(ops.gemm_skinny(lazy, w.to(DEV), swiglu=True), P.swiglu(ref[:, :N // 2], ref[:, N // 2:]), torch.bfloat16, scale=2)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (40, 96, 320), (64, 144, 104)])
+def test_gemm_skinny_residual(ops, M, N, K):
+    g = gen(M + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    res = torch.randn(M, N, generator=g)
+    r = res.clone().to(DEV)
+    ssq = ops.gemm_skinny_residual(x.to(DEV), w.to(DEV), r)
+    want = res.double() + (x.double() @ w.double().T)
+    close(r, want, torch.bfloat16)                       # the product is rounded to bfloat16 before the add
+    assert ssq.shape[0] == M
+    total = ssq.double().sum(1).cpu()
+    assert torch.allclose(total, (r.double().cpu() ** 2).sum(1), rtol=1e-5)
+    # and the partial sums feed a lazy norm that equals the norm kernel on the new stream
+    nw = torch.ones(N)
+    lazy = ops.LazyNorm(r, ssq, nw.to(DEV), 1e-5, torch.bfloat16)
+    if N % 8 == 0:
+        eye = torch.eye(N).bfloat16().to(DEV)
+        a = ops.gemm_skinny(lazy, eye, out_dtype=torch.float32)
+        b = ops.add_rmsnorm(r.clone(), None, nw.to(DEV), 1e-5, torch.bfloat16).float()
+        assert float((a - b).abs().max()) <= 1e-2 * float(b.abs().max())
+
+
+@pytest.mark.parametrize("M,H,W,bias", [(1, 64, 3, False), (8, 2048, 3, False), (20, 96, 4, True), (64, 48, 2, False)])
+def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias):
+    res, nw, lazy = lazy_case(ops, M, H, M + H)
+    g = gen(H + W)
+    w_in = (torch.randn(3 * H, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
+    taps = torch.randn(H, W, generator=g).to(DEV)
+    b = torch.randn(H, generator=g).to(DEV) if bias else None
+    state0 = torch.randn(M + 2, H, W - 1, generator=g)
+    slots = torch.randperm(M + 2, generator=g)[:M].to(torch.int32).to(DEV)
+    s1, s2 = state0.clone().to(DEV), state0.clone().to(DEV)
+    got = ops.gemm_skinny_conv(lazy, w_in, taps, b, s1, slots)
+    bcx = ops.gemm_skinny(lazy, w_in)
+    ar = torch.arange(M, dtype=torch.int32, device=DEV)
+    want = ops.short_conv(bcx, taps, b, s2, ar, torch.arange(M + 1, dtype=torch.int32, device=DEV), slots, M, True)
+    assert float((got.float() - want.float()).abs().max()) <= 1e-2 * max(1.0, float(want.float().abs().max()))
+    assert float((s1 - s2).abs().max()) <= 1e-2 * max(1.0, float(s2.abs().max()))
+    untouched = [i for i in range(M + 2) if i not in slots.tolist()]
+    assert torch.equal(s1[untouched].cpu(), state0[untouched])
+
+
+@pytest.mark.parametrize("M,nh,nkv,d,norm", [(1, 32, 8, 64, True), (8, 4, 2, 32, True), (33, 2, 1, 128, False), (64, 3, 3, 64, True)])
+def test_gemm_skinny_qkv_equals_the_separate_kernels(ops, M, nh, nkv, d, norm):
+    H = nh * d
+    res, nw, lazy = lazy_case(ops, M, H, M + H)
+    g = gen(nh + d)
+    wqkv = (torch.randn((nh + 2 * nkv) * d, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
+    qw = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV) if norm else None
+    kw = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV) if norm else None
+    ps = 16
+    cos, sin = rope_tables(d, 1e4, 256)
+    positions = torch.randint(0, 200, (M,), generator=g).to(torch.int32)
+    table = torch.zeros(M, 13, dtype=torch.int32)
+    for m in range(M):
+        table[m] = torch.arange(13, dtype=torch.int32) + 13 * m
+    kc1 = torch.zeros(13 * M, nkv, ps, d, dtype=torch.bfloat16, device=DEV)
+    vc1, kc2, vc2 = torch.zeros_like(kc1), torch.zeros_like(kc1), torch.zeros_like(kc1)
+    q = ops.gemm_skinny_qkv(lazy, wqkv, qw, kw, 1e-5, cos, sin, positions.to(DEV), table.to(DEV), ps, kc1, vc1, nh, nkv, d)
+    qkv = ops.gemm_skinny(lazy, wqkv)
+    ops.qknorm_rope_kv(qkv, qw, kw, 1e-5, cos, sin, d, positions.to(DEV), torch.arange(M, dtype=torch.int32, device=DEV),
+                       table.to(DEV), ps, kc2, vc2, nh, nkv, d)
+    ref_q = qkv[:, :nh * d].float()
+    assert float((q.float() - ref_q).abs().max()) <= 2e-2 * max(1.0, float(ref_q.abs().max()))
+    assert float((kc1.float() - kc2.float()).abs().max()) <= 2e-2 * max(1.0, float(kc2.float().abs().max()))
+    assert float((vc1.float() - vc2.float()).abs().max()) <= 2e-2 * max(1.0, float(vc2.float().abs().max()))
+    assert int((kc1.float().abs().sum(dim=(1, 3)) > 0).sum()) == M      # one row per token, nothing else
