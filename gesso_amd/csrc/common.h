@@ -41,16 +41,10 @@ struct bf16 {
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(bf16 v) { return __uint_as_float(((uint32_t)v.x) << 16); }
 
-// round to nearest, ties to even; NaN stays NaN
+// round to nearest, ties to even; NaN stays NaN (gfx950 converts in hardware: v_cvt_pk_bf16_f32)
 __device__ __forceinline__ bf16 f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
   bf16 r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {
-    r.x = (uint16_t)((u >> 16) | 0x40);
-    return r;
-  }
-  u += 0x7fffu + ((u >> 16) & 1u);
-  r.x = (uint16_t)(u >> 16);
+  r.x = __builtin_bit_cast(uint16_t, (__bf16)f);
   return r;
 }
 

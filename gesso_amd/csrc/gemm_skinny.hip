@@ -1,389 +1,13 @@
-// Y (M, N) = X (M, K) . W (N, K)^T for few rows (M <= 64): the weight-streaming product of decoding,
-// with what stands before and after it in a block folded in.
+// Entry points of the weight-streaming products (see gemm_skinny_impl.h for the kernel).
 //
-// Every weight is read once from HBM; the time of this kernel is the time of that stream.  bfloat16
-// inputs, float32 accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).  One MFMA takes a 16 x 32
-// tile of W as its A operand, straight from global memory in the operand's own layout (lane l: row
-// l % 16, eight consecutive k at 8 * (l / 16): one 16-byte load), and a 32 x 16 tile of X^T as its B
-// operand (lane l: token l % 16, the same eight k).  The result tile holds, per lane, four consecutive
-// output columns n for one token.
-//
-// A block of WAVES wavefronts owns R tiles of 16 rows of W; its wavefronts split K among themselves and
-// add their partial tiles through LDS in wavefront order.  Rows beyond N, tokens beyond M and k beyond K
-// are masked (K must be a multiple of 8 so that every 16-byte load is aligned).
-//
-// What feeds X (PRO):
-//   0  X is given, bfloat16.
-//   1  X is the RMSNorm of the float32 residual stream: x = res * inv_rms(row) * norm_weight, rounded to
-//      bfloat16 as the norm kernel would store it; the row's sum of squares comes as partial sums
-//      (row, nb), added in a fixed order.
-// What is done with Y (EPI):
-//   0  stored (bfloat16 or float32).
-//   1  SwiGLU: W holds gate rows [0, N/2) then up rows; stores silu(gate) * up, N/2 wide.
-//   2  added to the residual stream in place (float32), and the sums of squares of the new rows over this
-//      block's columns stored as partial sums for the next norm.
-//   3  gated short convolution of a decode step: tiles are the B, C, X rows of 16 channels; u = B X,
-//      y = taps . (history, u) + bias, out = C y, history shifted; one token per sequence.
-//   4  attention input of a decode step: the block owns one head (R = d / 16 tiles); per-head RMSNorm of
-//      q and k heads, half-split rotation, q stored, k and v written into the cache page.
+// Each takes the weight as stored, W (N, K), and optionally its tile-major copy Wt; with Wt the
+// kernels read that copy.  A tile-major copy exists only for K a multiple of 32 and row tiles that
+// do not straddle a boundary of the epilogue (N, N/2 or N/3 a multiple of 16).
 #include "common.h"
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-
-__device__ __forceinline__ bf16x8_t load8(const bf16* p) { return *reinterpret_cast<const bf16x8_t*>(p); }
-
-__device__ __forceinline__ bf16x8_t zero8() {
-  bf16x8_t z;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
-  return z;
-}
-
-template <typename T>
-__device__ __forceinline__ void store4(T* p, f32x4_t v, int valid);
-template <>
-__device__ __forceinline__ void store4<float>(float* p, f32x4_t v, int valid) {
-  if (valid >= 4 && ((uintptr_t)p & 15) == 0) {
-    *reinterpret_cast<f32x4_t*>(p) = v;
-  } else {
-    for (int i = 0; i < valid && i < 4; ++i) p[i] = v[i];
-  }
-}
-template <>
-__device__ __forceinline__ void store4<bf16>(bf16* p, f32x4_t v, int valid) {
-  if (valid >= 4 && ((uintptr_t)p & 7) == 0) {
-    uint2 o;
-    o.x = (uint32_t)f32_to_bf16(v[0]).x | ((uint32_t)f32_to_bf16(v[1]).x << 16);
-    o.y = (uint32_t)f32_to_bf16(v[2]).x | ((uint32_t)f32_to_bf16(v[3]).x << 16);
-    *reinterpret_cast<uint2*>(p) = o;
-  } else {
-    for (int i = 0; i < valid && i < 4; ++i) p[i] = f32_to_bf16(v[i]);
-  }
-}
-
-// Everything the prologues and epilogues need beside X, W, Y; unused fields stay null.
-struct SkinnyExtra {
-  // PRO 1
-  const float* res;      // (M, K) float32 residual stream
-  const float* ssq;      // (M, nb) partial sums of squares of res rows
-  int nb;
-  const float* norm_w;   // (K)
-  float eps;
-  // EPI 2
-  float* res_out;        // (M, N) float32, updated in place
-  float* ssq_out;        // (M, gridDim.x)
-  // EPI 3
-  const float* taps;     // (H, W)
-  const float* conv_bias;
-  float* state;          // (slots, H, W - 1)
-  const int* slots;      // (M)
-  int conv_w;
-  // EPI 4
-  const float* qw;       // (d) or null
-  const float* kw;
-  float head_eps;
-  const float* cos_t;    // (positions, d / 2)
-  const float* sin_t;
-  const int* positions;  // (M)
-  const int* block_table;
-  int max_blocks, page_size, nh, nkv, write_kv;
-  bf16* kcache;
-  bf16* vcache;
-};
-
-template <int R, int MT, int WAVES, int PRO, int EPI, typename TOut>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __restrict__ X, int ldx,
-                                                                  const bf16* __restrict__ W,
-                                                                  TOut* __restrict__ Y, int ldy, int M, int N,
-                                                                  int K, SkinnyExtra ex) {
-  extern __shared__ float red[];  // (WAVES - 1) x R x MT x 64 x 4 floats
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r16 = lane & 15, kg = lane >> 4;
-  const int half = N >> 1;
-  // rows of W this block owns
-  int rowbase[R];
-  if (EPI == 1) {
-    const int n0 = blockIdx.x * 16 * (R / 2);
-#pragma unroll
-    for (int r = 0; r < R; ++r) rowbase[r] = n0 + (r >> 1) * 16 + ((r & 1) ? half : 0);
-  } else if (EPI == 3) {
-    const int H = N / 3;
-#pragma unroll
-    for (int r = 0; r < R; ++r) rowbase[r] = blockIdx.x * 16 + r * H;  // B, C, X rows of the same channels
-  } else {
-    const int n0 = blockIdx.x * 16 * R;
-#pragma unroll
-    for (int r = 0; r < R; ++r) rowbase[r] = n0 + r * 16;
-  }
-  const bf16* wrow[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    int n = rowbase[r] + r16;
-    if (EPI == 1 && !(r & 1) && n >= half) n = half - 1;  // gate rows end at N/2
-    if (EPI == 3 && n >= (r + 1) * (N / 3)) n = (r + 1) * (N / 3) - 1;
-    if (n >= N) n = N - 1;                                // clamped: loaded, never stored
-    wrow[r] = W + (size_t)n * K;
-  }
-  bool xok[MT];
-  const bf16* xrow[MT];
-  const float* rrow[MT];
-  float inv[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int m = mt * 16 + r16;
-    xok[mt] = m < M;
-    xrow[mt] = nullptr;
-    rrow[mt] = nullptr;
-    inv[mt] = 0.f;
-    if (PRO == 0) {
-      xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * ldx;
-    } else {
-      rrow[mt] = ex.res + (size_t)(xok[mt] ? m : 0) * K;
-      // the row's sum of squares: this lane group adds every fourth partial, then the four groups are added
-      float s = 0.f;
-      if (xok[mt])
-        for (int b = kg; b < ex.nb; b += 4) s += ex.ssq[(size_t)m * ex.nb + b];
-      s += __shfl_xor(s, 16, 64);
-      s += __shfl_xor(s, 32, 64);
-      inv[mt] = 1.0f / sqrtf(s / (float)K + ex.eps);
-    }
-  }
-
-  f32x4_t acc[R][MT];
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-  auto load_x = [&](int mt, int k) -> bf16x8_t {
-    if (PRO == 0) {
-      return load8(xrow[mt] + k);
-    } else {
-      const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(rrow[mt] + k);
-      const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(rrow[mt] + k + 4);
-      const f32x4_t w0 = *reinterpret_cast<const f32x4_t*>(ex.norm_w + k);
-      const f32x4_t w1 = *reinterpret_cast<const f32x4_t*>(ex.norm_w + k + 4);
-      union {
-        bf16x8_t v;
-        uint16_t u[8];
-      } o;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        o.u[i] = f32_to_bf16(a0[i] * inv[mt] * w0[i]).x;
-        o.u[4 + i] = f32_to_bf16(a1[i] * inv[mt] * w1[i]).x;
-      }
-      return o.v;
-    }
-  };
-
-  // this wavefront's share of K, in steps of 32
-  const int ksteps = (K + 31) >> 5;
-  const int per = (ksteps + WAVES - 1) / WAVES;
-  const int s0 = wave * per, s1 = (s0 + per < ksteps) ? s0 + per : ksteps;
-  int s = s0;
-  constexpr int U = (R * MT <= 4) ? 4 : 2;  // steps whose loads are issued together
-  if ((K & 31) == 0) {
-    for (; s + U <= s1; s += U) {
-      bf16x8_t a[U][R], b[U][MT];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int k = ((s + u) << 5) + kg * 8;
-#pragma unroll
-        for (int r = 0; r < R; ++r) a[u][r] = load8(wrow[r] + k);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) b[u][mt] = xok[mt] ? load_x(mt, k) : zero8();
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r], b[u][mt], acc[r][mt], 0, 0, 0);
-    }
-  }
-  for (; s < s1; ++s) {
-    const int k = (s << 5) + kg * 8;
-    const bool kin = k < K;
-    bf16x8_t b[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) b[mt] = (kin && xok[mt]) ? load_x(mt, k) : zero8();
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      bf16x8_t a = kin ? load8(wrow[r] + k) : zero8();
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[mt], acc[r][mt], 0, 0, 0);
-    }
-  }
-
-  // add the wavefronts' partial tiles: wave 0 keeps its own, the others pass theirs through LDS
-  if (WAVES > 1) {
-    if (wave > 0) {
-      float* dst = red + ((size_t)(wave - 1) * R * MT) * 256;
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-          *reinterpret_cast<f32x4_t*>(dst + ((r * MT + mt) * 64 + lane) * 4) = acc[r][mt];
-    }
-    __syncthreads();
-    if (wave > 0) return;
-    for (int w = 0; w < WAVES - 1; ++w) {
-      const float* src = red + ((size_t)w * R * MT) * 256;
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          f32x4_t v = *reinterpret_cast<const f32x4_t*>(src + ((r * MT + mt) * 64 + lane) * 4);
-          acc[r][mt] += v;
-        }
-    }
-  }
-
-  // lane l holds, for token mt*16 + l%16, columns rowbase + 4*(l/16) + 0..3 of every tile
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + r16;
-    const bool live = m < M;
-    if (EPI == 0) {
-      if (!live) continue;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int n = rowbase[r] + kg * 4;
-        if (N - n > 0) store4<TOut>(Y + (size_t)m * ldy + n, acc[r][mt], N - n);
-      }
-    } else if (EPI == 1) {
-      if (!live) continue;
-#pragma unroll
-      for (int r = 0; r < R; r += 2) {
-        const int n = rowbase[r] + kg * 4;  // output column in [0, N/2)
-        f32x4_t g = acc[r][mt], u = acc[r + 1][mt], o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = g[i] / (1.0f + expf(-g[i])) * u[i];
-        if (half - n > 0) store4<TOut>(Y + (size_t)m * ldy + n, o, half - n);
-      }
-    } else if (EPI == 2) {
-      // every lane takes part in the shuffles, live or not
-      float ss = 0.f;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int n = rowbase[r] + kg * 4;
-        if (live && n < N) {
-          float* p = ex.res_out + (size_t)m * N + n;
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (n + i < N) {
-              // the product is rounded to bfloat16 first, as the unfused path stores it before the add
-              float v = p[i] + to_f32(f32_to_bf16(acc[r][mt][i]));
-              p[i] = v;
-              ss += v * v;
-            }
-        }
-      }
-      ss += __shfl_xor(ss, 16, 64);
-      ss += __shfl_xor(ss, 32, 64);
-      if (live && kg == 0) ex.ssq_out[(size_t)m * gridDim.x + blockIdx.x] = ss;
-    } else if (EPI == 3) {
-      if (!live) continue;
-      const int H = N / 3, Wd = ex.conv_w;
-      const int slot = ex.slots[m];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int c = blockIdx.x * 16 + kg * 4 + i;
-        if (c >= H) break;
-        // the products run on the values as the unfused path stores them: rounded to bfloat16
-        const float Bv = to_f32(f32_to_bf16(acc[0][mt][i])), Cv = to_f32(f32_to_bf16(acc[1][mt][i])),
-                    Xv = to_f32(f32_to_bf16(acc[2][mt][i]));
-        const float u = Bv * Xv;
-        const float* wt = ex.taps + (size_t)c * Wd;
-        float* hist = ex.state + ((size_t)slot * H + c) * (Wd - 1);
-        float y = 0.f;
-        for (int p = 0; p < Wd - 1; ++p) y += wt[p] * hist[p];
-        y += wt[Wd - 1] * u;
-        if (ex.conv_bias) y += ex.conv_bias[c];
-        Y[(size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
-        for (int p = 0; p < Wd - 2; ++p) hist[p] = hist[p + 1];
-        hist[Wd - 2] = u;
-      }
-    } else if (EPI == 4) {
-      // one head of d = 16 R features; tile r and tile r + R/2 hold the two halves of each rotation pair
-      constexpr int d = 16 * R;
-      const int hh = blockIdx.x;  // head among q heads, then k heads, then v heads
-      const bool is_q = hh < ex.nh, is_k = !is_q && hh < ex.nh + ex.nkv;
-      float v[R][4];
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[r][i] = to_f32(f32_to_bf16(acc[r][mt][i]));  // as the unfused path stores qkv
-      const float* nw = is_q ? ex.qw : ex.kw;
-      if (is_q || is_k) {
-        if (nw) {
-          float ss = 0.f;
-#pragma unroll
-          for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ss += v[r][i] * v[r][i];
-          ss += __shfl_xor(ss, 16, 64);
-          ss += __shfl_xor(ss, 32, 64);
-          const float hinv = 1.0f / sqrtf(ss / (float)d + ex.head_eps);
-#pragma unroll
-          for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) v[r][i] = v[r][i] * hinv * nw[r * 16 + kg * 4 + i];
-        }
-        if (live) {
-          const int pos = ex.positions[m];
-#pragma unroll
-          for (int r = 0; r < R / 2; ++r)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int j = r * 16 + kg * 4 + i;  // pair (j, j + d/2)
-              const float c = ex.cos_t[(size_t)pos * (d / 2) + j], sn = ex.sin_t[(size_t)pos * (d / 2) + j];
-              const float a = v[r][i], b = v[r + R / 2][i];
-              v[r][i] = a * c - b * sn;
-              v[r + R / 2][i] = a * sn + b * c;
-            }
-        }
-      }
-      if (!live) continue;
-      bf16* dst;
-      if (is_q) {
-        dst = (bf16*)Y + (size_t)m * ldy + (size_t)hh * d;
-      } else {
-        if (!ex.write_kv) continue;
-        const int pos = ex.positions[m];
-        const int kvh = is_k ? hh - ex.nh : hh - ex.nh - ex.nkv;
-        const int page = ex.block_table[(size_t)m * ex.max_blocks + pos / ex.page_size];
-        dst = (is_k ? ex.kcache : ex.vcache) + (((size_t)page * ex.nkv + kvh) * ex.page_size + pos % ex.page_size) * d;
-      }
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        f32x4_t o = {v[r][0], v[r][1], v[r][2], v[r][3]};
-        store4<bf16>(dst + r * 16 + kg * 4, o, 4);
-      }
-    }
-  }
-}
-
-template <int R, int MT, int WAVES, int PRO, int EPI, typename TOut>
-static void launch_skinny(int blocks, const bf16* X, int ldx, const bf16* W, TOut* Y, int ldy, int M, int N, int K,
-                          const SkinnyExtra& ex, hipStream_t stream) {
-  const size_t lds = (size_t)(WAVES - 1) * R * MT * 256 * sizeof(float);
-  gemm_skinny_kernel<R, MT, WAVES, PRO, EPI, TOut>
-      <<<blocks, WAVES * 64, lds, stream>>>(X, ldx, W, Y, ldy, M, N, K, ex);
-}
-
-// MT from M; the wavefronts per block are given per MT so that the LDS for the partial tiles,
-// (WAVES - 1) * R * MT KB, stays within 64 KB
-#define GS_BY_MT4(R, W1, W2, W3, W4, PRO, EPI, TOut, blocks)                                                       \
-  switch ((M + 15) / 16) {                                                                                         \
-    case 1: launch_skinny<R, 1, W1, PRO, EPI, TOut>(blocks, x, ldx, w, (TOut*)Y, ldy, M, N, K, ex, stream); break;  \
-    case 2: launch_skinny<R, 2, W2, PRO, EPI, TOut>(blocks, x, ldx, w, (TOut*)Y, ldy, M, N, K, ex, stream); break;  \
-    case 3: launch_skinny<R, 3, W3, PRO, EPI, TOut>(blocks, x, ldx, w, (TOut*)Y, ldy, M, N, K, ex, stream); break;  \
-    default: launch_skinny<R, 4, W4, PRO, EPI, TOut>(blocks, x, ldx, w, (TOut*)Y, ldy, M, N, K, ex, stream); break; \
-  }
-#define GS_BY_MT(R, WAVES, PRO, EPI, TOut, blocks) GS_BY_MT4(R, WAVES, WAVES, WAVES, WAVES, PRO, EPI, TOut, blocks)
+struct SkinnyExtra;
+struct SkinnyCall;
+#include "gemm_skinny_decl.h"
 
 static int check_common(const void* W, int M, int N, int K) {
   GS_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: %d rows; this kernel takes at most 64", M);
@@ -392,53 +16,35 @@ static int check_common(const void* W, int M, int N, int K) {
   return 0;
 }
 
+static int check_tiles(const void* Wt, int N, int K, int unit) {
+  if (!Wt) return 0;
+  GS_REQUIRE(K % 32 == 0 && unit % 16 == 0 && N % unit == 0 && ((uintptr_t)Wt & 15) == 0,
+             "gemm_skinny: no tile-major copy exists for N=%d K=%d (row unit %d)", N, K, unit);
+  return 0;
+}
+
+static int check_lazy(const float* res, const float* ssq, int nb, const float* norm_w, float eps) {
+  GS_REQUIRE(res && ssq && norm_w && nb > 0 && eps > 0.f, "gemm_skinny: the norm prologue needs the stream, partial sums, a weight and eps");
+  GS_REQUIRE(((uintptr_t)res & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemm_skinny: res and norm weight must be 16-byte aligned");
+  return 0;
+}
+
 // Plain and SwiGLU products of a given bfloat16 X, or of the normed residual stream (res != null).
 extern "C" int gs_gemm_skinny(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w,
-                              float eps, const void* W, void* Y, int y_dtype, int ldy, int M, int N, int K,
-                              int epilogue, hipStream_t stream) {
+                              float eps, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M, int N,
+                              int K, int epilogue, hipStream_t stream) {
   if (check_common(W, M, N, K)) return -1;
   GS_REQUIRE(epilogue == 0 || (epilogue == 1 && N % 2 == 0), "gemm_skinny: unknown epilogue %d (or odd N)", epilogue);
   GS_REQUIRE(ldy >= (epilogue == 1 ? N / 2 : N), "gemm_skinny: row stride %d of Y too small", ldy);
   GS_REQUIRE(y_dtype == GS_BF16 || y_dtype == GS_F32, "gemm_skinny: unknown output dtype %d", y_dtype);
-  const int pro = res ? 1 : 0;
-  if (pro) {
-    GS_REQUIRE(ssq && norm_w && nb > 0 && eps > 0.f, "gemm_skinny: the norm prologue needs partial sums, a weight and eps");
-    GS_REQUIRE(((uintptr_t)res & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemm_skinny: res and norm weight must be 16-byte aligned");
+  if (check_tiles(Wt, N, K, epilogue == 1 ? N / 2 : 16)) return -1;
+  if (res) {
+    if (check_lazy(res, ssq, nb, norm_w, eps)) return -1;
   } else {
     GS_REQUIRE(ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0, "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
   }
   if (M == 0) return 0;
-  const bf16* x = (const bf16*)X;
-  const bf16* w = (const bf16*)W;
-  SkinnyExtra ex = {};
-  ex.res = res; ex.ssq = ssq; ex.nb = nb; ex.norm_w = norm_w; ex.eps = eps;
-  const int cols = epilogue == 1 ? N / 2 : N;
-  const bool narrow = cols <= 4096;
-  // few output columns: more wavefronts per block split K further, so that the whole chip streams
-  if (epilogue == 1) {
-    const int blocks = gs_ceil_div(cols, 16);
-    if (pro) {
-      if (y_dtype == GS_BF16) { if (narrow) { GS_BY_MT(2, 8, 1, 1, bf16, blocks) } else { GS_BY_MT(2, 4, 1, 1, bf16, blocks) } }
-      else { GS_BY_MT(2, 4, 1, 1, float, blocks) }
-    } else {
-      if (y_dtype == GS_BF16) { if (narrow) { GS_BY_MT(2, 8, 0, 1, bf16, blocks) } else { GS_BY_MT(2, 4, 0, 1, bf16, blocks) } }
-      else { GS_BY_MT(2, 4, 0, 1, float, blocks) }
-    }
-  } else if (narrow) {
-    const int blocks = gs_ceil_div(cols, 16);
-    if (pro) {
-      if (y_dtype == GS_BF16) { GS_BY_MT(1, 8, 1, 0, bf16, blocks) } else { GS_BY_MT(1, 8, 1, 0, float, blocks) }
-    } else {
-      if (y_dtype == GS_BF16) { GS_BY_MT(1, 8, 0, 0, bf16, blocks) } else { GS_BY_MT(1, 8, 0, 0, float, blocks) }
-    }
-  } else {
-    const int blocks = gs_ceil_div(cols, 32);
-    if (pro) {
-      if (y_dtype == GS_BF16) { GS_BY_MT(2, 4, 1, 0, bf16, blocks) } else { GS_BY_MT(2, 4, 1, 0, float, blocks) }
-    } else {
-      if (y_dtype == GS_BF16) { GS_BY_MT(2, 4, 0, 0, bf16, blocks) } else { GS_BY_MT(2, 4, 0, 0, float, blocks) }
-    }
-  }
+  gs_skinny_run_plain(X, ldx, res, ssq, nb, norm_w, eps, W, Wt, Y, y_dtype, ldy, M, N, K, epilogue, stream);
   GS_LAUNCH_CHECK("gemm_skinny");
   return 0;
 }
@@ -447,43 +53,27 @@ extern "C" int gs_gemm_skinny(const void* X, int ldx, const float* res, const fl
 extern "C" int gs_gemm_skinny_residual_blocks(int N) { return gs_ceil_div(N, 16); }
 
 // res (M, N) += X W^T, and ssq_out (M, blocks) = partial sums of squares of the new rows.
-extern "C" int gs_gemm_skinny_residual(const void* X, int ldx, const void* W, float* res, float* ssq_out, int M,
-                                       int N, int K, hipStream_t stream) {
-  if (check_common(W, M, N, K)) return -1;
+extern "C" int gs_gemm_skinny_residual(const void* X, int ldx, const void* W, const void* Wt, float* res,
+                                       float* ssq_out, int M, int N, int K, hipStream_t stream) {
+  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16)) return -1;
   GS_REQUIRE(ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0, "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
   GS_REQUIRE(res && ssq_out, "gemm_skinny_residual: needs the stream and room for the partial sums");
   if (M == 0) return 0;
-  const bf16* x = (const bf16*)X;
-  const bf16* w = (const bf16*)W;
-  SkinnyExtra ex = {};
-  ex.res_out = res; ex.ssq_out = ssq_out;
-  float* Y = nullptr;
-  const int ldy = N;
-  const int blocks = gs_ceil_div(N, 16);
-  if (K >= 4096) { GS_BY_MT(1, 16, 0, 2, float, blocks) } else { GS_BY_MT(1, 8, 0, 2, float, blocks) }
+  gs_skinny_run_residual(X, ldx, W, Wt, res, ssq_out, M, N, K, stream);
   GS_LAUNCH_CHECK("gemm_skinny_residual");
   return 0;
 }
 
 // mixed (M, H) = gated short convolution of (normed res) W_in^T for a decode step; W_in (3H, K).
 extern "C" int gs_gemm_skinny_conv(const float* res, const float* ssq, int nb, const float* norm_w, float eps,
-                                   const void* W, const float* taps, const float* conv_bias, float* state,
-                                   const int* slots, int conv_w, void* Y, int M, int H, int K, hipStream_t stream) {
+                                   const void* W, const void* Wt, const float* taps, const float* conv_bias,
+                                   float* state, const int* slots, int conv_w, void* Y, int M, int H, int K,
+                                   hipStream_t stream) {
   const int N = 3 * H;
-  if (check_common(W, M, N, K)) return -1;
-  GS_REQUIRE(res && ssq && norm_w && nb > 0 && eps > 0.f, "gemm_skinny_conv: needs the normed stream");
-  GS_REQUIRE(((uintptr_t)res & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemm_skinny_conv: res and norm weight must be 16-byte aligned");
+  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, H) || check_lazy(res, ssq, nb, norm_w, eps)) return -1;
   GS_REQUIRE(conv_w >= 2 && conv_w <= 16 && taps && state && slots, "gemm_skinny_conv: bad convolution operands (width %d)", conv_w);
   if (M == 0) return 0;
-  const bf16* x = nullptr;
-  const int ldx = K;
-  const bf16* w = (const bf16*)W;
-  SkinnyExtra ex = {};
-  ex.res = res; ex.ssq = ssq; ex.nb = nb; ex.norm_w = norm_w; ex.eps = eps;
-  ex.taps = taps; ex.conv_bias = conv_bias; ex.state = state; ex.slots = slots; ex.conv_w = conv_w;
-  const int ldy = H;
-  const int blocks = gs_ceil_div(H, 16);
-  GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks)
+  gs_skinny_run_conv(res, ssq, nb, norm_w, eps, W, Wt, taps, conv_bias, state, slots, conv_w, Y, M, H, K, stream);
   GS_LAUNCH_CHECK("gemm_skinny_conv");
   return 0;
 }
@@ -495,33 +85,39 @@ extern "C" int gs_gemm_skinny_qkv_supports(int d, int rotary_dim) {
 
 // q (M, nh d) stored, k and v written to the cache, from (normed res) W_qkv^T for a decode step.
 extern "C" int gs_gemm_skinny_qkv(const float* res, const float* ssq, int nb, const float* norm_w, float eps,
-                                  const void* W, const float* qw, const float* kw, float head_eps, const float* cos_t,
-                                  const float* sin_t, const int* positions, const int* block_table, int max_blocks,
-                                  int page_size, void* kcache, void* vcache, int write_kv, void* Q, int M, int nh,
-                                  int nkv, int d, int K, hipStream_t stream) {
+                                  const void* W, const void* Wt, const float* qw, const float* kw, float head_eps,
+                                  const float* cos_t, const float* sin_t, const int* positions,
+                                  const int* block_table, int max_blocks, int page_size, void* kcache, void* vcache,
+                                  int write_kv, void* Q, int M, int nh, int nkv, int d, int K, hipStream_t stream) {
   const int N = (nh + 2 * nkv) * d;
-  if (check_common(W, M, N, K)) return -1;
+  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16) || check_lazy(res, ssq, nb, norm_w, eps)) return -1;
   GS_REQUIRE(gs_gemm_skinny_qkv_supports(d, d), "gemm_skinny_qkv: head width %d is not taken", d);
-  GS_REQUIRE(res && ssq && norm_w && nb > 0 && eps > 0.f, "gemm_skinny_qkv: needs the normed stream");
-  GS_REQUIRE(((uintptr_t)res & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemm_skinny_qkv: res and norm weight must be 16-byte aligned");
   GS_REQUIRE((qw == nullptr) == (kw == nullptr), "gemm_skinny_qkv: q and k norm weights come together");
   GS_REQUIRE(cos_t && sin_t && positions && block_table && kcache && vcache && page_size > 0 && max_blocks > 0,
              "gemm_skinny_qkv: missing rotation tables or cache");
   if (M == 0) return 0;
-  const bf16* x = nullptr;
-  const int ldx = K;
-  const bf16* w = (const bf16*)W;
-  SkinnyExtra ex = {};
-  ex.res = res; ex.ssq = ssq; ex.nb = nb; ex.norm_w = norm_w; ex.eps = eps;
-  ex.qw = qw; ex.kw = kw; ex.head_eps = head_eps; ex.cos_t = cos_t; ex.sin_t = sin_t; ex.positions = positions;
-  ex.block_table = block_table; ex.max_blocks = max_blocks; ex.page_size = page_size; ex.nh = nh; ex.nkv = nkv;
-  ex.write_kv = write_kv; ex.kcache = (bf16*)kcache; ex.vcache = (bf16*)vcache;
-  void* Y = Q;
-  const int ldy = nh * d;
-  const int blocks = nh + 2 * nkv;
-  if (d == 32) { GS_BY_MT4(2, 16, 16, 8, 8, 1, 4, bf16, blocks) }
-  else if (d == 64) { GS_BY_MT4(4, 16, 8, 4, 4, 1, 4, bf16, blocks) }
-  else { GS_BY_MT4(8, 8, 4, 2, 2, 1, 4, bf16, blocks) }
+  gs_skinny_run_qkv(res, ssq, nb, norm_w, eps, W, Wt, qw, kw, head_eps, cos_t, sin_t, positions, block_table,
+                    max_blocks, page_size, kcache, vcache, write_kv, Q, M, nh, nkv, d, K, stream);
   GS_LAUNCH_CHECK("gemm_skinny_qkv");
+  return 0;
+}
+
+// Tile-major copy: out[(t * ksteps + s) * 512 + lane * 8 + j] = W[16 t + lane % 16][32 s + 8 (lane / 16) + j].
+__global__ void tile_major_kernel(const bf16* __restrict__ W, bf16* __restrict__ out, int N, int K) {
+  const int ksteps = K >> 5;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);  // (row tile, k step)
+  const int lane = threadIdx.x & 63;
+  if (unit >= (long)(N >> 4) * ksteps) return;
+  const int t = (int)(unit / ksteps), s = (int)(unit - (long)t * ksteps);
+  const uint4 v = *reinterpret_cast<const uint4*>(W + (size_t)(16 * t + (lane & 15)) * K + 32 * s + 8 * (lane >> 4));
+  *reinterpret_cast<uint4*>(out + (size_t)unit * 512 + lane * 8) = v;
+}
+
+extern "C" int gs_tile_major(const void* W, void* out, int N, int K, hipStream_t stream) {
+  GS_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % 32 == 0, "tile_major: N=%d must be a multiple of 16 and K=%d of 32", N, K);
+  GS_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)out & 15) == 0, "tile_major: operands must be 16-byte aligned");
+  const long units = (long)(N / 16) * (K / 32);
+  tile_major_kernel<<<gs_ceil_div(units, 4), 256, 0, stream>>>((const bf16*)W, (bf16*)out, N, K);
+  GS_LAUNCH_CHECK("tile_major");
   return 0;
 }

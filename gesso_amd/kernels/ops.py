@@ -322,7 +322,18 @@ def _lazy_args(x):
     return (_p(x), c_int(x.stride(0) if M > 1 else K), None, None, c_int(0), None, c_float(0.0))
 
 
-def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, swiglu: bool = False):
+def tile_major(w: torch.Tensor) -> torch.Tensor:
+    """The tile-major copy of a bfloat16 weight ``(N, K)``, N a multiple of 16 and K of 32, that the
+    weight-streaming kernels read fastest: each 16 x 32 tile as 64 lanes x 16 bytes, in the MFMA operand's order."""
+    _dev(w)
+    N, K = w.shape
+    _need(w.dtype == torch.bfloat16 and N % 16 == 0 and K % 32 == 0, "tile_major: bfloat16 (N, K), N % 16 == 0, K % 32 == 0")
+    out = torch.empty_like(w)
+    _check(lib().gs_tile_major(_p(w), _p(out), c_int(N), c_int(K), _stream()))
+    return out
+
+
+def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, swiglu: bool = False, wt=None):
     """``x @ w.T`` for at most 64 rows, streaming the weights once; optionally ``silu(gate) * up`` of the result.
 
     ``x`` is a bfloat16 tensor or a :class:`LazyNorm`.  With ``swiglu`` the weight holds gate rows then up
@@ -339,13 +350,13 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, sw
     if out is None:
         out = torch.empty((M, cols), dtype=out_dtype or torch.bfloat16, device=w.device)
     _need(out.shape == (M, cols) and out.stride(1) == 1, "gemm_skinny: out has the wrong shape")
-    _check(lib().gs_gemm_skinny(*_lazy_args(x), _p(w), _p(out), c_int(_dt(out)),
+    _check(lib().gs_gemm_skinny(*_lazy_args(x), _p(w), _p(wt), _p(out), c_int(_dt(out)),
                                 c_int(out.stride(0) if M > 1 else cols), c_int(M), c_int(N), c_int(K),
                                 c_int(1 if swiglu else 0), _stream()))
     return out
 
 
-def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor) -> torch.Tensor:
+def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt=None) -> torch.Tensor:
     """``res += x @ w.T`` in place (float32); returns the new rows' sums of squares as partial sums ``(M, nb)``."""
     _dev(w, res)
     _need(skinny_ok(x, w), "gemm_skinny_residual: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
@@ -354,12 +365,12 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor) ->
     _need(w.shape == (N, K) and res.shape == (M, N) and res.dtype == torch.float32, "gemm_skinny_residual: shapes")
     nb = lib().gs_gemm_skinny_residual_blocks(c_int(N))
     ssq = torch.empty((M, nb), dtype=torch.float32, device=res.device)
-    _check(lib().gs_gemm_skinny_residual(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(res), _p(ssq), c_int(M),
+    _check(lib().gs_gemm_skinny_residual(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(wt), _p(res), _p(ssq), c_int(M),
                                          c_int(N), c_int(K), _stream()))
     return ssq
 
 
-def gemm_skinny_conv(x: "LazyNorm", w_in, taps, bias, state, slots) -> torch.Tensor:
+def gemm_skinny_conv(x: "LazyNorm", w_in, taps, bias, state, slots, wt=None) -> torch.Tensor:
     """A decode step's gated short convolution fused into its input product; ``state`` is advanced."""
     _dev(w_in, taps, bias, state, slots)
     _need(lazy_ok(x, w_in), "gemm_skinny_conv: needs a lazy norm and a bfloat16 weight")
@@ -372,7 +383,7 @@ def gemm_skinny_conv(x: "LazyNorm", w_in, taps, bias, state, slots) -> torch.Ten
     _i32(slots, M, "slots")
     out = torch.empty((M, H), dtype=torch.bfloat16, device=w_in.device)
     _check(lib().gs_gemm_skinny_conv(_p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps),
-                                     _p(w_in), _p(taps), _p(bias), _p(state), _p(slots), c_int(W), _p(out), c_int(M),
+                                     _p(w_in), _p(wt), _p(taps), _p(bias), _p(state), _p(slots), c_int(W), _p(out), c_int(M),
                                      c_int(H), c_int(K), _stream()))
     return out
 
@@ -382,7 +393,7 @@ def gemm_skinny_qkv_supports(d: int, rotary_dim: int) -> bool:
 
 
 def gemm_skinny_qkv(x: "LazyNorm", wqkv, q_weight, k_weight, head_eps, cos, sin, positions, block_table, page_size,
-                    kcache, vcache, nh, nkv, d, write_kv=True) -> torch.Tensor:
+                    kcache, vcache, nh, nkv, d, write_kv=True, wt=None) -> torch.Tensor:
     """A decode step's q, k, v: product, head norms, rotation and cache write in one kernel; returns q ``(M, nh d)``."""
     _dev(wqkv, q_weight, k_weight, cos, sin, positions, block_table, kcache, vcache)
     _need(lazy_ok(x, wqkv), "gemm_skinny_qkv: needs a lazy norm and a bfloat16 weight")
@@ -397,7 +408,7 @@ def gemm_skinny_qkv(x: "LazyNorm", wqkv, q_weight, k_weight, head_eps, cos, sin,
           and vcache.shape == kcache.shape, "cache must be bfloat16 (pages, nkv, page_size, d)")
     q = torch.empty((M, nh * d), dtype=torch.bfloat16, device=wqkv.device)
     _check(lib().gs_gemm_skinny_qkv(_p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps), _p(wqkv),
-                                    _p(q_weight), _p(k_weight), c_float(head_eps), _p(cos), _p(sin), _p(positions),
+                                    _p(wt), _p(q_weight), _p(k_weight), c_float(head_eps), _p(cos), _p(sin), _p(positions),
                                     _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
                                     _p(vcache), c_int(1 if write_kv else 0), _p(q), c_int(M), c_int(nh), c_int(nkv),
                                     c_int(d), c_int(K), _stream()))

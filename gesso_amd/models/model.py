@@ -68,7 +68,7 @@ class Model:
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         s = self.spec
         self.embed = tensors[s.names["embed"]]
-        self.head = self.embed if s.tie_embeddings else tensors[s.names["head"]]
+        self.head = self.rt.prepare(self.embed if s.tie_embeddings else tensors[s.names["head"]])
         self.final_norm.bind({k: tensors[s.names["final_norm." + k]]
                               for k in part_class("norm", s.final_norm).tensor_specs(s.final_norm)})
         for b, block in zip(s.blocks, self.blocks):

@@ -48,8 +48,8 @@ class Attention(Part):
         ws = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
         if len({w.dtype for w in ws}) > 1:
             ws = [w.float() for w in ws]
-        self.wqkv = torch.cat(ws, 0).contiguous()
-        self.wo = tensors["out_proj.weight"]
+        self.wqkv = self.rt.prepare(torch.cat(ws, 0).contiguous())
+        self.wo = self.rt.prepare(tensors["out_proj.weight"])
         self.bqkv = self.bo = None
         if self.spec.bias:
             self.bqkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]], 0).contiguous()

@@ -28,7 +28,7 @@ class ResidualStream:
         from .runtime import DeferredLinear
         if isinstance(out, DeferredLinear):
             self.flush(rt)
-            self.ssq = rt.ops.gemm_skinny_residual(out.x, out.w, self.res)
+            self.ssq = rt.ops.gemm_skinny_residual(out.x, out.w, self.res, wt=rt._wt(out.w))
         else:
             self.flush(rt)
             self.pending, self.ssq = out, None

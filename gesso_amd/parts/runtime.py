@@ -38,6 +38,8 @@ class Runtime:
         self._shared = {}
         self.no_library = False        # set while a HIP graph is recorded: only our own kernels go into it
         self.fused = False             # set while a decode step is recorded: norms, adds and small ops fold into products
+        self.tile_weights = dtype == torch.bfloat16   # keep a tile-major copy of weights for the streaming kernels
+        self._tiles = {}
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""
@@ -46,6 +48,22 @@ class Runtime:
         return self._shared[key]
 
     # ------------------------------------------------------------------ matrix products
+
+    def prepare(self, w: torch.Tensor, unit: int = 16) -> torch.Tensor:
+        """Called by a part for each weight of a matrix product, once, at bind time.
+
+        Makes the tile-major copy that the weight-streaming kernels read (a layout choice, the values
+        are the same); ``unit`` is the number of rows after which the part's epilogue starts a new
+        group (half the rows for gate|up, a third for B|C|X), which must be whole tiles.  The weight
+        as stored stays, for the products of many rows.  Returns ``w``.
+        """
+        if (self.tile_weights and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
+                and w.shape[1] % 32 == 0 and unit % 16 == 0 and w.shape[0] % unit == 0):
+            self._tiles[w.data_ptr()] = self.ops.tile_major(w)
+        return w
+
+    def _wt(self, w):
+        return self._tiles.get(w.data_ptr())
 
     def _dense(self, x):
         return x.materialize() if isinstance(x, self.ops.LazyNorm) else x
@@ -56,11 +74,11 @@ class Runtime:
         out_dtype = out_dtype or self.dtype
         if isinstance(x, ops.LazyNorm):
             if bias is None and ops.lazy_ok(x, w):
-                return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out)
+                return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self._wt(w))
             x = x.materialize()
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
             if ops.skinny_ok(x, w):
-                return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out)
+                return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self._wt(w))
             if out_dtype == torch.bfloat16 and not self.no_library:
                 return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
         return ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
@@ -70,10 +88,10 @@ class Runtime:
         ops = self.ops
         if isinstance(x, ops.LazyNorm):
             if ops.lazy_ok(x, w13):
-                return ops.gemm_skinny(x, w13, swiglu=True)
+                return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13))
             x = x.materialize()
         if ops.skinny_ok(x, w13):
-            return ops.gemm_skinny(x, w13, swiglu=True)
+            return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13))
         return ops.swiglu(self.linear(x, w13))
 
     def project(self, x: torch.Tensor, w: torch.Tensor, bias=None):
@@ -90,7 +108,7 @@ class Runtime:
         ops = self.ops
         if isinstance(x, ops.LazyNorm):
             if b_in is None and ctx.all_single and ops.lazy_ok(x, w_in) and taps.shape[1] <= 16:
-                return ops.gemm_skinny_conv(x, w_in, taps, b_conv, state, ctx.slots)
+                return ops.gemm_skinny_conv(x, w_in, taps, b_conv, state, ctx.slots, wt=self._wt(w_in))
             x = x.materialize()
         bcx = self.linear(x, w_in, b_in)
         return ops.short_conv(bcx, taps, b_conv, state, ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq,
@@ -105,7 +123,7 @@ class Runtime:
                     and ops.gemm_skinny_qkv_supports(d, position.rotary_dim)):
                 q = ops.gemm_skinny_qkv(x, wqkv, q_norm, k_norm, head_eps, position.cos, position.sin, ctx.positions,
                                         cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
-                                        write_kv=cache.write)
+                                        write_kv=cache.write, wt=self._wt(wqkv))
                 return q, nh * d
             x = x.materialize()
         qkv = self.linear(x, wqkv, bqkv)

@@ -32,8 +32,8 @@ class ShortConv(Part):
 
     def bind(self, tensors):
         H, W = self.spec.hidden, self.spec.width
-        self.w_in = tensors["in_proj.weight"]
-        self.w_out = tensors["out_proj.weight"]
+        self.w_in = self.rt.prepare(tensors["in_proj.weight"], unit=H)
+        self.w_out = self.rt.prepare(tensors["out_proj.weight"])
         self.taps = tensors["conv.weight"].reshape(H, W).contiguous()
         self.b_in = tensors.get("in_proj.bias")
         self.b_conv = tensors.get("conv.bias")

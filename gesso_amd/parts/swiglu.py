@@ -25,8 +25,8 @@ class SwiGLU(Part):
         w1, w3 = tensors["w1.weight"], tensors["w3.weight"]
         if w1.dtype != w3.dtype:
             w1, w3 = w1.float(), w3.float()
-        self.w13 = torch.cat([w1, w3], 0).contiguous()
-        self.w2 = tensors["w2.weight"]
+        self.w13 = self.rt.prepare(torch.cat([w1, w3], 0).contiguous(), unit=w1.shape[0])
+        self.w2 = self.rt.prepare(tensors["w2.weight"])
 
     def forward(self, x, ctx):
         a = self.rt.linear_swiglu(x, self.w13)

@@ -543,3 +543,20 @@ def test_gemm_skinny_qkv_equals_the_separate_kernels(ops, M, nh, nkv, d, norm):
     assert float((kc1.float() - kc2.float()).abs().max()) <= 2e-2 * max(1.0, float(kc2.float().abs().max()))
     assert float((vc1.float() - vc2.float()).abs().max()) <= 2e-2 * max(1.0, float(vc2.float().abs().max()))
     assert int((kc1.float().abs().sum(dim=(1, 3)) > 0).sum()) == M      # one row per token, nothing else
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 16384, 2048), (24, 96, 64), (64, 2048, 8192)])
+def test_tile_major_copy_gives_the_same_products(ops, M, N, K):
+    g = gen(M + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    wt = ops.tile_major(w)
+    # the copy holds the same values: tile (t, s), lane l, element j
+    t, s, l, j = N // 16 - 1, K // 32 - 1, 37, 5
+    assert wt.reshape(-1)[((t * (K // 32) + s) * 64 + l) * 8 + j] == w[16 * t + l % 16, 32 * s + 8 * (l // 16) + j]
+    for kw in ({}, {"swiglu": True}, {"out_dtype": torch.float32}):
+        assert torch.equal(ops.gemm_skinny(x, w, wt=wt, **kw), ops.gemm_skinny(x, w, **kw))
+    if N <= 2048:
+        r1, r2 = torch.ones(M, N, device=DEV), torch.ones(M, N, device=DEV)
+        s1, s2 = ops.gemm_skinny_residual(x, w, r1, wt=wt), ops.gemm_skinny_residual(x, w, r2)
+        assert torch.equal(r1, r2) and torch.equal(s1, s2)
