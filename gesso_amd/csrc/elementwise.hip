@@ -120,6 +120,38 @@ extern "C" int gs_add_rmsnorm(float* res, const void* delta, int delta_dtype, co
   return 0;
 }
 
+// out[t, :] = res[t, :] * inv_rms(t) * w, the row's sum of squares given as nb partial sums (added in a
+// fixed order).  The norm of a stream whose sums a product's epilogue has already taken: no pass over
+// the row is needed to find them.
+template <typename TO>
+__global__ void norm_from_ssq_kernel(const float* __restrict__ res, const float* __restrict__ ssq, int nb,
+                                     const float* __restrict__ w, float eps, TO* __restrict__ out, int H) {
+  __shared__ float red[17];
+  int t = blockIdx.x;
+  float s = 0.f;
+  for (int b = threadIdx.x; b < nb; b += blockDim.x) s += ssq[(size_t)t * nb + b];
+  s = block_sum(s, red);
+  float inv = 1.0f / sqrtf(s / (float)H + eps);
+  const float* x = res + (size_t)t * H;
+  TO* o = out + (size_t)t * H;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = from_f32<TO>(x[j] * inv * w[j]);
+}
+
+extern "C" int gs_norm_from_ssq(const float* res, const float* ssq, int nb, const float* w, float eps, void* out,
+                                int out_dtype, int T, int H, hipStream_t stream) {
+  GS_REQUIRE(T >= 0 && H > 0 && nb > 0 && eps > 0.f, "norm_from_ssq: bad sizes T=%d H=%d nb=%d", T, H, nb);
+  if (T == 0) return 0;
+  int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+  if (out_dtype == GS_BF16)
+    norm_from_ssq_kernel<bf16><<<T, threads, 0, stream>>>(res, ssq, nb, w, eps, (bf16*)out, H);
+  else if (out_dtype == GS_F32)
+    norm_from_ssq_kernel<float><<<T, threads, 0, stream>>>(res, ssq, nb, w, eps, (float*)out, H);
+  else
+    GS_REQUIRE(false, "norm_from_ssq: unknown dtype %d", out_dtype);
+  GS_LAUNCH_CHECK("norm_from_ssq");
+  return 0;
+}
+
 // res[t, :] += delta[t, :]   (the last sub-layer's output, when no norm follows it)
 template <typename TD>
 __global__ void add_kernel(float* __restrict__ res, const TD* __restrict__ delta, long n) {

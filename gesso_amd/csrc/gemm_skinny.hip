@@ -29,6 +29,15 @@ static int check_lazy(const float* res, const float* ssq, int nb, const float* n
   return 0;
 }
 
+// X is either given (bfloat16, aligned) or the normed residual stream (res != null).
+static int check_x(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps,
+                   int K) {
+  if (res) return check_lazy(res, ssq, nb, norm_w, eps);
+  GS_REQUIRE(X && ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0,
+             "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
+  return 0;
+}
+
 // Plain and SwiGLU products of a given bfloat16 X, or of the normed residual stream (res != null).
 extern "C" int gs_gemm_skinny(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w,
                               float eps, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M, int N,
@@ -65,15 +74,15 @@ extern "C" int gs_gemm_skinny_residual(const void* X, int ldx, const void* W, co
 }
 
 // mixed (M, H) = gated short convolution of (normed res) W_in^T for a decode step; W_in (3H, K).
-extern "C" int gs_gemm_skinny_conv(const float* res, const float* ssq, int nb, const float* norm_w, float eps,
+extern "C" int gs_gemm_skinny_conv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps,
                                    const void* W, const void* Wt, const float* taps, const float* conv_bias,
                                    float* state, const int* slots, int conv_w, void* Y, int M, int H, int K,
                                    hipStream_t stream) {
   const int N = 3 * H;
-  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, H) || check_lazy(res, ssq, nb, norm_w, eps)) return -1;
+  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, H) || check_x(X, ldx, res, ssq, nb, norm_w, eps, K)) return -1;
   GS_REQUIRE(conv_w >= 2 && conv_w <= 16 && taps && state && slots, "gemm_skinny_conv: bad convolution operands (width %d)", conv_w);
   if (M == 0) return 0;
-  gs_skinny_run_conv(res, ssq, nb, norm_w, eps, W, Wt, taps, conv_bias, state, slots, conv_w, Y, M, H, K, stream);
+  gs_skinny_run_conv(X, ldx, res, ssq, nb, norm_w, eps, W, Wt, taps, conv_bias, state, slots, conv_w, Y, M, H, K, stream);
   GS_LAUNCH_CHECK("gemm_skinny_conv");
   return 0;
 }
@@ -84,19 +93,19 @@ extern "C" int gs_gemm_skinny_qkv_supports(int d, int rotary_dim) {
 }
 
 // q (M, nh d) stored, k and v written to the cache, from (normed res) W_qkv^T for a decode step.
-extern "C" int gs_gemm_skinny_qkv(const float* res, const float* ssq, int nb, const float* norm_w, float eps,
+extern "C" int gs_gemm_skinny_qkv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps,
                                   const void* W, const void* Wt, const float* qw, const float* kw, float head_eps,
                                   const float* cos_t, const float* sin_t, const int* positions,
                                   const int* block_table, int max_blocks, int page_size, void* kcache, void* vcache,
                                   int write_kv, void* Q, int M, int nh, int nkv, int d, int K, hipStream_t stream) {
   const int N = (nh + 2 * nkv) * d;
-  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16) || check_lazy(res, ssq, nb, norm_w, eps)) return -1;
+  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16) || check_x(X, ldx, res, ssq, nb, norm_w, eps, K)) return -1;
   GS_REQUIRE(gs_gemm_skinny_qkv_supports(d, d), "gemm_skinny_qkv: head width %d is not taken", d);
   GS_REQUIRE((qw == nullptr) == (kw == nullptr), "gemm_skinny_qkv: q and k norm weights come together");
   GS_REQUIRE(cos_t && sin_t && positions && block_table && kcache && vcache && page_size > 0 && max_blocks > 0,
              "gemm_skinny_qkv: missing rotation tables or cache");
   if (M == 0) return 0;
-  gs_skinny_run_qkv(res, ssq, nb, norm_w, eps, W, Wt, qw, kw, head_eps, cos_t, sin_t, positions, block_table,
+  gs_skinny_run_qkv(X, ldx, res, ssq, nb, norm_w, eps, W, Wt, qw, kw, head_eps, cos_t, sin_t, positions, block_table,
                     max_blocks, page_size, kcache, vcache, write_kv, Q, M, nh, nkv, d, K, stream);
   GS_LAUNCH_CHECK("gemm_skinny_qkv");
   return 0;

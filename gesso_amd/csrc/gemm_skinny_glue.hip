@@ -38,22 +38,22 @@ void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* W
   Wt ? gs_skinny_residual_tiles(c) : gs_skinny_residual_rows(c);
 }
 
-void gs_skinny_run_conv(const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
+void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
                         const void* Wt, const float* taps, const float* conv_bias, float* state, const int* slots,
                         int conv_w, void* Y, int M, int H, int K, hipStream_t stream) {
-  SkinnyCall c = base(nullptr, K, W, Wt, Y, GS_BF16, H, M, 3 * H, K, 3, stream);
-  lazy(c, res, ssq, nb, norm_w, eps);
+  SkinnyCall c = base(X, ldx, W, Wt, Y, GS_BF16, H, M, 3 * H, K, 3, stream);
+  if (res) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.taps = taps; c.ex.conv_bias = conv_bias; c.ex.state = state; c.ex.slots = slots; c.ex.conv_w = conv_w;
   Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);
 }
 
-void gs_skinny_run_qkv(const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
+void gs_skinny_run_qkv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
                        const void* Wt, const float* qw, const float* kw, float head_eps, const float* cos_t,
                        const float* sin_t, const int* positions, const int* block_table, int max_blocks,
                        int page_size, void* kcache, void* vcache, int write_kv, void* Q, int M, int nh, int nkv, int d,
                        int K, hipStream_t stream) {
-  SkinnyCall c = base(nullptr, K, W, Wt, Q, GS_BF16, nh * d, M, (nh + 2 * nkv) * d, K, 4, stream);
-  lazy(c, res, ssq, nb, norm_w, eps);
+  SkinnyCall c = base(X, ldx, W, Wt, Q, GS_BF16, nh * d, M, (nh + 2 * nkv) * d, K, 4, stream);
+  if (res) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.qw = qw; c.ex.kw = kw; c.ex.head_eps = head_eps; c.ex.cos_t = cos_t; c.ex.sin_t = sin_t;
   c.ex.positions = positions; c.ex.block_table = block_table; c.ex.max_blocks = max_blocks; c.ex.page_size = page_size;
   c.ex.nh = nh; c.ex.nkv = nkv; c.ex.write_kv = write_kv; c.ex.kcache = (bf16*)kcache; c.ex.vcache = (bf16*)vcache;

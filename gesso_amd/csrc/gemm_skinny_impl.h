@@ -447,24 +447,30 @@ static void skinny_residual(const SkinnyCall& c) {
 
 template <int SHUF>
 static void skinny_conv(const SkinnyCall& c) {
-  const bf16 *x = nullptr, *w = c.w;
+  const bf16 *x = c.x, *w = c.w;
   void* Y = c.Y;
-  const int ldx = c.K, ldy = c.ldy, M = c.M, N = c.N, K = c.K;
+  const int ldx = c.ldx, ldy = c.ldy, M = c.M, N = c.N, K = c.K;
   const SkinnyExtra& ex = c.ex;
   hipStream_t stream = c.stream;
   const int blocks = gs_ceil_div(N / 3, 16);
-  GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks)
+  if (ex.res) { GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks) } else { GS_BY_MT4(3, 8, 8, 8, 4, 0, 3, bf16, blocks) }
 }
 
 template <int SHUF>
 static void skinny_qkv(const SkinnyCall& c, int d) {
-  const bf16 *x = nullptr, *w = c.w;
+  const bf16 *x = c.x, *w = c.w;
   void* Y = c.Y;
-  const int ldx = c.K, ldy = c.ldy, M = c.M, N = c.N, K = c.K;
+  const int ldx = c.ldx, ldy = c.ldy, M = c.M, N = c.N, K = c.K;
   const SkinnyExtra& ex = c.ex;
   hipStream_t stream = c.stream;
   const int blocks = N / d;
-  if (d == 32) { GS_BY_MT4(2, 16, 16, 8, 8, 1, 4, bf16, blocks) }
-  else if (d == 64) { GS_BY_MT4(4, 16, 8, 4, 4, 1, 4, bf16, blocks) }
-  else { GS_BY_MT4(8, 8, 4, 2, 2, 1, 4, bf16, blocks) }
+  if (ex.res) {
+    if (d == 32) { GS_BY_MT4(2, 16, 16, 8, 8, 1, 4, bf16, blocks) }
+    else if (d == 64) { GS_BY_MT4(4, 16, 8, 4, 4, 1, 4, bf16, blocks) }
+    else { GS_BY_MT4(8, 8, 4, 2, 2, 1, 4, bf16, blocks) }
+  } else {
+    if (d == 32) { GS_BY_MT4(2, 16, 16, 8, 8, 0, 4, bf16, blocks) }
+    else if (d == 64) { GS_BY_MT4(4, 16, 8, 4, 4, 0, 4, bf16, blocks) }
+    else { GS_BY_MT4(8, 8, 4, 2, 2, 0, 4, bf16, blocks) }
+  }
 }

@@ -293,7 +293,7 @@ class LazyNorm:
     """An RMSNorm not yet applied: the float32 stream, its rows' sums of squares as partial sums, weight and eps.
 
     The weight-streaming products take it in place of a tensor and norm on the fly; ``materialize``
-    runs the norm kernel for everything else.
+    runs a light norm kernel for everything else.
     """
 
     __slots__ = ("res", "ssq", "weight", "eps", "dtype")
@@ -306,7 +306,12 @@ class LazyNorm:
         return self.res.shape
 
     def materialize(self) -> torch.Tensor:
-        return add_rmsnorm(self.res, None, self.weight, self.eps, self.dtype)
+        """The normed rows as a tensor; the sums of squares are at hand, so one light pass does it."""
+        T, H = self.res.shape
+        out = torch.empty((T, H), dtype=self.dtype, device=self.res.device)
+        _check(lib().gs_norm_from_ssq(_p(self.res), _p(self.ssq), c_int(self.ssq.shape[1]), _p(self.weight),
+                                      c_float(self.eps), _p(out), c_int(_dt(out)), c_int(T), c_int(H), _stream()))
+        return out
 
 
 def lazy_ok(x, w: torch.Tensor) -> bool:
@@ -370,10 +375,11 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt
     return ssq
 
 
-def gemm_skinny_conv(x: "LazyNorm", w_in, taps, bias, state, slots, wt=None) -> torch.Tensor:
+def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None) -> torch.Tensor:
     """A decode step's gated short convolution fused into its input product; ``state`` is advanced."""
     _dev(w_in, taps, bias, state, slots)
-    _need(lazy_ok(x, w_in), "gemm_skinny_conv: needs a lazy norm and a bfloat16 weight")
+    _need(lazy_ok(x, w_in) if isinstance(x, LazyNorm) else skinny_ok(x, w_in),
+          "gemm_skinny_conv: needs bfloat16 rows or a lazy norm, and a bfloat16 weight")
     M, K = x.shape
     H, W = taps.shape
     _need(w_in.shape == (3 * H, K), "gemm_skinny_conv: the input weight must be (3H, K)")
@@ -382,8 +388,7 @@ def gemm_skinny_conv(x: "LazyNorm", w_in, taps, bias, state, slots, wt=None) -> 
     _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (H,)), "gemm_skinny_conv: bias float32 (H,)")
     _i32(slots, M, "slots")
     out = torch.empty((M, H), dtype=torch.bfloat16, device=w_in.device)
-    _check(lib().gs_gemm_skinny_conv(_p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps),
-                                     _p(w_in), _p(wt), _p(taps), _p(bias), _p(state), _p(slots), c_int(W), _p(out), c_int(M),
+    _check(lib().gs_gemm_skinny_conv(*_lazy_args(x), _p(w_in), _p(wt), _p(taps), _p(bias), _p(state), _p(slots), c_int(W), _p(out), c_int(M),
                                      c_int(H), c_int(K), _stream()))
     return out
 
@@ -392,11 +397,12 @@ def gemm_skinny_qkv_supports(d: int, rotary_dim: int) -> bool:
     return bool(lib().gs_gemm_skinny_qkv_supports(c_int(d), c_int(rotary_dim)))
 
 
-def gemm_skinny_qkv(x: "LazyNorm", wqkv, q_weight, k_weight, head_eps, cos, sin, positions, block_table, page_size,
+def gemm_skinny_qkv(x, wqkv, q_weight, k_weight, head_eps, cos, sin, positions, block_table, page_size,
                     kcache, vcache, nh, nkv, d, write_kv=True, wt=None) -> torch.Tensor:
     """A decode step's q, k, v: product, head norms, rotation and cache write in one kernel; returns q ``(M, nh d)``."""
     _dev(wqkv, q_weight, k_weight, cos, sin, positions, block_table, kcache, vcache)
-    _need(lazy_ok(x, wqkv), "gemm_skinny_qkv: needs a lazy norm and a bfloat16 weight")
+    _need(lazy_ok(x, wqkv) if isinstance(x, LazyNorm) else skinny_ok(x, wqkv),
+          "gemm_skinny_qkv: needs bfloat16 rows or a lazy norm, and a bfloat16 weight")
     M, K = x.shape
     _need(wqkv.shape == ((nh + 2 * nkv) * d, K), "gemm_skinny_qkv: the weight must be ((nh + 2 nkv) d, K)")
     for w in (q_weight, k_weight):
@@ -407,7 +413,7 @@ def gemm_skinny_qkv(x: "LazyNorm", wqkv, q_weight, k_weight, head_eps, cos, sin,
     _need(kcache.dtype == torch.bfloat16 and kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d)
           and vcache.shape == kcache.shape, "cache must be bfloat16 (pages, nkv, page_size, d)")
     q = torch.empty((M, nh * d), dtype=torch.bfloat16, device=wqkv.device)
-    _check(lib().gs_gemm_skinny_qkv(_p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps), _p(wqkv),
+    _check(lib().gs_gemm_skinny_qkv(*_lazy_args(x), _p(wqkv),
                                     _p(wt), _p(q_weight), _p(k_weight), c_float(head_eps), _p(cos), _p(sin), _p(positions),
                                     _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
                                     _p(vcache), c_int(1 if write_kv else 0), _p(q), c_int(M), c_int(nh), c_int(nkv),

@@ -10,6 +10,8 @@
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from ..errors import KernelError
@@ -40,6 +42,9 @@ class Runtime:
         self.fused = False             # set while a decode step is recorded: norms, adds and small ops fold into products
         self.tile_weights = dtype == torch.bfloat16   # keep a tile-major copy of weights for the streaming kernels
         self._tiles = {}
+        # a lazy norm is folded into the product that follows for up to this many rows; for more, one
+        # light kernel norms the rows first (the fold repeats the norm's arithmetic in every block)
+        self.fold_norm_rows = int(os.environ.get("GESSO_FOLD_NORM_ROWS", "0"))
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""
@@ -73,7 +78,7 @@ class Runtime:
         ops = self.ops
         out_dtype = out_dtype or self.dtype
         if isinstance(x, ops.LazyNorm):
-            if bias is None and ops.lazy_ok(x, w):
+            if bias is None and x.shape[0] <= self.fold_norm_rows and ops.lazy_ok(x, w):
                 return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self._wt(w))
             x = x.materialize()
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
@@ -87,7 +92,7 @@ class Runtime:
         """``silu(x @ w1.T) * (x @ w3.T)`` with ``w13`` holding w1's rows, then w3's."""
         ops = self.ops
         if isinstance(x, ops.LazyNorm):
-            if ops.lazy_ok(x, w13):
+            if x.shape[0] <= self.fold_norm_rows and ops.lazy_ok(x, w13):
                 return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13))
             x = x.materialize()
         if ops.skinny_ok(x, w13):
@@ -103,13 +108,20 @@ class Runtime:
 
     # ------------------------------------------------------------------ mixers' inner steps
 
+    def _rows(self, x):
+        """A lazy norm as the kernels of this step should take it: folded for few rows, else normed by one light pass."""
+        if isinstance(x, self.ops.LazyNorm) and x.shape[0] > self.fold_norm_rows:
+            return x.materialize()
+        return x
+
     def conv_in(self, x, w_in, b_in, taps, b_conv, state, ctx) -> torch.Tensor:
         """Input product and gated short convolution: ``(T, H)`` mixed rows; ``state`` is advanced."""
         ops = self.ops
-        if isinstance(x, ops.LazyNorm):
-            if b_in is None and ctx.all_single and ops.lazy_ok(x, w_in) and taps.shape[1] <= 16:
+        if self.fused and b_in is None and ctx.all_single and taps.shape[1] <= 16:
+            x = self._rows(x)
+            if ops.lazy_ok(x, w_in) or (not isinstance(x, ops.LazyNorm) and ops.skinny_ok(x, w_in)):
                 return ops.gemm_skinny_conv(x, w_in, taps, b_conv, state, ctx.slots, wt=self._wt(w_in))
-            x = x.materialize()
+        x = self._dense(x)
         bcx = self.linear(x, w_in, b_in)
         return ops.short_conv(bcx, taps, b_conv, state, ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq,
                               ctx.all_single)
@@ -118,14 +130,15 @@ class Runtime:
         """q, k, v products, head norms, position encoding, cache write.  Returns ``(q, q_stride)``:
         the queries as rows of a buffer, ``q_stride`` apart, head h at ``[h d, (h+1) d)``."""
         ops = self.ops
-        if isinstance(x, ops.LazyNorm):
-            if (bqkv is None and ctx.all_single and ops.lazy_ok(x, wqkv) and cache.k.dtype == torch.bfloat16
-                    and ops.gemm_skinny_qkv_supports(d, position.rotary_dim)):
+        if (self.fused and bqkv is None and ctx.all_single and cache.k.dtype == torch.bfloat16
+                and ops.gemm_skinny_qkv_supports(d, position.rotary_dim)):
+            x = self._rows(x)
+            if ops.lazy_ok(x, wqkv) or (not isinstance(x, ops.LazyNorm) and ops.skinny_ok(x, wqkv)):
                 q = ops.gemm_skinny_qkv(x, wqkv, q_norm, k_norm, head_eps, position.cos, position.sin, ctx.positions,
                                         cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
                                         write_kv=cache.write, wt=self._wt(wqkv))
                 return q, nh * d
-            x = x.materialize()
+        x = self._dense(x)
         qkv = self.linear(x, wqkv, bqkv)
         ops.qknorm_rope_kv(qkv, q_norm, k_norm, head_eps, position.cos, position.sin, position.rotary_dim,
                            ctx.positions, ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v,
