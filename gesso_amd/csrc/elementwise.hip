@@ -123,29 +123,39 @@ extern "C" int gs_add_rmsnorm(float* res, const void* delta, int delta_dtype, co
 // out[t, :] = res[t, :] * inv_rms(t) * w, the row's sum of squares given as nb partial sums (added in a
 // fixed order).  The norm of a stream whose sums a product's epilogue has already taken: no pass over
 // the row is needed to find them.
+// One wavefront per (row, chunk of 512 columns): every wavefront adds the row's partial sums itself
+// (a few loads and shuffles), so there is no block-wide barrier and the loads of the row's values
+// are under way while the sums are added.
 template <typename TO>
 __global__ void norm_from_ssq_kernel(const float* __restrict__ res, const float* __restrict__ ssq, int nb,
                                      const float* __restrict__ w, float eps, TO* __restrict__ out, int H) {
-  __shared__ float red[17];
-  int t = blockIdx.x;
+  const int t = blockIdx.y, lane = threadIdx.x;
+  const int j0 = blockIdx.x * 512 + lane * 8;
+  float x[8], wv[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    x[i] = (j0 + i < H) ? res[(size_t)t * H + j0 + i] : 0.f;
+    wv[i] = (j0 + i < H) ? w[j0 + i] : 0.f;
+  }
   float s = 0.f;
-  for (int b = threadIdx.x; b < nb; b += blockDim.x) s += ssq[(size_t)t * nb + b];
-  s = block_sum(s, red);
-  float inv = 1.0f / sqrtf(s / (float)H + eps);
-  const float* x = res + (size_t)t * H;
-  TO* o = out + (size_t)t * H;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = from_f32<TO>(x[j] * inv * w[j]);
+  for (int b = lane; b < nb; b += 64) s += ssq[(size_t)t * nb + b];
+  s = wave_sum(s);
+  const float inv = 1.0f / sqrtf(s / (float)H + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    if (j0 + i < H) out[(size_t)t * H + j0 + i] = from_f32<TO>(x[i] * inv * wv[i]);
 }
 
 extern "C" int gs_norm_from_ssq(const float* res, const float* ssq, int nb, const float* w, float eps, void* out,
                                 int out_dtype, int T, int H, hipStream_t stream) {
   GS_REQUIRE(T >= 0 && H > 0 && nb > 0 && eps > 0.f, "norm_from_ssq: bad sizes T=%d H=%d nb=%d", T, H, nb);
+  GS_REQUIRE(T <= 65535, "norm_from_ssq: more than 65535 rows");
   if (T == 0) return 0;
-  int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+  dim3 grid(gs_ceil_div(H, 512), T);
   if (out_dtype == GS_BF16)
-    norm_from_ssq_kernel<bf16><<<T, threads, 0, stream>>>(res, ssq, nb, w, eps, (bf16*)out, H);
+    norm_from_ssq_kernel<bf16><<<grid, 64, 0, stream>>>(res, ssq, nb, w, eps, (bf16*)out, H);
   else if (out_dtype == GS_F32)
-    norm_from_ssq_kernel<float><<<T, threads, 0, stream>>>(res, ssq, nb, w, eps, (float*)out, H);
+    norm_from_ssq_kernel<float><<<grid, 64, 0, stream>>>(res, ssq, nb, w, eps, (float*)out, H);
   else
     GS_REQUIRE(false, "norm_from_ssq: unknown dtype %d", out_dtype);
   GS_LAUNCH_CHECK("norm_from_ssq");

@@ -20,7 +20,33 @@ __device__ void row_argmax(const float* __restrict__ x, int V, int* id_out, int*
   float best = -INFINITY;
   int idx = 0x7fffffff;
   int notfinite = 0;
-  for (int j = threadIdx.x; j < V; j += blockDim.x) {
+  // 16-byte loads, four of them under way at a time; ids are visited in ascending order per thread, and a
+  // later equal value never replaces an earlier one
+  const int V4 = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) ? (V >> 2) : 0;
+  const float4* x4 = reinterpret_cast<const float4*>(x);
+  for (int q0 = threadIdx.x; q0 < V4; q0 += 4 * blockDim.x) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      int q = q0 + u * blockDim.x;
+      v[u] = q < V4 ? x4[q] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      int q = q0 + u * blockDim.x;
+      if (q >= V4) break;
+      const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (!(fabsf(e[i]) <= 3.402823466e38f)) notfinite = 1;
+        if (e[i] > best) {
+          best = e[i];
+          idx = 4 * q + i;
+        }
+      }
+    }
+  }
+  for (int j = 4 * V4 + threadIdx.x; j < V; j += blockDim.x) {
     float v = x[j];
     if (!(fabsf(v) <= 3.402823466e38f)) notfinite = 1;
     if (v > best || (v == best && j < idx)) {

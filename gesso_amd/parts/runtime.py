@@ -154,7 +154,8 @@ class Runtime:
         ops = self.ops
         if ctx.all_single and q.dtype == torch.bfloat16 and ops.attention_decode_supports(nh, nkv, d):
             # one query per sequence: the key stream is split so that the whole chip reads it
-            nsplit = max(1, min(16, 64 // max(1, ctx.nseq * nkv)))
+            # enough blocks that a wavefront rarely walks more than a tile or two of a few hundred keys
+            nsplit = max(1, min(16, 256 // max(1, ctx.nseq * nkv)))
             return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                         cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
         return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
