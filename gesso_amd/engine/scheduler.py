@@ -21,6 +21,11 @@ Decisions, all tested without a GPU:
   stopped).  This repeats until the step fits.  A request that does not fit into the empty pool
   on its own ends as ``failed`` with :class:`~gesso_amd.errors.ResourceLimit`; nothing else stops.
 * The token that ends a request (an id in ``eos_ids``/``stop_ids``) is returned and never fed.
+* When a step holds nothing but decoding requests and the executor has a recorded decode loop
+  (``decode``), several steps run back to back on the device: as many as every request still has
+  tokens to generate, at most ``decode_run_steps``, and one only while requests wait for admission.
+  Tokens come back together; a request that ends within the run (end token, callback) keeps its
+  tokens up to there, what the device computed beyond is dropped with the request's cache.
 """
 from __future__ import annotations
 
@@ -80,7 +85,7 @@ class Scheduled:
 
 class Scheduler:
     def __init__(self, executor, choose: Callable, max_num_seqs: int = 64, max_num_batched_tokens: int = 2048,
-                 chunk_size: int = 1024):
+                 chunk_size: int = 1024, decode_run_steps: int = 8):
         """``executor``: ``add_request``, ``finish_request``, ``step(entries) -> logits`` and ``manager``.
 
         ``choose(logits, samplers) -> ids or exceptions``, one per row.
@@ -93,6 +98,7 @@ class Scheduler:
         self.max_num_seqs = max_num_seqs
         self.max_num_batched_tokens = max_num_batched_tokens
         self.chunk_size = chunk_size
+        self.decode_run_steps = max(1, decode_run_steps)
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []          # in admission order
         self.finished: List[Request] = []
@@ -221,6 +227,9 @@ class Scheduler:
         plan = self.schedule()
         if not plan:
             return None
+        run = self._decode_run(plan)
+        if run is not None:
+            return run
         entries = []
         for s in plan:
             toks = s.request.tokens[s.start:s.start + s.count]
@@ -244,23 +253,61 @@ class Scheduler:
                 if isinstance(tok, Exception):
                     self._finish(r, "failed", error=tok)
                     continue
-                r.output.append(int(tok))
-                self.stats["decode_tokens"] += 1
-                emitted.append((r, int(tok)))
-                keep = True
-                if r.on_token is not None:
-                    try:
-                        keep = r.on_token(int(tok)) is not False
-                    except Exception as err:    # a failing callback ends its own request only
-                        self._finish(r, "failed", error=err)
-                        continue
-                if tok in r.eos_ids or tok in r.stop_ids:
-                    self._finish(r, "eos")
-                elif len(r.output) >= r.max_new_tokens:
-                    self._finish(r, "complete")
-                elif not keep or r.cancelled:
-                    self._finish(r, "cancelled")
+                self._emit(r, int(tok), emitted)
         return emitted
+
+    def _decode_run(self, plan: List[Scheduled]) -> Optional[List[Tuple[Request, int]]]:
+        """Several decode steps at once through the executor's recorded loop, when the plan allows it."""
+        ex = self.executor
+        if not hasattr(ex, "decode") or len(plan) > getattr(ex, "DECODE_MAX_BATCH", 0):
+            return None
+        if not all(s.count == 1 and s.samples for s in plan):
+            return None
+        reqs = [s.request for s in plan]
+        if any(r.sampler is not None and r.sampler.top_p < 1 for r in reqs):
+            return None
+        n = min(self.decode_run_steps, min(r.max_new_tokens - len(r.output) for r in reqs))
+        if self.waiting:
+            n = 1                     # someone waits: look at admission again after every step
+        while n > 1 and self._pages_short([Scheduled(r, r.computed, n, True) for r in reqs]):
+            n -= 1
+        ids, bad = ex.decode([r.rid for r in reqs], [r.tokens[-1] for r in reqs], n, [r.sampler for r in reqs])
+        self.stats["steps"] += n
+        emitted: List[Tuple[Request, int]] = []
+        for i, r in enumerate(reqs):
+            if r.computed < len(r.prompt):
+                self.stats["prompt_tokens"] += 1      # a prompt of one token decodes from its first step
+            r.computed += n
+            for s in range(n):
+                if bad[s][i]:
+                    from ..errors import NumericalInstability
+                    self._finish(r, "failed", error=NumericalInstability("non-finite logits: no token is emitted"))
+                    break
+                if self._emit(r, int(ids[s][i]), emitted):
+                    break
+        return emitted
+
+    def _emit(self, r: Request, tok: int, emitted: List[Tuple[Request, int]]) -> bool:
+        """Account one new token of a request; True when the request has ended with it."""
+        r.output.append(tok)
+        self.stats["decode_tokens"] += 1
+        emitted.append((r, tok))
+        keep = True
+        if r.on_token is not None:
+            try:
+                keep = r.on_token(tok) is not False
+            except Exception as err:    # a failing callback ends its own request only
+                self._finish(r, "failed", error=err)
+                return True
+        if tok in r.eos_ids or tok in r.stop_ids:
+            self._finish(r, "eos")
+        elif len(r.output) >= r.max_new_tokens:
+            self._finish(r, "complete")
+        elif not keep or r.cancelled:
+            self._finish(r, "cancelled")
+        else:
+            return False
+        return True
 
     def run(self) -> None:
         while self.has_work():

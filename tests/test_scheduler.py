@@ -235,3 +235,82 @@ def test_many_requests_under_pressure_all_come_out_right():
         assert r.finish_reason == "complete" and r.tokens == expected(p, r.max_new_tokens), r.rid
     assert eng.manager.stats()["pages_free"] == [20] and eng.manager.stats()["slots_free"] == 4
     assert s.stats["preemptions"] > 0
+
+
+class FakeDecodeEngine(FakeEngine):
+    """The stand-in with a recorded decode loop: n steps at once, tokens fed back inside."""
+
+    DECODE_MAX_BATCH = 4
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.runs = []
+
+    def decode(self, rids, tokens, n, samplers=None):
+        self.manager.reserve_many([(r, n) for r in rids])
+        self.runs.append((list(rids), n))
+        ids = np.zeros((n, len(rids)), dtype=np.int64)
+        bad = np.zeros((n, len(rids)), dtype=np.int64)
+        toks = list(tokens)
+        for s in range(n):
+            for i, r in enumerate(rids):
+                assert self.manager.get(r).length + s == len(self.fed[r])
+                self.fed[r].append(toks[i])
+                toks[i] = next_token(self.fed[r])
+                ids[s, i] = toks[i]
+                if samplers and samplers[i] is not None:
+                    samplers[i].unit()
+        for r in rids:
+            self.manager.commit(r, n)
+        self.manager.check()
+        return ids, bad
+
+
+def test_decode_runs_of_several_steps():
+    eng, s = make(FakeDecodeEngine(), decode_run_steps=5)
+    a = s.add(Request("a", [1, 2, 3], max_new_tokens=12))
+    b = s.add(Request("b", [9], max_new_tokens=7, sampler=Sampler(0.9, 1.0, 3)))
+    s.run()
+    assert a.tokens == expected([1, 2, 3], 12) and b.tokens == expected([9], 7)
+    # the first step holds a's prompt: an ordinary step; then runs of 5, bounded by what b may still generate
+    assert eng.runs[0][1] == 5 and all(n <= 5 for _, n in eng.runs)
+    assert sum(n for rids, n in eng.runs if "b" in rids) == 6            # b's first token came with a's prompt step
+    ref = Sampler(0.9, 1.0, 3)
+    for _ in range(7):
+        ref.unit()
+    assert b.sampler.state == ref.state
+    assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+
+
+def test_a_request_that_ends_inside_a_run_keeps_its_tokens_up_to_there():
+    full = expected([4, 5], 10)
+    eos = full[2 + 3]
+    eng, s = make(FakeDecodeEngine(), decode_run_steps=8)
+    seen = []
+    a = s.add(Request("a", [4, 5], max_new_tokens=10, eos_ids=(eos,)))
+    b = s.add(Request("b", [6, 7], max_new_tokens=10, on_token=lambda t: (seen.append(t), len(seen) < 5)[1]))
+    s.run()
+    assert a.tokens == full[:6] and a.finish_reason == "eos"
+    assert b.finish_reason == "cancelled" and b.tokens == expected([6, 7], 5) and seen == b.output
+    assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+
+
+def test_while_someone_waits_runs_are_single_steps():
+    eng, s = make(FakeDecodeEngine(num_slots=1), decode_run_steps=8)
+    a = s.add(Request("a", [1, 2], max_new_tokens=4))
+    b = s.add(Request("b", [3, 4], max_new_tokens=6))
+    s.run()
+    assert a.tokens == expected([1, 2], 4) and b.tokens == expected([3, 4], 6)
+    assert all(n == 1 for rids, n in eng.runs if rids == ["a"])           # b waited for the slot
+    assert any(n > 1 for rids, n in eng.runs if rids == ["b"])
+
+
+def test_runs_shrink_to_the_pages_that_are_left_and_nucleus_requests_step_singly():
+    eng, s = make(FakeDecodeEngine(num_pages=3, page_size=4), decode_run_steps=8)
+    a = s.add(Request("a", [1, 2, 3], max_new_tokens=8))
+    s.run()
+    assert a.tokens == expected([1, 2, 3], 8)
+    eng2, s2 = make(FakeDecodeEngine(), decode_run_steps=8)
+    c = s2.add(Request("c", [1, 2, 3], max_new_tokens=5, sampler=Sampler(0.9, 0.5, 3)))
+    s2.run()
+    assert c.tokens == expected([1, 2, 3], 5) and eng2.runs == []
