@@ -1,0 +1,219 @@
+// Prompt attention on the matrix cores: many queries per sequence over the paged cache, bfloat16.
+//
+// A block owns 16 consecutive queries of one sequence and one key head; its G wavefronts are the G query
+// heads that share the key head, so keys and values are fetched once per group.  Keys are walked in steps
+// of 32 with a running maximum and sum per query (online softmax, float32).
+//
+// Both products are computed transposed, so that everything a lane holds concerns one query (lane % 16):
+//   S^T = K Q^T   A = K tile (16 keys x 32 features, 16-byte loads straight from the page, lane l: key
+//                 l % 16, features 8 (l / 16) ..), B = Q^T (the wavefront's query fragment, kept in
+//                 registers), result: lane l holds keys 4 (l / 16) + 0..3 for query l % 16.
+//   O^T = V^T P^T B = P^T is exactly the lane's own eight probabilities of a step (two key blocks of
+//                 four), A = V^T read from LDS, where the step's 32 value rows are staged transposed once
+//                 per block.  Result: lane l holds features 4 (l / 16) + 0..3 (per tile of 16) of query l % 16.
+// No probability ever crosses lanes; the only cross-lane traffic is the maximum and the sum over the four
+// lane groups.  v_mfma_f32_16x16x32_bf16 throughout.
+//
+// Causal rule: the query at position p sees keys lo..p, lo = 0 or p - window + 1.  Tiles of queries come
+// from the host: tile i covers rows tile_row[i] .. + tile_n[i] of the flattened tokens, of sequence
+// tile_seq[i].  q (T, q_stride), head h at [h D, (h+1) D); caches (pages, nkv, page_size, D); out (T, nh D).
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+#define PF_KSTEP 32
+#define PF_PAD 8
+
+template <int D, int G>
+__global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
+    const int* __restrict__ positions, const int* __restrict__ tile_seq, const int* __restrict__ tile_row,
+    const int* __restrict__ tile_n, const int* __restrict__ block_table, int max_blocks, int page_size, int window,
+    float scale, bf16* __restrict__ out, int nh, int nkv) {
+  constexpr int KK = D / 32;   // feature steps of the score product
+  constexpr int DT = D / 16;   // feature tiles of the output
+  __shared__ uint16_t vt[D][PF_KSTEP + PF_PAD];
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
+  const int h = kvh * G + wave;
+  const int seq = tile_seq[tile], row0 = tile_row[tile], nq = tile_n[tile];
+  const int* bt = block_table + (size_t)seq * max_blocks;
+  const int pos0 = positions[row0];                  // positions of a tile are consecutive
+  const int my_pos = pos0 + (r16 < nq ? r16 : nq - 1);
+  const bool my_live = r16 < nq;
+  const int last_key = pos0 + nq - 1;
+  const int first_key = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
+  const int my_lo = window > 0 ? (my_pos - window + 1 > 0 ? my_pos - window + 1 : 0) : 0;
+
+  // this wavefront's queries as the B operand: lane (query r16, features 8 kg ..)
+  bf16x8_t qf[KK];
+  {
+    const bf16* qrow = q + (size_t)(row0 + (my_live ? r16 : 0)) * q_stride + (size_t)h * D + kg * 8;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8_t*>(qrow + kk * 32);
+  }
+  float m = -INFINITY, l = 0.f;
+  f32x4_t acc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int k0 = (first_key / PF_KSTEP) * PF_KSTEP; k0 <= last_key; k0 += PF_KSTEP) {
+    // stage the step's value rows transposed: thread (key, chunk of 8 features)
+    __syncthreads();
+    for (int i = tid; i < PF_KSTEP * (D / 8); i += G * 64) {
+      const int key = i / (D / 8), c = i - key * (D / 8);
+      const int u = k0 + key;
+      uint4 w = make_uint4(0, 0, 0, 0);
+      if (u >= first_key && u <= last_key) {   // rows no query of the tile sees are staged as zeros
+        const int page = bt[u / page_size];
+        w = *reinterpret_cast<const uint4*>(vcache + (((size_t)page * nkv + kvh) * page_size + u % page_size) * D + c * 8);
+      }
+      const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        vt[c * 8 + 2 * e][key] = (uint16_t)(ww[e] & 0xffffu);
+        vt[c * 8 + 2 * e + 1][key] = (uint16_t)(ww[e] >> 16);
+      }
+    }
+    // scores of two blocks of 16 keys: S^T = K Q^T
+    float s[8];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int u = k0 + b * 16 + r16;               // the key whose row this lane loads
+      f32x4_t st = {0.f, 0.f, 0.f, 0.f};
+      const bool kin = u >= first_key && u <= last_key;
+      const bf16* krow = kcache;
+      if (kin) {
+        const int page = bt[u / page_size];
+        krow = kcache + (((size_t)page * nkv + kvh) * page_size + u % page_size) * D + kg * 8;
+      }
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        bf16x8_t kf;
+        if (kin) {
+          kf = *reinterpret_cast<const bf16x8_t*>(krow + kk * 32);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) kf[e] = (__bf16)0.0f;
+        }
+        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kk], st, 0, 0, 0);
+      }
+      // lane holds keys k0 + 16 b + 4 kg + i for its query
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + b * 16 + kg * 4 + i;
+        s[b * 4 + i] = (my_live && key <= my_pos && key >= my_lo) ? st[i] * scale : -INFINITY;
+      }
+    }
+    float mloc = s[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) mloc = fmaxf(mloc, s[j]);
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    const float m_new = fmaxf(m, mloc);
+    float p[8], lsum = 0.f;
+    float alpha = 1.f;
+    if (m_new > -INFINITY) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        p[j] = expf(s[j] - m_new);
+        lsum += p[j];
+      }
+      alpha = expf(m - m_new);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) p[j] = 0.f;
+    }
+    lsum += __shfl_xor(lsum, 16, 64);
+    lsum += __shfl_xor(lsum, 32, 64);
+    l = l * alpha + lsum;
+    m = m_new;
+    bf16x8_t pf;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pf[j] = (__bf16)p[j];
+    __syncthreads();   // the staged values are in place
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      // A = V^T tile: lane (feature 16 t + r16, key slots 8 kg + j <-> block j / 4, key 4 kg + j % 4)
+      union {
+        bf16x8_t v;
+        uint2 u2[2];
+      } a;
+      a.u2[0] = *reinterpret_cast<const uint2*>(&vt[t * 16 + r16][kg * 4]);
+      a.u2[1] = *reinterpret_cast<const uint2*>(&vt[t * 16 + r16][16 + kg * 4]);
+      acc[t] *= alpha;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf, acc[t], 0, 0, 0);
+    }
+  }
+  if (!my_live) return;
+  const float inv = 1.0f / l;
+  bf16* orow = out + (size_t)(row0 + r16) * nh * D + (size_t)h * D;
+#pragma unroll
+  for (int t = 0; t < DT; ++t) {
+    uint2 o;
+    o.x = (uint32_t)f32_to_bf16(acc[t][0] * inv).x | ((uint32_t)f32_to_bf16(acc[t][1] * inv).x << 16);
+    o.y = (uint32_t)f32_to_bf16(acc[t][2] * inv).x | ((uint32_t)f32_to_bf16(acc[t][3] * inv).x << 16);
+    *reinterpret_cast<uint2*>(orow + t * 16 + kg * 4) = o;
+  }
+}
+
+// Head widths 32, 64, 128; groups of 1 to 8 heads (the block has one wavefront per head of the group).
+extern "C" int gs_attention_prefill_supports(int nh, int nkv, int d) {
+  if (nkv <= 0 || nh % nkv) return 0;
+  int g = nh / nkv;
+  return (d == 32 || d == 64 || d == 128) && g >= 1 && g <= 8;
+}
+
+template <int D>
+static int launch_prefill(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
+                          const bf16* vc, const int* positions, const int* tile_seq, const int* tile_row,
+                          const int* tile_n, const int* bt, int max_blocks, int page_size, int window, float scale,
+                          bf16* out, int nh, int nkv) {
+#define GS_RUN(GG)                                                                                                   \
+  attention_prefill_kernel<D, GG><<<grid, GG * 64, 0, stream>>>(q, q_stride, kc, vc, positions, tile_seq, tile_row, \
+                                                                tile_n, bt, max_blocks, page_size, window, scale,   \
+                                                                out, nh, nkv)
+  switch (G) {
+    case 1: GS_RUN(1); break;
+    case 2: GS_RUN(2); break;
+    case 3: GS_RUN(3); break;
+    case 4: GS_RUN(4); break;
+    case 5: GS_RUN(5); break;
+    case 6: GS_RUN(6); break;
+    case 7: GS_RUN(7); break;
+    case 8: GS_RUN(8); break;
+    default: return -1;
+  }
+#undef GS_RUN
+  return 0;
+}
+
+extern "C" int gs_attention_prefill(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                    const int* positions, const int* tile_seq, const int* tile_row,
+                                    const int* tile_n, int ntiles, const int* block_table, int max_blocks,
+                                    int page_size, int window, float scale, void* out, int nh, int nkv, int d,
+                                    hipStream_t stream) {
+  GS_REQUIRE(gs_attention_prefill_supports(nh, nkv, d), "attention_prefill: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
+  GS_REQUIRE(ntiles >= 0 && nkv <= 65535, "attention_prefill: bad grid");
+  GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill: bad page_size/max_blocks/window");
+  GS_REQUIRE(q_stride >= nh * d && q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_prefill: q rows must be 16-byte aligned");
+  GS_REQUIRE(((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0 && ((uintptr_t)out & 7) == 0,
+             "attention_prefill: cache and output must be aligned");
+  if (ntiles == 0) return 0;
+  dim3 grid(ntiles, nkv);
+  int rc = -1;
+#define GS_ARGS                                                                                                      \
+  nh / nkv, grid, stream, (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions, tile_seq,  \
+      tile_row, tile_n, block_table, max_blocks, page_size, window, scale, (bf16*)out, nh, nkv
+  switch (d) {
+    case 32: rc = launch_prefill<32>(GS_ARGS); break;
+    case 64: rc = launch_prefill<64>(GS_ARGS); break;
+    case 128: rc = launch_prefill<128>(GS_ARGS); break;
+  }
+#undef GS_ARGS
+  GS_REQUIRE(rc == 0, "attention_prefill: no kernel for this group size");
+  GS_LAUNCH_CHECK("attention_prefill");
+  return 0;
+}

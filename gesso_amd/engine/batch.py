@@ -98,8 +98,25 @@ class StepContext:
         (self.token_ids, self.positions, self.seq_of_token, self.q_start, self.kv_len, self.slots,
          self.want_rows, flat_tables) = views
         self.block_tables = [flat_tables.view(n_groups, nseq, max_blocks)[g] for g in range(n_groups)] if n_groups else []
+        self._tiles = None
         self._host = host          # keeps the pinned buffer alive until the copy has run
         self._storage = storage
 
     def cache_view(self, call: int):
         return self._storage.view(call, self.block_tables)
+
+    def query_tiles(self, rows: int = 16) -> torch.Tensor:
+        """int32 ``(3, ntiles)``: sequence, first row, row count of each tile of at most ``rows`` consecutive
+        queries of one sequence; made once per step, on first use."""
+        if self._tiles is None or self._tiles[0] != rows:
+            seq, row, cnt = [], [], []
+            at = 0
+            for i, n in enumerate(self.q_lens):
+                for a in range(0, n, rows):
+                    seq.append(i)
+                    row.append(at + a)
+                    cnt.append(min(rows, n - a))
+                at += n
+            t = torch.tensor([seq, row, cnt], dtype=torch.int32).pin_memory().to(self.token_ids.device, non_blocking=True)
+            self._tiles = (rows, t)
+        return self._tiles[1]

@@ -478,3 +478,34 @@ def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_s
                                      _p(out), _p(ws), c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit),
                                      _stream()))
     return out
+
+
+def attention_prefill_supports(nh: int, nkv: int, d: int) -> bool:
+    return bool(lib().gs_attention_prefill_supports(c_int(nh), c_int(nkv), c_int(d)))
+
+
+def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv, d,
+                      ntok, out: torch.Tensor = None) -> torch.Tensor:
+    """Causal GQA of many queries per sequence on the matrix cores (bfloat16).
+
+    ``tiles``: int32 ``(3, ntiles)``: sequence, first row and number of rows (<= 16) of each tile of
+    consecutive queries of one sequence.
+    """
+    _dev(q, kcache, vcache, positions, tiles, block_table, out)
+    _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
+          "attention_prefill takes bfloat16")
+    _need(q.numel() >= (ntok - 1) * q_stride + nh * d if ntok else True, "attention_prefill: q is too small")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
+          "cache must be (pages, nkv, page_size, d)")
+    _i32(positions, ntok, "positions")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[0] == 3, "tiles must be int32 (3, ntiles)")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
+    if out is None:
+        out = torch.empty((ntok, nh * d), dtype=q.dtype, device=q.device)
+    _need(out.shape == (ntok, nh * d) and out.dtype == q.dtype, "attention_prefill: out has the wrong shape or type")
+    nt = tiles.shape[1]
+    _check(lib().gs_attention_prefill(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(tiles[0]),
+                                      _p(tiles[1]), _p(tiles[2]), c_int(nt), _p(block_table),
+                                      c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
+                                      _p(out), c_int(nh), c_int(nkv), c_int(d), _stream()))
+    return out

@@ -158,5 +158,10 @@ class Runtime:
             nsplit = max(1, min(16, 256 // max(1, ctx.nseq * nkv)))
             return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                         cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
+        if (not ctx.all_single and q.dtype == torch.bfloat16 and q_stride % 8 == 0
+                and ops.attention_prefill_supports(nh, nkv, d)):
+            # prompts: queries in tiles of 16 per sequence, both products on the matrix cores
+            return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(16),
+                                         cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)
         return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
                                      cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)

@@ -560,3 +560,78 @@ def test_tile_major_copy_gives_the_same_products(ops, M, N, K):
         r1, r2 = torch.ones(M, N, device=DEV), torch.ones(M, N, device=DEV)
         s1, s2 = ops.gemm_skinny_residual(x, w, r1, wt=wt), ops.gemm_skinny_residual(x, w, r2)
         assert torch.equal(r1, r2) and torch.equal(s1, s2)
+
+
+# ------------------------------------------------------------------ prompt attention on the matrix cores
+
+@pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 32, 8), (32, 8, 64, 16), (3, 1, 64, 16), (8, 1, 128, 16), (5, 5, 64, 4)])
+@pytest.mark.parametrize("window", [None, 37])
+def test_attention_prefill(ops, nh, nkv, d, ps, window):
+    """Three sequences in one launch: a chunk over a cached prefix, a fresh prompt, a single token."""
+    g = gen(nh + d + ps)
+    prefix = [70, 0, 45]
+    new = [41, 33, 1]
+    nseq = 3
+    K = [a + b for a, b in zip(prefix, new)]
+    nblk = [-(-k // ps) for k in K]
+    total = sum(nblk)
+    perm = torch.randperm(total + 2, generator=g)[:total] + 1
+    kc = torch.randn(total + 3, nkv, ps, d, generator=g).bfloat16()
+    vc = torch.randn(total + 3, nkv, ps, d, generator=g).bfloat16()
+    table = torch.zeros(nseq, max(nblk), dtype=torch.int32)
+    qs, want, at = [], [], 0
+    for i in range(nseq):
+        pages = perm[at:at + nblk[i]]
+        at += nblk[i]
+        table[i, :nblk[i]] = pages.to(torch.int32)
+        k = kc[pages].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:K[i]]
+        v = vc[pages].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:K[i]]
+        q = torch.randn(new[i], nh, d, generator=g)
+        if i == 0:
+            q[-1] *= 3.0
+        q = q.bfloat16()
+        qs.append(q.reshape(new[i], -1))
+        want.append(P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(new[i], -1))
+    qall, want = torch.cat(qs), torch.cat(want)
+    positions = torch.tensor([p + j for p, n in zip(prefix, new) for j in range(n)], dtype=torch.int32)
+    seq_of = torch.tensor([i for i, n in enumerate(new) for _ in range(n)], dtype=torch.int32)
+    tiles, row = [[], [], []], 0
+    for i, n in enumerate(new):
+        for a in range(0, n, 16):
+            tiles[0].append(i); tiles[1].append(row + a); tiles[2].append(min(16, n - a))
+        row += n
+    tiles = torch.tensor(tiles, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    # q as a strided view, as the attention mixer hands it over (q, k, v side by side)
+    wide = torch.zeros(sum(new), (nh + 2 * nkv) * d, dtype=torch.bfloat16)
+    wide[:, :nh * d] = qall
+    got = ops.attention_prefill(wide.to(DEV), (nh + 2 * nkv) * d, kc.to(DEV), vc.to(DEV), positions.to(DEV),
+                                tiles.to(DEV), table.to(DEV), ps, window, scale, nh, nkv, d, sum(new))
+    close(got, want, torch.bfloat16)
+    same = ops.attention_generic(wide.to(DEV), (nh + 2 * nkv) * d, kc.to(DEV), vc.to(DEV), positions.to(DEV),
+                                 seq_of.to(DEV), table.to(DEV), ps, window, scale, nh, nkv, d, sum(new))
+    close(got, same.double().cpu(), torch.bfloat16)
+
+
+def test_attention_prefill_far_key_and_supports(ops):
+    assert ops.attention_prefill_supports(32, 8, 64) and not ops.attention_prefill_supports(3, 3, 48)
+    assert not ops.attention_prefill_supports(18, 2, 64)
+    # 600 cached keys; key 5 carries most of the weight for the last query of a 20-token chunk
+    g = gen(77)
+    nh, nkv, d, ps, prefix, new = 4, 2, 64, 16, 600, 20
+    K = prefix + new
+    k, v, q = torch.randn(K, nkv, d, generator=g), torch.randn(K, nkv, d, generator=g), torch.randn(new, nh, d, generator=g)
+    q[-1] *= 4.0
+    k[5] = q[-1, ::2][:nkv] / 4.0 * 2.0
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    nblk = -(-K // ps)
+    kc = torch.zeros(nblk, nkv, ps, d, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    for u in range(K):
+        kc[u // ps, :, u % ps], vc[u // ps, :, u % ps] = k[u], v[u]
+    table = torch.arange(nblk, dtype=torch.int32)[None]
+    tiles = torch.tensor([[0, 0], [0, 16], [16, 4]], dtype=torch.int32)
+    got = ops.attention_prefill(q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV),
+                                torch.arange(prefix, K, dtype=torch.int32, device=DEV), tiles.to(DEV), table.to(DEV), ps,
+                                None, 1.0 / math.sqrt(d), nh, nkv, d, new)
+    close(got, P.causal_attention(q.double(), k.double(), v.double()).reshape(new, -1), torch.bfloat16)
