@@ -15,8 +15,8 @@
 // lane groups.  v_mfma_f32_16x16x32_bf16 throughout.
 //
 // Causal rule: the query at position p sees keys lo..p, lo = 0 or p - window + 1.  Tiles of queries come
-// from the host: tile i covers rows tile_row[i] .. + tile_n[i] of the flattened tokens, of sequence
-// tile_seq[i].  q (T, q_stride), head h at [h D, (h+1) D); caches (pages, nkv, page_size, D); out (T, nh D).
+// from the host: tile i covers rows tile_row[i] .. + tile_n[i] (at most 16 QT) of the flattened tokens, of
+// sequence tile_seq[i].  Exponentials are base 2 on scores scaled by log2(e): one v_exp_f32 each.  q (T, q_stride), head h at [h D, (h+1) D); caches (pages, nkv, page_size, D); out (T, nh D).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -24,8 +24,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 #define PF_KSTEP 32
 #define PF_PAD 8
+#define PF_LOG2E 1.4426950408889634f
 
-template <int D, int G>
+// QT: tiles of 16 queries per wavefront; a key fragment and a value fragment feed QT products each.
+template <int D, int G, int QT>
 __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int* __restrict__ positions, const int* __restrict__ tile_seq, const int* __restrict__ tile_row,
@@ -41,23 +43,33 @@ __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
   const int seq = tile_seq[tile], row0 = tile_row[tile], nq = tile_n[tile];
   const int* bt = block_table + (size_t)seq * max_blocks;
   const int pos0 = positions[row0];                  // positions of a tile are consecutive
-  const int my_pos = pos0 + (r16 < nq ? r16 : nq - 1);
-  const bool my_live = r16 < nq;
   const int last_key = pos0 + nq - 1;
   const int first_key = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
-  const int my_lo = window > 0 ? (my_pos - window + 1 > 0 ? my_pos - window + 1 : 0) : 0;
+  // scores are kept in units of log2(e), so that the exponentials are single v_exp_f32
+  const float sc = scale * PF_LOG2E;
 
-  // this wavefront's queries as the B operand: lane (query r16, features 8 kg ..)
-  bf16x8_t qf[KK];
-  {
-    const bf16* qrow = q + (size_t)(row0 + (my_live ? r16 : 0)) * q_stride + (size_t)h * D + kg * 8;
+  bool live[QT];
+  int my_pos[QT], my_lo[QT];
+  bf16x8_t qf[QT][KK];   // the queries as the B operand: lane (query r16, features 8 kg ..)
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8_t*>(qrow + kk * 32);
+  for (int t = 0; t < QT; ++t) {
+    const int r = t * 16 + r16;
+    live[t] = r < nq;
+    my_pos[t] = pos0 + (live[t] ? r : nq - 1);
+    my_lo[t] = window > 0 ? (my_pos[t] - window + 1 > 0 ? my_pos[t] - window + 1 : 0) : 0;
+    const bf16* qrow = q + (size_t)(row0 + (live[t] ? r : 0)) * q_stride + (size_t)h * D + kg * 8;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) qf[t][kk] = *reinterpret_cast<const bf16x8_t*>(qrow + kk * 32);
   }
-  float m = -INFINITY, l = 0.f;
-  f32x4_t acc[DT];
+  float m[QT], l[QT];
+  f32x4_t acc[QT][DT];
 #pragma unroll
-  for (int t = 0; t < DT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < QT; ++t) {
+    m[t] = -INFINITY;
+    l[t] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[t][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
 
   for (int k0 = (first_key / PF_KSTEP) * PF_KSTEP; k0 <= last_key; k0 += PF_KSTEP) {
     // stage the step's value rows transposed: thread (key, chunk of 8 features)
@@ -77,18 +89,22 @@ __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
         vt[c * 8 + 2 * e + 1][key] = (uint16_t)(ww[e] >> 16);
       }
     }
+    // a step every query of the tile sees whole needs no mask
+    const bool whole = (k0 + PF_KSTEP - 1 <= pos0) && (window <= 0 || k0 >= pos0 + nq - window);
     // scores of two blocks of 16 keys: S^T = K Q^T
-    float s[8];
+    float s[QT][8];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       const int u = k0 + b * 16 + r16;               // the key whose row this lane loads
-      f32x4_t st = {0.f, 0.f, 0.f, 0.f};
       const bool kin = u >= first_key && u <= last_key;
       const bf16* krow = kcache;
       if (kin) {
         const int page = bt[u / page_size];
         krow = kcache + (((size_t)page * nkv + kvh) * page_size + u % page_size) * D + kg * 8;
       }
+      f32x4_t st[QT];
+#pragma unroll
+      for (int t = 0; t < QT; ++t) st[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         bf16x8_t kf;
@@ -98,64 +114,78 @@ __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
 #pragma unroll
           for (int e = 0; e < 8; ++e) kf[e] = (__bf16)0.0f;
         }
-        st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kk], st, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][kk], st[t], 0, 0, 0);
       }
       // lane holds keys k0 + 16 b + 4 kg + i for its query
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + b * 16 + kg * 4 + i;
-        s[b * 4 + i] = (my_live && key <= my_pos && key >= my_lo) ? st[i] * scale : -INFINITY;
-      }
+      for (int t = 0; t < QT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + b * 16 + kg * 4 + i;
+          const bool see = whole ? live[t] : (live[t] && key <= my_pos[t] && key >= my_lo[t]);
+          s[t][b * 4 + i] = see ? st[t][i] * sc : -INFINITY;
+        }
     }
-    float mloc = s[0];
+    bf16x8_t pf[QT];
+    float alpha[QT];
 #pragma unroll
-    for (int j = 1; j < 8; ++j) mloc = fmaxf(mloc, s[j]);
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-    const float m_new = fmaxf(m, mloc);
-    float p[8], lsum = 0.f;
-    float alpha = 1.f;
-    if (m_new > -INFINITY) {
+    for (int t = 0; t < QT; ++t) {
+      float mloc = s[t][0];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        p[j] = expf(s[j] - m_new);
-        lsum += p[j];
+      for (int j = 1; j < 8; ++j) mloc = fmaxf(mloc, s[t][j]);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+      const float m_new = fmaxf(m[t], mloc);
+      float p[8], lsum = 0.f;
+      alpha[t] = 1.f;
+      if (m_new > -INFINITY) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          p[j] = exp2f(s[t][j] - m_new);
+          lsum += p[j];
+        }
+        alpha[t] = exp2f(m[t] - m_new);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) p[j] = 0.f;
       }
-      alpha = expf(m - m_new);
-    } else {
+      lsum += __shfl_xor(lsum, 16, 64);
+      lsum += __shfl_xor(lsum, 32, 64);
+      l[t] = l[t] * alpha[t] + lsum;
+      m[t] = m_new;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) p[j] = 0.f;
+      for (int j = 0; j < 8; ++j) pf[t][j] = (__bf16)p[j];
     }
-    lsum += __shfl_xor(lsum, 16, 64);
-    lsum += __shfl_xor(lsum, 32, 64);
-    l = l * alpha + lsum;
-    m = m_new;
-    bf16x8_t pf;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) pf[j] = (__bf16)p[j];
     __syncthreads();   // the staged values are in place
 #pragma unroll
-    for (int t = 0; t < DT; ++t) {
-      // A = V^T tile: lane (feature 16 t + r16, key slots 8 kg + j <-> block j / 4, key 4 kg + j % 4)
+    for (int dt = 0; dt < DT; ++dt) {
+      // A = V^T tile: lane (feature 16 dt + r16, key slots 8 kg + j <-> block j / 4, key 4 kg + j % 4)
       union {
         bf16x8_t v;
         uint2 u2[2];
       } a;
-      a.u2[0] = *reinterpret_cast<const uint2*>(&vt[t * 16 + r16][kg * 4]);
-      a.u2[1] = *reinterpret_cast<const uint2*>(&vt[t * 16 + r16][16 + kg * 4]);
-      acc[t] *= alpha;
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf, acc[t], 0, 0, 0);
+      a.u2[0] = *reinterpret_cast<const uint2*>(&vt[dt * 16 + r16][kg * 4]);
+      a.u2[1] = *reinterpret_cast<const uint2*>(&vt[dt * 16 + r16][16 + kg * 4]);
+#pragma unroll
+      for (int t = 0; t < QT; ++t) {
+        acc[t][dt] *= alpha[t];
+        acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf[t], acc[t][dt], 0, 0, 0);
+      }
     }
   }
-  if (!my_live) return;
-  const float inv = 1.0f / l;
-  bf16* orow = out + (size_t)(row0 + r16) * nh * D + (size_t)h * D;
 #pragma unroll
-  for (int t = 0; t < DT; ++t) {
-    uint2 o;
-    o.x = (uint32_t)f32_to_bf16(acc[t][0] * inv).x | ((uint32_t)f32_to_bf16(acc[t][1] * inv).x << 16);
-    o.y = (uint32_t)f32_to_bf16(acc[t][2] * inv).x | ((uint32_t)f32_to_bf16(acc[t][3] * inv).x << 16);
-    *reinterpret_cast<uint2*>(orow + t * 16 + kg * 4) = o;
+  for (int t = 0; t < QT; ++t) {
+    if (!live[t]) continue;
+    const float inv = 1.0f / l[t];
+    bf16* orow = out + (size_t)(row0 + t * 16 + r16) * nh * D + (size_t)h * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 o;
+      o.x = (uint32_t)f32_to_bf16(acc[t][dt][0] * inv).x | ((uint32_t)f32_to_bf16(acc[t][dt][1] * inv).x << 16);
+      o.y = (uint32_t)f32_to_bf16(acc[t][dt][2] * inv).x | ((uint32_t)f32_to_bf16(acc[t][dt][3] * inv).x << 16);
+      *reinterpret_cast<uint2*>(orow + dt * 16 + kg * 4) = o;
+    }
   }
 }
 
@@ -166,13 +196,13 @@ extern "C" int gs_attention_prefill_supports(int nh, int nkv, int d) {
   return (d == 32 || d == 64 || d == 128) && g >= 1 && g <= 8;
 }
 
-template <int D>
+template <int D, int QT>
 static int launch_prefill(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
                           const bf16* vc, const int* positions, const int* tile_seq, const int* tile_row,
                           const int* tile_n, const int* bt, int max_blocks, int page_size, int window, float scale,
                           bf16* out, int nh, int nkv) {
 #define GS_RUN(GG)                                                                                                   \
-  attention_prefill_kernel<D, GG><<<grid, GG * 64, 0, stream>>>(q, q_stride, kc, vc, positions, tile_seq, tile_row, \
+  attention_prefill_kernel<D, GG, QT><<<grid, GG * 64, 0, stream>>>(q, q_stride, kc, vc, positions, tile_seq, tile_row, \
                                                                 tile_n, bt, max_blocks, page_size, window, scale,   \
                                                                 out, nh, nkv)
   switch (G) {
@@ -194,9 +224,10 @@ extern "C" int gs_attention_prefill(const void* q, int q_stride, const void* kca
                                     const int* positions, const int* tile_seq, const int* tile_row,
                                     const int* tile_n, int ntiles, const int* block_table, int max_blocks,
                                     int page_size, int window, float scale, void* out, int nh, int nkv, int d,
-                                    hipStream_t stream) {
+                                    int tile_rows, hipStream_t stream) {
   GS_REQUIRE(gs_attention_prefill_supports(nh, nkv, d), "attention_prefill: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
   GS_REQUIRE(ntiles >= 0 && nkv <= 65535, "attention_prefill: bad grid");
+  GS_REQUIRE(tile_rows == 16 || tile_rows == 32, "attention_prefill: tiles hold 16 or 32 queries, not %d", tile_rows);
   GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill: bad page_size/max_blocks/window");
   GS_REQUIRE(q_stride >= nh * d && q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_prefill: q rows must be 16-byte aligned");
   GS_REQUIRE(((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0 && ((uintptr_t)out & 7) == 0,
@@ -207,10 +238,18 @@ extern "C" int gs_attention_prefill(const void* q, int q_stride, const void* kca
 #define GS_ARGS                                                                                                      \
   nh / nkv, grid, stream, (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions, tile_seq,  \
       tile_row, tile_n, block_table, max_blocks, page_size, window, scale, (bf16*)out, nh, nkv
-  switch (d) {
-    case 32: rc = launch_prefill<32>(GS_ARGS); break;
-    case 64: rc = launch_prefill<64>(GS_ARGS); break;
-    case 128: rc = launch_prefill<128>(GS_ARGS); break;
+  if (tile_rows == 16) {
+    switch (d) {
+      case 32: rc = launch_prefill<32, 1>(GS_ARGS); break;
+      case 64: rc = launch_prefill<64, 1>(GS_ARGS); break;
+      case 128: rc = launch_prefill<128, 1>(GS_ARGS); break;
+    }
+  } else {
+    switch (d) {
+      case 32: rc = launch_prefill<32, 2>(GS_ARGS); break;
+      case 64: rc = launch_prefill<64, 2>(GS_ARGS); break;
+      case 128: rc = launch_prefill<128, 2>(GS_ARGS); break;
+    }
   }
 #undef GS_ARGS
   GS_REQUIRE(rc == 0, "attention_prefill: no kernel for this group size");

@@ -91,4 +91,35 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return red[16];
 }
 
+// Eight consecutive values as float, from float32 or bfloat16 storage (16-byte aligned), and back.
+__device__ __forceinline__ void load8f(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8f(const bf16* p, float* v) {
+  const uint4 w = *reinterpret_cast<const uint4*>(p);
+  const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[2 * e] = __uint_as_float(ww[e] << 16);
+    v[2 * e + 1] = __uint_as_float(ww[e] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void store8f(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8f(bf16* p, const float* v) {
+  uint4 w;
+  w.x = (uint32_t)f32_to_bf16(v[0]).x | ((uint32_t)f32_to_bf16(v[1]).x << 16);
+  w.y = (uint32_t)f32_to_bf16(v[2]).x | ((uint32_t)f32_to_bf16(v[3]).x << 16);
+  w.z = (uint32_t)f32_to_bf16(v[4]).x | ((uint32_t)f32_to_bf16(v[5]).x << 16);
+  w.w = (uint32_t)f32_to_bf16(v[6]).x | ((uint32_t)f32_to_bf16(v[7]).x << 16);
+  *reinterpret_cast<uint4*>(p) = w;
+}
+template <typename T>
+__device__ __forceinline__ bool aligned16(const T* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
 static inline int gs_ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -79,6 +79,57 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict
   float* x = res + (size_t)s * H;
   const TD* dl = delta ? delta + (size_t)s * H : nullptr;
   float ss = 0.f;
+  TO* o = out + (size_t)r * H;
+  if ((H & 7) == 0 && aligned16(x) && aligned16(o) && aligned16(w) && (!dl || aligned16(dl))) {
+    // eight values per thread and turn, 16-byte loads and stores; the row stays in registers between the passes
+    constexpr int MAXV = 4;                       // turns kept in registers: rows up to 8 * 256 * 4 values
+    float keep[MAXV][8];
+    const int turns = (H / 8 + blockDim.x - 1) / blockDim.x;
+    for (int u = 0; u < turns; ++u) {
+      const int j = (u * blockDim.x + threadIdx.x) * 8;
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (j < H) {
+        load8f(x + j, v);
+        if (dl) {
+          float d8[8];
+          load8f(dl + j, d8);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] += d8[i];
+          if (!rows) store8f(x + j, v);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+      }
+      if (u < MAXV) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) keep[u][i] = v[i];
+      }
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int u = 0; u < turns; ++u) {
+      const int j = (u * blockDim.x + threadIdx.x) * 8;
+      if (j >= H) break;
+      float v[8], w8[8];
+      if (u < MAXV) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = keep[u][i];
+      } else {
+        load8f(x + j, v);
+        if (dl && rows) {
+          float d8[8];
+          load8f(dl + j, d8);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] += d8[i];
+        }
+      }
+      load8f(w + j, w8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = v[i] * inv * w8[i];
+      store8f(o + j, v);
+    }
+    return;
+  }
   for (int j = threadIdx.x; j < H; j += blockDim.x) {
     float v = x[j];
     if (dl) {
@@ -89,7 +140,6 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict
   }
   ss = block_sum(ss, red);
   float inv = 1.0f / sqrtf(ss / (float)H + eps);
-  TO* o = out + (size_t)r * H;
   for (int j = threadIdx.x; j < H; j += blockDim.x) {
     float v = x[j];
     if (dl && rows) v += to_f32(dl[j]);
@@ -186,6 +236,22 @@ extern "C" int gs_residual_add(float* res, const void* delta, int delta_dtype, l
 // ------------------------------------------------------------------ SwiGLU
 
 // in (T, 2F): gate in columns [0, F), up in [F, 2F).  out[t, j] = silu(gate) * up, silu(g) = g / (1 + exp(-g)).
+// Eight outputs per thread with 16-byte loads and stores; F a multiple of 8, rows 16-byte aligned.
+template <typename T>
+__global__ void swiglu8_kernel(const T* __restrict__ in, T* __restrict__ out, int F, long n8) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n8) return;
+  const int f8 = F / 8;
+  long t = i / f8;
+  int j = (int)(i - t * f8) * 8;
+  float g[8], u[8];
+  load8f(in + t * 2 * F + j, g);
+  load8f(in + t * 2 * F + F + j, u);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) g[k] = g[k] / (1.0f + expf(-g[k])) * u[k];
+  store8f(out + t * F + j, g);
+}
+
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ in, T* __restrict__ out, int F, long n) {
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -201,6 +267,15 @@ extern "C" int gs_swiglu(const void* in, void* out, int dtype, int T, int F, hip
   GS_REQUIRE(T >= 0 && F > 0, "swiglu: bad sizes T=%d F=%d", T, F);
   long n = (long)T * F;
   if (n == 0) return 0;
+  if (F % 8 == 0 && ((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0 && (dtype == GS_F32 || dtype == GS_BF16)) {
+    long n8 = n / 8;
+    if (dtype == GS_F32)
+      swiglu8_kernel<float><<<gs_ceil_div(n8, 256), 256, 0, stream>>>((const float*)in, (float*)out, F, n8);
+    else
+      swiglu8_kernel<bf16><<<gs_ceil_div(n8, 256), 256, 0, stream>>>((const bf16*)in, (bf16*)out, F, n8);
+    GS_LAUNCH_CHECK("swiglu");
+    return 0;
+  }
   int blocks = gs_ceil_div(n, 256);
   if (dtype == GS_F32)
     swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, F, n);

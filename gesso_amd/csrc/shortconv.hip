@@ -54,6 +54,51 @@ __global__ void short_conv_kernel(const T* __restrict__ bcx, const float* __rest
   }
 }
 
+// Eight channels per thread: 16-byte loads of B, C and X rows.  H a multiple of 8, rows 16-byte aligned.
+template <typename T>
+__global__ void short_conv8_kernel(const T* __restrict__ bcx, const float* __restrict__ taps,
+                                   const float* __restrict__ bias, float* __restrict__ state,
+                                   const int* __restrict__ seq_of_token, const int* __restrict__ q_start,
+                                   const int* __restrict__ slots, T* __restrict__ out, int ntok, int H, int W,
+                                   int update_state) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (c >= H) return;
+  for (int t = blockIdx.y; t < ntok; t += gridDim.y) {
+    const int s = seq_of_token[t];
+    const int t0 = q_start[s];
+    float* hist = state + ((size_t)slots[s] * H + c) * (W - 1);   // channel c + i at hist + i (W - 1)
+    float y[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, u[8];
+    for (int p = 0; p < W; ++p) {
+      const int j = t - (W - 1) + p;
+      if (j >= t0) {
+        float b8[8], x8[8];
+        load8f(bcx + (size_t)j * 3 * H + c, b8);
+        load8f(bcx + (size_t)j * 3 * H + 2 * H + c, x8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) u[i] = b8[i] * x8[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) u[i] = hist[i * (W - 1) + (W - 1) - (t0 - j)];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] += taps[(size_t)(c + i) * W + p] * u[i];
+    }
+    float c8[8];
+    load8f(bcx + (size_t)t * 3 * H + H + c, c8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = c8[i] * (bias ? y[i] + bias[c + i] : y[i]);
+    store8f(out + (size_t)t * H + c, y);
+    if (update_state) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float* h = hist + i * (W - 1);
+        for (int p = 0; p < W - 2; ++p) h[p] = h[p + 1];
+        h[W - 2] = u[i];
+      }
+    }
+  }
+}
+
 template <typename T>
 __global__ void short_conv_state_kernel(const T* __restrict__ bcx, float* __restrict__ state,
                                         const int* __restrict__ q_start, const int* __restrict__ slots, int H,
@@ -87,7 +132,18 @@ extern "C" int gs_short_conv(const void* bcx, int dtype, const float* taps, cons
   int threads = H >= 256 ? 256 : 64;
   int cx = gs_ceil_div(H, threads);
   dim3 grid(cx, ntok < 65535 ? ntok : 65535);  // the kernel strides over tokens beyond gridDim.y
-  if (dtype == GS_F32)
+  const bool vec = H % 8 == 0 && ((uintptr_t)bcx & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
+                   (dtype == GS_F32 || dtype == GS_BF16);
+  if (vec) {
+    int th = H / 8 >= 256 ? 256 : 64;
+    dim3 g8(gs_ceil_div(H / 8, th), grid.y);
+    if (dtype == GS_F32)
+      short_conv8_kernel<float><<<g8, th, 0, stream>>>((const float*)bcx, taps, bias, state, seq_of_token, q_start,
+                                                       slots, (float*)out, ntok, H, W, all_single);
+    else
+      short_conv8_kernel<bf16><<<g8, th, 0, stream>>>((const bf16*)bcx, taps, bias, state, seq_of_token, q_start,
+                                                      slots, (bf16*)out, ntok, H, W, all_single);
+  } else if (dtype == GS_F32)
     short_conv_kernel<float><<<grid, threads, 0, stream>>>((const float*)bcx, taps, bias, state, seq_of_token,
                                                             q_start, slots, (float*)out, ntok, H, W, all_single);
   else if (dtype == GS_BF16)

@@ -485,11 +485,11 @@ def attention_prefill_supports(nh: int, nkv: int, d: int) -> bool:
 
 
 def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv, d,
-                      ntok, out: torch.Tensor = None) -> torch.Tensor:
+                      ntok, out: torch.Tensor = None, tile_rows: int = 16) -> torch.Tensor:
     """Causal GQA of many queries per sequence on the matrix cores (bfloat16).
 
-    ``tiles``: int32 ``(3, ntiles)``: sequence, first row and number of rows (<= 16) of each tile of
-    consecutive queries of one sequence.
+    ``tiles``: int32 ``(3, ntiles)``: sequence, first row and number of rows (at most ``tile_rows``, 16 or
+    32) of each tile of consecutive queries of one sequence.
     """
     _dev(q, kcache, vcache, positions, tiles, block_table, out)
     _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
@@ -507,5 +507,5 @@ def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table
     _check(lib().gs_attention_prefill(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(tiles[0]),
                                       _p(tiles[1]), _p(tiles[2]), c_int(nt), _p(block_table),
                                       c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
-                                      _p(out), c_int(nh), c_int(nkv), c_int(d), _stream()))
+                                      _p(out), c_int(nh), c_int(nkv), c_int(d), c_int(tile_rows), _stream()))
     return out

@@ -160,8 +160,11 @@ class Runtime:
                                         cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
         if (not ctx.all_single and q.dtype == torch.bfloat16 and q_stride % 8 == 0
                 and ops.attention_prefill_supports(nh, nkv, d)):
-            # prompts: queries in tiles of 16 per sequence, both products on the matrix cores
-            return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(16),
-                                         cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)
+            # prompts: queries in tiles per sequence, both products on the matrix cores; tiles of 32 share
+            # every key and value fragment between two products, which pays when portions are long
+            rows = 32 if ctx.max_q_len >= 64 else 16
+            return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows),
+                                         cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T,
+                                         tile_rows=rows)
         return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
                                      cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)

@@ -566,7 +566,8 @@ def test_tile_major_copy_gives_the_same_products(ops, M, N, K):
 
 @pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 32, 8), (32, 8, 64, 16), (3, 1, 64, 16), (8, 1, 128, 16), (5, 5, 64, 4)])
 @pytest.mark.parametrize("window", [None, 37])
-def test_attention_prefill(ops, nh, nkv, d, ps, window):
+@pytest.mark.parametrize("rows", [16, 32])
+def test_attention_prefill(ops, nh, nkv, d, ps, window, rows):
     """Three sequences in one launch: a chunk over a cached prefix, a fresh prompt, a single token."""
     g = gen(nh + d + ps)
     prefix = [70, 0, 45]
@@ -597,8 +598,8 @@ def test_attention_prefill(ops, nh, nkv, d, ps, window):
     seq_of = torch.tensor([i for i, n in enumerate(new) for _ in range(n)], dtype=torch.int32)
     tiles, row = [[], [], []], 0
     for i, n in enumerate(new):
-        for a in range(0, n, 16):
-            tiles[0].append(i); tiles[1].append(row + a); tiles[2].append(min(16, n - a))
+        for a in range(0, n, rows):
+            tiles[0].append(i); tiles[1].append(row + a); tiles[2].append(min(rows, n - a))
         row += n
     tiles = torch.tensor(tiles, dtype=torch.int32)
     scale = 1.0 / math.sqrt(d)
@@ -606,7 +607,7 @@ def test_attention_prefill(ops, nh, nkv, d, ps, window):
     wide = torch.zeros(sum(new), (nh + 2 * nkv) * d, dtype=torch.bfloat16)
     wide[:, :nh * d] = qall
     got = ops.attention_prefill(wide.to(DEV), (nh + 2 * nkv) * d, kc.to(DEV), vc.to(DEV), positions.to(DEV),
-                                tiles.to(DEV), table.to(DEV), ps, window, scale, nh, nkv, d, sum(new))
+                                tiles.to(DEV), table.to(DEV), ps, window, scale, nh, nkv, d, sum(new), tile_rows=rows)
     close(got, want, torch.bfloat16)
     same = ops.attention_generic(wide.to(DEV), (nh + 2 * nkv) * d, kc.to(DEV), vc.to(DEV), positions.to(DEV),
                                  seq_of.to(DEV), table.to(DEV), ps, window, scale, nh, nkv, d, sum(new))
