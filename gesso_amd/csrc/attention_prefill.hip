@@ -17,13 +17,17 @@
 // Causal rule: the query at position p sees keys lo..p, lo = 0 or p - window + 1.  Tiles of queries come
 // from the host: tile i covers rows tile_row[i] .. + tile_n[i] (at most 16 QT) of the flattened tokens, of
 // sequence tile_seq[i].  Exponentials are base 2 on scores scaled by log2(e): one v_exp_f32 each.  q (T, q_stride), head h at [h D, (h+1) D); caches (pages, nkv, page_size, D); out (T, nh D).
+#include <type_traits>
+
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 #define PF_KSTEP 32
-#define PF_PAD 8
+#define PF_PAD 4
+#define PF_MAXPAGES 2048
+#define PF_SLACK 6.0f
 #define PF_LOG2E 1.4426950408889634f
 
 // QT: tiles of 16 queries per wavefront; a key fragment and a value fragment feed QT products each.
@@ -36,7 +40,8 @@ __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
   constexpr int KK = D / 32;   // feature steps of the score product
   constexpr int DT = D / 16;   // feature tiles of the output
   __shared__ uint16_t vt[D][PF_KSTEP + PF_PAD];
-  const int tile = blockIdx.x, kvh = blockIdx.y;
+  __shared__ int pages[PF_MAXPAGES];
+  const int tile = gridDim.x - 1 - blockIdx.x, kvh = blockIdx.y;   // late tiles walk the most keys: they start first
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int h = kvh * G + wave;
@@ -47,6 +52,7 @@ __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
   const int first_key = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
   // scores are kept in units of log2(e), so that the exponentials are single v_exp_f32
   const float sc = scale * PF_LOG2E;
+  const int ps_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
 
   bool live[QT];
   int my_pos[QT], my_lo[QT];
@@ -71,89 +77,126 @@ __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
     for (int dt = 0; dt < DT; ++dt) acc[t][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int k0 = (first_key / PF_KSTEP) * PF_KSTEP; k0 <= last_key; k0 += PF_KSTEP) {
+  // The tile's part of the block table goes to LDS first: a key's row is then one global load away, not
+  // two dependent ones (page number, then row).  Longer ranges than the LDS copy holds look pages up in memory.
+  const int blk0 = ps_shift >= 0 ? (first_key >> ps_shift) : first_key / page_size;
+  const int blk1 = ps_shift >= 0 ? (last_key >> ps_shift) : last_key / page_size;
+  const bool in_lds = blk1 - blk0 < PF_MAXPAGES;
+  if (in_lds)
+    for (int i = tid; i <= blk1 - blk0; i += G * 64) pages[i] = bt[blk0 + i];
+  __syncthreads();
+  // Rows outside first_key..last_key are never seen (their scores are masked): their addresses are clamped
+  // into the range, so that every load is of a row the sequence holds and no load needs a branch.
+  auto row_of = [&](int u) -> size_t {
+    u = u < first_key ? first_key : (u > last_key ? last_key : u);
+    int blk, offs;
+    if (ps_shift >= 0) {
+      blk = u >> ps_shift;
+      offs = u & ((1 << ps_shift) - 1);
+    } else {
+      blk = u / page_size;
+      offs = u % page_size;
+    }
+    const int page = in_lds ? pages[blk - blk0] : bt[blk];
+    return (((size_t)page * nkv + kvh) * page_size + offs) * D;
+  };
+  // The loads of a step are issued one step ahead and land in registers while the step before is computed.
+  constexpr int VPT = (PF_KSTEP * (D / 8) + G * 64 - 1) / (G * 64);   // value chunks per thread and step
+  bf16x8_t kn[2][KK];
+  uint4 vn[VPT];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const bf16* krow = kcache + row_of(k0 + b * 16 + r16) + kg * 8;   // the key whose row this lane loads
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) kn[b][kk] = *reinterpret_cast<const bf16x8_t*>(krow + kk * 32);
+    }
+#pragma unroll
+    for (int x = 0; x < VPT; ++x) {
+      const int i = (tid + x * G * 64) % (PF_KSTEP * (D / 8));
+      const int key = i / (D / 8), c = i % (D / 8);
+      vn[x] = *reinterpret_cast<const uint4*>(vcache + row_of(k0 + key) + c * 8);
+    }
+  };
+  // per query: the last key it sees and the first, relative to this lane's rows of a score tile (4 kg + i)
+  int hi[QT], lo[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    hi[t] = live[t] ? my_pos[t] - kg * 4 : -(1 << 30);
+    lo[t] = my_lo[t] - kg * 4;
+  }
+  const int kstart = (first_key / PF_KSTEP) * PF_KSTEP;
+  fetch(kstart);
+  for (int k0 = kstart; k0 <= last_key; k0 += PF_KSTEP) {
+    bf16x8_t kc[2][KK];
+    uint4 vc[VPT];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) kc[b][kk] = kn[b][kk];
+#pragma unroll
+    for (int x = 0; x < VPT; ++x) vc[x] = vn[x];
+    fetch(k0 + PF_KSTEP);          // beyond the last step the addresses are clamped and the loads are spare
     // stage the step's value rows transposed: thread (key, chunk of 8 features)
     __syncthreads();
-    for (int i = tid; i < PF_KSTEP * (D / 8); i += G * 64) {
-      const int key = i / (D / 8), c = i - key * (D / 8);
-      const int u = k0 + key;
-      uint4 w = make_uint4(0, 0, 0, 0);
-      if (u >= first_key && u <= last_key) {   // rows no query of the tile sees are staged as zeros
-        const int page = bt[u / page_size];
-        w = *reinterpret_cast<const uint4*>(vcache + (((size_t)page * nkv + kvh) * page_size + u % page_size) * D + c * 8);
-      }
-      const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        vt[c * 8 + 2 * e][key] = (uint16_t)(ww[e] & 0xffffu);
-        vt[c * 8 + 2 * e + 1][key] = (uint16_t)(ww[e] >> 16);
+    for (int x = 0; x < VPT; ++x) {
+      const int i = tid + x * G * 64;
+      if (i < PF_KSTEP * (D / 8)) {
+        const int key = i / (D / 8), c = i % (D / 8);
+        const uint32_t ww[4] = {vc[x].x, vc[x].y, vc[x].z, vc[x].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vt[c * 8 + 2 * e][key] = (uint16_t)(ww[e] & 0xffffu);
+          vt[c * 8 + 2 * e + 1][key] = (uint16_t)(ww[e] >> 16);
+        }
       }
     }
-    // a step every query of the tile sees whole needs no mask
-    const bool whole = (k0 + PF_KSTEP - 1 <= pos0) && (window <= 0 || k0 >= pos0 + nq - window);
-    // scores of two blocks of 16 keys: S^T = K Q^T
+    // scores of two blocks of 16 keys: S^T = K Q^T; lane holds keys k0 + 16 b + 4 kg + i for its query
     float s[QT][8];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const int u = k0 + b * 16 + r16;               // the key whose row this lane loads
-      const bool kin = u >= first_key && u <= last_key;
-      const bf16* krow = kcache;
-      if (kin) {
-        const int page = bt[u / page_size];
-        krow = kcache + (((size_t)page * nkv + kvh) * page_size + u % page_size) * D + kg * 8;
-      }
       f32x4_t st[QT];
 #pragma unroll
       for (int t = 0; t < QT; ++t) st[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        bf16x8_t kf;
-        if (kin) {
-          kf = *reinterpret_cast<const bf16x8_t*>(krow + kk * 32);
-        } else {
+      for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-          for (int e = 0; e < 8; ++e) kf[e] = (__bf16)0.0f;
-        }
-#pragma unroll
-        for (int t = 0; t < QT; ++t) st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][kk], st[t], 0, 0, 0);
-      }
-      // lane holds keys k0 + 16 b + 4 kg + i for its query
+        for (int t = 0; t < QT; ++t) st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc[b][kk], qf[t][kk], st[t], 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < QT; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int key = k0 + b * 16 + kg * 4 + i;
-          const bool see = whole ? live[t] : (live[t] && key <= my_pos[t] && key >= my_lo[t]);
-          s[t][b * 4 + i] = see ? st[t][i] * sc : -INFINITY;
+          const int key = k0 + b * 16 + i;           // + 4 kg, which hi and lo already hold
+          s[t][b * 4 + i] = (key <= hi[t] && key >= lo[t]) ? st[t][i] * sc : -INFINITY;
         }
     }
     bf16x8_t pf[QT];
-    float alpha[QT];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
       float mloc = s[t][0];
 #pragma unroll
       for (int j = 1; j < 8; ++j) mloc = fmaxf(mloc, s[t][j]);
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-      const float m_new = fmaxf(m[t], mloc);
-      float p[8], lsum = 0.f;
-      alpha[t] = 1.f;
-      if (m_new > -INFINITY) {
+      mloc = group4_max(mloc);
+      // The reference point of the exponentials moves only when the maximum has grown by more than 2^PF_SLACK
+      // (or at the first keys): probabilities then stay below 2^PF_SLACK, well inside float32 and bfloat16,
+      // and the accumulators are rescaled on few steps instead of on every one.
+      if (mloc > m[t] + PF_SLACK || m[t] == -INFINITY) {
+        if (mloc > -INFINITY) {
+          const float a = m[t] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[t] - mloc);
+          l[t] *= a;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          p[j] = exp2f(s[t][j] - m_new);
-          lsum += p[j];
+          for (int dt = 0; dt < DT; ++dt) acc[t][dt] *= a;
+          m[t] = mloc;
         }
-        alpha[t] = exp2f(m[t] - m_new);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) p[j] = 0.f;
       }
-      lsum += __shfl_xor(lsum, 16, 64);
-      lsum += __shfl_xor(lsum, 32, 64);
-      l[t] = l[t] * alpha[t] + lsum;
-      m[t] = m_new;
+      float p[8], lsum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        p[j] = m[t] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[t][j] - m[t]);
+        lsum += p[j];
+      }
+      l[t] += group4_sum(lsum);
 #pragma unroll
       for (int j = 0; j < 8; ++j) pf[t][j] = (__bf16)p[j];
     }
@@ -168,10 +211,7 @@ __global__ __launch_bounds__(G * 64) void attention_prefill_kernel(
       a.u2[0] = *reinterpret_cast<const uint2*>(&vt[dt * 16 + r16][kg * 4]);
       a.u2[1] = *reinterpret_cast<const uint2*>(&vt[dt * 16 + r16][16 + kg * 4]);
 #pragma unroll
-      for (int t = 0; t < QT; ++t) {
-        acc[t][dt] *= alpha[t];
-        acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf[t], acc[t][dt], 0, 0, 0);
-      }
+      for (int t = 0; t < QT; ++t) acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pf[t], acc[t][dt], 0, 0, 0);
     }
   }
 #pragma unroll

@@ -75,6 +75,21 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
   return v;
 }
 
+// Maximum and sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the lane groups that share a column of an
+// MFMA result), by gfx950's row swaps: VALU moves, no trip through the LDS crossbar.
+__device__ __forceinline__ float group4_max(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float group4_sum(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.  `red` holds 17 floats.
 __device__ __forceinline__ float block_sum(float v, float* red) {
   int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
