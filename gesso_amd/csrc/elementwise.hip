@@ -19,15 +19,17 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 2; }
+extern "C" int gs_abi_version() { return 3; }
 
 // ------------------------------------------------------------------ embedding
 
 // out[t, :] = table[ids[t], :] as float32; an id outside the table gives a NaN row.
 // With ssq: ssq[t] = sum of squares of the row (one partial sum per row, for a norm that follows).
+// With next_w and xs: xs[t, :] = bfloat16(row * next_w), the rows pre-weighted for the first norm's consumer.
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
-                             float* __restrict__ ssq, int H, int V) {
+                             float* __restrict__ ssq, const float* __restrict__ next_w, bf16* __restrict__ xs, int H,
+                             int V) {
   __shared__ float red[17];
   int t = blockIdx.x;
   int id = ids[t];
@@ -42,6 +44,7 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
       float v = to_f32(row[j]);
       o[j] = v;
       ss += v * v;
+      if (xs) xs[(size_t)t * H + j] = f32_to_bf16(v * next_w[j]);
     }
   }
   if (ssq) {
@@ -50,14 +53,14 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
   }
 }
 
-extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, float* out, float* ssq, int T, int H,
-                        int V, hipStream_t stream) {
+extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, float* out, float* ssq,
+                        const float* next_w, void* xs, int T, int H, int V, hipStream_t stream) {
   GS_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
   if (T == 0) return 0;
   if (table_dtype == GS_F32)
-    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, ssq, H, V);
+    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, ssq, next_w, (bf16*)xs, H, V);
   else if (table_dtype == GS_BF16)
-    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, ssq, H, V);
+    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, ssq, next_w, (bf16*)xs, H, V);
   else
     GS_REQUIRE(false, "embed: unknown dtype %d", table_dtype);
   GS_LAUNCH_CHECK("embed");

@@ -33,6 +33,7 @@ static int check_lazy(const float* res, const float* ssq, int nb, const float* n
 static int check_x(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps,
                    int K) {
   if (res) return check_lazy(res, ssq, nb, norm_w, eps);
+  GS_REQUIRE(!ssq || (nb > 0 && eps > 0.f), "gemm_skinny: pre-weighted rows need their partial sums and eps");
   GS_REQUIRE(X && ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0,
              "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
   return 0;
@@ -47,11 +48,7 @@ extern "C" int gs_gemm_skinny(const void* X, int ldx, const float* res, const fl
   GS_REQUIRE(ldy >= (epilogue == 1 ? N / 2 : N), "gemm_skinny: row stride %d of Y too small", ldy);
   GS_REQUIRE(y_dtype == GS_BF16 || y_dtype == GS_F32, "gemm_skinny: unknown output dtype %d", y_dtype);
   if (check_tiles(Wt, N, K, epilogue == 1 ? N / 2 : 16)) return -1;
-  if (res) {
-    if (check_lazy(res, ssq, nb, norm_w, eps)) return -1;
-  } else {
-    GS_REQUIRE(ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0, "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
-  }
+  if (check_x(X, ldx, res, ssq, nb, norm_w, eps, K)) return -1;
   if (M == 0) return 0;
   gs_skinny_run_plain(X, ldx, res, ssq, nb, norm_w, eps, W, Wt, Y, y_dtype, ldy, M, N, K, epilogue, stream);
   GS_LAUNCH_CHECK("gemm_skinny");
@@ -63,12 +60,14 @@ extern "C" int gs_gemm_skinny_residual_blocks(int N) { return gs_ceil_div(N, 16)
 
 // res (M, N) += X W^T, and ssq_out (M, blocks) = partial sums of squares of the new rows.
 extern "C" int gs_gemm_skinny_residual(const void* X, int ldx, const void* W, const void* Wt, float* res,
-                                       float* ssq_out, int M, int N, int K, hipStream_t stream) {
+                                       float* ssq_out, const float* next_w, void* xs_out, int M, int N, int K,
+                                       hipStream_t stream) {
   if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16)) return -1;
   GS_REQUIRE(ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0, "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
   GS_REQUIRE(res && ssq_out, "gemm_skinny_residual: needs the stream and room for the partial sums");
   if (M == 0) return 0;
-  gs_skinny_run_residual(X, ldx, W, Wt, res, ssq_out, M, N, K, stream);
+  GS_REQUIRE((next_w == nullptr) == (xs_out == nullptr), "gemm_skinny_residual: the next norm's weight and the room for the weighted rows come together");
+  gs_skinny_run_residual(X, ldx, W, Wt, res, ssq_out, next_w, xs_out, M, N, K, stream);
   GS_LAUNCH_CHECK("gemm_skinny_residual");
   return 0;
 }

@@ -5,8 +5,8 @@
 void gs_skinny_run_plain(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w,
                          float eps, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M, int N, int K,
                          int epilogue, hipStream_t stream);
-void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out, int M,
-                            int N, int K, hipStream_t stream);
+void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out,
+                            const float* next_w, void* xs_out, int M, int N, int K, hipStream_t stream);
 void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
                         const void* Wt, const float* taps, const float* conv_bias, float* state, const int* slots,
                         int conv_w, void* Y, int M, int H, int K, hipStream_t stream);

@@ -27,14 +27,14 @@ void gs_skinny_run_plain(const void* X, int ldx, const float* res, const float* 
                          float eps, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M, int N, int K,
                          int epilogue, hipStream_t stream) {
   SkinnyCall c = base(X, ldx, W, Wt, Y, y_dtype, ldy, M, N, K, epilogue, stream);
-  if (res) lazy(c, res, ssq, nb, norm_w, eps);
+  if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   Wt ? gs_skinny_plain_tiles(c) : gs_skinny_plain_rows(c);
 }
 
-void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out, int M,
-                            int N, int K, hipStream_t stream) {
+void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out,
+                            const float* next_w, void* xs_out, int M, int N, int K, hipStream_t stream) {
   SkinnyCall c = base(X, ldx, W, Wt, nullptr, GS_F32, N, M, N, K, 2, stream);
-  c.ex.res_out = res; c.ex.ssq_out = ssq_out;
+  c.ex.res_out = res; c.ex.ssq_out = ssq_out; c.ex.next_w = next_w; c.ex.xs_out = (bf16*)xs_out;
   Wt ? gs_skinny_residual_tiles(c) : gs_skinny_residual_rows(c);
 }
 
@@ -42,7 +42,7 @@ void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* s
                         const void* Wt, const float* taps, const float* conv_bias, float* state, const int* slots,
                         int conv_w, void* Y, int M, int H, int K, hipStream_t stream) {
   SkinnyCall c = base(X, ldx, W, Wt, Y, GS_BF16, H, M, 3 * H, K, 3, stream);
-  if (res) lazy(c, res, ssq, nb, norm_w, eps);
+  if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.taps = taps; c.ex.conv_bias = conv_bias; c.ex.state = state; c.ex.slots = slots; c.ex.conv_w = conv_w;
   Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);
 }
@@ -53,7 +53,7 @@ void gs_skinny_run_qkv(const void* X, int ldx, const float* res, const float* ss
                        int page_size, void* kcache, void* vcache, int write_kv, void* Q, int M, int nh, int nkv, int d,
                        int K, hipStream_t stream) {
   SkinnyCall c = base(X, ldx, W, Wt, Q, GS_BF16, nh * d, M, (nh + 2 * nkv) * d, K, 4, stream);
-  if (res) lazy(c, res, ssq, nb, norm_w, eps);
+  if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.qw = qw; c.ex.kw = kw; c.ex.head_eps = head_eps; c.ex.cos_t = cos_t; c.ex.sin_t = sin_t;
   c.ex.positions = positions; c.ex.block_table = block_table; c.ex.max_blocks = max_blocks; c.ex.page_size = page_size;
   c.ex.nh = nh; c.ex.nkv = nkv; c.ex.write_kv = write_kv; c.ex.kcache = (bf16*)kcache; c.ex.vcache = (bf16*)vcache;

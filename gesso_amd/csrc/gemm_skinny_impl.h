@@ -23,6 +23,10 @@
 //   1  X is the RMSNorm of the float32 residual stream: x = res * inv_rms(row) * norm_weight, rounded to
 //      bfloat16 as the norm kernel would store it; the row's sum of squares comes as partial sums
 //      (row, nb), added in a fixed order.
+//   0 with partial sums given: X holds rows already multiplied by the norm's weight (res * norm_weight,
+//      written by the product that last added to the stream, EPI 2); the row's inverse root mean square,
+//      which no single block of that product knew, multiplies this product's result instead:
+//      (x inv) W^T = inv (x W^T).  The norm costs no kernel and no pass of its own.
 // What is done with Y (EPI):
 //   0  stored (bfloat16 or float32).
 //   1  SwiGLU: W holds gate rows [0, N/2) then up rows; stores silu(gate) * up, N/2 wide.
@@ -80,6 +84,8 @@ struct SkinnyExtra {
   // EPI 2
   float* res_out;        // (M, N) float32, updated in place
   float* ssq_out;        // (M, gridDim.x)
+  const float* next_w;   // (N) weight of the norm that reads the stream next, or null
+  bf16* xs_out;          // (M, N) res * next_w, for that norm's consumer
   // EPI 3
   const float* taps;     // (H, W)
   const float* conv_bias;
@@ -151,6 +157,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * ldx;
     } else {
       rrow[mt] = ex.res + (size_t)(xok[mt] ? m : 0) * K;
+    }
+    if (PRO == 1) {
       // the row's sum of squares: this lane group adds every fourth partial, then the four groups are added
       float s = 0.f;
       if (xok[mt])
@@ -159,6 +167,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       s += __shfl_xor(s, 32, 64);
       inv[mt] = 1.0f / sqrtf(s / (float)K + ex.eps);
     }
+  }
+
+  // Pre-weighted rows: the rows' inverse root mean squares are needed only at the end.  The wavefronts share
+  // the rows; a lane adds every 64th partial sum and the wavefront adds its lanes (an order that depends on
+  // nothing but the number of partials).  The first row's loads start here, under the product's own.
+  __shared__ float inv_s[64];
+  const bool scaled = PRO == 0 && ex.ssq != nullptr;
+  float pre0 = 0.f, pre1 = 0.f;
+  if (scaled && wave < M) {
+    if (lane < ex.nb) pre0 = ex.ssq[(size_t)wave * ex.nb + lane];
+    if (lane + 64 < ex.nb) pre1 = ex.ssq[(size_t)wave * ex.nb + lane + 64];
   }
 
   f32x4_t acc[R][MT];
@@ -229,6 +248,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     }
   }
 
+  if (scaled) {
+    for (int m = wave; m < M; m += WAVES) {
+      float ssum = pre0 + pre1;
+      for (int b = (m == wave ? 128 : 0) + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
+      ssum = wave_sum(ssum);
+      if (lane == 0) inv_s[m] = 1.0f / sqrtf(ssum / (float)K + ex.eps);
+      pre0 = pre1 = 0.f;
+    }
+    if (WAVES == 1) __syncthreads();
+  }
+
   // add the wavefronts' partial tiles: wave 0 keeps its own, the others pass theirs through LDS
   if (WAVES > 1) {
     if (wave > 0) {
@@ -250,6 +280,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
           f32x4_t v = *reinterpret_cast<const f32x4_t*>(src + ((r * MT + mt) * 64 + lane) * 4);
           acc[r][mt] += v;
         }
+    }
+  }
+
+  // rows that came pre-weighted get their inverse root mean square now
+  if (scaled) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const float iv = inv_s[(mt * 16 + r16 < M) ? mt * 16 + r16 : 0];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r][mt] *= iv;
     }
   }
 
@@ -283,6 +323,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         const int n = rowbase[r] + kg * 4;
         if (live && n < N) {
           float* p = ex.res_out + (size_t)m * N + n;
+          f32x4_t xv = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             if (n + i < N) {
@@ -290,7 +331,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
               float v = p[i] + to_f32(f32_to_bf16(acc[r][mt][i]));
               p[i] = v;
               ss += v * v;
+              if (ex.xs_out) xv[i] = v * ex.next_w[n + i];
             }
+          if (ex.xs_out) store4<bf16>(ex.xs_out + (size_t)m * N + n, xv, N - n);
         }
       }
       ss += __shfl_xor(ss, 16, 64);

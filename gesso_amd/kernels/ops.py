@@ -67,9 +67,11 @@ def _i32(t, n=None, what="index"):
 
 # ---------------------------------------------------------------------- elementwise
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq: torch.Tensor = None) -> torch.Tensor:
-    """``out[t] = table[ids[t]]`` as float32 ``(T, H)``; with ``ssq (T, 1)`` also each row's sum of squares."""
-    _dev(ids, table, out, ssq)
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq: torch.Tensor = None,
+          next_weight: torch.Tensor = None, xs: torch.Tensor = None) -> torch.Tensor:
+    """``out[t] = table[ids[t]]`` as float32 ``(T, H)``; with ``ssq (T, 1)`` also each row's sum of squares;
+    with ``next_weight (H,)`` and ``xs (T, H)`` bfloat16 also ``xs = out * next_weight``."""
+    _dev(ids, table, out, ssq, next_weight, xs)
     _i32(ids, what="token ids")
     V, H = table.shape
     T = ids.numel()
@@ -77,7 +79,12 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq:
         out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     _need(out.dtype == torch.float32 and out.shape == (T, H), "embed: out must be float32 (T, H)")
     _need(ssq is None or (ssq.dtype == torch.float32 and ssq.numel() == T), "embed: ssq must be float32 (T, 1)")
-    _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), _p(ssq), c_int(T), c_int(H), c_int(V), _stream()))
+    _need((next_weight is None) == (xs is None), "embed: next_weight and xs come together")
+    if xs is not None:
+        _need(next_weight.dtype == torch.float32 and next_weight.shape == (H,) and xs.dtype == torch.bfloat16
+              and xs.shape == (T, H) and xs.is_contiguous(), "embed: next_weight float32 (H,), xs bfloat16 (T, H)")
+    _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), _p(ssq), _p(next_weight), _p(xs), c_int(T), c_int(H),
+                          c_int(V), _stream()))
     return out
 
 
@@ -293,13 +300,15 @@ class LazyNorm:
     """An RMSNorm not yet applied: the float32 stream, its rows' sums of squares as partial sums, weight and eps.
 
     The weight-streaming products take it in place of a tensor and norm on the fly; ``materialize``
-    runs a light norm kernel for everything else.
+    runs a light norm kernel for everything else.  ``xs``, when given, holds ``res * weight`` in bfloat16,
+    written by whatever last added to the stream: then a product reads ``xs`` and multiplies its result by the
+    row's inverse root mean square, and the norm costs nothing of its own.
     """
 
-    __slots__ = ("res", "ssq", "weight", "eps", "dtype")
+    __slots__ = ("res", "ssq", "weight", "eps", "dtype", "xs")
 
-    def __init__(self, res, ssq, weight, eps, dtype):
-        self.res, self.ssq, self.weight, self.eps, self.dtype = res, ssq, weight, eps, dtype
+    def __init__(self, res, ssq, weight, eps, dtype, xs=None):
+        self.res, self.ssq, self.weight, self.eps, self.dtype, self.xs = res, ssq, weight, eps, dtype, xs
 
     @property
     def shape(self):
@@ -322,6 +331,8 @@ def lazy_ok(x, w: torch.Tensor) -> bool:
 
 def _lazy_args(x):
     if isinstance(x, LazyNorm):
+        if x.xs is not None:
+            return (_p(x.xs), c_int(x.res.shape[1]), None, _p(x.ssq), c_int(x.ssq.shape[1]), None, c_float(x.eps))
         return (None, c_int(x.res.shape[1]), _p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps))
     M, K = x.shape
     return (_p(x), c_int(x.stride(0) if M > 1 else K), None, None, c_int(0), None, c_float(0.0))
@@ -361,17 +372,23 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, sw
     return out
 
 
-def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt=None) -> torch.Tensor:
-    """``res += x @ w.T`` in place (float32); returns the new rows' sums of squares as partial sums ``(M, nb)``."""
-    _dev(w, res)
+def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt=None, next_weight=None,
+                         xs: torch.Tensor = None) -> torch.Tensor:
+    """``res += x @ w.T`` in place (float32); returns the new rows' sums of squares as partial sums ``(M, nb)``.
+    With ``next_weight (N,)`` and ``xs (M, N)`` bfloat16 also ``xs = res * next_weight``."""
+    _dev(w, res, next_weight, xs)
     _need(skinny_ok(x, w), "gemm_skinny_residual: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
     M, K = x.shape
     N = w.shape[0]
     _need(w.shape == (N, K) and res.shape == (M, N) and res.dtype == torch.float32, "gemm_skinny_residual: shapes")
     nb = lib().gs_gemm_skinny_residual_blocks(c_int(N))
     ssq = torch.empty((M, nb), dtype=torch.float32, device=res.device)
-    _check(lib().gs_gemm_skinny_residual(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(wt), _p(res), _p(ssq), c_int(M),
-                                         c_int(N), c_int(K), _stream()))
+    _need((next_weight is None) == (xs is None), "gemm_skinny_residual: next_weight and xs come together")
+    if xs is not None:
+        _need(next_weight.dtype == torch.float32 and next_weight.shape == (N,) and xs.dtype == torch.bfloat16
+              and xs.shape == (M, N) and xs.is_contiguous(), "gemm_skinny_residual: next_weight float32 (N,), xs bfloat16 (M, N)")
+    _check(lib().gs_gemm_skinny_residual(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(wt), _p(res), _p(ssq),
+                                         _p(next_weight), _p(xs), c_int(M), c_int(N), c_int(K), _stream()))
     return ssq
 
 

@@ -15,7 +15,7 @@ from ..config.spec import ModelSpec
 from ..errors import ConfigError
 from ..parts.base import MATRIX, TABLE, TensorSpec, sub_tensors
 from ..parts.registry import build, part_class
-from ..parts.rmsnorm import ResidualStream
+from ..parts.rmsnorm import ResidualStream, row_weight_of
 
 
 def tensor_table(spec: ModelSpec) -> Dict[str, TensorSpec]:
@@ -82,16 +82,26 @@ class Model:
     def forward(self, ctx) -> Optional[torch.Tensor]:
         """Run the tokens of ``ctx`` through every scheduled block; float32 logits at ``ctx.want_rows``."""
         ops, rt = self.rt.ops, self.rt
+        decode_only = getattr(ctx, "decode_only", False)
+        # the norm that reads the stream after the i-th scheduled block: the next block's first, then the final one
+        order = [self.blocks[call.layer] for call in self.spec.schedule]
+        readers = [getattr(b, "first_norm", None) for b in order[1:]] + [self.final_norm if decode_only else None]
         if rt.fused:
             ssq = torch.empty((ctx.T, 1), dtype=torch.float32, device=rt.device)
-            stream = ResidualStream(ops.embed(ctx.token_ids, self.embed, ssq=ssq), ssq=ssq)
+            first = getattr(order[0], "first_norm", None) if order else None
+            res = torch.empty((ctx.T, self.embed.shape[1]), dtype=torch.float32, device=rt.device)
+            w = row_weight_of(first, res, rt)
+            xs = torch.empty(res.shape, dtype=torch.bfloat16, device=rt.device) if w is not None else None
+            ops.embed(ctx.token_ids, self.embed, out=res, ssq=ssq, next_weight=w, xs=xs)
+            stream = ResidualStream(res, ssq=ssq, xs=xs, xs_for=first if xs is not None else None)
         else:
             stream = ResidualStream(ops.embed(ctx.token_ids, self.embed))
         for i, call in enumerate(self.spec.schedule):
-            self.blocks[call.layer].forward(stream, ctx, ctx.cache_view(i))
+            stream.following = readers[i]
+            order[i].forward(stream, ctx, ctx.cache_view(i))
         if ctx.n_want == 0:
             return None
         # every row wanted, in order (a decode step): no gather, and the norm may stay lazy
-        rows = None if getattr(ctx, "decode_only", False) else ctx.want_rows
+        rows = None if decode_only else ctx.want_rows
         normed = self.final_norm.add_norm(stream, rows=rows)
         return self.rt.linear(normed, self.head, out_dtype=torch.float32)

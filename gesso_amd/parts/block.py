@@ -45,12 +45,18 @@ class PreNormBlock(Part):
             self.ffn_norm.bind(sub_tensors(tensors, "ffn_norm"))
             self.ffn.bind(sub_tensors(tensors, "ffn"))
 
+    @property
+    def first_norm(self):
+        """The norm that reads the stream first when this block runs (a hint for whoever writes the stream before)."""
+        return self.mixer_norm
+
     def forward(self, stream, ctx, cache):
+        after = stream.following
         x = self.mixer_norm.add_norm(stream)
-        stream.push(self.mixer.forward(x, ctx, cache), self.rt)
+        stream.push(self.mixer.forward(x, ctx, cache), self.rt, next_norm=self.ffn_norm if self.ffn is not None else after)
         if self.ffn is not None:
             x = self.ffn_norm.add_norm(stream)
-            stream.push(self.ffn.forward(x, ctx), self.rt)
+            stream.push(self.ffn.forward(x, ctx), self.rt, next_norm=after)
 
     @property
     def graph_safe(self) -> bool:

@@ -5,6 +5,8 @@ the norm into the same pass, as the reference's seam does (``src/Inference/Infer
 """
 from __future__ import annotations
 
+import torch
+
 from .base import VECTOR, Part, TensorSpec
 from .registry import register
 
@@ -15,22 +17,33 @@ class ResidualStream:
     ``push`` takes a sub-layer's output: a tensor becomes ``pending`` (the next norm adds it), a
     deferred product (:class:`~gesso_amd.parts.runtime.DeferredLinear`) is computed straight into
     ``res``, which leaves the new rows' sums of squares in ``ssq`` for a lazy norm.
+
+    Whoever knows which norm reads the stream next may say so (``next_norm`` of ``push``; ``following``, set
+    by the model, names the norm after the current block).  If that norm offers ``row_weight`` (a float32
+    vector ``w`` with ``norm(x) = inv_rms(x) * (x * w)``), the deferred product also leaves ``xs = res * w``
+    in bfloat16, and the norm's consumer needs no norm pass at all.  ``xs_for`` is the norm ``xs`` was made for.
     """
 
-    __slots__ = ("res", "pending", "ssq")
+    __slots__ = ("res", "pending", "ssq", "xs", "xs_for", "following")
 
-    def __init__(self, res, pending=None, ssq=None):
+    def __init__(self, res, pending=None, ssq=None, xs=None, xs_for=None):
         self.res = res
         self.pending = pending
         self.ssq = ssq
+        self.xs, self.xs_for = xs, xs_for
+        self.following = None
 
-    def push(self, out, rt) -> None:
+    def push(self, out, rt, next_norm=None) -> None:
         from .runtime import DeferredLinear
+        self.flush(rt)
+        self.xs = self.xs_for = None
         if isinstance(out, DeferredLinear):
-            self.flush(rt)
-            self.ssq = rt.ops.gemm_skinny_residual(out.x, out.w, self.res, wt=rt._wt(out.w))
+            w = row_weight_of(next_norm, self.res, rt)
+            if w is not None:
+                self.xs = torch.empty(self.res.shape, dtype=torch.bfloat16, device=self.res.device)
+                self.xs_for = next_norm
+            self.ssq = rt.ops.gemm_skinny_residual(out.x, out.w, self.res, wt=rt._wt(out.w), next_weight=w, xs=self.xs)
         else:
-            self.flush(rt)
             self.pending, self.ssq = out, None
 
     def flush(self, rt) -> None:
@@ -38,6 +51,15 @@ class ResidualStream:
         if self.pending is not None:
             rt.ops.residual_add(self.res, self.pending)
             self.pending, self.ssq = None, None
+            self.xs = self.xs_for = None
+
+
+def row_weight_of(norm, res, rt):
+    """``norm.row_weight`` if the norm offers one that fits the stream's width and the rows are few enough, else None."""
+    w = getattr(norm, "row_weight", None)
+    if w is None or w.dtype != res.dtype or w.shape != (res.shape[1],) or res.shape[0] > rt.weighted_rows_max:
+        return None
+    return w
 
 
 class RMSNorm(Part):
@@ -50,6 +72,11 @@ class RMSNorm(Part):
     def bind(self, tensors):
         self.weight = tensors["weight"]
 
+    @property
+    def row_weight(self):
+        """``norm(x) = inv_rms(x) * (x * row_weight)``: what lets a producer pre-weight the rows for this norm."""
+        return self.weight if self.rt.dtype == torch.bfloat16 else None
+
     def add_norm(self, stream: ResidualStream, rows=None, out=None):
         """Add what is pending to the stream, then norm it (only ``rows`` of it when given).
 
@@ -58,7 +85,8 @@ class RMSNorm(Part):
         follows, which norms on the fly.
         """
         if self.rt.fused and rows is None and stream.pending is None and stream.ssq is not None:
-            return self.rt.ops.LazyNorm(stream.res, stream.ssq, self.weight, self.spec.eps, self.rt.dtype)
+            xs = stream.xs if stream.xs_for is self else None
+            return self.rt.ops.LazyNorm(stream.res, stream.ssq, self.weight, self.spec.eps, self.rt.dtype, xs=xs)
         y = self.rt.ops.add_rmsnorm(stream.res, stream.pending, self.weight, self.spec.eps, self.rt.dtype,
                                     rows=rows, out=out)
         if rows is None:

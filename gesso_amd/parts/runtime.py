@@ -45,6 +45,10 @@ class Runtime:
         # a lazy norm is folded into the product that follows for up to this many rows; for more, one
         # light kernel norms the rows first (the fold repeats the norm's arithmetic in every block)
         self.fold_norm_rows = int(os.environ.get("GESSO_FOLD_NORM_ROWS", "0"))
+        # up to this many rows a deferred product also leaves the rows weighted for the next norm, whose consumer
+        # then only scales its result; for more rows every block's reading of the partial sums costs more than
+        # one light norm pass
+        self.weighted_rows_max = int(os.environ.get("GESSO_WEIGHTED_ROWS_MAX", "32"))
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""
@@ -78,7 +82,7 @@ class Runtime:
         ops = self.ops
         out_dtype = out_dtype or self.dtype
         if isinstance(x, ops.LazyNorm):
-            if bias is None and x.shape[0] <= self.fold_norm_rows and ops.lazy_ok(x, w):
+            if bias is None and self._keep_lazy(x) and ops.lazy_ok(x, w):
                 return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self._wt(w))
             x = x.materialize()
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
@@ -92,7 +96,7 @@ class Runtime:
         """``silu(x @ w1.T) * (x @ w3.T)`` with ``w13`` holding w1's rows, then w3's."""
         ops = self.ops
         if isinstance(x, ops.LazyNorm):
-            if x.shape[0] <= self.fold_norm_rows and ops.lazy_ok(x, w13):
+            if self._keep_lazy(x) and ops.lazy_ok(x, w13):
                 return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13))
             x = x.materialize()
         if ops.skinny_ok(x, w13):
@@ -108,9 +112,14 @@ class Runtime:
 
     # ------------------------------------------------------------------ mixers' inner steps
 
+    def _keep_lazy(self, x) -> bool:
+        """Whether a lazy norm goes to the product as it is: always when its rows come pre-weighted (the product
+        only scales its result), else for few rows (the fold repeats the norm's arithmetic in every block)."""
+        return x.xs is not None or x.shape[0] <= self.fold_norm_rows
+
     def _rows(self, x):
-        """A lazy norm as the kernels of this step should take it: folded for few rows, else normed by one light pass."""
-        if isinstance(x, self.ops.LazyNorm) and x.shape[0] > self.fold_norm_rows:
+        """A lazy norm as the kernels of this step should take it: kept, or normed by one light pass."""
+        if isinstance(x, self.ops.LazyNorm) and not self._keep_lazy(x):
             return x.materialize()
         return x
 

@@ -448,14 +448,15 @@ def test_attention_decode_supports(ops):
 
 # ------------------------------------------------------------------ the decode step's fused products
 
-def lazy_case(ops, M, K, seed):
+def lazy_case(ops, M, K, seed, weighted=False):
     g = gen(seed)
     res = torch.randn(M, K, generator=g)
     nw = 1 + 0.1 * torch.randn(K, generator=g)
     nb = 5
     part = torch.rand(M, nb, generator=g)
     part = part / part.sum(1, keepdim=True) * (res * res).sum(1, keepdim=True)      # partial sums of the true sums
-    lazy = ops.LazyNorm(res.to(DEV), part.to(DEV), nw.to(DEV), 1e-5, torch.bfloat16)
+    xs = (res * nw).bfloat16().to(DEV) if weighted else None     # as a producer would have left them
+    lazy = ops.LazyNorm(res.to(DEV), part.to(DEV), nw.to(DEV), 1e-5, torch.bfloat16, xs=xs)
     return res, nw, lazy
 
 
@@ -498,9 +499,48 @@ def test_gemm_skinny_residual(ops, M, N, K):
         assert float((a - b).abs().max()) <= 1e-2 * float(b.abs().max())
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (40, 96, 320), (64, 144, 104)])
+def test_gemm_skinny_residual_leaves_rows_weighted_for_the_next_norm(ops, M, N, K):
+    g = gen(M + N + K + 1)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    res = torch.randn(M, N, generator=g)
+    nw = 1 + 0.3 * torch.randn(N, generator=g)
+    r1, r2 = res.clone().to(DEV), res.clone().to(DEV)
+    xs = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ssq1 = ops.gemm_skinny_residual(x.to(DEV), w.to(DEV), r1, next_weight=nw.to(DEV), xs=xs)
+    ssq2 = ops.gemm_skinny_residual(x.to(DEV), w.to(DEV), r2)
+    assert torch.equal(r1, r2) and torch.equal(ssq1, ssq2)
+    assert torch.equal(xs.cpu(), (r1.cpu() * nw).bfloat16())
+    # a product that reads the weighted rows and scales its result equals the product of the normed rows
+    N2 = 112
+    w2 = (torch.randn(N2, N, generator=g) / math.sqrt(N)).bfloat16()
+    lazy = ops.LazyNorm(r1, ssq1, nw.to(DEV), 1e-5, torch.bfloat16, xs=xs)
+    if N % 8 == 0:
+        ref = P.rmsnorm(r1.double().cpu(), nw.double(), 1e-5) @ w2.double().T
+        close(ops.gemm_skinny(lazy, w2.to(DEV), out_dtype=torch.float32), ref, torch.bfloat16)
+        close(ops.gemm_skinny(lazy, w2.to(DEV), swiglu=True), P.swiglu(ref[:, :N2 // 2], ref[:, N2 // 2:]), torch.bfloat16, scale=2)
+
+
+@pytest.mark.parametrize("T,H,V", [(1, 2048, 1000), (9, 104, 301)])
+def test_embed_leaves_rows_weighted_for_the_first_norm(ops, T, H, V):
+    g = gen(T + H)
+    table = torch.randn(V, H, generator=g).bfloat16()
+    ids = torch.randint(0, V, (T,), generator=g).to(torch.int32)
+    nw = 1 + 0.3 * torch.randn(H, generator=g)
+    ssq = torch.empty(T, 1, device=DEV)
+    xs = torch.empty(T, H, dtype=torch.bfloat16, device=DEV)
+    out = ops.embed(ids.to(DEV), table.to(DEV), ssq=ssq, next_weight=nw.to(DEV), xs=xs)
+    rows = table[ids.long()].float()
+    assert torch.equal(out.cpu(), rows)
+    assert torch.equal(xs.cpu(), (rows * nw).bfloat16())
+    assert torch.allclose(ssq.cpu()[:, 0].double(), (rows.double() ** 2).sum(1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("weighted", [False, True])
 @pytest.mark.parametrize("M,H,W,bias", [(1, 64, 3, False), (8, 2048, 3, False), (20, 96, 4, True), (64, 48, 2, False)])
-def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias):
-    res, nw, lazy = lazy_case(ops, M, H, M + H)
+def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias, weighted):
+    res, nw, lazy = lazy_case(ops, M, H, M + H, weighted)
     g = gen(H + W)
     w_in = (torch.randn(3 * H, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
     taps = torch.randn(H, W, generator=g).to(DEV)
@@ -518,10 +558,11 @@ def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias):
     assert torch.equal(s1[untouched].cpu(), state0[untouched])
 
 
+@pytest.mark.parametrize("weighted", [False, True])
 @pytest.mark.parametrize("M,nh,nkv,d,norm", [(1, 32, 8, 64, True), (8, 4, 2, 32, True), (33, 2, 1, 128, False), (64, 3, 3, 64, True)])
-def test_gemm_skinny_qkv_equals_the_separate_kernels(ops, M, nh, nkv, d, norm):
+def test_gemm_skinny_qkv_equals_the_separate_kernels(ops, M, nh, nkv, d, norm, weighted):
     H = nh * d
-    res, nw, lazy = lazy_case(ops, M, H, M + H)
+    res, nw, lazy = lazy_case(ops, M, H, M + H, weighted)
     g = gen(nh + d)
     wqkv = (torch.randn((nh + 2 * nkv) * d, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
     qw = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV) if norm else None
