@@ -56,7 +56,9 @@ extern "C" int gs_gemm_skinny(const void* X, int ldx, const float* res, const fl
 }
 
 // Partial sums per row that gs_gemm_skinny_residual writes for N columns.
-extern "C" int gs_gemm_skinny_residual_blocks(int N) { return gs_ceil_div(N, 16); }
+extern "C" int gs_gemm_skinny_residual_blocks(int N, int tile_major) {
+  return gs_ceil_div(N, tile_major && gs_skinny_residual_halves(N) ? 8 : 16);
+}
 
 // res (M, N) += X W^T, and ssq_out (M, blocks) = partial sums of squares of the new rows.
 extern "C" int gs_gemm_skinny_residual(const void* X, int ldx, const void* W, const void* Wt, float* res,

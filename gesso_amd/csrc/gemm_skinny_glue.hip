@@ -8,6 +8,7 @@ void gs_skinny_conv_rows(const SkinnyCall& c);
 void gs_skinny_qkv_rows(const SkinnyCall& c, int d);
 void gs_skinny_plain_tiles(const SkinnyCall& c);
 void gs_skinny_residual_tiles(const SkinnyCall& c);
+void gs_skinny_residual_half_tiles(const SkinnyCall& c);
 void gs_skinny_conv_tiles(const SkinnyCall& c);
 void gs_skinny_qkv_tiles(const SkinnyCall& c, int d);
 
@@ -31,11 +32,15 @@ void gs_skinny_run_plain(const void* X, int ldx, const float* res, const float* 
   Wt ? gs_skinny_plain_tiles(c) : gs_skinny_plain_rows(c);
 }
 
+// A weight of few rows is shared out in half tiles, so that twice as many blocks stream it.
+bool gs_skinny_residual_halves(int N) { return N % 16 == 0 && N / 16 <= 160; }
+
 void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out,
                             const float* next_w, void* xs_out, int M, int N, int K, hipStream_t stream) {
   SkinnyCall c = base(X, ldx, W, Wt, nullptr, GS_F32, N, M, N, K, 2, stream);
   c.ex.res_out = res; c.ex.ssq_out = ssq_out; c.ex.next_w = next_w; c.ex.xs_out = (bf16*)xs_out;
-  Wt ? gs_skinny_residual_tiles(c) : gs_skinny_residual_rows(c);
+  if (Wt && gs_skinny_residual_halves(N)) gs_skinny_residual_half_tiles(c);
+  else Wt ? gs_skinny_residual_tiles(c) : gs_skinny_residual_rows(c);
 }
 
 void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,

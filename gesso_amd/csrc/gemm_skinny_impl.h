@@ -124,11 +124,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     const int H = N / 3;
 #pragma unroll
     for (int r = 0; r < R; ++r) rowbase[r] = blockIdx.x * 16 + r * H;  // B, C, X rows of the same channels
+  } else if (SHUF == 2) {
+    rowbase[0] = blockIdx.x * 8;  // half a tile: twice the blocks for a weight of few rows
   } else {
     const int n0 = blockIdx.x * 16 * R;
 #pragma unroll
     for (int r = 0; r < R; ++r) rowbase[r] = n0 + r * 16;
   }
+  static_assert(SHUF != 2 || (R == 1 && EPI == 2), "half tiles are written for the residual epilogue, one tile a block");
+  const bool wact = SHUF != 2 || r16 < 8;  // half tiles: the lanes of the other eight rows load nothing
   const bf16* wrow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -136,7 +140,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     if (EPI == 1 && !(r & 1) && n >= half) n = half - 1;  // gate rows end at N/2
     if (EPI == 3 && n >= (r + 1) * (N / 3)) n = (r + 1) * (N / 3) - 1;
     if (n >= N) n = N - 1;                                // clamped: loaded, never stored
-    if (SHUF)
+    if (SHUF == 2)
+      wrow[r] = W + ((size_t)(blockIdx.x >> 1) * ((K + 31) >> 5)) * 512 + (kg * 16 + (blockIdx.x & 1) * 8 + (r16 & 7)) * 8;
+    else if (SHUF)
       // tile-major: the 16 x 32 tile of (row tile, k step) is 64 lanes x 16 bytes in the operand's own order
       wrow[r] = W + ((size_t)(rowbase[r] >> 4) * ((K + 31) >> 5)) * 512 + lane * 8;
     else
@@ -174,10 +180,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   // nothing but the number of partials).  The first row's loads start here, under the product's own.
   __shared__ float inv_s[64];
   const bool scaled = PRO == 0 && ex.ssq != nullptr;
-  float pre0 = 0.f, pre1 = 0.f;
+  float pre[4] = {0.f, 0.f, 0.f, 0.f};
   if (scaled && wave < M) {
-    if (lane < ex.nb) pre0 = ex.ssq[(size_t)wave * ex.nb + lane];
-    if (lane + 64 < ex.nb) pre1 = ex.ssq[(size_t)wave * ex.nb + lane + 64];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (lane + 64 * j < ex.nb) pre[j] = ex.ssq[(size_t)wave * ex.nb + lane + 64 * j];
   }
 
   f32x4_t acc[R][MT];
@@ -221,7 +228,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       for (int u = 0; u < U; ++u) {
         const int k = ((s + u) << 5) + kg * 8;
 #pragma unroll
-        for (int r = 0; r < R; ++r) a[u][r] = load8(wrow[r] + (size_t)(s + u) * WSTEP);
+        for (int r = 0; r < R; ++r) a[u][r] = wact ? load8(wrow[r] + (size_t)(s + u) * WSTEP) : zero8();
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) b[u][mt] = xok[mt] ? load_x(mt, k) : zero8();
       }
@@ -242,7 +249,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     for (int mt = 0; mt < MT; ++mt) b[mt] = (kin && xok[mt]) ? load_x(mt, k) : zero8();
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      bf16x8_t a = (kin || SHUF) ? load8(wrow[r] + (size_t)s * WSTEP) : zero8();
+      bf16x8_t a = ((kin || SHUF) && wact) ? load8(wrow[r] + (size_t)s * WSTEP) : zero8();
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[mt], acc[r][mt], 0, 0, 0);
     }
@@ -250,11 +257,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 
   if (scaled) {
     for (int m = wave; m < M; m += WAVES) {
-      float ssum = pre0 + pre1;
-      for (int b = (m == wave ? 128 : 0) + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
+      float ssum = 0.f;
+      if (m == wave) ssum = (pre[0] + pre[1]) + (pre[2] + pre[3]);
+      for (int b = (m == wave ? 256 : 0) + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
       ssum = wave_sum(ssum);
       if (lane == 0) inv_s[m] = 1.0f / sqrtf(ssum / (float)K + ex.eps);
-      pre0 = pre1 = 0.f;
     }
     if (WAVES == 1) __syncthreads();
   }
@@ -321,7 +328,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int n = rowbase[r] + kg * 4;
-        if (live && n < N) {
+        if (live && n < N && (SHUF != 2 || kg < 2)) {
           float* p = ex.res_out + (size_t)m * N + n;
           f32x4_t xv = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -484,8 +491,9 @@ static void skinny_residual(const SkinnyCall& c) {
   const int ldx = c.ldx, ldy = c.N, M = c.M, N = c.N, K = c.K;
   const SkinnyExtra& ex = c.ex;
   hipStream_t stream = c.stream;
-  const int blocks = gs_ceil_div(N, 16);
-  if (K >= 4096) { GS_BY_MT(1, 16, 0, 2, float, blocks) } else { GS_BY_MT(1, 8, 0, 2, float, blocks) }
+  const int blocks = gs_ceil_div(N, SHUF == 2 ? 8 : 16);
+  if (SHUF == 2) { GS_BY_MT(1, 8, 0, 2, float, blocks) }
+  else if (K >= 4096) { GS_BY_MT(1, 16, 0, 2, float, blocks) } else { GS_BY_MT(1, 8, 0, 2, float, blocks) }
 }
 
 template <int SHUF>

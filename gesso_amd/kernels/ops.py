@@ -381,7 +381,7 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt
     M, K = x.shape
     N = w.shape[0]
     _need(w.shape == (N, K) and res.shape == (M, N) and res.dtype == torch.float32, "gemm_skinny_residual: shapes")
-    nb = lib().gs_gemm_skinny_residual_blocks(c_int(N))
+    nb = lib().gs_gemm_skinny_residual_blocks(c_int(N), c_int(0 if wt is None else 1))
     ssq = torch.empty((M, nb), dtype=torch.float32, device=res.device)
     _need((next_weight is None) == (xs is None), "gemm_skinny_residual: next_weight and xs come together")
     if xs is not None:

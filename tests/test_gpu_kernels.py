@@ -600,7 +600,12 @@ def test_tile_major_copy_gives_the_same_products(ops, M, N, K):
     if N <= 2048:
         r1, r2 = torch.ones(M, N, device=DEV), torch.ones(M, N, device=DEV)
         s1, s2 = ops.gemm_skinny_residual(x, w, r1, wt=wt), ops.gemm_skinny_residual(x, w, r2)
-        assert torch.equal(r1, r2) and torch.equal(s1, s2)
+        # a weight of few rows is shared out in half tiles: twice the partial sums, and K split over other
+        # numbers of wavefronts, so the float32 sums differ by rounding (and a bfloat16 rounding may flip)
+        assert s1.shape == (M, N // 8) and s2.shape == (M, N // 16)
+        assert float((r1 - r2).abs().max()) <= 2.0 ** -7 * float((r2 - 1).abs().max())
+        assert torch.allclose(s1.sum(1), s2.sum(1), rtol=1e-3)
+        assert torch.allclose(s1.double().sum(1), (r1.double() ** 2).sum(1), rtol=1e-5)
 
 
 # ------------------------------------------------------------------ prompt attention on the matrix cores
