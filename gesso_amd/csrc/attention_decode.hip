@@ -1,44 +1,59 @@
 // Decode attention: one query token per sequence over its paged keys and values, bfloat16 cache.
 //
 // The step reads every cached key and value of the live sequences once; that stream is all the
-// work there is.  A block owns (split, key head, sequence): a contiguous share of the sequence's
-// keys, for all G query heads that share the key head, so keys and values are read once per group.
+// work there is, and for a few hundred keys the kernel's time is a chain of memory round trips
+// (position, page number, rows), so the chain is kept short: a wavefront issues all the loads of a
+// tile of 64 keys, keys and values, before it computes anything, and (where registers allow) the next
+// tile's loads before it computes the current one.
 //
-// Inside a block each wavefront takes tiles of 64 keys.  Scores: lane = key; the lane reads its key row
-// (D bfloat16, 16-byte loads) and dots it with the G queries held in LDS as float32.  Softmax
-// runs online per head across the wavefront (running maximum and sum).  Values: lane = (key
-// group of 8, chunk of 8 features); 16-byte loads of V rows, probabilities broadcast from LDS.
-// Wavefronts, then splits, are merged by the usual (max, sum, accumulator) rule in a fixed order.
-// With one split the block writes the output itself; with more, each block writes its partial
-// (accumulator, max, sum) and a second small kernel merges them in split order.  (Merging in the
-// last block to arrive would save that launch, but the device-wide fence it needs writes back and
-// invalidates the L2 in every block, which costs far more than the launch.)  Scores, maxima, sums
-// and accumulators are float32.
+// A block owns (split, key head, sequence): a contiguous share of the sequence's keys, for all G
+// query heads that share the key head, so keys and values are read once per group.  Inside a block
+// each wavefront takes tiles of 64 keys.  Scores run on the matrix cores (v_mfma_f32_16x16x32_bf16:
+// 16 keys x 16 head columns, of which G are used, per instruction), with the key rows loaded straight
+// in operand order and the queries held in registers.  Softmax runs online per head (running maximum
+// and sum, base-2 exponentials of scores scaled by log2 e).  Values: lane = (key group, chunk of 8
+// features); 16-byte loads of V rows, probabilities broadcast from LDS.  Wavefronts, then splits, are merged by the usual (max, sum, accumulator) rule
+// in a fixed order.  With one split the block writes the output itself; with more, each block writes
+// its partial (accumulator, max, sum) and a second small kernel merges them in split order.  (Merging
+// in the last block to arrive would save that launch, but the device-wide fence it needs writes back
+// and invalidates the L2 in every block, which costs far more than the launch.)  A block has eight
+// wavefronts, so that for contexts of up to about a thousand keys one block per (sequence, key head)
+// covers them in a pass or two and no merge kernel is needed.  Scores, maxima, sums and accumulators
+// are float32.
 //
 // Everything that changes between steps (positions, block table) is read from device memory, so the
 // launch can be recorded into a graph.  q (T, q_stride), head h at [h D, (h+1) D); caches
 // (pages, nkv, page_size, D); out (T, nh D).  Window: keys lo..pos with lo = pos - window + 1.
 #include "common.h"
 
-#define DEC_WAVES 4
 #define DEC_MAXG 8
+#define DEC_LOG2E 1.4426950408889634f
 
-template <int D, int G>
-__global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+template <int D, int G, int W>
+__global__ __launch_bounds__(W * 64) void attention_decode_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
-    const int* __restrict__ positions, const int* __restrict__ block_table, int max_blocks, int page_size, int window,
-    float scale, bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv) {
-  constexpr int DC = D / 8;        // 16-byte chunks per row
-  constexpr int KG = 64 / DC;      // key groups per wavefront in the value phase
-  static_assert(D % 8 == 0 && 64 % DC == 0, "head width must be 8, 16, 32, 64, 128, 256 or 512");
-  __shared__ float qs[G][D];
-  __shared__ float ps[DEC_WAVES][64][G];
-  __shared__ long vrow[DEC_WAVES][64];
-  __shared__ float wm[DEC_WAVES][G], wl[DEC_WAVES][G];
-  __shared__ float wacc[DEC_WAVES][G][D];
+    const int* __restrict__ positions, const int* __restrict__ block_table, int max_blocks, int page_size,
+    int page_shift, int window, float scale, bf16* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int nh, int nkv) {
+  constexpr int DC = D / 8;               // 16-byte chunks per row
+  constexpr int KG = 64 / DC;             // key groups per wavefront in the value phase
+  constexpr int NI = 64 / KG;             // keys per lane in the value phase
+  constexpr int KS = (D + 31) / 32;       // steps of 32 features in the score products
+  static_assert(D % 8 == 0 && 64 % DC == 0 && G <= 16, "head width must be 8, 16, 32, 64, 128, 256 or 512");
+  // What the registers allow (256 a lane at eight wavefronts a block): the next tile's rows in flight while
+  // this one is computed, for rows of up to 64.
+  constexpr bool PIPE = D <= 64;
+  __shared__ float ps[W][G][64];          // a tile's probabilities, then read per key in the value phase
+  __shared__ float al[W][G];              // by how much a tile shrinks what was accumulated before it
+  __shared__ float wm[W][G], wl[W][G];
+  __shared__ float wacc[W][G][D];
 
   const int split = blockIdx.x, nsplit = gridDim.x, kvh = blockIdx.y, seq = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kg = lane >> 4;
   const int pos = positions[seq];
   const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
   const int nkeys = pos - lo + 1;
@@ -47,69 +62,122 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
   const int tper = (tiles + nsplit - 1) / nsplit;
   const int t0 = split * tper, t1 = (t0 + tper < tiles) ? t0 + tper : tiles;
   const int* bt = block_table + (size_t)seq * max_blocks;
-
-  for (int i = tid; i < G * D; i += blockDim.x) {
-    int g = i / D, j = i - g * D;
-    qs[g][j] = to_f32(q[(size_t)seq * q_stride + (size_t)(kvh * G + g) * D + j]) * scale;
-  }
-  __syncthreads();
-
-  float m[G], l[G], acc[G][8];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m[g] = -INFINITY;
-    l[g] = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[g][j] = 0.f;
-  }
   const int dc = lane % DC, kq = lane / DC;
 
-  for (int t = t0 + wave; t < t1; t += DEC_WAVES) {
-    const int u = lo + (t << 6) + lane;  // this lane's key
-    float s[G];
-    long off = 0;
-    if (u <= pos) {
-      const int page = bt[u / page_size];
-      off = (((long)page * nkv + kvh) * page_size + u % page_size) * D;
-      const uint4* kr = reinterpret_cast<const uint4*>(kcache + off);
-#pragma unroll
-      for (int g = 0; g < G; ++g) s[g] = 0.f;
-#pragma unroll
-      for (int c = 0; c < DC; ++c) {
-        uint4 w = kr[c];
-        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float k0 = __uint_as_float(ww[e] << 16), k1 = __uint_as_float(ww[e] & 0xffff0000u);
-#pragma unroll
-          for (int g = 0; g < G; ++g) s[g] += qs[g][c * 8 + 2 * e] * k0 + qs[g][c * 8 + 2 * e + 1] * k1;
-        }
-      }
+  // where key u's row starts in the caches (u <= pos)
+  auto row_off = [&](int u) -> long {
+    int pg, r;
+    if (page_shift >= 0) {
+      pg = u >> page_shift;
+      r = u & (page_size - 1);
     } else {
-#pragma unroll
-      for (int g = 0; g < G; ++g) s[g] = -INFINITY;
+      pg = u / page_size;
+      r = u - pg * page_size;
     }
-    float alpha[G];
+    return (((long)bt[pg] * nkv + kvh) * page_size + r) * D;
+  };
+  // The loads of tile t.  Keys, as the first operand of the score products: lane (r16, kg) holds, of the four
+  // keys 4 r16 + kt, features 32 s + 8 kg .. + 8.  Values: the lane's chunk of eight features of the value rows
+  // of its NI keys.  Keys beyond pos are read from key pos (they are masked, their probabilities are zero).
+  auto issue = [&](int t, bf16x8_t (*kreg)[KS], uint4* vreg) {
+    const int base = lo + (t << 6);
+    long ko[4], vo[NI];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float mn = fmaxf(m[g], wave_max(s[g]));
-      float p = u <= pos ? expf(s[g] - mn) : 0.f;
-      alpha[g] = expf(m[g] - mn);
-      l[g] = l[g] * alpha[g] + wave_sum(p);
-      m[g] = mn;
-      ps[wave][lane][g] = p;
+    for (int kt = 0; kt < 4; ++kt) {
+      const int u = base + 4 * r16 + kt;
+      ko[kt] = row_off(u <= pos ? u : pos) + kg * 8;
     }
-    vrow[wave][lane] = off;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int uu = base + kq + i * KG;
+      vo[i] = row_off(uu <= pos ? uu : pos) + dc * 8;
+    }
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int st = 0; st < KS; ++st) {
+        if (32 * st + 8 * kg < D)
+          kreg[kt][st] = *reinterpret_cast<const bf16x8_t*>(kcache + ko[kt] + 32 * st);
+        else
+          kreg[kt][st] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) vreg[i] = *reinterpret_cast<const uint4*>(vcache + vo[i]);
+  };
+
+  bf16x8_t kn[4][KS];
+  uint4 vn[NI];
+  int t = t0 + wave;
+  if (t < t1) issue(t, kn, vn);
+
+  // the queries as the second operand: lane (r16, kg) holds head r16's features 32 s + 8 kg .. + 8
+  bf16x8_t qreg[KS];
+#pragma unroll
+  for (int st = 0; st < KS; ++st) {
+    if (r16 < G && 32 * st + 8 * kg < D)
+      qreg[st] = *reinterpret_cast<const bf16x8_t*>(q + (size_t)seq * q_stride + (size_t)(kvh * G + r16) * D + 32 * st + 8 * kg);
+    else
+      qreg[st] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  const float qscale = scale * DEC_LOG2E;   // scores are scaled after the product, in float32
+
+  // lanes r16 < G keep the running maximum and sum of head r16; every lane keeps its share of all heads' sums
+  float m = -INFINITY, l = 0.f;
+  float acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[g][j] = 0.f;
+
+  // one tile: scores, online softmax, values
+  auto compute = [&](int t, bf16x8_t (*kc)[KS], const uint4* vc) {
+    const int base = lo + (t << 6);
+    // sc[kt][i]: head r16, key base + 4 (4 kg + i) + kt
+    f32x4_t sc[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      sc[kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < KS; ++st) sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc[kt][st], qreg[st], sc[kt], 0, 0, 0);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool valid = base + 4 * (4 * kg + i) + kt <= pos;
+        sc[kt][i] = valid ? sc[kt][i] * qscale : -INFINITY;
+        mx = fmaxf(mx, sc[kt][i]);
+      }
+    const float mn = fmaxf(m, group4_max(mx));   // finite: a tile holds at least one key
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sc[kt][i] = __builtin_amdgcn_exp2f(sc[kt][i] - mn);   // 0 for masked keys
+        sum += sc[kt][i];
+      }
+    const float alpha = __builtin_amdgcn_exp2f(m - mn);
+    l = l * alpha + group4_sum(sum);
+    m = mn;
+    if (r16 < G) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<f32x4_t*>(&ps[wave][r16][4 * (4 * kg + i)]) = f32x4_t{sc[0][i], sc[1][i], sc[2][i], sc[3][i]};
+      if (kg == 0) al[wave][r16] = alpha;
+    }
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_s_waitcnt(0xc07f);  // LDS writes of this wavefront are visible to its own lanes
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int g = 0; g < G; ++g) {
+      const float a = al[wave][g];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[g][j] *= alpha[g];
-    const int nk = pos - (lo + (t << 6)) + 1 < 64 ? pos - (lo + (t << 6)) + 1 : 64;
-    for (int kk = kq; kk < nk; kk += KG) {
-      uint4 w = *reinterpret_cast<const uint4*>(vcache + vrow[wave][kk] + dc * 8);
-      const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+      for (int j = 0; j < 8; ++j) acc[g][j] *= a;
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const uint32_t ww[4] = {vc[i].x, vc[i].y, vc[i].z, vc[i].w};
       float v[8];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -118,12 +186,38 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
       }
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        float p = ps[wave][kk][g];
+        const float p = ps[wave][g][kq + i * KG];
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[g][j] += p * v[j];
       }
     }
     __builtin_amdgcn_wave_barrier();
+  };
+
+  if (PIPE) {
+    // the next tile's loads are in flight while this one is computed: two sets of row registers
+    for (; t < t1; t += W) {
+      bf16x8_t kc[4][KS];
+      uint4 vc[NI];
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int st = 0; st < KS; ++st) kc[kt][st] = kn[kt][st];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) vc[i] = vn[i];
+      if (t + W < t1) issue(t + W, kn, vn);
+      compute(t, kc, vc);
+    }
+  } else {
+    // one set of row registers: the first tile's loads were issued above
+    if (t < t1) {
+      compute(t, kn, vn);
+      t += W;
+    }
+    for (; t < t1; t += W) {
+      issue(t, kn, vn);
+      compute(t, kn, vn);
+    }
   }
   // key groups of a wavefront hold partial sums over different keys for the same features: add them
 #pragma unroll
@@ -140,12 +234,9 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
 #pragma unroll
       for (int j = 0; j < 8; ++j) wacc[wave][g][dc * 8 + j] = acc[g][j];
   }
-  if (lane == 0) {
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      wm[wave][g] = m[g];
-      wl[wave][g] = l[g];
-    }
+  if (lane < G) {
+    wm[wave][lane] = m;
+    wl[wave][lane] = l;
   }
   __syncthreads();
 
@@ -154,12 +245,12 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
   for (int i = tid; i < G * D; i += blockDim.x) {
     int g = i / D, j = i - g * D;
     float M = -INFINITY;
-    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, wm[w][g]);
+    for (int w = 0; w < W; ++w) M = fmaxf(M, wm[w][g]);
     float o = 0.f, L = 0.f;
     if (M > -INFINITY)
-      for (int w = 0; w < DEC_WAVES; ++w)
+      for (int w = 0; w < W; ++w)
         if (wm[w][g] > -INFINITY) {
-          float f = expf(wm[w][g] - M);
+          float f = __builtin_amdgcn_exp2f(wm[w][g] - M);
           o += wacc[w][g][j] * f;
           L += wl[w][g] * f;
         }
@@ -188,7 +279,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
     for (int sp = 0; sp < nsplit; ++sp) {
       float ms = part_ml[((base + sp) * G + g) * 2];
       if (ms > -INFINITY) {
-        float f = expf(ms - M);
+        float f = __builtin_amdgcn_exp2f(ms - M);   // maxima are in base-2 units
         o += part_o[((base + sp) * G + g) * D + j] * f;
         L += part_ml[((base + sp) * G + g) * 2 + 1] * f;
       }
@@ -197,14 +288,17 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
   }
 }
 
+#define DEC_WAVES 8
+
 template <int D>
 static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
                          const bf16* vc, const int* positions, const int* bt, int max_blocks, int page_size,
-                         int window, float scale, bf16* out, float* part_o, float* part_ml, int nh, int nkv) {
-#define GS_RUN(GG)                                                                                                  \
-  attention_decode_kernel<D, GG><<<grid, DEC_WAVES * 64, 0, stream>>>(q, q_stride, kc, vc, positions, bt, max_blocks, \
-                                                                      page_size, window, scale, out, part_o,       \
-                                                                      part_ml, nh, nkv)
+                         int page_shift, int window, float scale, bf16* out, float* part_o, float* part_ml, int nh,
+                         int nkv) {
+#define GS_RUN(GG)                                                                                                     \
+  attention_decode_kernel<D, GG, DEC_WAVES><<<grid, DEC_WAVES * 64, 0, stream>>>(                                      \
+      q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_shift, window, scale, out, part_o, part_ml, nh, \
+      nkv)
   switch (G) {
     case 1: GS_RUN(1); break;
     case 2: GS_RUN(2); break;
@@ -240,18 +334,22 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
   GS_REQUIRE(nseq >= 0 && nseq <= 65535 && nkv <= 65535, "attention_decode: bad batch %d", nseq);
   GS_REQUIRE(nsplit >= 1 && nsplit <= 64, "attention_decode: %d splits outside [1, 64]", nsplit);
   GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_decode: bad page_size/max_blocks/window");
-  GS_REQUIRE(q_stride >= nh * d && q_stride % 1 == 0, "attention_decode: q_stride %d below nh*d", q_stride);
+  GS_REQUIRE(q_stride >= nh * d, "attention_decode: q_stride %d below nh*d", q_stride);
+  GS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_decode: query rows must be 16-byte aligned");
   GS_REQUIRE((d * (int)sizeof(bf16)) % 16 == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0,
              "attention_decode: cache rows must be 16-byte aligned");
   if (nseq == 0) return 0;
   int G = nh / nkv;
   dim3 grid(nsplit, nkv, nseq);
+  int page_shift = -1;
+  for (int b = 0; b < 30; ++b)
+    if (page_size == (1 << b)) page_shift = b;
   float* part_o = workspace;
   float* part_ml = workspace + (size_t)nseq * nh * nsplit * d;
   int rc = -1;
 #define GS_ARGS                                                                                                   \
-  G, grid, stream, (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions, block_table,    \
-      max_blocks, page_size, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
+  G, grid, stream, (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions,       \
+      block_table, max_blocks, page_size, page_shift, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
   switch (d) {
     case 16: rc = launch_decode<16>(GS_ARGS); break;
     case 32: rc = launch_decode<32>(GS_ARGS); break;

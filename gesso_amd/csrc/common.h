@@ -90,6 +90,27 @@ __device__ __forceinline__ float group4_sum(float x) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// Maximum and sum over the wavefront without the LDS crossbar: data-parallel moves within rows of 16 lanes
+// (quad swaps, then mirrors of 8 and of 16 lanes), then the row swaps.  The order of the additions is fixed.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float wave_max_dpp(float x) {
+  x = fmaxf(x, dpp_move<0xB1>(x));   // quad_perm [1,0,3,2]
+  x = fmaxf(x, dpp_move<0x4E>(x));   // quad_perm [2,3,0,1]
+  x = fmaxf(x, dpp_move<0x141>(x));  // row_half_mirror
+  x = fmaxf(x, dpp_move<0x140>(x));  // row_mirror
+  return group4_max(x);
+}
+__device__ __forceinline__ float wave_sum_dpp(float x) {
+  x += dpp_move<0xB1>(x);
+  x += dpp_move<0x4E>(x);
+  x += dpp_move<0x141>(x);
+  x += dpp_move<0x140>(x);
+  return group4_sum(x);
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.  `red` holds 17 floats.
 __device__ __forceinline__ float block_sum(float v, float* red) {
   int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;

@@ -42,7 +42,7 @@ class _DecodeContext:
         self.q_lens = [1] * r.cap
         self.all_single = True
         self.max_q_len = 1
-        self.max_kv_len = None            # not known on the host: kernels read kv_len on the device
+        self.max_kv_len = None            # an upper bound, set per recording; kernels read kv_len on the device
         self.decode_only = True
         self.token_ids, self.positions, self.kv_len, self.slots = r.tok, r.pos, r.kv_len, r.slots
         self.seq_of_token, self.q_start, self.want_rows = r.seq_of_token, r.q_start, r.seq_of_token
@@ -78,7 +78,8 @@ class DecodeRunner:
         self.ring = torch.zeros((self.MAX_STEPS, cap), **i32)
         self.bad_ring = torch.zeros((self.MAX_STEPS, cap), **i32)
         self.ctx = _DecodeContext(self)
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        # one recording per bound on the context length: launch shapes (how attention splits its keys) depend on it
+        self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
 
     def _body(self) -> None:
         ops = self.engine.rt.ops
@@ -93,8 +94,16 @@ class DecodeRunner:
         ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring)
         ops.decode_advance(self.pos, self.kv_len, self.live, self.counter)
 
-    def _record(self) -> None:
+    def _bound(self, longest: int) -> int:
+        """The recording that serves contexts of up to ``longest`` tokens: 1024, 2048, 4096, ... tokens."""
+        b = 1024
+        while b < longest:
+            b *= 2
+        return b
+
+    def _record(self, bound: int) -> None:
         """One eager run on scratch rows (everything lazily initialised gets initialised), then the capture."""
+        self.ctx.max_kv_len = bound
         side = torch.cuda.Stream(device=self.engine.device)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -104,7 +113,7 @@ class DecodeRunner:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             self._body()
-        self.graph = graph
+        self.graphs[bound] = graph
 
     def run(self, rids: Sequence[Hashable], tokens: Sequence[int], n: int, samplers=None
             ) -> Tuple[np.ndarray, np.ndarray]:
@@ -116,10 +125,19 @@ class DecodeRunner:
         eng, cap, B = self.engine, self.cap, len(rids)
         if not 1 <= n <= self.MAX_STEPS:
             raise InvalidPlan(f"a decode run takes 1 to {self.MAX_STEPS} steps, not {n}")
-        if self.graph is None:
-            self._record()                       # before any live row is set: the eager run sees scratch rows only
         mgr, st = eng.manager, eng.storage
         rcs = [mgr.get(r) for r in rids]
+        bound = self._bound(max(rc.length for rc in rcs) + n)
+        if bound not in self.graphs:
+            # before any live row is set: the eager run sees scratch rows only
+            self.slots.fill_(st.scratch_slot)
+            self.live.zero_()
+            self.pos.zero_()
+            self.kv_len.fill_(1)
+            for g, bt in enumerate(self.block_tables):
+                bt.fill_(st.num_pages[g])
+            self._record(bound)
+        graph = self.graphs[bound]
         for t in tokens:
             if not 0 <= int(t) < eng.spec.vocab:
                 raise InvalidPlan(f"token id {int(t)} outside the vocabulary of {eng.spec.vocab}")
@@ -158,7 +176,7 @@ class DecodeRunner:
         self.temperature.copy_(torch.from_numpy(temp).pin_memory().to(eng.device, non_blocking=True))
         self.counter.zero_()
         for _ in range(n):
-            self.graph.replay()
+            graph.replay()
         ids = self.ring[:n, :B].cpu().numpy()
         bad = self.bad_ring[:n, :B].cpu().numpy()
         for r in rids:

@@ -162,9 +162,13 @@ class Runtime:
         """
         ops = self.ops
         if ctx.all_single and q.dtype == torch.bfloat16 and ops.attention_decode_supports(nh, nkv, d):
-            # one query per sequence: the key stream is split so that the whole chip reads it
-            # enough blocks that a wavefront rarely walks more than a tile or two of a few hundred keys
-            nsplit = max(1, min(16, 256 // max(1, ctx.nseq * nkv)))
+            # one query per sequence.  A block of eight wavefronts takes a tile of 64 keys per wavefront and pass;
+            # up to two passes stay in one block (no merge kernel), longer key streams are split over blocks
+            longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
+            if window:
+                longest = min(longest, window)
+            tiles = max(1, -(-longest // 64))
+            nsplit = max(1, min(-(-tiles // 16), 64, max(1, 2048 // max(1, ctx.nseq * nkv))))
             return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                         cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
         if (not ctx.all_single and q.dtype == torch.bfloat16 and q_stride % 8 == 0

@@ -409,7 +409,8 @@ def test_gemm_skinny_refuses(ops):
 @pytest.mark.parametrize("window", [None, 70])
 def test_attention_decode(ops, nh, nkv, d, ps, nsplit, window):
     g = gen(nh + d + nsplit)
-    lens = [1, 2, 63, 64, 65, 300, 700, 129]            # keys per sequence, the query's own included
+    lens = [1, 2, 63, 64, 65, 300, 700, 129, 1500]      # keys per sequence, the query's own included; the last
+                                                          # takes a block of eight wavefronts three passes
     nseq = len(lens)
     nblk = [-(-n // ps) for n in lens]
     total = sum(nblk)
