@@ -57,7 +57,7 @@ extern "C" int gs_gemm_skinny(const void* X, int ldx, const float* res, const fl
 
 // Partial sums per row that gs_gemm_skinny_residual writes for N columns.
 extern "C" int gs_gemm_skinny_residual_blocks(int N, int tile_major) {
-  return gs_ceil_div(N, tile_major && gs_skinny_residual_halves(N) ? 8 : 16);
+  return gs_ceil_div(N, tile_major && gs_skinny_halves(N) ? 8 : 16);
 }
 
 // res (M, N) += X W^T, and ssq_out (M, blocks) = partial sums of squares of the new rows.
@@ -67,6 +67,7 @@ extern "C" int gs_gemm_skinny_residual(const void* X, int ldx, const void* W, co
   if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16)) return -1;
   GS_REQUIRE(ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0, "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
   GS_REQUIRE(res && ssq_out, "gemm_skinny_residual: needs the stream and room for the partial sums");
+  GS_REQUIRE(((uintptr_t)res & 15) == 0 && ((uintptr_t)next_w & 15) == 0, "gemm_skinny_residual: the stream and the norm weight must be 16-byte aligned");
   if (M == 0) return 0;
   GS_REQUIRE((next_w == nullptr) == (xs_out == nullptr), "gemm_skinny_residual: the next norm's weight and the room for the weighted rows come together");
   gs_skinny_run_residual(X, ldx, W, Wt, res, ssq_out, next_w, xs_out, M, N, K, stream);

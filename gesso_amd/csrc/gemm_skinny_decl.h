@@ -5,7 +5,7 @@
 void gs_skinny_run_plain(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w,
                          float eps, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M, int N, int K,
                          int epilogue, hipStream_t stream);
-bool gs_skinny_residual_halves(int N);
+bool gs_skinny_halves(int N);
 void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out,
                             const float* next_w, void* xs_out, int M, int N, int K, hipStream_t stream);
 void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,

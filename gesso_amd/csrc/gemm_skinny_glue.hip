@@ -10,6 +10,7 @@ void gs_skinny_plain_tiles(const SkinnyCall& c);
 void gs_skinny_residual_tiles(const SkinnyCall& c);
 void gs_skinny_residual_half_tiles(const SkinnyCall& c);
 void gs_skinny_conv_tiles(const SkinnyCall& c);
+void gs_skinny_conv_half_tiles(const SkinnyCall& c);
 void gs_skinny_qkv_tiles(const SkinnyCall& c, int d);
 
 static SkinnyCall base(const void* X, int ldx, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M,
@@ -33,13 +34,13 @@ void gs_skinny_run_plain(const void* X, int ldx, const float* res, const float* 
 }
 
 // A weight of few rows is shared out in half tiles, so that twice as many blocks stream it.
-bool gs_skinny_residual_halves(int N) { return N % 16 == 0 && N / 16 <= 160; }
+bool gs_skinny_halves(int N) { return N % 16 == 0 && N / 16 <= 160; }
 
 void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out,
                             const float* next_w, void* xs_out, int M, int N, int K, hipStream_t stream) {
   SkinnyCall c = base(X, ldx, W, Wt, nullptr, GS_F32, N, M, N, K, 2, stream);
   c.ex.res_out = res; c.ex.ssq_out = ssq_out; c.ex.next_w = next_w; c.ex.xs_out = (bf16*)xs_out;
-  if (Wt && gs_skinny_residual_halves(N)) gs_skinny_residual_half_tiles(c);
+  if (Wt && gs_skinny_halves(N)) gs_skinny_residual_half_tiles(c);
   else Wt ? gs_skinny_residual_tiles(c) : gs_skinny_residual_rows(c);
 }
 
@@ -49,7 +50,8 @@ void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* s
   SkinnyCall c = base(X, ldx, W, Wt, Y, GS_BF16, H, M, 3 * H, K, 3, stream);
   if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.taps = taps; c.ex.conv_bias = conv_bias; c.ex.state = state; c.ex.slots = slots; c.ex.conv_w = conv_w;
-  Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);
+  if (Wt && gs_skinny_halves(c.N / 3)) gs_skinny_conv_half_tiles(c);   // c.N / 3 channels, as few as a narrow weight's rows
+  else Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);
 }
 
 void gs_skinny_run_qkv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,

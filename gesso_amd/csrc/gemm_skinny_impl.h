@@ -123,7 +123,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   } else if (EPI == 3) {
     const int H = N / 3;
 #pragma unroll
-    for (int r = 0; r < R; ++r) rowbase[r] = blockIdx.x * 16 + r * H;  // B, C, X rows of the same channels
+    for (int r = 0; r < R; ++r) rowbase[r] = blockIdx.x * (SHUF == 2 ? 8 : 16) + r * H;  // B, C, X rows of the same channels
   } else if (SHUF == 2) {
     rowbase[0] = blockIdx.x * 8;  // half a tile: twice the blocks for a weight of few rows
   } else {
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
     for (int r = 0; r < R; ++r) rowbase[r] = n0 + r * 16;
   }
-  static_assert(SHUF != 2 || (R == 1 && EPI == 2), "half tiles are written for the residual epilogue, one tile a block");
+  static_assert(SHUF != 2 || (R == 1 && EPI == 2) || EPI == 3, "half tiles are written for the residual and the convolution epilogues");
   const bool wact = SHUF != 2 || r16 < 8;  // half tiles: the lanes of the other eight rows load nothing
   const bf16* wrow[R];
 #pragma unroll
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     if (EPI == 3 && n >= (r + 1) * (N / 3)) n = (r + 1) * (N / 3) - 1;
     if (n >= N) n = N - 1;                                // clamped: loaded, never stored
     if (SHUF == 2)
-      wrow[r] = W + ((size_t)(blockIdx.x >> 1) * ((K + 31) >> 5)) * 512 + (kg * 16 + (blockIdx.x & 1) * 8 + (r16 & 7)) * 8;
+      wrow[r] = W + ((size_t)(rowbase[r] >> 4) * ((K + 31) >> 5)) * 512 + (kg * 16 + (rowbase[r] & 8) + (r16 & 7)) * 8;
     else if (SHUF)
       // tile-major: the 16 x 32 tile of (row tile, k step) is 64 lanes x 16 bytes in the operand's own order
       wrow[r] = W + ((size_t)(rowbase[r] >> 4) * ((K + 31) >> 5)) * 512 + lane * 8;
@@ -185,6 +185,86 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (lane + 64 * j < ex.nb) pre[j] = ex.ssq[(size_t)wave * ex.nb + lane + 64 * j];
+  }
+
+  // What the epilogue reads besides the product (the stream's old rows, the convolution's history and taps, the
+  // positions and rotation factors) is loaded here, by the wavefront that runs the epilogue, so that these
+  // round trips pass under the product's own instead of after it.
+  constexpr int PRE_TAPS = 4;                       // convolutions of up to this width are held in registers
+  constexpr bool PRE_ROT = R * MT <= 8;             // rotation factors too, while the registers allow
+  const bool half_ok = SHUF != 2 || kg < 2;
+  f32x4_t rold[EPI == 2 ? R : 1][EPI == 2 ? MT : 1], nextw[EPI == 2 ? R : 1];
+  float chist[EPI == 3 ? MT : 1][4][PRE_TAPS - 1], ctap[4][PRE_TAPS], cbias[4];
+  int epos[EPI == 4 ? MT : 1], epage[EPI == 4 ? MT : 1];
+  float ecos[(EPI == 4 && PRE_ROT) ? MT : 1][(EPI == 4 && PRE_ROT) ? R / 2 + 1 : 1][4],
+      esin[(EPI == 4 && PRE_ROT) ? MT : 1][(EPI == 4 && PRE_ROT) ? R / 2 + 1 : 1][4];
+  const bool vec4 = (N & 3) == 0;
+  if (EPI == 2 && wave == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = rowbase[r] + kg * 4;
+      const bool ok = n < N && half_ok;
+      nextw[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (ok && ex.next_w) {
+        if (vec4) nextw[r] = *reinterpret_cast<const f32x4_t*>(ex.next_w + n);
+        else
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) nextw[r][i] = ex.next_w[n + i];
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        rold[r][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (ok && xok[mt]) {
+          const float* p = ex.res_out + (size_t)(mt * 16 + r16) * N + n;
+          if (vec4) rold[r][mt] = *reinterpret_cast<const f32x4_t*>(p);
+          else
+            for (int i = 0; i < 4; ++i)
+              if (n + i < N) rold[r][mt][i] = p[i];
+        }
+      }
+    }
+  }
+  const bool pre_conv = EPI == 3 && ex.conv_w <= PRE_TAPS;
+  if (EPI == 3 && wave == 0 && pre_conv) {
+    const int H = N / 3, Wd = ex.conv_w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4 + i;
+      const bool ok = c < H && half_ok;
+      cbias[i] = (ok && ex.conv_bias) ? ex.conv_bias[c] : 0.f;
+#pragma unroll
+      for (int p = 0; p < PRE_TAPS; ++p) ctap[i][p] = (ok && p < Wd) ? ex.taps[(size_t)c * Wd + p] : 0.f;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int slot = xok[mt] ? ex.slots[mt * 16 + r16] : 0;
+#pragma unroll
+        for (int p = 0; p < PRE_TAPS - 1; ++p)
+          chist[mt][i][p] = (ok && xok[mt] && p < Wd - 1) ? ex.state[((size_t)slot * H + c) * (Wd - 1) + p] : 0.f;
+      }
+    }
+  }
+  if (EPI == 4 && wave == 0) {
+    constexpr int d = 16 * R;
+    const int hh = blockIdx.x;
+    const bool is_q = hh < ex.nh, is_k = !is_q && hh < ex.nh + ex.nkv;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      epos[mt] = xok[mt] ? ex.positions[mt * 16 + r16] : 0;
+      epage[mt] = (xok[mt] && !is_q && ex.write_kv)
+                      ? ex.block_table[(size_t)(mt * 16 + r16) * ex.max_blocks + epos[mt] / ex.page_size] : 0;
+      if (PRE_ROT && (is_q || is_k)) {
+#pragma unroll
+        for (int r = 0; r < R / 2; ++r) {
+          const float* cp = ex.cos_t + (size_t)epos[mt] * (d / 2) + r * 16 + kg * 4;
+          const float* sp = ex.sin_t + (size_t)epos[mt] * (d / 2) + r * 16 + kg * 4;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            ecos[mt][r][i] = cp[i];
+            esin[mt][r][i] = sp[i];
+          }
+        }
+      }
+    }
   }
 
   f32x4_t acc[R][MT];
@@ -328,18 +408,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int n = rowbase[r] + kg * 4;
-        if (live && n < N && (SHUF != 2 || kg < 2)) {
+        if (live && n < N && half_ok) {
           float* p = ex.res_out + (size_t)m * N + n;
-          f32x4_t xv = {0.f, 0.f, 0.f, 0.f};
+          f32x4_t nv, xv;
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (n + i < N) {
-              // the product is rounded to bfloat16 first, as the unfused path stores it before the add
-              float v = p[i] + to_f32(f32_to_bf16(acc[r][mt][i]));
-              p[i] = v;
-              ss += v * v;
-              if (ex.xs_out) xv[i] = v * ex.next_w[n + i];
-            }
+          for (int i = 0; i < 4; ++i) {
+            // the product is rounded to bfloat16 first, as the unfused path stores it before the add
+            nv[i] = rold[r][mt][i] + to_f32(f32_to_bf16(acc[r][mt][i]));
+            if (n + i < N) ss += nv[i] * nv[i];
+            xv[i] = nv[i] * nextw[r][i];
+          }
+          if (vec4) *reinterpret_cast<f32x4_t*>(p) = nv;
+          else
+            for (int i = 0; i < 4; ++i)
+              if (n + i < N) p[i] = nv[i];
           if (ex.xs_out) store4<bf16>(ex.xs_out + (size_t)m * N + n, xv, N - n);
         }
       }
@@ -352,21 +434,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       const int slot = ex.slots[m];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int c = blockIdx.x * 16 + kg * 4 + i;
-        if (c >= H) break;
+        const int c = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4 + i;
+        if (c >= H || !half_ok) break;
         // the products run on the values as the unfused path stores them: rounded to bfloat16
         const float Bv = to_f32(f32_to_bf16(acc[0][mt][i])), Cv = to_f32(f32_to_bf16(acc[1][mt][i])),
                     Xv = to_f32(f32_to_bf16(acc[2][mt][i]));
         const float u = Bv * Xv;
-        const float* wt = ex.taps + (size_t)c * Wd;
         float* hist = ex.state + ((size_t)slot * H + c) * (Wd - 1);
-        float y = 0.f;
-        for (int p = 0; p < Wd - 1; ++p) y += wt[p] * hist[p];
-        y += wt[Wd - 1] * u;
-        if (ex.conv_bias) y += ex.conv_bias[c];
-        Y[(size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
-        for (int p = 0; p < Wd - 2; ++p) hist[p] = hist[p + 1];
-        hist[Wd - 2] = u;
+        if (pre_conv) {
+          float y = 0.f;
+#pragma unroll
+          for (int p = 0; p < PRE_TAPS - 1; ++p)
+            if (p < Wd - 1) y += ctap[i][p] * chist[mt][i][p];
+#pragma unroll
+          for (int p = 0; p < PRE_TAPS; ++p)
+            if (p == Wd - 1) y += ctap[i][p] * u;
+          if (ex.conv_bias) y += cbias[i];
+          Y[(size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
+#pragma unroll
+          for (int p = 0; p < PRE_TAPS - 2; ++p)
+            if (p < Wd - 2) hist[p] = chist[mt][i][p + 1];
+          if (Wd >= 2) hist[Wd - 2] = u;
+        } else {
+          const float* wt = ex.taps + (size_t)c * Wd;
+          float y = 0.f;
+          for (int p = 0; p < Wd - 1; ++p) y += wt[p] * hist[p];
+          y += wt[Wd - 1] * u;
+          if (ex.conv_bias) y += ex.conv_bias[c];
+          Y[(size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
+          for (int p = 0; p < Wd - 2; ++p) hist[p] = hist[p + 1];
+          hist[Wd - 2] = u;
+        }
       }
     } else if (EPI == 4) {
       // one head of d = 16 R features; tile r and tile r + R/2 hold the two halves of each rotation pair
@@ -395,13 +493,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
             for (int i = 0; i < 4; ++i) v[r][i] = v[r][i] * hinv * nw[r * 16 + kg * 4 + i];
         }
         if (live) {
-          const int pos = ex.positions[m];
+          const int pos = epos[mt];
 #pragma unroll
           for (int r = 0; r < R / 2; ++r)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int j = r * 16 + kg * 4 + i;  // pair (j, j + d/2)
-              const float c = ex.cos_t[(size_t)pos * (d / 2) + j], sn = ex.sin_t[(size_t)pos * (d / 2) + j];
+              const float c = PRE_ROT ? ecos[mt][r][i] : ex.cos_t[(size_t)pos * (d / 2) + j];
+              const float sn = PRE_ROT ? esin[mt][r][i] : ex.sin_t[(size_t)pos * (d / 2) + j];
               const float a = v[r][i], b = v[r + R / 2][i];
               v[r][i] = a * c - b * sn;
               v[r + R / 2][i] = a * sn + b * c;
@@ -414,9 +513,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         dst = (bf16*)Y + (size_t)m * ldy + (size_t)hh * d;
       } else {
         if (!ex.write_kv) continue;
-        const int pos = ex.positions[m];
+        const int pos = epos[mt];
         const int kvh = is_k ? hh - ex.nh : hh - ex.nh - ex.nkv;
-        const int page = ex.block_table[(size_t)m * ex.max_blocks + pos / ex.page_size];
+        const int page = epage[mt];
         dst = (is_k ? ex.kcache : ex.vcache) + (((size_t)page * ex.nkv + kvh) * ex.page_size + pos % ex.page_size) * d;
       }
 #pragma unroll
@@ -503,7 +602,7 @@ static void skinny_conv(const SkinnyCall& c) {
   const int ldx = c.ldx, ldy = c.ldy, M = c.M, N = c.N, K = c.K;
   const SkinnyExtra& ex = c.ex;
   hipStream_t stream = c.stream;
-  const int blocks = gs_ceil_div(N / 3, 16);
+  const int blocks = gs_ceil_div(N / 3, SHUF == 2 ? 8 : 16);
   if (ex.res) { GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks) } else { GS_BY_MT4(3, 8, 8, 8, 4, 0, 3, bf16, blocks) }
 }
 
