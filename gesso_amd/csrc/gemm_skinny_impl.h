@@ -299,7 +299,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   const int per = (ksteps + WAVES - 1) / WAVES;
   const int s0 = wave * per, s1 = (s0 + per < ksteps) ? s0 + per : ksteps;
   int s = s0;
-  constexpr int U = R * MT == 1 ? 8 : (R * MT == 2 ? 4 : (R * MT <= 4 ? 2 : 1));  // steps whose loads are issued together
+  // steps whose loads are issued together: as many as about a hundred registers hold (16 bytes a lane per tile)
+  constexpr int UQ = (WAVES >= 16 ? 12 : 24) / (R + MT);   // sixteen wavefronts leave a lane 128 registers
+  constexpr int U = UQ >= 8 ? 8 : (UQ >= 4 ? 4 : (UQ >= 2 ? 2 : 1));
   constexpr int WSTEP = SHUF ? 512 : 32;  // elements between a row tile's consecutive k steps
   if ((K & 31) == 0 || SHUF) {
     for (; s + U <= s1; s += U) {
