@@ -40,11 +40,29 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
     ss = __uint_as_float(0x7fc00000u);
   } else {
     const T* row = table + (size_t)id * H;
-    for (int j = threadIdx.x; j < H; j += blockDim.x) {
-      float v = to_f32(row[j]);
-      o[j] = v;
-      ss += v * v;
-      if (xs) xs[(size_t)t * H + j] = f32_to_bf16(v * next_w[j]);
+    if ((H & 7) == 0 && aligned16(row) && aligned16(o) && (!xs || (aligned16(next_w) && aligned16(xs)))) {
+      // eight values per thread and turn, 16-byte loads and stores
+      for (int j = threadIdx.x * 8; j < H; j += blockDim.x * 8) {
+        float v[8];
+        load8f(row + j, v);
+        store8f(o + j, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+        if (xs) {
+          float w[8];
+          load8f(next_w + j, w);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) w[i] *= v[i];
+          store8f(xs + (size_t)t * H + j, w);
+        }
+      }
+    } else {
+      for (int j = threadIdx.x; j < H; j += blockDim.x) {
+        float v = to_f32(row[j]);
+        o[j] = v;
+        ss += v * v;
+        if (xs) xs[(size_t)t * H + j] = f32_to_bf16(v * next_w[j]);
+      }
     }
   }
   if (ssq) {

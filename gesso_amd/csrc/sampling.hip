@@ -169,14 +169,18 @@ __global__ void sample_temperature_kernel(const float* __restrict__ logits, int 
 
 // The decode loop's choice, made to be recorded into a HIP graph: everything that changes from step to
 // step is read from device memory.  Row r: temperature[r] <= 0 means greedy, else a draw with
-// u[step * rows + r], step = *counter.  The chosen id goes to next_ids[r] (the token fed back) and,
-// with the row's flag, to ring[step * rows + r] and bad_ring[...], which the host reads once per run.
+// u[step * rows + r], step = counter[r] (each row counts its own steps, so no block waits for another).
+// The chosen id goes to next_ids[r] (the token fed back) and, with the row's flag, to
+// ring[step * rows + r] and bad_ring[...], which the host reads once per run.  Then the row moves on:
+// its counter counts up and, if the row is live, so do its position and its number of keys.
 __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
-                                     const double* __restrict__ u, const int* __restrict__ counter,
-                                     int* __restrict__ next_ids, int* __restrict__ ring, int* __restrict__ bad_ring) {
+                                     const double* __restrict__ u, int* __restrict__ counter,
+                                     int* __restrict__ next_ids, int* __restrict__ ring, int* __restrict__ bad_ring,
+                                     int* __restrict__ positions, int* __restrict__ kv_len,
+                                     const int* __restrict__ live) {
   __shared__ int sid, sbad;
   int row = blockIdx.x, rows = gridDim.x;
-  int step = *counter;
+  int step = counter[row];
   double T = temperature[row];
   const float* x = logits + (size_t)row * V;
   if (T > 0.0)
@@ -187,33 +191,22 @@ __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, co
     next_ids[row] = sid;
     ring[(size_t)step * rows + row] = sid;
     bad_ring[(size_t)step * rows + row] = sbad;
+    counter[row] = step + 1;
+    if (live[row]) {
+      positions[row] += 1;
+      kv_len[row] += 1;
+    }
   }
-}
-
-// After a decode step: live rows move one position on; the step counter counts up.  One block.
-__global__ void decode_advance_kernel(int* __restrict__ positions, int* __restrict__ kv_len,
-                                      const int* __restrict__ live, int* __restrict__ counter, int rows) {
-  int r = threadIdx.x;
-  if (r < rows && live[r]) {
-    positions[r] += 1;
-    kv_len[r] += 1;
-  }
-  if (r == 0) *counter += 1;
 }
 
 extern "C" int gs_decode_choose(const float* logits, int rows, int V, const double* temperature, const double* u,
-                                const int* counter, int* next_ids, int* ring, int* bad_ring, hipStream_t stream) {
+                                int* counter, int* next_ids, int* ring, int* bad_ring, int* positions, int* kv_len,
+                                const int* live, hipStream_t stream) {
   GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
-  decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, counter, next_ids, ring, bad_ring);
+  GS_REQUIRE(counter && positions && kv_len && live, "decode_choose: needs the rows' counters, positions, key counts and live flags");
+  decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, counter, next_ids, ring, bad_ring,
+                                                          positions, kv_len, live);
   GS_LAUNCH_CHECK("decode_choose");
-  return 0;
-}
-
-extern "C" int gs_decode_advance(int* positions, int* kv_len, const int* live, int* counter, int rows,
-                                 hipStream_t stream) {
-  GS_REQUIRE(rows > 0 && rows <= 1024, "decode_advance: %d rows; at most 1024", rows);
-  decode_advance_kernel<<<1, 1024, 0, stream>>>(positions, kv_len, live, counter, rows);
-  GS_LAUNCH_CHECK("decode_advance");
   return 0;
 }
 

@@ -4,7 +4,7 @@ A decode step of a small batch is bound by launch overhead, not by arithmetic: m
 hundred kernels of a few microseconds each.  So the step (embedding, all blocks, head, the choice
 of the next token, the advance of positions) is recorded into a graph per batch capacity and
 replayed; everything that changes between steps lives in device buffers the kernels read
-(tokens, positions, block tables, slots, the step counter).  The token a step chooses is written
+(tokens, positions, block tables, slots, the rows' step counters).  The token a step chooses is written
 where the next step's embedding reads it, so ``n`` steps run back to back without the host; the
 host reads the chosen tokens once per call.  The reference decodes one row per call with one
 host round trip per token (``src/Inference/Inference.jl:2547-2712``).
@@ -12,7 +12,7 @@ host round trip per token (``src/Inference/Inference.jl:2547-2712``).
 Rows beyond the live batch (the capacity is the batch rounded up to a power of two) point at the
 scratch page and the scratch slot, so they compute and write garbage that nobody reads.
 
-Graph hygiene: nothing in the graph clears memory with a memset node; the step counter is reset by
+Graph hygiene: nothing in the graph clears memory with a memset node; the step counters are reset by
 an ordinary fill before the replays.
 """
 from __future__ import annotations
@@ -74,7 +74,7 @@ class DecodeRunner:
         self.block_tables = [torch.full((cap, self.max_blocks), n, **i32) for n in st.num_pages]
         self.temperature = torch.zeros(cap, dtype=torch.float64, device=dev)
         self.u = torch.zeros((self.MAX_STEPS, cap), dtype=torch.float64, device=dev)
-        self.counter = torch.zeros(1, **i32)
+        self.counter = torch.zeros(cap, **i32)          # steps made since the host last looked, per row
         self.ring = torch.zeros((self.MAX_STEPS, cap), **i32)
         self.bad_ring = torch.zeros((self.MAX_STEPS, cap), **i32)
         self.ctx = _DecodeContext(self)
@@ -91,8 +91,8 @@ class DecodeRunner:
         finally:
             rt.no_library = rt.fused = False
         self.logits = logits
-        ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring)
-        ops.decode_advance(self.pos, self.kv_len, self.live, self.counter)
+        ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring,
+                          self.pos, self.kv_len, self.live)
 
     def _bound(self, longest: int) -> int:
         """The recording that serves contexts of up to ``longest`` tokens: 1024, 2048, 4096, ... tokens."""

@@ -438,27 +438,21 @@ def gemm_skinny_qkv(x, wqkv, q_weight, k_weight, head_eps, cos, sin, positions, 
     return q
 
 
-def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring) -> None:
-    """Per row: greedy (temperature <= 0) or a draw with ``u[counter, row]``; results into the loop's buffers."""
-    _dev(logits, temperature, u, counter, next_ids, ring, bad_ring)
-    _need(logits.dtype == torch.float32 and logits.dim() == 2, "decode_choose: logits are float32 (rows, V)")
+def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live) -> None:
+    """Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``; results into the loop's buffers;
+    then the row's counter counts up and a live row moves one position on."""
+    _dev(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "decode_choose: logits are float32 (rows, V)")
     rows, V = logits.shape
     _need(temperature.dtype == torch.float64 and temperature.numel() == rows, "decode_choose: temperature float64 (rows,)")
     _need(u.dtype == torch.float64 and u.dim() == 2 and u.shape[1] == rows, "decode_choose: u is float64 (steps, rows)")
-    for t in (counter, next_ids, ring, bad_ring):
+    for t in (counter, next_ids, positions, kv_len, live):
+        _i32(t, rows)
+    for t in (ring, bad_ring):
         _i32(t)
-    _need(ring.shape == u.shape and bad_ring.shape == u.shape and next_ids.numel() == rows, "decode_choose: buffer shapes")
+    _need(ring.shape == u.shape and bad_ring.shape == u.shape, "decode_choose: buffer shapes")
     _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(u), _p(counter), _p(next_ids),
-                                  _p(ring), _p(bad_ring), _stream()))
-
-
-def decode_advance(positions, kv_len, live, counter) -> None:
-    _dev(positions, kv_len, live, counter)
-    rows = positions.numel()
-    for t in (positions, kv_len, live, counter):
-        _i32(t)
-    _need(kv_len.numel() == rows and live.numel() == rows, "decode_advance: buffer shapes")
-    _check(lib().gs_decode_advance(_p(positions), _p(kv_len), _p(live), _p(counter), c_int(rows), _stream()))
+                                  _p(ring), _p(bad_ring), _p(positions), _p(kv_len), _p(live), _stream()))
 
 
 def attention_decode_supports(nh: int, nkv: int, d: int) -> bool:
