@@ -99,6 +99,72 @@ __global__ void short_conv8_kernel(const T* __restrict__ bcx, const float* __res
   }
 }
 
+// Prompt portions: a thread takes eight channels and a run of TT consecutive tokens, so every B and X row is read
+// once (plus W - 1 rows of run-in), all loads of the run are issued before anything is computed, and the products
+// u = B x stay in registers for the W tokens that use them.  Sums run over the taps in the same order as in the
+// kernels above.  The first W - 1 tokens of a sequence take what they miss from the history, read where needed.
+template <typename T, int W, int TT>
+__global__ __launch_bounds__(64) void short_conv_run_kernel(const T* __restrict__ bcx, const float* __restrict__ taps,
+                                                            const float* __restrict__ bias,
+                                                            const float* __restrict__ state,
+                                                            const int* __restrict__ seq_of_token,
+                                                            const int* __restrict__ q_start,
+                                                            const int* __restrict__ slots, T* __restrict__ out,
+                                                            int ntok, int H) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (c >= H) return;
+  const int ta = blockIdx.y * TT;
+  float u[TT + W - 1][8], cc[TT][8];
+#pragma unroll
+  for (int r = 0; r < TT + W - 1; ++r) {
+    const int j = ta - (W - 1) + r;
+    if (j >= 0 && j < ntok) {
+      float b8[8], x8[8];
+      load8f(bcx + (size_t)j * 3 * H + c, b8);
+      load8f(bcx + (size_t)j * 3 * H + 2 * H + c, x8);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) u[r][k] = b8[k] * x8[k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) u[r][k] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TT; ++i) {
+    if (ta + i < ntok) load8f(bcx + (size_t)(ta + i) * 3 * H + H + c, cc[i]);
+  }
+  float tp[8][W], bs[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    bs[k] = bias ? bias[c + k] : 0.f;
+#pragma unroll
+    for (int p = 0; p < W; ++p) tp[k][p] = taps[(size_t)(c + k) * W + p];
+  }
+#pragma unroll
+  for (int i = 0; i < TT; ++i) {
+    const int t = ta + i;
+    if (t >= ntok) break;
+    const int s = seq_of_token[t];
+    const int t0 = q_start[s];
+    float y[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int p = 0; p < W; ++p) {
+      const int j = t - (W - 1) + p;
+      if (j >= t0) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) y[k] += tp[k][p] * u[i + p][k];
+      } else {
+        const float* hist = state + ((size_t)slots[s] * H + c) * (W - 1);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) y[k] += tp[k][p] * hist[k * (W - 1) + (W - 1) - (t0 - j)];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) y[k] = cc[i][k] * (bias ? y[k] + bs[k] : y[k]);
+    store8f(out + (size_t)t * H + c, y);
+  }
+}
+
 template <typename T>
 __global__ void short_conv_state_kernel(const T* __restrict__ bcx, float* __restrict__ state,
                                         const int* __restrict__ q_start, const int* __restrict__ slots, int H,
@@ -134,7 +200,20 @@ extern "C" int gs_short_conv(const void* bcx, int dtype, const float* taps, cons
   dim3 grid(cx, ntok < 65535 ? ntok : 65535);  // the kernel strides over tokens beyond gridDim.y
   const bool vec = H % 8 == 0 && ((uintptr_t)bcx & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
                    (dtype == GS_F32 || dtype == GS_BF16);
-  if (vec) {
+  if (vec && !all_single && W <= 4) {
+    constexpr int TT = 8;
+    dim3 gr(gs_ceil_div(H / 8, 64), gs_ceil_div(ntok, TT));
+    GS_REQUIRE(gr.y <= 65535, "short_conv: %d tokens in one call; at most %d", ntok, 65535 * TT);
+#define GS_RUN_CONV(TY, WW)                                                                                          \
+  short_conv_run_kernel<TY, WW, TT><<<gr, 64, 0, stream>>>((const TY*)bcx, taps, bias, state, seq_of_token, q_start, \
+                                                           slots, (TY*)out, ntok, H)
+    if (dtype == GS_F32) {
+      if (W == 2) GS_RUN_CONV(float, 2); else if (W == 3) GS_RUN_CONV(float, 3); else GS_RUN_CONV(float, 4);
+    } else {
+      if (W == 2) GS_RUN_CONV(bf16, 2); else if (W == 3) GS_RUN_CONV(bf16, 3); else GS_RUN_CONV(bf16, 4);
+    }
+#undef GS_RUN_CONV
+  } else if (vec) {
     int th = H / 8 >= 256 ? 256 : 64;
     dim3 g8(gs_ceil_div(H / 8, th), grid.y);
     if (dtype == GS_F32)

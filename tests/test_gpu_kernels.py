@@ -99,7 +99,8 @@ def test_residual_add_and_zero_slots(ops):
 
 # ------------------------------------------------------------------ short convolution
 
-@pytest.mark.parametrize("H,W,bias", [(13, 3, False), (200, 4, True), (64, 2, False), (1, 3, True)])
+@pytest.mark.parametrize("H,W,bias", [(13, 3, False), (200, 4, True), (64, 2, False), (1, 3, True), (72, 6, True),
+                                      (520, 3, True)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_short_conv_segments_and_history(ops, H, W, bias, dtype):
     g = gen(10 * H + W)
@@ -134,6 +135,31 @@ def test_short_conv_segments_and_history(ops, H, W, bias, dtype):
     assert torch.equal(state[1].cpu(), torch.full((H, W - 1), 7.0)) and torch.equal(state[4].cpu(), torch.full((H, W - 1), 7.0))
 
 
+@pytest.mark.parametrize("W", [2, 3, 4])
+def test_short_conv_long_portions_beside_short_ones(ops, W):
+    """Portions longer than a thread's run of tokens, beside ones of one and two tokens, each with its own history."""
+    H = 136
+    g = gen(W)
+    taps = torch.randn(H, W, generator=g)
+    b = torch.randn(H, generator=g)
+    n = [37, 1, 2, 19, 8, 3]
+    state0 = torch.randn(len(n) + 1, H, W - 1, generator=g)
+    slots = torch.tensor([4, 0, 6, 2, 1, 5], dtype=torch.int32)
+    rows = [torch.randn(k, 3 * H, generator=g).bfloat16() for k in n]
+    state = state0.clone().to(DEV)
+    q_start = torch.tensor([0] + list(torch.tensor(n).cumsum(0)), dtype=torch.int32, device=DEV)
+    seq_of = torch.cat([torch.full((k,), i, dtype=torch.int32) for i, k in enumerate(n)]).to(DEV)
+    out = ops.short_conv(torch.cat(rows).to(DEV), taps.to(DEV), b.to(DEV), state, seq_of, q_start, slots.to(DEV),
+                         len(n), False).cpu()
+    o = 0
+    for i, k in enumerate(n):
+        want, hist = P.short_conv(rows[i].double(), taps.double(), b.double(), state0[slots[i]].double())
+        close(out[o:o + k], want, torch.bfloat16)
+        close(state[slots[i]], hist, torch.float32)
+        o += k
+    assert torch.equal(state[3].cpu(), state0[3])
+
+
 def test_short_conv_refuses_a_width_it_cannot_take(ops):
     from gesso_amd.errors import KernelError
     H, W = 4, 17
@@ -152,7 +178,8 @@ def rope_tables(rd, theta, n):
 
 
 @pytest.mark.parametrize("nh,nkv,d,rd,norm", [(4, 2, 16, 16, True), (3, 1, 48, 48, True), (2, 2, 128, 64, False),
-                                               (5, 5, 80, 80, True), (8, 2, 256, 256, True)])
+                                               (5, 5, 80, 80, True), (8, 2, 256, 256, True), (32, 8, 64, 64, True),
+                                               (3, 1, 32, 32, False), (2, 1, 128, 128, True)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_qknorm_rope_kv(ops, nh, nkv, d, rd, norm, dtype):
     g = gen(nh * 100 + d)
