@@ -36,7 +36,7 @@ template <int D, int G, int W>
 __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int* __restrict__ positions, const int* __restrict__ block_table, int max_blocks, int page_size,
-    int page_shift, int window, float scale, bf16* __restrict__ out, float* __restrict__ part_o,
+    unsigned page_magic, int window, float scale, bf16* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int nh, int nkv) {
   constexpr int DC = D / 8;               // 16-byte chunks per row
   constexpr int KG = 64 / DC;             // key groups per wavefront in the value phase
@@ -65,15 +65,11 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
   const int dc = lane % DC, kq = lane / DC;
 
   // where key u's row starts in the caches (u <= pos)
+  // (u / page_size as one multiplication, page_magic = floor(2^32 / page_size) + 1, exact while u page_size < 2^32:
+  // no branch near the loads, which would make the compiler wait for every load in flight)
   auto row_off = [&](int u) -> long {
-    int pg, r;
-    if (page_shift >= 0) {
-      pg = u >> page_shift;
-      r = u & (page_size - 1);
-    } else {
-      pg = u / page_size;
-      r = u - pg * page_size;
-    }
+    const int pg = (int)__umulhi((unsigned)u, page_magic);
+    const int r = u - pg * page_size;
     return (((long)bt[pg] * nkv + kvh) * page_size + r) * D;
   };
   // The loads of tile t.  Keys, as the first operand of the score products: lane (r16, kg) holds, of the four
@@ -293,11 +289,11 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
 template <int D>
 static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
                          const bf16* vc, const int* positions, const int* bt, int max_blocks, int page_size,
-                         int page_shift, int window, float scale, bf16* out, float* part_o, float* part_ml, int nh,
+                         unsigned page_magic, int window, float scale, bf16* out, float* part_o, float* part_ml, int nh,
                          int nkv) {
 #define GS_RUN(GG)                                                                                                     \
   attention_decode_kernel<D, GG, DEC_WAVES><<<grid, DEC_WAVES * 64, 0, stream>>>(                                      \
-      q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_shift, window, scale, out, part_o, part_ml, nh, \
+      q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_magic, window, scale, out, part_o, part_ml, nh, \
       nkv)
   switch (G) {
     case 1: GS_RUN(1); break;
@@ -341,15 +337,15 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
   if (nseq == 0) return 0;
   int G = nh / nkv;
   dim3 grid(nsplit, nkv, nseq);
-  int page_shift = -1;
-  for (int b = 0; b < 30; ++b)
-    if (page_size == (1 << b)) page_shift = b;
+  GS_REQUIRE(page_size >= 2 && (long)max_blocks * page_size * page_size < (1L << 32),
+             "attention_decode: page_size %d with %d blocks a sequence is outside what the kernel's division takes", page_size, max_blocks);
+  const unsigned page_magic = (unsigned)((1ull << 32) / (unsigned)page_size + 1);
   float* part_o = workspace;
   float* part_ml = workspace + (size_t)nseq * nh * nsplit * d;
   int rc = -1;
 #define GS_ARGS                                                                                                   \
   G, grid, stream, (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions,       \
-      block_table, max_blocks, page_size, page_shift, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
+      block_table, max_blocks, page_size, page_magic, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
   switch (d) {
     case 16: rc = launch_decode<16>(GS_ARGS); break;
     case 32: rc = launch_decode<32>(GS_ARGS); break;

@@ -161,7 +161,8 @@ class Runtime:
         shapes they are written for.
         """
         ops = self.ops
-        if ctx.all_single and q.dtype == torch.bfloat16 and ops.attention_decode_supports(nh, nkv, d):
+        if (ctx.all_single and q.dtype == torch.bfloat16 and cache.page_size >= 2
+                and ops.attention_decode_supports(nh, nkv, d)):
             # one query per sequence.  A block of eight wavefronts takes a tile of 64 keys per wavefront and pass;
             # up to two passes stay in one block (no merge kernel), longer key streams are split over blocks
             longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
@@ -171,11 +172,12 @@ class Runtime:
             nsplit = max(1, min(-(-tiles // 16), 64, max(1, 2048 // max(1, ctx.nseq * nkv))))
             return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                         cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
-        if (not ctx.all_single and q.dtype == torch.bfloat16 and q_stride % 8 == 0
+        if (not ctx.all_single and q.dtype == torch.bfloat16 and q_stride % 8 == 0 and cache.page_size >= 2
                 and ops.attention_prefill_supports(nh, nkv, d)):
             # prompts: queries in tiles per sequence, both products on the matrix cores; tiles of 32 share
             # every key and value fragment between two products, which pays when portions are long
-            rows = 32 if ctx.max_q_len >= 64 else 16
+            # (groups of more than four heads have no registers for tiles of 32)
+            rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16
             return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows),
                                          cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T,
                                          tile_rows=rows)
