@@ -6,7 +6,8 @@ A step is one decode step of the whole batch: every live request gets its next t
 model's forward from the cache, the head, and greedy choice of the token that is fed back).
 The default run: 16 layers of the 1.2B sizes, bfloat16, batch 8, 512-token random prompts,
 context 4,096 with 16-token pages.  Prints one JSON line; for more than one GPU it prints
-one line that says so and exits with 2 (this engine runs on one GPU).
+one line that says so and exits with 2 (this engine runs on one GPU).  ``--workload serve`` and
+``--workload long`` measure two other workloads and print a line of their own.
 
 Roofline of the decode step: the bytes it has to read (every weight it uses once, the keys and
 values of the live requests, their convolution state) over its time, against 8 TB/s.  Prefill:
@@ -23,14 +24,22 @@ HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def model_config():
+SIZES = {   # hidden, layers, heads, attention layers, block_ff_dim (before the 2/3 adjustment)
+    "1.2b": (2048, 16, 32, [2, 5, 8, 10, 12, 14], 12288),
+    "350m": (1024, 16, 16, [2, 5, 8, 10, 12, 14], 6656),
+    "2.6b": (2048, 30, 32, [2, 6, 10, 14, 18, 21, 24, 27], 10752),
+}
+
+
+def model_config(size: str = "1.2b", max_position: int = 4096):
     from gesso_amd.config import Lfm2Config
+    hidden, layers, heads, attn, ff = SIZES[size]
     return Lfm2Config.from_dict({
-        "architectures": ["Lfm2ForCausalLM"], "vocab_size": 65536, "hidden_size": 2048, "num_hidden_layers": 16,
-        "num_attention_heads": 32, "num_key_value_heads": 8, "full_attn_idxs": [2, 5, 8, 10, 12, 14],
-        "conv_L_cache": 3, "conv_bias": False, "block_ff_dim": 12288, "block_auto_adjust_ff_dim": True,
+        "architectures": ["Lfm2ForCausalLM"], "vocab_size": 65536, "hidden_size": hidden, "num_hidden_layers": layers,
+        "num_attention_heads": heads, "num_key_value_heads": 8, "full_attn_idxs": attn,
+        "conv_L_cache": 3, "conv_bias": False, "block_ff_dim": ff, "block_auto_adjust_ff_dim": True,
         "block_multiple_of": 256, "block_ffn_dim_multiplier": 1.0, "norm_eps": 1e-5, "rope_theta": 1000000.0,
-        "tie_word_embeddings": True, "max_position_embeddings": 4096})
+        "tie_word_embeddings": True, "max_position_embeddings": max_position})
 
 
 def weight_bytes(engine) -> int:
@@ -117,6 +126,90 @@ def prefill_run(engine, cfg, tokens: int, reps: int = 5):
     return times[len(times) // 2]
 
 
+def serve_workload(seed: int = 5) -> dict:
+    """LFM2-350M sizes: 64 requests at once, prompts of 64 to 2,048 tokens, 32 to 512 new tokens each, prompt
+    portions of 512 tokens beside the decodes of the others; the scheduler's own loop, greedy."""
+    from gesso_amd import Session
+    from gesso_amd.engine.scheduler import Request
+    cfg = model_config("350m")
+    g = torch.Generator().manual_seed(seed)
+    n = 64
+    plen = torch.randint(64, 2049, (n,), generator=g).tolist()
+    olen = torch.randint(32, 513, (n,), generator=g).tolist()
+    sess = Session(cfg, random_weights_seed=0, context_length=4096, max_num_seqs=64, chunk_size=512,
+                   max_num_batched_tokens=1024, max_tokens=n * 2624)
+    stamps = {}
+
+    def run():
+        sched = sess.scheduler()
+        reqs = []
+        for i in range(n):
+            prompt = torch.randint(0, cfg.vocab_size, (plen[i],), generator=g).tolist()
+            stamps[i] = []
+            reqs.append(sched.add(Request(("serve", i), prompt, olen[i], None, (), (),
+                                          lambda tok, i=i: stamps[i].append(time.perf_counter()))))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while sched.has_work():
+            sched.step()
+        torch.cuda.synchronize()
+        return t0, time.perf_counter(), sched, reqs
+
+    run()                                   # once to record the decode graphs and warm the library
+    t0, t1, sched, reqs = run()
+    new = sum(len(r.output) for r in reqs)
+    ttft = [stamps[i][0] - t0 for i in range(n)]
+    tpot = [(stamps[i][-1] - stamps[i][0]) / (len(stamps[i]) - 1) for i in range(n) if len(stamps[i]) > 1]
+    return {"metric": "continuous batching, LFM2-350M sizes: new tokens a second over the whole run",
+            "value": round(new / (t1 - t0), 1), "unit": "tok/s", "seconds": round(t1 - t0, 3), "requests": n,
+            "prompt_tokens": sum(plen), "new_tokens": new, "prompt_tok_s": round(sum(plen) / (t1 - t0), 1),
+            "mean_ttft_ms": round(1e3 * sum(ttft) / n, 2), "mean_tpot_ms": round(1e3 * sum(tpot) / len(tpot), 3),
+            "steps": sched.stats["steps"], "preemptions": sched.stats["preemptions"], "chunk": 512,
+            "token_budget": 1024, "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
+
+
+def long_workload(seed: int = 6) -> dict:
+    """LFM2-2.6B sizes: prompts of 32,768 tokens in portions of 2,048, then 256 decode steps of 8 such requests."""
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.engine.decode import DecodeLoop
+    ctx_len, chunk, batch, steps = 32768, 2048, 8, 256
+    cfg = model_config("2.6b", max_position=ctx_len + 512)
+    engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=16, max_context=ctx_len + 512,
+                                max_tokens=batch * (ctx_len + 512), num_slots=batch + 1)
+    g = torch.Generator().manual_seed(seed)
+    rids, first, times = [("long", i) for i in range(batch)], [], []
+    for rid in rids:
+        engine.add_request(rid)
+        ids = torch.randint(0, cfg.vocab_size, (ctx_len,), generator=g).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for at in range(0, ctx_len, chunk):
+            last = at + chunk >= ctx_len
+            logits = engine.step([StepEntry(rid, ids[at:at + chunk], [chunk - 1] if last else [])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        first.append(int(logits.argmax(1)[0]))
+    prefill = sorted(times[1:])[len(times[1:]) // 2]            # the first prompt warms the library up
+    loop = DecodeLoop(engine, rids, first)
+    loop.run(8)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    loop.run(steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    wbytes = weight_bytes(engine)
+    mean_ctx = ctx_len + 8 + steps / 2.0
+    bytes_step = wbytes + kv_bytes(cfg, engine, [mean_ctx] * batch)
+    flops = step_flops(cfg, ctx_len, ctx_len * (ctx_len + 1) // 2, 1)
+    return {"metric": "LFM2-2.6B sizes at a context of 32,768: decode tok/s at batch 8", "value": round(batch * steps / dt, 1),
+            "unit": "tok/s", "ms_per_step": round(dt / steps * 1e3, 4), "decode_gb_per_step": round(bytes_step / 1e9, 3),
+            "decode_roofline_frac": round(bytes_step / (dt / steps) / 1e9 / HBM_GBPS, 4),
+            "prefill_tok_s": round(ctx_len / prefill, 1), "prefill_s": round(prefill, 4), "prefill_chunk": chunk,
+            "prefill_frac": round(flops / prefill / PEAK_FLOPS["bf16"], 4), "layers": cfg.num_hidden_layers,
+            "weights_gb": round(wbytes / 1e9, 3), "dtype": "bf16",
+            "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -127,10 +220,16 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="measure the 2,048-token prefill alone (for profiling)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long"],
+                    help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
+                         "sizes at a context of 32,768")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
         return 2
+    if args.workload != "decode":
+        print(json.dumps(serve_workload() if args.workload == "serve" else long_workload()))
+        return 0
 
     from gesso_amd import Engine
 

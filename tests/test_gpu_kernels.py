@@ -688,6 +688,33 @@ def test_attention_prefill(ops, nh, nkv, d, ps, window, rows):
     close(got, same.double().cpu(), torch.bfloat16)
 
 
+@pytest.mark.parametrize("rows,window", [(32, None), (16, 3000)])
+def test_attention_prefill_over_more_pages_than_the_kernel_keeps_at_hand(ops, rows, window):
+    """4,700 keys in pages of two: the kernel keeps 2,048 page numbers in LDS and walks the rest window by window.
+    One key far back, in the first window, carries weight for the last query."""
+    g = gen(5)
+    nh, nkv, d, ps, prefix, new = 2, 1, 64, 2, 4650, 50
+    K = prefix + new
+    k, v, q = torch.randn(K, nkv, d, generator=g), torch.randn(K, nkv, d, generator=g), torch.randn(new, nh, d, generator=g)
+    far = 1999 if window is None else K - 2990
+    k[far, 0] = q[-1, 0] * 1.5
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    nblk = -(-K // ps)
+    perm = torch.randperm(nblk, generator=g)
+    kc = torch.zeros(nblk, nkv, ps, d, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    kc[perm] = k.reshape(nblk, ps, nkv, d).permute(0, 2, 1, 3)
+    vc[perm] = v.reshape(nblk, ps, nkv, d).permute(0, 2, 1, 3)
+    table = perm.to(torch.int32)[None].contiguous()
+    tiles = torch.tensor([[0] * -(-new // rows), list(range(0, new, rows)),
+                          [min(rows, new - a) for a in range(0, new, rows)]], dtype=torch.int32)
+    got = ops.attention_prefill(q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV),
+                                torch.arange(prefix, K, dtype=torch.int32, device=DEV), tiles.to(DEV), table.to(DEV), ps,
+                                window, 1.0 / math.sqrt(d), nh, nkv, d, new, tile_rows=rows)
+    want = P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(new, -1)
+    close(got, want, torch.bfloat16)
+
+
 def test_attention_prefill_far_key_and_supports(ops):
     assert ops.attention_prefill_supports(32, 8, 64) and not ops.attention_prefill_supports(3, 3, 48)
     assert not ops.attention_prefill_supports(18, 2, 64)
