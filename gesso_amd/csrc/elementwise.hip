@@ -19,7 +19,7 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 3; }
+extern "C" int gs_abi_version() { return 4; }
 
 // ------------------------------------------------------------------ embedding
 
@@ -82,6 +82,84 @@ extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, floa
   else
     GS_REQUIRE(false, "embed: unknown dtype %d", table_dtype);
   GS_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ------------------------------------------------------------------ residual add from partial sums (+ RMSNorm)
+
+// One block per row: delta = sum over the parts of K (in order), rounded to bfloat16 as a product's result is
+// before the add; res += delta; ssq[row] = sum of squares of the new row; and, with next_w, the row normed for
+// the norm that reads the stream next: normed = res / sqrt(mean(res^2) + eps) * next_w.
+template <typename TO>
+__global__ void residual_from_parts_kernel(const float* __restrict__ part, int parts, float* __restrict__ res,
+                                           float* __restrict__ ssq, const float* __restrict__ next_w, float eps,
+                                           TO* __restrict__ normed, int M, int N) {
+  __shared__ float red[17];
+  const int m = blockIdx.x;
+  float* x = res + (size_t)m * N;
+  constexpr int MAXV = 4;                         // values kept in registers between the passes: rows up to 4096
+  float keep[MAXV][4];
+  float ss = 0.f;
+  const bool vec = (N & 3) == 0;
+  const int turns = (N + 4 * blockDim.x - 1) / (4 * blockDim.x);
+  for (int u = 0; u < turns; ++u) {
+    const int j = (u * blockDim.x + threadIdx.x) * 4;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (j < N) {
+      float d[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int p = 0; p < parts; ++p) {
+        const float* src = part + ((size_t)p * M + m) * N + j;
+        if (vec) {
+          const float4 a = *reinterpret_cast<const float4*>(src);
+          d[0] += a.x; d[1] += a.y; d[2] += a.z; d[3] += a.w;
+        } else {
+          for (int i = 0; i < 4; ++i)
+            if (j + i < N) d[i] += src[i];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (j + i < N) {
+          v[i] = x[j + i] + to_f32(f32_to_bf16(d[i]));
+          x[j + i] = v[i];
+          ss += v[i] * v[i];
+        }
+    }
+    if (u < MAXV) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) keep[u][i] = v[i];
+    }
+  }
+  ss = block_sum(ss, red);
+  if (threadIdx.x == 0) ssq[m] = ss;
+  if (!normed) return;
+  const float inv = 1.0f / sqrtf(ss / (float)N + eps);
+  for (int u = 0; u < turns; ++u) {
+    const int j = (u * blockDim.x + threadIdx.x) * 4;
+    if (j >= N) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (j + i < N) {
+        const float v = u < MAXV ? keep[u][i] : x[j + i];
+        normed[(size_t)m * N + j + i] = from_f32<TO>(v * inv * next_w[j + i]);
+      }
+  }
+}
+
+extern "C" int gs_residual_from_parts(const float* part, int parts, float* res, float* ssq, const float* next_w,
+                                      float eps, void* normed, int normed_dtype, int M, int N, hipStream_t stream) {
+  GS_REQUIRE(M >= 0 && N > 0 && parts >= 1, "residual_from_parts: bad sizes M=%d N=%d parts=%d", M, N, parts);
+  GS_REQUIRE(part && res && ssq, "residual_from_parts: needs the partial sums, the stream and room for the sums of squares");
+  GS_REQUIRE((next_w == nullptr) == (normed == nullptr), "residual_from_parts: the next norm's weight and the room for the normed rows come together");
+  GS_REQUIRE(((uintptr_t)part & 15) == 0, "residual_from_parts: the partial sums must be 16-byte aligned");
+  if (M == 0) return 0;
+  if (!normed || normed_dtype == GS_BF16)
+    residual_from_parts_kernel<bf16><<<M, 256, 0, stream>>>(part, parts, res, ssq, next_w, eps, (bf16*)normed, M, N);
+  else if (normed_dtype == GS_F32)
+    residual_from_parts_kernel<float><<<M, 256, 0, stream>>>(part, parts, res, ssq, next_w, eps, (float*)normed, M, N);
+  else
+    GS_REQUIRE(false, "residual_from_parts: unknown dtype %d", normed_dtype);
+  GS_LAUNCH_CHECK("residual_from_parts");
   return 0;
 }
 

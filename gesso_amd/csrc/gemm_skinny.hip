@@ -75,6 +75,18 @@ extern "C" int gs_gemm_skinny_residual(const void* X, int ldx, const void* W, co
   return 0;
 }
 
+// part (parts, M, N) float32 = partial sums of X W^T over `parts` parts of K; gs_residual_from_parts adds them up.
+extern "C" int gs_gemm_skinny_parts(const void* X, int ldx, const void* W, const void* Wt, float* part, int parts,
+                                    int M, int N, int K, hipStream_t stream) {
+  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16)) return -1;
+  GS_REQUIRE(ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0, "gemm_skinny: X must be 16-byte aligned with a row stride that is a multiple of 8");
+  GS_REQUIRE(part && parts >= 1 && parts <= 64 && ((uintptr_t)part & 15) == 0, "gemm_skinny_parts: 1 to 64 parts and an aligned buffer");
+  if (M == 0) return 0;
+  gs_skinny_run_parts(X, ldx, W, Wt, part, parts, M, N, K, stream);
+  GS_LAUNCH_CHECK("gemm_skinny_parts");
+  return 0;
+}
+
 // mixed (M, H) = gated short convolution of (normed res) W_in^T for a decode step; W_in (3H, K).
 extern "C" int gs_gemm_skinny_conv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps,
                                    const void* W, const void* Wt, const float* taps, const float* conv_bias,

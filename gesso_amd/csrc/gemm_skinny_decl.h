@@ -16,3 +16,5 @@ void gs_skinny_run_qkv(const void* X, int ldx, const float* res, const float* ss
                        const float* sin_t, const int* positions, const int* block_table, int max_blocks,
                        int page_size, void* kcache, void* vcache, int write_kv, void* Q, int M, int nh, int nkv, int d,
                        int K, hipStream_t stream);
+void gs_skinny_run_parts(const void* X, int ldx, const void* W, const void* Wt, float* part, int parts, int M, int N,
+                         int K, hipStream_t stream);

@@ -10,6 +10,8 @@ void gs_skinny_plain_tiles(const SkinnyCall& c);
 void gs_skinny_residual_tiles(const SkinnyCall& c);
 void gs_skinny_residual_half_tiles(const SkinnyCall& c);
 void gs_skinny_conv_tiles(const SkinnyCall& c);
+void gs_skinny_parts_rows(const SkinnyCall& c, int parts);
+void gs_skinny_parts_tiles(const SkinnyCall& c, int parts);
 void gs_skinny_conv_half_tiles(const SkinnyCall& c);
 void gs_skinny_qkv_tiles(const SkinnyCall& c, int d);
 
@@ -65,4 +67,10 @@ void gs_skinny_run_qkv(const void* X, int ldx, const float* res, const float* ss
   c.ex.positions = positions; c.ex.block_table = block_table; c.ex.max_blocks = max_blocks; c.ex.page_size = page_size;
   c.ex.nh = nh; c.ex.nkv = nkv; c.ex.write_kv = write_kv; c.ex.kcache = (bf16*)kcache; c.ex.vcache = (bf16*)vcache;
   Wt ? gs_skinny_qkv_tiles(c, d) : gs_skinny_qkv_rows(c, d);
+}
+
+void gs_skinny_run_parts(const void* X, int ldx, const void* W, const void* Wt, float* part, int parts, int M, int N,
+                         int K, hipStream_t stream) {
+  SkinnyCall c = base(X, ldx, W, Wt, part, GS_F32, N, M, N, K, 5, stream);
+  Wt ? gs_skinny_parts_tiles(c, parts) : gs_skinny_parts_rows(c, parts);
 }

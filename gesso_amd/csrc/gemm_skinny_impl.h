@@ -30,6 +30,9 @@
 // What is done with Y (EPI):
 //   0  stored (bfloat16 or float32).
 //   1  SwiGLU: W holds gate rows [0, N/2) then up rows; stores silu(gate) * up, N/2 wide.
+//   5  partial sums: K is shared out over gridDim.y blocks as well, each writes its float32 (M, N) sheet; a second
+//      kernel adds the sheets.  For many rows: every block reads all rows of X for its part of K, so the fewer
+//      weight rows and the more of K a block takes, the more X traffic; sharing K over blocks caps it.
 //   2  added to the residual stream in place (float32), and the sums of squares of the new rows over this
 //      block's columns stored as partial sums for the next norm.
 //   3  gated short convolution of a decode step: tiles are the B, C, X rows of 16 channels; u = B X,
@@ -295,9 +298,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   };
 
   // this wavefront's share of K, in steps of 32
-  const int ksteps = (K + 31) >> 5;
-  const int per = (ksteps + WAVES - 1) / WAVES;
-  const int s0 = wave * per, s1 = (s0 + per < ksteps) ? s0 + per : ksteps;
+  // (EPI 5: the blocks of one column of the grid share K among themselves first, blockIdx.y taking its part)
+  const int ksteps_all = (K + 31) >> 5;
+  int kbeg = 0, kend = ksteps_all;
+  if (EPI == 5) {
+    const int part = (ksteps_all + (int)gridDim.y - 1) / (int)gridDim.y;
+    kbeg = blockIdx.y * part;
+    kend = kbeg + part < ksteps_all ? kbeg + part : ksteps_all;
+    if (kend < kbeg) kend = kbeg;
+  }
+  const int per = (kend - kbeg + WAVES - 1) / WAVES;
+  const int s0 = kbeg + wave * per, s1 = (s0 + per < kend) ? s0 + per : kend;
   int s = s0;
   // steps whose loads are issued together: as many as about a hundred registers hold (16 bytes a lane per tile)
   constexpr int UQ = (WAVES >= 16 ? 12 : 24) / (R + MT);   // sixteen wavefronts leave a lane 128 registers
@@ -387,12 +398,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r16;
     const bool live = m < M;
-    if (EPI == 0) {
+    if (EPI == 0 || EPI == 5) {
       if (!live) continue;
+      TOut* Yp = EPI == 5 ? Y + (size_t)blockIdx.y * M * ldy : Y;   // partial sums: one (M, N) sheet per part of K
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int n = rowbase[r] + kg * 4;
-        if (N - n > 0) store4<TOut>(Y + (size_t)m * ldy + n, acc[r][mt], N - n);
+        if (N - n > 0) store4<TOut>(Yp + (size_t)m * ldy + n, acc[r][mt], N - n);
       }
     } else if (EPI == 1) {
       if (!live) continue;
@@ -537,6 +549,14 @@ static void launch_skinny(int blocks, const bf16* X, int ldx, const bf16* W, TOu
       <<<blocks, WAVES * 64, lds, stream>>>(X, ldx, W, Y, ldy, M, N, K, ex);
 }
 
+template <int R, int MT, int WAVES, int SHUF>
+static void launch_skinny_parts(int blocks, int parts, const bf16* X, int ldx, const bf16* W, float* Y, int M, int N,
+                                int K, const SkinnyExtra& ex, hipStream_t stream) {
+  const size_t lds = (size_t)(WAVES - 1) * R * MT * 256 * sizeof(float);
+  gemm_skinny_kernel<R, MT, WAVES, 0, 5, SHUF, float>
+      <<<dim3(blocks, parts), WAVES * 64, lds, stream>>>(X, ldx, W, Y, N, M, N, K, ex);
+}
+
 // MT from M; the wavefronts per block are given per MT so that the LDS for the partial tiles,
 // (WAVES - 1) * R * MT KB, stays within 64 KB
 #define GS_BY_MT4(R, W1, W2, W3, W4, PRO, EPI, TOut, blocks)                                                            \
@@ -595,6 +615,18 @@ static void skinny_residual(const SkinnyCall& c) {
   const int blocks = gs_ceil_div(N, SHUF == 2 ? 8 : 16);
   if (SHUF == 2) { GS_BY_MT(1, 8, 0, 2, float, blocks) }
   else if (K >= 4096) { GS_BY_MT(1, 16, 0, 2, float, blocks) } else { GS_BY_MT(1, 8, 0, 2, float, blocks) }
+}
+
+// Partial sums over `parts` parts of K into Y (parts, M, N) float32: two weight tiles a block, four wavefronts.
+template <int SHUF>
+static void skinny_parts(const SkinnyCall& c, int parts) {
+  const int blocks = gs_ceil_div(c.N, 32);
+  switch ((c.M + 15) / 16) {
+    case 1: launch_skinny_parts<2, 1, 4, SHUF>(blocks, parts, c.x, c.ldx, c.w, (float*)c.Y, c.M, c.N, c.K, c.ex, c.stream); break;
+    case 2: launch_skinny_parts<2, 2, 4, SHUF>(blocks, parts, c.x, c.ldx, c.w, (float*)c.Y, c.M, c.N, c.K, c.ex, c.stream); break;
+    case 3: launch_skinny_parts<2, 3, 4, SHUF>(blocks, parts, c.x, c.ldx, c.w, (float*)c.Y, c.M, c.N, c.K, c.ex, c.stream); break;
+    default: launch_skinny_parts<2, 4, 4, SHUF>(blocks, parts, c.x, c.ldx, c.w, (float*)c.Y, c.M, c.N, c.K, c.ex, c.stream); break;
+  }
 }
 
 template <int SHUF>

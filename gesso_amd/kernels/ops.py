@@ -305,10 +305,11 @@ class LazyNorm:
     row's inverse root mean square, and the norm costs nothing of its own.
     """
 
-    __slots__ = ("res", "ssq", "weight", "eps", "dtype", "xs")
+    __slots__ = ("res", "ssq", "weight", "eps", "dtype", "xs", "ready")
 
-    def __init__(self, res, ssq, weight, eps, dtype, xs=None):
+    def __init__(self, res, ssq, weight, eps, dtype, xs=None, ready=None):
         self.res, self.ssq, self.weight, self.eps, self.dtype, self.xs = res, ssq, weight, eps, dtype, xs
+        self.ready = ready            # the normed rows themselves, where whatever wrote the stream last made them
 
     @property
     def shape(self):
@@ -316,6 +317,8 @@ class LazyNorm:
 
     def materialize(self) -> torch.Tensor:
         """The normed rows as a tensor; the sums of squares are at hand, so one light pass does it."""
+        if self.ready is not None:
+            return self.ready
         T, H = self.res.shape
         out = torch.empty((T, H), dtype=self.dtype, device=self.res.device)
         _check(lib().gs_norm_from_ssq(_p(self.res), _p(self.ssq), c_int(self.ssq.shape[1]), _p(self.weight),
@@ -390,6 +393,32 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt
     _check(lib().gs_gemm_skinny_residual(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(wt), _p(res), _p(ssq),
                                          _p(next_weight), _p(xs), c_int(M), c_int(N), c_int(K), _stream()))
     return ssq
+
+
+def gemm_skinny_residual_parts(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, parts: int, wt=None,
+                               next_weight=None, eps: float = 0.0, out_dtype=None):
+    """``res += x @ w.T`` for up to 64 rows in two kernels: partial sums over ``parts`` parts of K from many blocks,
+    then one pass that adds them to the stream.  Returns ``(ssq (M, 1), normed)``: the new rows' sums of squares and,
+    with ``next_weight``, the rows normed with that weight and ``eps`` (else None)."""
+    _dev(w, res, next_weight)
+    _need(skinny_ok(x, w), "gemm_skinny_residual_parts: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape == (N, K) and res.shape == (M, N) and res.dtype == torch.float32 and res.is_contiguous(),
+          "gemm_skinny_residual_parts: shapes")
+    _need(1 <= parts <= 64, "gemm_skinny_residual_parts: 1 to 64 parts")
+    part = torch.empty((parts, M, N), dtype=torch.float32, device=res.device)
+    _check(lib().gs_gemm_skinny_parts(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(wt), _p(part), c_int(parts),
+                                      c_int(M), c_int(N), c_int(K), _stream()))
+    ssq = torch.empty((M, 1), dtype=torch.float32, device=res.device)
+    normed = None
+    if next_weight is not None:
+        _need(next_weight.dtype == torch.float32 and next_weight.shape == (N,), "next_weight must be float32 (N,)")
+        normed = torch.empty((M, N), dtype=out_dtype or torch.bfloat16, device=res.device)
+    _check(lib().gs_residual_from_parts(_p(part), c_int(parts), _p(res), _p(ssq), _p(next_weight), c_float(eps),
+                                        _p(normed), c_int(_dt(normed) if normed is not None else 1), c_int(M), c_int(N),
+                                        _stream()))
+    return ssq, normed
 
 
 def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None) -> torch.Tensor:

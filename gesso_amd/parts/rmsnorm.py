@@ -24,7 +24,7 @@ class ResidualStream:
     in bfloat16, and the norm's consumer needs no norm pass at all.  ``xs_for`` is the norm ``xs`` was made for.
     """
 
-    __slots__ = ("res", "pending", "ssq", "xs", "xs_for", "following")
+    __slots__ = ("res", "pending", "ssq", "xs", "xs_for", "following", "normed")
 
     def __init__(self, res, pending=None, ssq=None, xs=None, xs_for=None):
         self.res = res
@@ -32,12 +32,24 @@ class ResidualStream:
         self.ssq = ssq
         self.xs, self.xs_for = xs, xs_for
         self.following = None
+        self.normed = None            # the rows normed for ``xs_for``, where the last push made them
 
     def push(self, out, rt, next_norm=None) -> None:
         from .runtime import DeferredLinear
         self.flush(rt)
-        self.xs = self.xs_for = None
-        if isinstance(out, DeferredLinear):
+        self.xs = self.xs_for = self.normed = None
+        if isinstance(out, DeferredLinear) and self.res.shape[0] > rt.weighted_rows_max:
+            # many rows: K is shared out over many blocks, and the pass that adds their partial sums to the stream
+            # norms the rows for the next norm on its way (it sees whole rows)
+            w = getattr(next_norm, "row_weight", None)
+            eps = getattr(getattr(next_norm, "spec", None), "eps", None)
+            if w is not None and (w.shape != (self.res.shape[1],) or eps is None):
+                w = None
+            eps = eps if w is not None else 0.0
+            self.ssq, self.normed = rt.ops.gemm_skinny_residual_parts(
+                out.x, out.w, self.res, rt.split_parts(out.w), wt=rt._wt(out.w), next_weight=w, eps=eps, out_dtype=rt.dtype)
+            self.xs_for = next_norm if self.normed is not None else None
+        elif isinstance(out, DeferredLinear):
             w = row_weight_of(next_norm, self.res, rt)
             if w is not None:
                 self.xs = torch.empty(self.res.shape, dtype=torch.bfloat16, device=self.res.device)
@@ -51,7 +63,7 @@ class ResidualStream:
         if self.pending is not None:
             rt.ops.residual_add(self.res, self.pending)
             self.pending, self.ssq = None, None
-            self.xs = self.xs_for = None
+            self.xs = self.xs_for = self.normed = None
 
 
 def row_weight_of(norm, res, rt):
@@ -85,8 +97,9 @@ class RMSNorm(Part):
         follows, which norms on the fly.
         """
         if self.rt.fused and rows is None and stream.pending is None and stream.ssq is not None:
-            xs = stream.xs if stream.xs_for is self else None
-            return self.rt.ops.LazyNorm(stream.res, stream.ssq, self.weight, self.spec.eps, self.rt.dtype, xs=xs)
+            mine = stream.xs_for is self
+            return self.rt.ops.LazyNorm(stream.res, stream.ssq, self.weight, self.spec.eps, self.rt.dtype,
+                                        xs=stream.xs if mine else None, ready=stream.normed if mine else None)
         y = self.rt.ops.add_rmsnorm(stream.res, stream.pending, self.weight, self.spec.eps, self.rt.dtype,
                                     rows=rows, out=out)
         if rows is None:

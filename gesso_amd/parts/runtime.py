@@ -112,6 +112,12 @@ class Runtime:
 
     # ------------------------------------------------------------------ mixers' inner steps
 
+    def split_parts(self, w) -> int:
+        """Into how many parts a deferred product of many rows shares K out: enough blocks to fill the chip
+        (a block takes 32 weight rows), each part at least 256 wide."""
+        blocks = max(1, w.shape[0] // 32)
+        return max(1, min(16, 512 // blocks, w.shape[1] // 256))
+
     def _keep_lazy(self, x) -> bool:
         """Whether a lazy norm goes to the product as it is: always when its rows come pre-weighted (the product
         only scales its result), else for few rows (the fold repeats the norm's arithmetic in every block)."""

@@ -550,6 +550,27 @@ def test_gemm_skinny_residual_leaves_rows_weighted_for_the_next_norm(ops, M, N, 
         close(ops.gemm_skinny(lazy, w2.to(DEV), swiglu=True), P.swiglu(ref[:, :N2 // 2], ref[:, N2 // 2:]), torch.bfloat16, scale=2)
 
 
+@pytest.mark.parametrize("M,N,K,parts", [(64, 2048, 8192, 8), (40, 96, 320, 3), (33, 144, 104, 1), (17, 2048, 2048, 16),
+                                          (5, 100, 64, 4)])
+def test_gemm_skinny_residual_in_parts(ops, M, N, K, parts):
+    g = gen(M + N + K + parts)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    res = torch.randn(M, N, generator=g)
+    nw = 1 + 0.3 * torch.randn(N, generator=g)
+    r = res.clone().to(DEV)
+    wt = ops.tile_major(w.to(DEV)) if N % 16 == 0 and K % 32 == 0 else None
+    ssq, normed = ops.gemm_skinny_residual_parts(x.to(DEV), w.to(DEV), r, parts, wt=wt, next_weight=nw.to(DEV), eps=1e-5)
+    want = res.double() + (x.double() @ w.double().T)
+    close(r, want, torch.bfloat16)                       # the product is rounded to bfloat16 before the add
+    assert torch.allclose(ssq.double().cpu()[:, 0], (r.double().cpu() ** 2).sum(1), rtol=1e-5)
+    close(normed, P.rmsnorm(r.double().cpu(), nw.double(), 1e-5), torch.bfloat16)
+    # and without a norm to prepare for
+    r2 = res.clone().to(DEV)
+    ssq2, none = ops.gemm_skinny_residual_parts(x.to(DEV), w.to(DEV), r2, parts, wt=wt)
+    assert none is None and torch.equal(r2, r) and torch.equal(ssq2, ssq)
+
+
 @pytest.mark.parametrize("T,H,V", [(1, 2048, 1000), (9, 104, 301)])
 def test_embed_leaves_rows_weighted_for_the_first_norm(ops, T, H, V):
     g = gen(T + H)
