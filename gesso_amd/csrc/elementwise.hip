@@ -107,12 +107,24 @@ __global__ void residual_from_parts_kernel(const float* __restrict__ part, int p
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (j < N) {
       float d[4] = {0.f, 0.f, 0.f, 0.f};
-      for (int p = 0; p < parts; ++p) {
-        const float* src = part + ((size_t)p * M + m) * N + j;
-        if (vec) {
-          const float4 a = *reinterpret_cast<const float4*>(src);
-          d[0] += a.x; d[1] += a.y; d[2] += a.z; d[3] += a.w;
-        } else {
+      if (vec) {
+        // eight parts' loads are issued together, then added in the order of the parts
+        for (int p0 = 0; p0 < parts; p0 += 8) {
+          float4 a[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const int p = p0 + q < parts ? p0 + q : parts - 1;
+            a[q] = *reinterpret_cast<const float4*>(part + ((size_t)p * M + m) * N + j);
+          }
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+            if (p0 + q < parts) {
+              d[0] += a[q].x; d[1] += a[q].y; d[2] += a[q].z; d[3] += a[q].w;
+            }
+        }
+      } else {
+        for (int p = 0; p < parts; ++p) {
+          const float* src = part + ((size_t)p * M + m) * N + j;
           for (int i = 0; i < 4; ++i)
             if (j + i < N) d[i] += src[i];
         }
@@ -153,10 +165,11 @@ extern "C" int gs_residual_from_parts(const float* part, int parts, float* res, 
   GS_REQUIRE((next_w == nullptr) == (normed == nullptr), "residual_from_parts: the next norm's weight and the room for the normed rows come together");
   GS_REQUIRE(((uintptr_t)part & 15) == 0, "residual_from_parts: the partial sums must be 16-byte aligned");
   if (M == 0) return 0;
+  const int threads = N >= 4096 ? 1024 : (N >= 2048 ? 512 : 256);   // four values a thread and turn
   if (!normed || normed_dtype == GS_BF16)
-    residual_from_parts_kernel<bf16><<<M, 256, 0, stream>>>(part, parts, res, ssq, next_w, eps, (bf16*)normed, M, N);
+    residual_from_parts_kernel<bf16><<<M, threads, 0, stream>>>(part, parts, res, ssq, next_w, eps, (bf16*)normed, M, N);
   else if (normed_dtype == GS_F32)
-    residual_from_parts_kernel<float><<<M, 256, 0, stream>>>(part, parts, res, ssq, next_w, eps, (float*)normed, M, N);
+    residual_from_parts_kernel<float><<<M, threads, 0, stream>>>(part, parts, res, ssq, next_w, eps, (float*)normed, M, N);
   else
     GS_REQUIRE(false, "residual_from_parts: unknown dtype %d", normed_dtype);
   GS_LAUNCH_CHECK("residual_from_parts");

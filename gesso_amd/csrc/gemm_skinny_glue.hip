@@ -52,7 +52,8 @@ void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* s
   SkinnyCall c = base(X, ldx, W, Wt, Y, GS_BF16, H, M, 3 * H, K, 3, stream);
   if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.taps = taps; c.ex.conv_bias = conv_bias; c.ex.state = state; c.ex.slots = slots; c.ex.conv_w = conv_w;
-  if (Wt && gs_skinny_halves(c.N / 3)) gs_skinny_conv_half_tiles(c);   // c.N / 3 channels, as few as a narrow weight's rows
+  // c.N / 3 channels, as few as a narrow weight's rows; with many rows of X the blocks' reading of X outweighs that
+  if (Wt && gs_skinny_halves(c.N / 3) && M <= 32) gs_skinny_conv_half_tiles(c);
   else Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);
 }
 

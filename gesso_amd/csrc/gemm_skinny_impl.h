@@ -590,7 +590,11 @@ static void skinny_plain(const SkinnyCall& c) {
   const int cols = c.epilogue == 1 ? N / 2 : N;
   const bool narrow = cols <= 8192;
   // few output columns: more wavefronts per block split K further, so that the whole chip streams
-  if (c.epilogue == 1) {
+  if (c.epilogue == 1 && M > 32 && !pro && cols % 32 == 0 && cols >= 8192) {
+    // many rows: a block that takes four weight tiles reads X half as often per weight byte
+    const int blocks = cols / 32;
+    if (f32) { GS_BY_MT4(4, 4, 4, 4, 4, 0, 1, float, blocks) } else { GS_BY_MT4(4, 4, 4, 4, 4, 0, 1, bf16, blocks) }
+  } else if (c.epilogue == 1) {
     const int blocks = gs_ceil_div(cols, 16);
     if (pro) { if (f32) { GS_BY_MT4(2, 8, 8, 4, 4, 1, 1, float, blocks) } else { GS_BY_MT4(2, 8, 8, 4, 4, 1, 1, bf16, blocks) } }
     else     { if (f32) { GS_BY_MT4(2, 8, 8, 4, 4, 0, 1, float, blocks) } else { GS_BY_MT4(2, 8, 8, 4, 4, 0, 1, bf16, blocks) } }
