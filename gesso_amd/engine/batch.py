@@ -105,18 +105,27 @@ class StepContext:
     def cache_view(self, call: int):
         return self._storage.view(call, self.block_tables)
 
-    def query_tiles(self, rows: int = 16) -> torch.Tensor:
+    @property
+    def lead_single(self) -> int:
+        """How many sequences at the batch's head bring one token each (decoded tokens come before prompt portions)."""
+        n = 0
+        while n < len(self.q_lens) and self.q_lens[n] == 1:
+            n += 1
+        return n
+
+    def query_tiles(self, rows: int = 16, skip: int = 0) -> torch.Tensor:
         """int32 ``(3, ntiles)``: sequence, first row, row count of each tile of at most ``rows`` consecutive
-        queries of one sequence; made once per step, on first use."""
-        if self._tiles is None or self._tiles[0] != rows:
+        queries of one sequence, for the sequences from ``skip`` on; made once per step, on first use."""
+        if self._tiles is None or self._tiles[0] != (rows, skip):
             seq, row, cnt = [], [], []
             at = 0
             for i, n in enumerate(self.q_lens):
-                for a in range(0, n, rows):
-                    seq.append(i)
-                    row.append(at + a)
-                    cnt.append(min(rows, n - a))
+                if i >= skip:
+                    for a in range(0, n, rows):
+                        seq.append(i)
+                        row.append(at + a)
+                        cnt.append(min(rows, n - a))
                 at += n
             t = torch.tensor([seq, row, cnt], dtype=torch.int32).pin_memory().to(self.token_ids.device, non_blocking=True)
-            self._tiles = (rows, t)
+            self._tiles = ((rows, skip), t)
         return self._tiles[1]

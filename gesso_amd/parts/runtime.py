@@ -160,6 +160,18 @@ class Runtime:
                            nh, nkv, d, write_kv=cache.write)
         return qkv, (nh + 2 * nkv) * d
 
+    def _attention_single(self, q, q_stride, cache, ctx, window, scale, nh, nkv, d, nseq, out):
+        """The first ``nseq`` sequences, one query each (their rows are the first ``nseq`` rows).  A block of eight
+        wavefronts takes a tile of 64 keys per wavefront and pass; up to two passes stay in one block (no merge
+        kernel), longer key streams are split over blocks."""
+        longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
+        if window:
+            longest = min(longest, window)
+        tiles = max(1, -(-longest // 64))
+        nsplit = max(1, min(-(-tiles // 16), 64, max(1, 2048 // max(1, nseq * nkv))))
+        return self.ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
+                                         cache.page_size, window, scale, nh, nkv, d, nseq, nsplit, out=out)
+
     def attention(self, q, q_stride, cache, ctx, window, scale, nh, nkv, d) -> torch.Tensor:
         """Causal attention of this step's queries over the paged cache; ``(T, nh * d)``.
 
@@ -167,25 +179,24 @@ class Runtime:
         shapes they are written for.
         """
         ops = self.ops
-        if (ctx.all_single and q.dtype == torch.bfloat16 and cache.page_size >= 2
-                and ops.attention_decode_supports(nh, nkv, d)):
-            # one query per sequence.  A block of eight wavefronts takes a tile of 64 keys per wavefront and pass;
-            # up to two passes stay in one block (no merge kernel), longer key streams are split over blocks
-            longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
-            if window:
-                longest = min(longest, window)
-            tiles = max(1, -(-longest // 64))
-            nsplit = max(1, min(-(-tiles // 16), 64, max(1, 2048 // max(1, ctx.nseq * nkv))))
-            return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
-                                        cache.page_size, window, scale, nh, nkv, d, ctx.nseq, nsplit)
-        if (not ctx.all_single and q.dtype == torch.bfloat16 and q_stride % 8 == 0 and cache.page_size >= 2
-                and ops.attention_prefill_supports(nh, nkv, d)):
+        fast = q.dtype == torch.bfloat16 and cache.page_size >= 2
+        if ctx.all_single and fast and ops.attention_decode_supports(nh, nkv, d):
+            return self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, ctx.nseq, None)
+        if (not ctx.all_single and fast and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d)):
             # prompts: queries in tiles per sequence, both products on the matrix cores; tiles of 32 share
             # every key and value fragment between two products, which pays when portions are long
             # (groups of more than four heads have no registers for tiles of 32)
             rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16
-            return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows),
+            # decoded tokens at the batch's head go to the kernel for single queries: as tiles of one query they
+            # would each hold a whole block that walks all the keys alone
+            lead = getattr(ctx, "lead_single", 0)
+            if not ops.attention_decode_supports(nh, nkv, d):
+                lead = 0
+            out = torch.empty((ctx.T, nh * d), dtype=q.dtype, device=q.device)
+            if lead:
+                self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, lead, out[:lead])
+            return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows, lead),
                                          cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T,
-                                         tile_rows=rows)
+                                         out=out, tile_rows=rows)
         return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
                                      cache.block_table, cache.page_size, window, scale, nh, nkv, d, ctx.T)
