@@ -269,28 +269,31 @@ def test_recorded_decode_loop_equals_single_steps(folders, name, dtype):
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_recorded_decode_logits_follow_the_plain_model(folders, name):
-    """The fused kernels of the recorded step, row by row against the plain implementation (bfloat16)."""
+@pytest.mark.parametrize("nreq,steps", [(3, 20), (20, 4), (40, 4)])
+def test_recorded_decode_logits_follow_the_plain_model(folders, name, nreq, steps):
+    """The fused kernels of the recorded step, row by row against the plain implementation (bfloat16): few rows
+    (rows pre-weighted for the next norm), more than sixteen, and more than thirty-two (products in parts of K)."""
     from gesso_amd import Engine, StepEntry
+    from gesso_amd.engine.decode import _capacity
     d = write_tiny(folders, name, torch.bfloat16)
     cfg, w = P.read_config(d), P.read_weights(d)
-    prompts = [random_ids(n, cfg["V"], 700 + n) for n in (3, 18, 40)]
-    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=512)
+    prompts = [random_ids(n, cfg["V"], 700 + n) for n in ([3, 18, 40] + [5 + (7 * i) % 23 for i in range(nreq)])[:nreq]]
+    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=64 * nreq + 256, num_slots=nreq + 1)
     seqs, toks = [list(p) for p in prompts], []
     for i, p in enumerate(prompts):
         eng.add_request(i)
         toks.append(int(eng.step([StepEntry(i, p, [len(p) - 1])]).argmax()))
     worst = 0.0
-    for step in range(20):
+    for step in range(steps):
         for s, t in zip(seqs, toks):
             s.append(t)
-        ids, bad = eng.decode([0, 1, 2], toks, 1)
+        ids, bad = eng.decode(list(range(nreq)), toks, 1)
         assert not bad.any()
-        logits = eng._runners[4].logits[:3].double().cpu()
+        logits = eng._runners[_capacity(nreq)].logits[:nreq].double().cpu()
         for i, s in enumerate(seqs):
             ref = P.forward(cfg, w, s)[-1]
             scale = max(1.0, float(ref.abs().max()))
             worst = max(worst, float((logits[i] - ref).abs().max()) / scale)
         toks = ids[0].tolist()
-    print(f"{name}: worst relative difference of the recorded step's logits {worst:.3e}")
+    print(f"{name}, {nreq} requests: worst relative difference of the recorded step's logits {worst:.3e}")
     assert worst <= 1.5e-2
