@@ -262,25 +262,48 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
   }
 }
 
-// Merge the splits of each (sequence, head), in split order.  One block per (sequence, key head).
+// Merge the splits of each (sequence, head), in split order.  One block per (sequence, key head).  The splits'
+// maxima and sums go through LDS, so that each head's weights are computed once and the loads of the partial
+// outputs are independent of one another.
+#define DEC_MAXSPLIT 64
 __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                               bf16* __restrict__ out, int nsplit, int nh, int nkv, int G, int D) {
+  __shared__ float sm[DEC_MAXSPLIT][DEC_MAXG], sl[DEC_MAXSPLIT][DEC_MAXG], sf[DEC_MAXSPLIT][DEC_MAXG];
+  __shared__ float sinv[DEC_MAXG];
   const int kvh = blockIdx.x, seq = blockIdx.y;
   const size_t base = ((size_t)seq * nkv + kvh) * nsplit;
-  for (int i = threadIdx.x; i < G * D; i += blockDim.x) {
-    int g = i / D, j = i - g * D;
+  for (int i = threadIdx.x; i < nsplit * G; i += blockDim.x) {
+    const int sp = i / G, g = i - sp * G;
+    sm[sp][g] = part_ml[((base + sp) * G + g) * 2];
+    sl[sp][g] = part_ml[((base + sp) * G + g) * 2 + 1];
+  }
+  __syncthreads();
+  if (threadIdx.x < G) {
+    const int g = threadIdx.x;
     float M = -INFINITY;
-    for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, part_ml[((base + sp) * G + g) * 2]);
-    float o = 0.f, L = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) M = fmaxf(M, sm[sp][g]);
+    float L = 0.f;
     for (int sp = 0; sp < nsplit; ++sp) {
-      float ms = part_ml[((base + sp) * G + g) * 2];
-      if (ms > -INFINITY) {
-        float f = __builtin_amdgcn_exp2f(ms - M);   // maxima are in base-2 units
-        o += part_o[((base + sp) * G + g) * D + j] * f;
-        L += part_ml[((base + sp) * G + g) * 2 + 1] * f;
-      }
+      const float f = sm[sp][g] > -INFINITY ? __builtin_amdgcn_exp2f(sm[sp][g] - M) : 0.f;   // maxima are in base-2 units
+      sf[sp][g] = f;
+      L += sl[sp][g] * f;
     }
-    out[((size_t)seq * nh + kvh * G + g) * D + j] = f32_to_bf16(o / L);
+    sinv[g] = 1.0f / L;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < G * D; i += blockDim.x) {
+    const int g = i / D, j = i - g * D;
+    float o = 0.f;
+    int sp = 0;
+    for (; sp + 8 <= nsplit; sp += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = part_o[((base + sp + u) * G + g) * D + j];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) o += v[u] * sf[sp + u][g];
+    }
+    for (; sp < nsplit; ++sp) o += part_o[((base + sp) * G + g) * D + j] * sf[sp][g];
+    out[((size_t)seq * nh + kvh * G + g) * D + j] = f32_to_bf16(o * sinv[g]);
   }
 }
 
