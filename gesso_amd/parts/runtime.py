@@ -49,6 +49,10 @@ class Runtime:
         # then only scales its result; for more rows every block's reading of the partial sums costs more than
         # one light norm pass
         self.weighted_rows_max = int(os.environ.get("GESSO_WEIGHTED_ROWS_MAX", "32"))
+        # q|k|v with head norm, rotation and cache write as the product's epilogue needs a whole head in one block:
+        # 48 blocks for LFM2-1.2B, and a block streams weights no faster than about 45 GB/s.  The plain product over
+        # the whole chip plus the small kernel for norm, rotation and cache write measured half a percent faster.
+        self.fuse_qkv = os.environ.get("GESSO_FUSE_QKV", "0") != "0"
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""
@@ -145,7 +149,7 @@ class Runtime:
         """q, k, v products, head norms, position encoding, cache write.  Returns ``(q, q_stride)``:
         the queries as rows of a buffer, ``q_stride`` apart, head h at ``[h d, (h+1) d)``."""
         ops = self.ops
-        if (self.fused and bqkv is None and ctx.all_single and cache.k.dtype == torch.bfloat16
+        if (self.fused and self.fuse_qkv and bqkv is None and ctx.all_single and cache.k.dtype == torch.bfloat16
                 and ops.gemm_skinny_qkv_supports(d, position.rotary_dim)):
             x = self._rows(x)
             if ops.lazy_ok(x, wqkv) or (not isinstance(x, ops.LazyNorm) and ops.skinny_ok(x, wqkv)):
@@ -153,8 +157,7 @@ class Runtime:
                                         cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
                                         write_kv=cache.write, wt=self._wt(wqkv))
                 return q, nh * d
-        x = self._dense(x)
-        qkv = self.linear(x, wqkv, bqkv)
+        qkv = self.linear(x, wqkv, bqkv)          # a lazy norm goes through as it is where the product takes it
         ops.qknorm_rope_kv(qkv, q_norm, k_norm, head_eps, position.cos, position.sin, position.rotary_dim,
                            ctx.positions, ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v,
                            nh, nkv, d, write_kv=cache.write)
