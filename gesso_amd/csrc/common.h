@@ -13,6 +13,9 @@
 
 #define GS_WAVE 64
 
+// The float32 products add k in chunks of this many, and then the chunks' sums, both in ascending order.
+#define GS_SUM_CHUNK 64
+
 extern "C" const char* gs_last_error();
 void gs_set_error(const char* fmt, ...);
 

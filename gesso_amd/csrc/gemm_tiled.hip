@@ -2,9 +2,10 @@
 //
 // Every size is taken (bounds are checked per element), every mix of float32 and bfloat16
 // storage for X, W and Y.  Products and sums are float32 FMAs: with float32 storage this is the
-// true 32-bit path (no matrix-core input rounding).  Each output element sums over k in
-// ascending order, in one accumulator, so its value does not depend on M or on which rows share
-// the launch.
+// true 32-bit path (no matrix-core input rounding).  Each output element is summed in one fixed order,
+// so its value does not depend on M or on which rows share the launch: k in chunks of 64, each chunk
+// from zero in ascending k, the chunks' sums added in ascending order.  (The streaming kernel for few
+// rows, gemv_f32.hip, adds in the same order; a chunk is what one of its lanes takes.)
 //
 // 64 x 64 tile per block of 256 threads, 4 x 4 outputs per thread, k in steps of 16 through LDS.
 #include "common.h"
@@ -12,6 +13,7 @@
 #define TM 64
 #define TN 64
 #define TK 16
+static_assert(GS_SUM_CHUNK % TK == 0 && ((GS_SUM_CHUNK / TK) & (GS_SUM_CHUNK / TK - 1)) == 0, "chunks are whole k steps");
 
 template <typename TX, typename TW, typename TY>
 __global__ void gemm_tiled_kernel(const TX* __restrict__ X, int ldx, const TW* __restrict__ W,
@@ -21,11 +23,11 @@ __global__ void gemm_tiled_kernel(const TX* __restrict__ X, int ldx, const TW* _
   int tid = threadIdx.x;
   int tx = tid & 15, ty = tid >> 4;  // tx: columns (n), ty: rows (m)
   int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
-  float acc[4][4];
+  float acc[4][4], tot[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j] = 0.f;
 
   for (int k0 = 0; k0 < K; k0 += TK) {
     // 64 rows x 16 k = 1024 elements per operand, 4 per thread
@@ -51,6 +53,15 @@ __global__ void gemm_tiled_kernel(const TX* __restrict__ X, int ldx, const TW* _
         for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
     }
     __syncthreads();
+    if (((k0 / TK) & (GS_SUM_CHUNK / TK - 1)) == GS_SUM_CHUNK / TK - 1 || k0 + TK >= K) {   // a chunk is complete
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          tot[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -60,7 +71,7 @@ __global__ void gemm_tiled_kernel(const TX* __restrict__ X, int ldx, const TW* _
     for (int j = 0; j < 4; ++j) {
       int n = n0 + tx * 4 + j;
       if (n >= N) continue;
-      float v = acc[i][j];
+      float v = tot[i][j];
       if (bias) v += bias[n];
       Y[(size_t)m * ldy + n] = from_f32<TY>(v);
     }

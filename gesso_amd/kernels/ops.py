@@ -236,6 +236,13 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, bias=None, out_dtype=None, out:
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype or x.dtype, device=x.device)
     _need(out.shape == (M, N) and out.stride(1) == 1, "gemm: out has the wrong shape")
+    ldx = x.stride(0) if M > 1 else K
+    if (x.dtype == torch.float32 and w.dtype == torch.float32 and w.is_contiguous()
+            and lib().gs_gemv_f32_supports(c_int(M), c_int(K), c_int(ldx), _p(x), _p(w))):
+        # few rows: the weights are streamed once, each output summed in an order that depends on K alone
+        _check(lib().gs_gemv_f32(_p(x), c_int(ldx), _p(w), _p(bias), _p(out), c_int(_dt(out)),
+                                 c_int(out.stride(0) if M > 1 else N), c_int(M), c_int(N), c_int(K), _stream()))
+        return out
     _check(lib().gs_gemm_tiled(_p(x), c_int(_dt(x)), c_int(x.stride(0) if M > 1 else K), _p(w), c_int(_dt(w)),
                                _p(bias), _p(out), c_int(_dt(out)), c_int(out.stride(0) if M > 1 else N), c_int(M),
                                c_int(N), c_int(K), _stream()))

@@ -324,6 +324,20 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
     assert torch.equal(ops.gemm_tiled(wide[:, 50:150], w), ops.gemm_tiled(wide[:, 50:150].contiguous(), w))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 301, 8192), (16, 96, 100), (5, 7, 64), (3, 130, 4)])
+def test_float32_product_of_few_rows_streams_the_weights_and_adds_in_the_same_order(ops, M, N, K):
+    g = gen(M * N + K)
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(N, K, generator=g)
+    b = torch.randn(N, generator=g)
+    got = ops.gemm_tiled(x.to(DEV), w.to(DEV), b.to(DEV))                    # few aligned rows: the streaming kernel
+    close(got, x.double() @ w.double().T + b.double(), torch.float32, scale=math.sqrt(K) / 4)
+    # the same rows inside a launch of many rows go through the tiled kernel: equal to the bit
+    many = torch.cat([x, torch.randn(40, K, generator=g)]).to(DEV)
+    assert torch.equal(ops.gemm_tiled(many, w.to(DEV), b.to(DEV))[:M], got)
+    close(ops.gemm_tiled(x.to(DEV), w.to(DEV), out_dtype=torch.bfloat16), x.double() @ w.double().T, torch.bfloat16)
+
+
 # ------------------------------------------------------------------ choosing tokens
 
 def test_argmax_rows(ops):
