@@ -353,7 +353,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       float ssum = 0.f;
       if (m == wave) ssum = (pre[0] + pre[1]) + (pre[2] + pre[3]);
       for (int b = (m == wave ? 256 : 0) + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
-      ssum = wave_sum(ssum);
+      ssum = wave_sum_dpp(ssum);
       if (lane == 0) inv_s[m] = 1.0f / sqrtf(ssum / (float)K + ex.eps);
     }
     if (WAVES == 1) __syncthreads();
