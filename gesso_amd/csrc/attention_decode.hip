@@ -32,12 +32,27 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int D, int G, int W>
+// With RAW, q points at rows of q|k|v as their product left them (q heads, then k heads, then v heads), and the
+// kernel does what comes between that product and attention itself: the head norms of q and k, the rotation, and
+// the write of the new key and value into their page.  Every block norms and rotates its own queries; the block
+// whose keys end with the new one norms and rotates it, keeps it and the value in LDS for its scores, and writes
+// both to the cache for the steps to come.  Heads of 64 or 128, rotated whole.
+struct DecodeRaw {
+  const float* qw;       // (D) head norm weights, or null for no norm
+  const float* kw;
+  float eps;
+  const float* cos_t;    // (positions, D / 2)
+  const float* sin_t;
+  int write_kv;          // 0: another layer owns the cache; the new key is already in it
+};
+
+template <int D, int G, int W, int RAW>
 __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
-    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
+    const bf16* __restrict__ q, int q_stride, bf16* kcache, bf16* vcache,
     const int* __restrict__ positions, const int* __restrict__ block_table, int max_blocks, int page_size,
     unsigned page_magic, int window, float scale, bf16* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int nh, int nkv) {
+    float* __restrict__ part_ml, int nh, int nkv, DecodeRaw raw) {
+  static_assert(!RAW || D == 64 || D == 128, "the fused head norm and rotation are written for heads of 64 and 128");
   constexpr int DC = D / 8;               // 16-byte chunks per row
   constexpr int KG = 64 / DC;             // key groups per wavefront in the value phase
   constexpr int NI = 64 / KG;             // keys per lane in the value phase
@@ -115,6 +130,89 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
     else
       qreg[st] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
   }
+  __shared__ __align__(16) uint16_t knew[RAW ? D : 8], vnew[RAW ? D : 8];
+  const bool has_new = RAW && raw.write_kv && t0 < t1 && t1 == tiles;   // this block's keys end with the new one
+  if constexpr (RAW != 0) {
+    // head norm and rotation of this lane's part of its query: float32 arithmetic on the product's bfloat16
+    // values, rounded to bfloat16 again, as the separate kernel does.  The halves of a rotation pair (i, i + D/2)
+    // are steps KS/2 apart in the same lane.
+    float qf[KS][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int st = 0; st < KS; ++st)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        qf[st][j] = (float)qreg[st][j];
+        ss += qf[st][j] * qf[st][j];
+      }
+    // (weights and rotation factors in 16-byte loads: the tables' rows and this lane's offsets are multiples of 8)
+    float c8[KS / 2][8], s8[KS / 2][8];
+#pragma unroll
+    for (int st = 0; st < KS / 2; ++st) {
+      load8f(raw.cos_t + (size_t)pos * (D / 2) + 32 * st + 8 * kg, c8[st]);
+      load8f(raw.sin_t + (size_t)pos * (D / 2) + 32 * st + 8 * kg, s8[st]);
+    }
+    if (raw.qw) {
+      const float inv = 1.0f / sqrtf(group4_sum(ss) / (float)D + raw.eps);
+#pragma unroll
+      for (int st = 0; st < KS; ++st) {
+        float w8[8];
+        load8f(raw.qw + 32 * st + 8 * kg, w8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[st][j] = qf[st][j] * inv * w8[j];
+      }
+    }
+#pragma unroll
+    for (int st = 0; st < KS / 2; ++st)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float a = qf[st][j], b = qf[st + KS / 2][j];
+        qf[st][j] = a * c8[st][j] - b * s8[st][j];
+        qf[st + KS / 2][j] = a * s8[st][j] + b * c8[st][j];
+      }
+#pragma unroll
+    for (int st = 0; st < KS; ++st)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qreg[st][j] = (r16 < G) ? (__bf16)qf[st][j] : (__bf16)0.f;
+    // the new key and value: wavefront 0, lane = feature (and feature + 64 for heads of 128)
+    if (has_new && wave == 0) {
+      constexpr int E = D >= 64 ? D / 64 : 1;
+      const bf16* kraw = q + (size_t)seq * q_stride + (size_t)(nh + kvh) * D;
+      const bf16* vraw = q + (size_t)seq * q_stride + (size_t)(nh + nkv + kvh) * D;
+      float kf[E];
+      float ks = 0.f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        kf[e] = to_f32(kraw[lane + 64 * e]);
+        ks += kf[e] * kf[e];
+      }
+      if (raw.kw) {
+        const float inv = 1.0f / sqrtf(wave_sum_dpp(ks) / (float)D + raw.eps);
+#pragma unroll
+        for (int e = 0; e < E; ++e) kf[e] = kf[e] * inv * raw.kw[lane + 64 * e];
+      }
+      const int i = E == 2 ? lane : (lane & 31);          // index of this lane's pair
+      const float c = raw.cos_t[(size_t)pos * (D / 2) + i], sn = raw.sin_t[(size_t)pos * (D / 2) + i];
+      if (E == 2) {
+        const float a = kf[0], b = kf[E - 1];
+        kf[0] = a * c - b * sn;
+        kf[E - 1] = a * sn + b * c;
+      } else {
+        const float other = __shfl_xor(kf[0], 32, 64);
+        kf[0] = lane < 32 ? kf[0] * c - other * sn : other * sn + kf[0] * c;
+      }
+      const long row = row_off(pos);
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const bf16 kb = f32_to_bf16(kf[e]), vb = vraw[lane + 64 * e];
+        knew[lane + 64 * e] = kb.x;
+        vnew[lane + 64 * e] = vb.x;
+        kcache[row + lane + 64 * e] = kb;
+        vcache[row + lane + 64 * e] = vb;
+      }
+    }
+    __syncthreads();
+  }
   const float qscale = scale * DEC_LOG2E;   // scores are scaled after the product, in float32
 
   // lanes r16 < G keep the running maximum and sum of head r16; every lane keeps its share of all heads' sums
@@ -126,8 +224,21 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
     for (int j = 0; j < 8; ++j) acc[g][j] = 0.f;
 
   // one tile: scores, online softmax, values
-  auto compute = [&](int t, bf16x8_t (*kc)[KS], const uint4* vc) {
+  auto compute = [&](int t, bf16x8_t (*kc)[KS], uint4* vc) {
     const int base = lo + (t << 6);
+    if (RAW && has_new && t == tiles - 1) {
+      // the new key's row and the new value's row come from LDS: the cache's rows were loaded before they were written
+      const int rel = pos - base;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+        if (4 * r16 + kt == rel) {
+#pragma unroll
+          for (int st = 0; st < KS; ++st) kc[kt][st] = *reinterpret_cast<const bf16x8_t*>(&knew[32 * st + 8 * kg]);
+        }
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        if (kq + i * KG == rel) vc[i] = *reinterpret_cast<const uint4*>(&vnew[dc * 8]);
+    }
     // sc[kt][i]: head r16, key base + 4 (4 kg + i) + kt
     f32x4_t sc[4];
 #pragma unroll
@@ -309,15 +420,15 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
 
 #define DEC_WAVES 8
 
-template <int D>
-static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
-                         const bf16* vc, const int* positions, const int* bt, int max_blocks, int page_size,
-                         unsigned page_magic, int window, float scale, bf16* out, float* part_o, float* part_ml, int nh,
-                         int nkv) {
+template <int D, int RAW>
+static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, bf16* kc, bf16* vc,
+                         const int* positions, const int* bt, int max_blocks, int page_size, unsigned page_magic,
+                         int window, float scale, bf16* out, float* part_o, float* part_ml, int nh, int nkv,
+                         DecodeRaw raw) {
 #define GS_RUN(GG)                                                                                                     \
-  attention_decode_kernel<D, GG, DEC_WAVES><<<grid, DEC_WAVES * 64, 0, stream>>>(                                      \
+  attention_decode_kernel<D, GG, DEC_WAVES, RAW><<<grid, DEC_WAVES * 64, 0, stream>>>(                                 \
       q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_magic, window, scale, out, part_o, part_ml, nh, \
-      nkv)
+      nkv, raw)
   switch (G) {
     case 1: GS_RUN(1); break;
     case 2: GS_RUN(2); break;
@@ -345,15 +456,15 @@ extern "C" long gs_attention_decode_workspace(int nseq, int nh, int nkv, int d, 
   return (long)nseq * nh * nsplit * (d + 2);
 }
 
-extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcache, const void* vcache,
-                                   const int* positions, const int* block_table, int max_blocks, int page_size,
-                                   int window, float scale, void* out, float* workspace, int nseq, int nh, int nkv,
-                                   int d, int nsplit, hipStream_t stream) {
+static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache, const int* positions,
+                        const int* block_table, int max_blocks, int page_size, int window, float scale, void* out,
+                        float* workspace, int nseq, int nh, int nkv, int d, int nsplit, const DecodeRaw* raw,
+                        hipStream_t stream) {
   GS_REQUIRE(gs_attention_decode_supports(nh, nkv, d), "attention_decode: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
   GS_REQUIRE(nseq >= 0 && nseq <= 65535 && nkv <= 65535, "attention_decode: bad batch %d", nseq);
   GS_REQUIRE(nsplit >= 1 && nsplit <= 64, "attention_decode: %d splits outside [1, 64]", nsplit);
   GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_decode: bad page_size/max_blocks/window");
-  GS_REQUIRE(q_stride >= nh * d, "attention_decode: q_stride %d below nh*d", q_stride);
+  GS_REQUIRE(q_stride >= (raw ? nh + 2 * nkv : nh) * d, "attention_decode: q_stride %d below the row's width", q_stride);
   GS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_decode: query rows must be 16-byte aligned");
   GS_REQUIRE((d * (int)sizeof(bf16)) % 16 == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0,
              "attention_decode: cache rows must be 16-byte aligned");
@@ -366,17 +477,25 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
   float* part_o = workspace;
   float* part_ml = workspace + (size_t)nseq * nh * nsplit * d;
   int rc = -1;
-#define GS_ARGS                                                                                                   \
-  G, grid, stream, (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions,       \
-      block_table, max_blocks, page_size, page_magic, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
-  switch (d) {
-    case 16: rc = launch_decode<16>(GS_ARGS); break;
-    case 32: rc = launch_decode<32>(GS_ARGS); break;
-    case 64: rc = launch_decode<64>(GS_ARGS); break;
-    case 128: rc = launch_decode<128>(GS_ARGS); break;
+  const DecodeRaw none = {};
+#define GS_ARGS                                                                                             \
+  G, grid, stream, (const bf16*)q, q_stride, (bf16*)kcache, (bf16*)vcache, positions, block_table, max_blocks, \
+      page_size, page_magic, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
+  if (raw) {
+    switch (d) {
+      case 64: rc = launch_decode<64, 1>(GS_ARGS, *raw); break;
+      case 128: rc = launch_decode<128, 1>(GS_ARGS, *raw); break;
+    }
+  } else {
+    switch (d) {
+      case 16: rc = launch_decode<16, 0>(GS_ARGS, none); break;
+      case 32: rc = launch_decode<32, 0>(GS_ARGS, none); break;
+      case 64: rc = launch_decode<64, 0>(GS_ARGS, none); break;
+      case 128: rc = launch_decode<128, 0>(GS_ARGS, none); break;
+    }
   }
 #undef GS_ARGS
-  GS_REQUIRE(rc == 0, "attention_decode: no kernel for group %d", G);
+  GS_REQUIRE(rc == 0, "attention_decode: no kernel for group %d and head width %d", G, d);
   GS_LAUNCH_CHECK("attention_decode");
   if (nsplit > 1) {
     dim3 mgrid(nkv, nseq);
@@ -384,4 +503,32 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
     GS_LAUNCH_CHECK("attention_decode_merge");
   }
   return 0;
+}
+
+extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                   const int* positions, const int* block_table, int max_blocks, int page_size,
+                                   int window, float scale, void* out, float* workspace, int nseq, int nh, int nkv,
+                                   int d, int nsplit, hipStream_t stream) {
+  return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
+                      scale, out, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream);
+}
+
+// Whether the kernel also takes the head norms, the rotation and the cache write: heads of 64 or 128 rotated whole.
+extern "C" int gs_attention_decode_raw_supports(int nh, int nkv, int d, int rotary_dim) {
+  return gs_attention_decode_supports(nh, nkv, d) && (d == 64 || d == 128) && rotary_dim == d;
+}
+
+// qkv (nseq, q_stride): the rows of q|k|v as their product left them.  The kernel norms and rotates q and the new
+// key, writes the new key and value into their pages (unless write_kv is 0), and attends.
+extern "C" int gs_attention_decode_raw(const void* qkv, int q_stride, void* kcache, void* vcache, const int* positions,
+                                       const int* block_table, int max_blocks, int page_size, int window, float scale,
+                                       const float* qw, const float* kw, float eps, const float* cos_t,
+                                       const float* sin_t, int rotary_dim, int write_kv, void* out, float* workspace,
+                                       int nseq, int nh, int nkv, int d, int nsplit, hipStream_t stream) {
+  GS_REQUIRE(gs_attention_decode_raw_supports(nh, nkv, d, rotary_dim), "attention_decode_raw: sizes nh=%d nkv=%d d=%d rotary=%d are not taken", nh, nkv, d, rotary_dim);
+  GS_REQUIRE((qw == nullptr) == (kw == nullptr) && cos_t && sin_t, "attention_decode_raw: q and k norm weights come together; the rotation needs its tables");
+  GS_REQUIRE((((uintptr_t)qw | (uintptr_t)kw | (uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0, "attention_decode_raw: weights and tables must be 16-byte aligned");
+  DecodeRaw raw = {qw, kw, eps, cos_t, sin_t, write_kv};
+  return decode_entry(qkv, q_stride, kcache, vcache, positions, block_table, max_blocks, page_size, window, scale, out,
+                      workspace, nseq, nh, nkv, d, nsplit, &raw, stream);
 }

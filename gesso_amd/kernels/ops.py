@@ -498,6 +498,17 @@ def attention_decode_supports(nh: int, nkv: int, d: int) -> bool:
 _decode_ws = {}
 
 
+def _decode_workspace(device, nseq, nh, nkv, d, nsplit):
+    key = (device, nseq, nh, nkv, d, nsplit)
+    ws = _decode_ws.get(key)
+    if ws is None:
+        n = lib().gs_attention_decode_workspace
+        n.restype = c_long
+        floats = n(c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit))
+        ws = _decode_ws[key] = torch.empty(max(1, floats), dtype=torch.float32, device=device)
+    return ws
+
+
 def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_size, window, scale, nh, nkv, d, nseq,
                      nsplit: int, out: torch.Tensor = None) -> torch.Tensor:
     """One query per sequence over its paged keys (bfloat16), keys split over ``nsplit`` blocks per key head."""
@@ -510,13 +521,7 @@ def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_s
     _i32(positions, nseq, "positions")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= nseq,
           "block_table must be int32 (nseq, max_blocks)")
-    key = (q.device, nseq, nh, nkv, d, nsplit)
-    ws = _decode_ws.get(key)
-    if ws is None:
-        n = lib().gs_attention_decode_workspace
-        n.restype = c_long
-        floats = n(c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit))
-        ws = _decode_ws[key] = torch.empty(max(1, floats), dtype=torch.float32, device=q.device)
+    ws = _decode_workspace(q.device, nseq, nh, nkv, d, nsplit)
     if out is None:
         out = torch.empty((nseq, nh * d), dtype=q.dtype, device=q.device)
     _need(out.shape == (nseq, nh * d) and out.dtype == q.dtype, "attention_decode: out has the wrong shape or type")
@@ -524,6 +529,40 @@ def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_s
                                      c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
                                      _p(out), _p(ws), c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit),
                                      _stream()))
+    return out
+
+
+def attention_decode_raw_supports(nh: int, nkv: int, d: int, rotary_dim: int) -> bool:
+    return bool(lib().gs_attention_decode_raw_supports(c_int(nh), c_int(nkv), c_int(d), c_int(rotary_dim)))
+
+
+def attention_decode_raw(qkv, q_stride, kcache, vcache, positions, block_table, page_size, window, scale, q_weight,
+                         k_weight, head_eps, cos, sin, nh, nkv, d, nseq, nsplit: int, write_kv: bool = True,
+                         out: torch.Tensor = None) -> torch.Tensor:
+    """Decode attention straight from the rows of q|k|v as their product left them: the kernel norms and rotates
+    the queries and the new key, writes the new key and value into their pages, and attends."""
+    _dev(qkv, kcache, vcache, positions, block_table, q_weight, k_weight, cos, sin, out)
+    _need(qkv.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
+          "attention_decode_raw takes bfloat16")
+    _need(qkv.numel() >= (nseq - 1) * q_stride + (nh + 2 * nkv) * d if nseq else True, "attention_decode_raw: qkv is too small")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
+          "cache must be (pages, nkv, page_size, d)")
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "head norm weight float32 (d,)")
+    _need(cos.dtype == torch.float32 and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == d // 2
+          and cos.is_contiguous() and sin.is_contiguous(), "rotation tables (positions, d/2) float32")
+    _i32(positions, nseq, "positions")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= nseq,
+          "block_table must be int32 (nseq, max_blocks)")
+    ws = _decode_workspace(qkv.device, nseq, nh, nkv, d, nsplit)
+    if out is None:
+        out = torch.empty((nseq, nh * d), dtype=qkv.dtype, device=qkv.device)
+    _need(out.shape == (nseq, nh * d) and out.dtype == qkv.dtype, "attention_decode_raw: out has the wrong shape or type")
+    _check(lib().gs_attention_decode_raw(_p(qkv), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
+                                         c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0),
+                                         c_float(scale), _p(q_weight), _p(k_weight), c_float(head_eps), _p(cos), _p(sin),
+                                         c_int(d), c_int(1 if write_kv else 0), _p(out), _p(ws), c_int(nseq), c_int(nh),
+                                         c_int(nkv), c_int(d), c_int(nsplit), _stream()))
     return out
 
 

@@ -26,6 +26,17 @@ class DeferredLinear:
         self.x, self.w = x, w
 
 
+class RawQKV:
+    """Rows of q|k|v as their product left them, with what the attention kernel needs to finish them itself
+    (head norms, rotation, cache write).  Opaque to the mixer: it hands it from ``attention_in`` to ``attention``."""
+
+    __slots__ = ("qkv", "q_norm", "k_norm", "eps", "position", "dtype")
+
+    def __init__(self, qkv, q_norm, k_norm, eps, position):
+        self.qkv, self.q_norm, self.k_norm, self.eps, self.position = qkv, q_norm, k_norm, eps, position
+        self.dtype = qkv.dtype
+
+
 class Runtime:
     def __init__(self, device, dtype: torch.dtype):
         if dtype not in (torch.float32, torch.bfloat16):
@@ -158,6 +169,11 @@ class Runtime:
                                         write_kv=cache.write, wt=self._wt(wqkv))
                 return q, nh * d
         qkv = self.linear(x, wqkv, bqkv)          # a lazy norm goes through as it is where the product takes it
+        if (self.fused and ctx.all_single and cache.k.dtype == torch.bfloat16 and qkv.dtype == torch.bfloat16
+                and cache.page_size >= 2 and (q_norm is None) == (k_norm is None)
+                and ops.attention_decode_raw_supports(nh, nkv, d, position.rotary_dim)):
+            # a decode step: the attention kernel norms, rotates and writes the cache itself
+            return RawQKV(qkv, q_norm, k_norm, head_eps, position), (nh + 2 * nkv) * d
         ops.qknorm_rope_kv(qkv, q_norm, k_norm, head_eps, position.cos, position.sin, position.rotary_dim,
                            ctx.positions, ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v,
                            nh, nkv, d, write_kv=cache.write)
@@ -172,6 +188,11 @@ class Runtime:
             longest = min(longest, window)
         tiles = max(1, -(-longest // 64))
         nsplit = max(1, min(-(-tiles // 16), 64, max(1, 2048 // max(1, nseq * nkv))))
+        if isinstance(q, RawQKV):
+            return self.ops.attention_decode_raw(q.qkv, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
+                                                 cache.page_size, window, scale, q.q_norm, q.k_norm, q.eps,
+                                                 q.position.cos, q.position.sin, nh, nkv, d, nseq, nsplit,
+                                                 write_kv=cache.write, out=out)
         return self.ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                          cache.page_size, window, scale, nh, nkv, d, nseq, nsplit, out=out)
 
@@ -182,6 +203,8 @@ class Runtime:
         shapes they are written for.
         """
         ops = self.ops
+        if isinstance(q, RawQKV):
+            return self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, ctx.nseq, None)
         fast = q.dtype == torch.bfloat16 and cache.page_size >= 2
         if ctx.all_single and fast and ops.attention_decode_supports(nh, nkv, d):
             return self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, ctx.nseq, None)

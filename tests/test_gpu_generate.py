@@ -268,7 +268,7 @@ def test_recorded_decode_loop_equals_single_steps(folders, name, dtype):
     assert [eng2.length(i) for i in range(3)] == [len(p) + 21 for p in prompts]
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("nreq,steps", [(3, 20), (20, 4), (40, 4)])
 def test_recorded_decode_logits_follow_the_plain_model(folders, name, nreq, steps):
     """The fused kernels of the recorded step, row by row against the plain implementation (bfloat16): few rows

@@ -483,6 +483,45 @@ def test_attention_decode(ops, nh, nkv, d, ps, nsplit, window):
     close(got, same.double().cpu(), torch.bfloat16)
 
 
+@pytest.mark.parametrize("nh,nkv,d,norm,nsplit,write", [(32, 8, 64, True, 1, True), (2, 1, 64, False, 3, True),
+                                                        (8, 1, 128, True, 2, True), (5, 5, 64, True, 1, False)])
+def test_attention_decode_from_raw_rows_equals_the_separate_kernels(ops, nh, nkv, d, norm, nsplit, write):
+    """Head norms, rotation and cache write inside the attention kernel against the kernel that does them alone."""
+    g = gen(nh * 7 + d + nsplit)
+    ps, lens = 16, [1, 64, 65, 300, 17, 129]
+    nseq = len(lens)
+    nblk = [-(-n // ps) for n in lens]
+    total = sum(nblk)
+    kc = torch.randn(total + 1, nkv, ps, d, generator=g).bfloat16()
+    vc = torch.randn(total + 1, nkv, ps, d, generator=g).bfloat16()
+    table = torch.zeros(nseq, max(nblk), dtype=torch.int32)
+    at = 0
+    for i in range(nseq):
+        table[i, :nblk[i]] = torch.arange(at, at + nblk[i], dtype=torch.int32)
+        at += nblk[i]
+    qkv = torch.randn(nseq, (nh + 2 * nkv) * d, generator=g).bfloat16()
+    qw = (1 + 0.2 * torch.randn(d, generator=g)).to(DEV) if norm else None
+    kw = (1 + 0.2 * torch.randn(d, generator=g)).to(DEV) if norm else None
+    cos, sin = rope_tables(d, 1e4, 512)
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32).to(DEV)
+    seq_of = torch.arange(nseq, dtype=torch.int32, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    stride = (nh + 2 * nkv) * d
+    # the separate kernels
+    k1, v1, q1 = kc.clone().to(DEV), vc.clone().to(DEV), qkv.clone().to(DEV)
+    ops.qknorm_rope_kv(q1, qw, kw, 1e-5, cos, sin, d, positions, seq_of, table.to(DEV), ps, k1, v1, nh, nkv, d, write_kv=write)
+    want = ops.attention_decode(q1, stride, k1, v1, positions, table.to(DEV), ps, None, scale, nh, nkv, d, nseq, nsplit)
+    # all in one
+    k2, v2 = kc.clone().to(DEV), vc.clone().to(DEV)
+    got = ops.attention_decode_raw(qkv.to(DEV), stride, k2, v2, positions, table.to(DEV), ps, None, scale, qw, kw, 1e-5,
+                                   cos, sin, nh, nkv, d, nseq, nsplit, write_kv=write)
+    assert float((got.float() - want.float()).abs().max()) <= 2e-2 * max(1.0, float(want.float().abs().max()))
+    assert float((k2.float() - k1.float()).abs().max()) <= 2e-2 * max(1.0, float(k1.float().abs().max()))
+    assert torch.equal(v2, v1)
+    if not write:
+        assert torch.equal(k2.cpu(), kc) and torch.equal(v2.cpu(), vc)
+
+
 def test_attention_decode_supports(ops):
     assert ops.attention_decode_supports(32, 8, 64) and ops.attention_decode_supports(3, 1, 32)
     assert not ops.attention_decode_supports(3, 3, 48) and not ops.attention_decode_supports(18, 2, 64)

@@ -22,7 +22,8 @@ pytestmark = pytest.mark.gpu
 TOL = {"float32": 1e-4, "bfloat16": 1.5e-2}
 
 # sequence lengths: the benchmark description's prompts plus generated tokens
-LENGTHS = {"A": (5 + 16, 17 + 16, 32 + 16, 70), "B": (1 + 24, 9 + 24, 40 + 24, 100 + 24), "C": (3, 50, 97)}
+LENGTHS = {"A": (5 + 16, 17 + 16, 32 + 16, 70), "B": (1 + 24, 9 + 24, 40 + 24, 100 + 24), "C": (3, 50, 97),
+           "D": (2, 40, 66, 150)}
 
 
 @pytest.fixture(scope="module")
@@ -36,7 +37,7 @@ def sequences(name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_replay_four_ways(name, dtype, folders, tmp_path):
     cfg, _ = CONFIGS[name]
     model_dir = write_tiny(folders, name, torch.float32 if dtype == "float32" else torch.bfloat16)

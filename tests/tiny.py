@@ -2,7 +2,7 @@
 
 A and B are the two configurations the benchmark description names; C adds sizes that are no
 power of two anywhere (a feed-forward width that is no multiple of 8, an odd vocabulary, as
-many key heads as query heads, two taps).  Weights are drawn with a standard deviation of
+many key heads as query heads, two taps); D has heads 64 wide.  Weights are drawn with a standard deviation of
 0.1 rather than 0.02, so that every sub-layer moves the stream by about as much as the stream
 itself holds and a fault in any of them shows in the logits.
 """
@@ -31,7 +31,15 @@ TINY_C = Lfm2Config(
     layer_types=("full_attention", "full_attention", "conv"), conv_L_cache=2, conv_bias=False,
     intermediate_size=100, norm_eps=1e-4, rope_theta=5e5, tie_word_embeddings=True, max_position_embeddings=384)
 
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# D has the head width of the benchmark's model (64), so that the kernels written for it (attention on the matrix
+# cores for prompts and for decoding, the 16-byte head norm and rotation) run inside a whole model, two query
+# heads to a key head
+TINY_D = Lfm2Config(
+    vocab_size=200, hidden_size=128, num_hidden_layers=3, num_attention_heads=2, num_key_value_heads=1,
+    layer_types=("full_attention", "conv", "full_attention"), conv_L_cache=3, conv_bias=False,
+    intermediate_size=136, norm_eps=1e-5, rope_theta=1e5, tie_word_embeddings=True, max_position_embeddings=320)
+
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 def write_tiny(root: str, name: str, dtype=torch.float32) -> str:
