@@ -34,13 +34,17 @@ _MUST_BE_TRUE = ("block_use_swiglu", "use_pos_enc")
 # Features of other members of the family that dense LFM2 does not have (lfm2.jl:1-15).
 _REFUSED = ("sliding_window", "sliding_window_pattern", "rope_scaling", "rope_freq_factors",
             "num_experts", "num_local_experts", "num_experts_per_tok", "moe_intermediate_size",
-            "attention_bias", "partial_rotary_factor", "head_dim")
+            "attention_bias", "partial_rotary_factor", "attention_dropout")
+# The architecture's published defaults for keys a config.json may leave out.
+DEFAULTS = {"conv_L_cache": 3, "norm_eps": 1e-5, "rope_theta": 1000000.0, "max_position_embeddings": 128000,
+            "block_auto_adjust_ff_dim": True, "block_multiple_of": 256, "block_ffn_dim_multiplier": 1.0}
 _KNOWN = frozenset({
     "architectures", "vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
     "num_key_value_heads", "layer_types", "full_attn_idxs", "conv_L_cache", "conv_bias",
     "block_ff_dim", "block_auto_adjust_ff_dim", "block_multiple_of", "block_ffn_dim_multiplier",
     "intermediate_size", "norm_eps", "rope_theta", "tie_word_embeddings", "tie_embedding",
     "max_position_embeddings", "eos_token_id", "bos_token_id", "pad_token_id",
+    "head_dim", "rms_norm_eps", "rope_parameters", "hidden_act",
 }) | _IGNORED | frozenset(_MUST_EQUAL) | frozenset(_MUST_BE_TRUE) | frozenset(_REFUSED)
 
 
@@ -124,8 +128,28 @@ class Lfm2Config:
             if raw.get(key) not in (None, False, 0):
                 raise ConfigError(f"config.json asks for {key!r}, which dense LFM2 does not have", key=key)
 
+        raw = dict(raw)
+        # other spellings of the same facts: they must agree where both are given
+        if "rms_norm_eps" in raw:
+            if "norm_eps" in raw and raw["norm_eps"] != raw["rms_norm_eps"]:
+                raise ConfigError("norm_eps and rms_norm_eps disagree")
+            raw["norm_eps"] = raw.pop("rms_norm_eps")
+        rp = raw.pop("rope_parameters", None)
+        if rp is not None:
+            if not isinstance(rp, dict) or rp.get("rope_type", "default") not in (None, "default") or \
+                    set(rp) - {"rope_type", "rope_theta"}:
+                raise ConfigError("rope_parameters: dense LFM2 has plain rotation only (rope_type default, rope_theta)")
+            if "rope_theta" in rp:
+                if "rope_theta" in raw and raw["rope_theta"] != rp["rope_theta"]:
+                    raise ConfigError("rope_theta and rope_parameters.rope_theta disagree")
+                raw["rope_theta"] = rp["rope_theta"]
+        if raw.pop("hidden_act", "silu") != "silu":
+            raise ConfigError("hidden_act: the LFM2 feed-forward is SwiGLU (silu)")
+
         def need(key, kind):
             if key not in raw:
+                if key in DEFAULTS:
+                    return DEFAULTS[key]
                 raise ConfigError(f"config.json lacks the required key {key!r}", key=key)
             v = raw[key]
             if kind is float and isinstance(v, int) and not isinstance(v, bool):
@@ -201,8 +225,11 @@ class Lfm2Config:
             pad_token_id=raw.get("pad_token_id"),
             block_ff_dim=block_ff, block_multiple_of=mult_of, block_ffn_dim_multiplier=mult,
         )
+        if raw.get("head_dim") is not None and raw["head_dim"] != cfg.head_dim:
+            raise ConfigError("head_dim must equal hidden_size / num_attention_heads (the attention width is the "
+                              "hidden width)", head_dim=raw["head_dim"], expected=cfg.head_dim)
         for key, other in _MUST_EQUAL.items():
-            if key in raw and raw[key] != raw[other]:
+            if key in raw and other in raw and raw[key] != raw[other]:
                 raise ConfigError(f"config.json key {key!r} must equal {other!r}",
                                   **{key: raw[key], other: raw[other]})
         for key in _MUST_BE_TRUE:

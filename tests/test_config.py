@@ -100,13 +100,40 @@ def test_malformed_fields_raise(change, match):
 
 
 @pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
-                                 "num_key_value_heads", "conv_L_cache", "norm_eps", "rope_theta",
-                                 "max_position_embeddings", "block_ff_dim", "block_multiple_of"])
+                                 "num_key_value_heads", "block_ff_dim"])
 def test_required_keys(key):
     raw = dict(BASE)
     del raw[key]
     with pytest.raises(ConfigError, match=key):
         Lfm2Config.from_dict(raw)
+
+
+def test_keys_that_may_be_left_out_take_the_published_defaults():
+    raw = dict(BASE)
+    for key in ("conv_L_cache", "norm_eps", "rope_theta", "max_position_embeddings", "block_multiple_of",
+                "block_auto_adjust_ff_dim", "block_ffn_dim_multiplier"):
+        raw.pop(key, None)
+    c = Lfm2Config.from_dict(raw)
+    assert (c.conv_L_cache, c.norm_eps, c.rope_theta, c.max_position_embeddings) == (3, 1e-5, 1e6, 128000)
+    assert c.intermediate_size == 8192                      # 12288 -> two thirds -> up to a multiple of 256
+
+
+def test_other_spellings_of_the_same_facts():
+    raw = dict(BASE)
+    eps = raw.pop("norm_eps")
+    theta = raw.pop("rope_theta")
+    raw.update(rms_norm_eps=eps, rope_parameters={"rope_type": "default", "rope_theta": theta}, head_dim=64,
+               hidden_act="silu")
+    c = Lfm2Config.from_dict(raw)
+    assert c.norm_eps == eps and c.rope_theta == theta
+    with pytest.raises(ConfigError, match="head_dim"):
+        Lfm2Config.from_dict(dict(BASE, head_dim=32))
+    with pytest.raises(ConfigError, match="disagree"):
+        Lfm2Config.from_dict(dict(BASE, rms_norm_eps=BASE["norm_eps"] * 2))
+    with pytest.raises(ConfigError, match="rope_parameters"):
+        Lfm2Config.from_dict(dict(BASE, rope_parameters={"rope_type": "yarn", "factor": 4.0}))
+    with pytest.raises(ConfigError, match="hidden_act"):
+        Lfm2Config.from_dict(dict(BASE, hidden_act="gelu"))
 
 
 def test_layer_list_length_and_kinds():
