@@ -54,7 +54,7 @@ def load_tensors(model_dir: str, table: Dict[str, TensorSpec], mode: torch.dtype
     for name, ts in table.items():
         if name in where:
             f = where[name]
-            if tuple(f.shape(name)) != tuple(ts.shape):
+            if _core(f.shape(name)) != _core(ts.shape):
                 wrong_shape.append(f"{name}: file has {tuple(f.shape(name))}, the configuration needs {tuple(ts.shape)}")
             if f.dtype(name) not in _FLOATS:
                 wrong_type.append(f"{name}: {f.dtype(name)}")
@@ -75,7 +75,7 @@ def load_tensors(model_dir: str, table: Dict[str, TensorSpec], mode: torch.dtype
                           wrong_type=wrong_type, duplicates=sorted(duplicates))
     out = {}
     for name, ts in table.items():
-        t = where[name].tensor(name)
+        t = where[name].tensor(name).reshape(ts.shape)      # axes of length one may be stored or left out
         out[name] = t.to(device=device, dtype=held_dtype(t.dtype, ts.role, mode)).contiguous()
     for alias, target in aliases.items():
         if alias in where:
@@ -86,6 +86,12 @@ def load_tensors(model_dir: str, table: Dict[str, TensorSpec], mode: torch.dtype
     for f in files:
         f.close()
     return out
+
+
+def _core(shape) -> tuple:
+    """A shape without its axes of length one: a depthwise convolution's taps are (H, 1, W) in some files, (H, W) in
+    others, and mean the same."""
+    return tuple(int(n) for n in shape if int(n) != 1)
 
 
 def random_tensors(table: Dict[str, TensorSpec], seed: int, dtype: torch.dtype, device="cpu",

@@ -63,6 +63,15 @@ def test_a_tensor_stored_in_32_bit_stays_so(tmp_path):
     assert held_dtype(torch.int64, "table", torch.bfloat16) == torch.int32
 
 
+def test_axes_of_length_one_may_be_stored_or_left_out(tmp_path):
+    d = folder(tmp_path)
+    want = load(d)["model.layers.0.conv.conv.weight"]
+    assert want.shape == (64, 1, 3)
+    rewrite(d, lambda t: t.__setitem__("model.layers.0.conv.conv.weight", t["model.layers.0.conv.conv.weight"].reshape(64, 3)))
+    got = load(d)["model.layers.0.conv.conv.weight"]
+    assert got.shape == (64, 1, 3) and torch.equal(got, want)
+
+
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     d = folder(tmp_path)
 
