@@ -297,3 +297,31 @@ def test_recorded_decode_logits_follow_the_plain_model(folders, name, nreq, step
         toks = ids[0].tolist()
     print(f"{name}, {nreq} requests: worst relative difference of the recorded step's logits {worst:.3e}")
     assert worst <= 1.5e-2
+
+
+def test_recorded_decode_across_a_bound_on_the_context(tmp_path):
+    """The decode step is recorded per bound on the context length (1024, 2048, ...); a request that grows past a
+    bound moves to another recording in the middle of its decoding, and its logits stay those of the plain model."""
+    import dataclasses
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.weights import write_model_folder
+    from tiny import TINY_D, STD
+    cfg_d = dataclasses.replace(TINY_D, max_position_embeddings=1536)
+    d = write_model_folder(str(tmp_path / "long_d"), cfg_d, 11, torch.bfloat16, std=STD)
+    cfg, w = P.read_config(d), P.read_weights(d)
+    seq = random_ids(1010, cfg["V"], 4242)
+    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=2048, num_slots=2)
+    eng.add_request("r")
+    tok = int(eng.step([StepEntry("r", seq, [len(seq) - 1])]).argmax())
+    checked = 0
+    for step in range(24):
+        seq.append(tok)
+        ids, bad = eng.decode(["r"], [tok], 1)
+        assert not bad.any()
+        if len(seq) in (1020, 1023, 1024, 1025, 1030):          # around the bound: the second recording takes over
+            logits = eng._runners[1].logits[0].double().cpu()
+            ref = P.forward(cfg, w, seq)[-1]
+            assert float((logits - ref).abs().max()) <= 1.5e-2 * max(1.0, float(ref.abs().max()))
+            checked += 1
+        tok = int(ids[0][0])
+    assert checked == 5 and len(eng._runners[1].graphs) == 2
