@@ -67,3 +67,57 @@ def test_replay_four_ways(name, dtype, folders, tmp_path):
         w, where = R.worst(mine, ref)
         print(f"{name} {dtype} {way}: worst |diff| {w:.3e} at {where} (tolerance {tol:.3e}, scale {scale:.2f})")
         assert w <= tol, f"{way}: first look at {where}"
+
+
+def random_config(seed: int):
+    """A configuration drawn from a seed: head widths in steps of 16, any number of heads and groups, widths and
+    vocabularies that are no powers of two, two to five layers of either kind."""
+    import random
+    from gesso_amd.config import Lfm2Config
+    rng = random.Random(seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 128])
+    nkv = rng.choice([1, 2, 3])
+    nh = nkv * (rng.choice([1, 2, 3, 4]) if d <= 64 else rng.choice([1, 2]))
+    layers = rng.randint(2, 5)
+    types = [rng.choice(["conv", "full_attention"]) for _ in range(layers)]
+    types[rng.randrange(layers)] = "full_attention"
+    types[(types.index("full_attention") + 1) % layers] = "conv"
+    return Lfm2Config(vocab_size=rng.choice([97, 200, 301, 512, 1000]), hidden_size=nh * d, num_hidden_layers=layers,
+                      num_attention_heads=nh, num_key_value_heads=nkv, layer_types=tuple(types),
+                      conv_L_cache=rng.choice([2, 3, 4]), conv_bias=rng.random() < 0.4,
+                      intermediate_size=rng.choice([40, 100, 136, 192, 320, 500]),
+                      norm_eps=rng.choice([1e-5, 1e-6, 1e-4]), rope_theta=rng.choice([1e4, 1e5, 1e6]),
+                      tie_word_embeddings=rng.random() < 0.5, max_position_embeddings=rng.choice([192, 256, 400]))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_replay_of_configurations_drawn_at_random(seed, dtype, tmp_path):
+    import random
+    from gesso_amd.weights import write_model_folder
+    from tiny import STD
+    cfg = random_config(seed)
+    rng = random.Random(seed)
+    model_dir = write_model_folder(str(tmp_path / "m"), cfg, seed, torch.float32 if dtype == "float32" else torch.bfloat16,
+                                   std=STD)
+    lens = [rng.randint(1, 6), rng.randint(20, 60), rng.randint(61, 110), rng.randint(111, 170)]
+    seqs = {f"s{i}": random_ids(n, cfg.vocab_size, seed * 10 + i) for i, n in enumerate(lens)}
+    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
+    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    ways = {"whole": R.trace_whole, "tail": R.trace_tail, "portions": R.trace_portions,
+            "mixed": lambda s: R.trace_mixed(s, seed=seed)}
+    big = R.Trace()
+    for way, make in ways.items():
+        t = make({f"{way}.{k}": v for k, v in seqs.items()})
+        for rec, rows in zip(t.steps, t.rows):
+            big.steps.append(dict(rec, step=len(big.steps)))
+            big.rows.append(rows)
+        big.max_tokens = max(big.max_tokens, t.max_tokens)
+    got, rc = R.run_trace(model_dir, dtype, str(tmp_path / "out"), big, cfg.vocab_size)
+    assert rc == 0
+    for way in ways:
+        mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
+        w, where = R.worst(mine, ref)
+        print(f"seed {seed} ({cfg.num_attention_heads}/{cfg.num_key_value_heads} heads of {cfg.head_dim}) {dtype} {way}: "
+              f"worst |diff| {w:.3e} at {where}")
+        assert w <= TOL[dtype] * scale, f"{way}: first look at {where}"
