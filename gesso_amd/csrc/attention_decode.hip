@@ -37,6 +37,12 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 // the write of the new key and value into their page.  Every block norms and rotates its own queries; the block
 // whose keys end with the new one norms and rotates it, keeps it and the value in LDS for its scores, and writes
 // both to the cache for the steps to come.  Heads of 64 or 128, rotated whole.
+// Where column c of sequence seq's output goes: a row of `width`, or tiled rows (out_tiles = ceil(nseq / 16) > 0),
+// the order in which the product that follows takes them.
+__device__ __forceinline__ size_t out_index(int seq, int c, int width, int out_tiles) {
+  return out_tiles ? tiled_index(seq, c, out_tiles) : (size_t)seq * width + c;
+}
+
 struct DecodeRaw {
   const float* qw;       // (D) head norm weights, or null for no norm
   const float* kw;
@@ -51,7 +57,7 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
     const bf16* __restrict__ q, int q_stride, bf16* kcache, bf16* vcache,
     const int* __restrict__ positions, const int* __restrict__ block_table, int max_blocks, int page_size,
     unsigned page_magic, int window, float scale, bf16* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int nh, int nkv, DecodeRaw raw) {
+    float* __restrict__ part_ml, int nh, int nkv, int out_tiles, DecodeRaw raw) {
   static_assert(!RAW || D == 64 || D == 128, "the fused head norm and rotation are written for heads of 64 and 128");
   constexpr int DC = D / 8;               // 16-byte chunks per row
   constexpr int KG = 64 / DC;             // key groups per wavefront in the value phase
@@ -362,7 +368,7 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
           L += wl[w][g] * f;
         }
     if (nsplit == 1) {
-      out[((size_t)seq * nh + kvh * G + g) * D + j] = f32_to_bf16(o / L);
+      out[out_index(seq, (kvh * G + g) * D + j, nh * D, out_tiles)] = f32_to_bf16(o / L);
     } else {
       part_o[(unit * G + g) * D + j] = o;
       if (j == 0) {
@@ -378,7 +384,8 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
 // outputs are independent of one another.
 #define DEC_MAXSPLIT 64
 __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                              bf16* __restrict__ out, int nsplit, int nh, int nkv, int G, int D) {
+                                              bf16* __restrict__ out, int nsplit, int nh, int nkv, int G, int D,
+                                              int out_tiles) {
   __shared__ float sm[DEC_MAXSPLIT][DEC_MAXG], sl[DEC_MAXSPLIT][DEC_MAXG], sf[DEC_MAXSPLIT][DEC_MAXG];
   __shared__ float sinv[DEC_MAXG];
   const int kvh = blockIdx.x, seq = blockIdx.y;
@@ -414,7 +421,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
       for (int u = 0; u < 8; ++u) o += v[u] * sf[sp + u][g];
     }
     for (; sp < nsplit; ++sp) o += part_o[((base + sp) * G + g) * D + j] * sf[sp][g];
-    out[((size_t)seq * nh + kvh * G + g) * D + j] = f32_to_bf16(o * sinv[g]);
+    out[out_index(seq, (kvh * G + g) * D + j, nh * D, out_tiles)] = f32_to_bf16(o * sinv[g]);
   }
 }
 
@@ -424,11 +431,11 @@ template <int D, int RAW>
 static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, bf16* kc, bf16* vc,
                          const int* positions, const int* bt, int max_blocks, int page_size, unsigned page_magic,
                          int window, float scale, bf16* out, float* part_o, float* part_ml, int nh, int nkv,
-                         DecodeRaw raw) {
+                         int out_tiles, DecodeRaw raw) {
 #define GS_RUN(GG)                                                                                                     \
   attention_decode_kernel<D, GG, DEC_WAVES, RAW><<<grid, DEC_WAVES * 64, 0, stream>>>(                                 \
       q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_magic, window, scale, out, part_o, part_ml, nh, \
-      nkv, raw)
+      nkv, out_tiles, raw)
   switch (G) {
     case 1: GS_RUN(1); break;
     case 2: GS_RUN(2); break;
@@ -458,8 +465,10 @@ extern "C" long gs_attention_decode_workspace(int nseq, int nh, int nkv, int d, 
 
 static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache, const int* positions,
                         const int* block_table, int max_blocks, int page_size, int window, float scale, void* out,
-                        float* workspace, int nseq, int nh, int nkv, int d, int nsplit, const DecodeRaw* raw,
-                        hipStream_t stream) {
+                        int out_tiled, float* workspace, int nseq, int nh, int nkv, int d, int nsplit,
+                        const DecodeRaw* raw, hipStream_t stream) {
+  GS_REQUIRE(!out_tiled || (nh * d) % 32 == 0, "attention_decode: tiled rows need a width that is a multiple of 32, not %d", nh * d);
+  const int out_tiles = out_tiled ? gs_ceil_div(nseq, 16) : 0;
   GS_REQUIRE(gs_attention_decode_supports(nh, nkv, d), "attention_decode: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
   GS_REQUIRE(nseq >= 0 && nseq <= 65535 && nkv <= 65535, "attention_decode: bad batch %d", nseq);
   GS_REQUIRE(nsplit >= 1 && nsplit <= 64, "attention_decode: %d splits outside [1, 64]", nsplit);
@@ -480,7 +489,7 @@ static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache,
   const DecodeRaw none = {};
 #define GS_ARGS                                                                                             \
   G, grid, stream, (const bf16*)q, q_stride, (bf16*)kcache, (bf16*)vcache, positions, block_table, max_blocks, \
-      page_size, page_magic, window, scale, (bf16*)out, part_o, part_ml, nh, nkv
+      page_size, page_magic, window, scale, (bf16*)out, part_o, part_ml, nh, nkv, out_tiles
   if (raw) {
     switch (d) {
       case 64: rc = launch_decode<64, 1>(GS_ARGS, *raw); break;
@@ -499,7 +508,7 @@ static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache,
   GS_LAUNCH_CHECK("attention_decode");
   if (nsplit > 1) {
     dim3 mgrid(nkv, nseq);
-    attention_decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, (bf16*)out, nsplit, nh, nkv, G, d);
+    attention_decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, (bf16*)out, nsplit, nh, nkv, G, d, out_tiles);
     GS_LAUNCH_CHECK("attention_decode_merge");
   }
   return 0;
@@ -507,10 +516,10 @@ static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache,
 
 extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcache, const void* vcache,
                                    const int* positions, const int* block_table, int max_blocks, int page_size,
-                                   int window, float scale, void* out, float* workspace, int nseq, int nh, int nkv,
-                                   int d, int nsplit, hipStream_t stream) {
+                                   int window, float scale, void* out, int out_tiled, float* workspace, int nseq, int nh,
+                                   int nkv, int d, int nsplit, hipStream_t stream) {
   return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
-                      scale, out, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream);
+                      scale, out, out_tiled, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream);
 }
 
 // Whether the kernel also takes the head norms, the rotation and the cache write: heads of 64 or 128 rotated whole.
@@ -523,12 +532,13 @@ extern "C" int gs_attention_decode_raw_supports(int nh, int nkv, int d, int rota
 extern "C" int gs_attention_decode_raw(const void* qkv, int q_stride, void* kcache, void* vcache, const int* positions,
                                        const int* block_table, int max_blocks, int page_size, int window, float scale,
                                        const float* qw, const float* kw, float eps, const float* cos_t,
-                                       const float* sin_t, int rotary_dim, int write_kv, void* out, float* workspace,
-                                       int nseq, int nh, int nkv, int d, int nsplit, hipStream_t stream) {
+                                       const float* sin_t, int rotary_dim, int write_kv, void* out, int out_tiled,
+                                       float* workspace, int nseq, int nh, int nkv, int d, int nsplit,
+                                       hipStream_t stream) {
   GS_REQUIRE(gs_attention_decode_raw_supports(nh, nkv, d, rotary_dim), "attention_decode_raw: sizes nh=%d nkv=%d d=%d rotary=%d are not taken", nh, nkv, d, rotary_dim);
   GS_REQUIRE((qw == nullptr) == (kw == nullptr) && cos_t && sin_t, "attention_decode_raw: q and k norm weights come together; the rotation needs its tables");
   GS_REQUIRE((((uintptr_t)qw | (uintptr_t)kw | (uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0, "attention_decode_raw: weights and tables must be 16-byte aligned");
   DecodeRaw raw = {qw, kw, eps, cos_t, sin_t, write_kv};
   return decode_entry(qkv, q_stride, kcache, vcache, positions, block_table, max_blocks, page_size, window, scale, out,
-                      workspace, nseq, nh, nkv, d, nsplit, &raw, stream);
+                      out_tiled, workspace, nseq, nh, nkv, d, nsplit, &raw, stream);
 }

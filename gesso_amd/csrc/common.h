@@ -161,4 +161,12 @@ __device__ __forceinline__ bool aligned16(const T* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
 }
 
+// "Tiled rows": M rows of K columns (K a multiple of 32) in the order a matrix-core product takes them as its
+// second operand: the 16 rows x 32 columns tile of (k step, row tile) lies as 64 lanes x 16 bytes, lane l holding
+// row l % 16, columns 8 (l / 16) .. + 7; the row tiles of a k step follow each other, then the next k step.
+// `tiles` = ceil(M / 16); the buffer holds (K / 32) * tiles * 512 elements.
+__host__ __device__ __forceinline__ size_t tiled_index(int m, int k, int tiles) {
+  return ((((size_t)(k >> 5) * tiles + (m >> 4)) * 64) + ((k & 31) >> 3) * 16 + (m & 15)) * 8 + (k & 7);
+}
+
 static inline int gs_ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

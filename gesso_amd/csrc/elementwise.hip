@@ -19,17 +19,18 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 4; }
+extern "C" int gs_abi_version() { return 5; }
 
 // ------------------------------------------------------------------ embedding
 
 // out[t, :] = table[ids[t], :] as float32; an id outside the table gives a NaN row.
 // With ssq: ssq[t] = sum of squares of the row (one partial sum per row, for a norm that follows).
-// With next_w and xs: xs[t, :] = bfloat16(row * next_w), the rows pre-weighted for the first norm's consumer.
+// With next_w and xs: xs[t, :] = bfloat16(row * next_w), the rows pre-weighted for the first norm's consumer,
+// as rows of H or, with xs_tiles = ceil(T / 16) > 0, as tiled rows.
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
-                             float* __restrict__ ssq, const float* __restrict__ next_w, bf16* __restrict__ xs, int H,
-                             int V) {
+                             float* __restrict__ ssq, const float* __restrict__ next_w, bf16* __restrict__ xs,
+                             int xs_tiles, int H, int V) {
   __shared__ float red[17];
   int t = blockIdx.x;
   int id = ids[t];
@@ -53,7 +54,7 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
           load8f(next_w + j, w);
 #pragma unroll
           for (int i = 0; i < 8; ++i) w[i] *= v[i];
-          store8f(xs + (size_t)t * H + j, w);
+          store8f(xs + (xs_tiles ? tiled_index(t, j, xs_tiles) : (size_t)t * H + j), w);
         }
       }
     } else {
@@ -61,7 +62,7 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
         float v = to_f32(row[j]);
         o[j] = v;
         ss += v * v;
-        if (xs) xs[(size_t)t * H + j] = f32_to_bf16(v * next_w[j]);
+        if (xs) xs[xs_tiles ? tiled_index(t, j, xs_tiles) : (size_t)t * H + j] = f32_to_bf16(v * next_w[j]);
       }
     }
   }
@@ -72,13 +73,15 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
 }
 
 extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, float* out, float* ssq,
-                        const float* next_w, void* xs, int T, int H, int V, hipStream_t stream) {
+                        const float* next_w, void* xs, int xs_tiled, int T, int H, int V, hipStream_t stream) {
   GS_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+  GS_REQUIRE(!xs_tiled || (xs && H % 32 == 0), "embed: tiled rows need a width that is a multiple of 32, not %d", H);
+  const int xs_tiles = xs_tiled ? gs_ceil_div(T, 16) : 0;
   if (T == 0) return 0;
   if (table_dtype == GS_F32)
-    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, ssq, next_w, (bf16*)xs, H, V);
+    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, ssq, next_w, (bf16*)xs, xs_tiles, H, V);
   else if (table_dtype == GS_BF16)
-    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, ssq, next_w, (bf16*)xs, H, V);
+    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, ssq, next_w, (bf16*)xs, xs_tiles, H, V);
   else
     GS_REQUIRE(false, "embed: unknown dtype %d", table_dtype);
   GS_LAUNCH_CHECK("embed");
@@ -89,11 +92,12 @@ extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, floa
 
 // One block per row: delta = sum over the parts of K (in order), rounded to bfloat16 as a product's result is
 // before the add; res += delta; ssq[row] = sum of squares of the new row; and, with next_w, the row normed for
-// the norm that reads the stream next: normed = res / sqrt(mean(res^2) + eps) * next_w.
+// the norm that reads the stream next: normed = res / sqrt(mean(res^2) + eps) * next_w (as rows of N or, with
+// tiles = ceil(M / 16) > 0, as tiled rows).
 template <typename TO>
 __global__ void residual_from_parts_kernel(const float* __restrict__ part, int parts, float* __restrict__ res,
                                            float* __restrict__ ssq, const float* __restrict__ next_w, float eps,
-                                           TO* __restrict__ normed, int M, int N) {
+                                           TO* __restrict__ normed, int tiles, int M, int N) {
   __shared__ float red[17];
   const int m = blockIdx.x;
   float* x = res + (size_t)m * N;
@@ -153,13 +157,17 @@ __global__ void residual_from_parts_kernel(const float* __restrict__ part, int p
     for (int i = 0; i < 4; ++i)
       if (j + i < N) {
         const float v = u < MAXV ? keep[u][i] : x[j + i];
-        normed[(size_t)m * N + j + i] = from_f32<TO>(v * inv * next_w[j + i]);
+        normed[tiles ? tiled_index(m, j + i, tiles) : (size_t)m * N + j + i] = from_f32<TO>(v * inv * next_w[j + i]);
       }
   }
 }
 
 extern "C" int gs_residual_from_parts(const float* part, int parts, float* res, float* ssq, const float* next_w,
-                                      float eps, void* normed, int normed_dtype, int M, int N, hipStream_t stream) {
+                                      float eps, void* normed, int normed_dtype, int normed_tiled, int M, int N,
+                                      hipStream_t stream) {
+  GS_REQUIRE(!normed_tiled || (normed && normed_dtype == GS_BF16 && N % 32 == 0),
+             "residual_from_parts: tiled rows are bfloat16 and a multiple of 32 wide, not %d", N);
+  const int tiles = normed_tiled ? gs_ceil_div(M, 16) : 0;
   GS_REQUIRE(M >= 0 && N > 0 && parts >= 1, "residual_from_parts: bad sizes M=%d N=%d parts=%d", M, N, parts);
   GS_REQUIRE(part && res && ssq, "residual_from_parts: needs the partial sums, the stream and room for the sums of squares");
   GS_REQUIRE((next_w == nullptr) == (normed == nullptr), "residual_from_parts: the next norm's weight and the room for the normed rows come together");
@@ -167,12 +175,38 @@ extern "C" int gs_residual_from_parts(const float* part, int parts, float* res, 
   if (M == 0) return 0;
   const int threads = N >= 4096 ? 1024 : (N >= 2048 ? 512 : 256);   // four values a thread and turn
   if (!normed || normed_dtype == GS_BF16)
-    residual_from_parts_kernel<bf16><<<M, threads, 0, stream>>>(part, parts, res, ssq, next_w, eps, (bf16*)normed, M, N);
+    residual_from_parts_kernel<bf16><<<M, threads, 0, stream>>>(part, parts, res, ssq, next_w, eps, (bf16*)normed, tiles, M, N);
   else if (normed_dtype == GS_F32)
-    residual_from_parts_kernel<float><<<M, threads, 0, stream>>>(part, parts, res, ssq, next_w, eps, (float*)normed, M, N);
+    residual_from_parts_kernel<float><<<M, threads, 0, stream>>>(part, parts, res, ssq, next_w, eps, (float*)normed, tiles, M, N);
   else
     GS_REQUIRE(false, "residual_from_parts: unknown dtype %d", normed_dtype);
   GS_LAUNCH_CHECK("residual_from_parts");
+  return 0;
+}
+
+// ------------------------------------------------------------------ rows <-> tiled rows
+
+// One thread per eight consecutive columns of a row: out = the same values in the other order.
+__global__ void retile_rows_kernel(const bf16* __restrict__ in, bf16* __restrict__ out, int M, int K, int ld,
+                                   int tiles, int to_tiled) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int k8 = K >> 3;
+  if (i >= (long)M * k8) return;
+  const int m = (int)(i / k8), k = (int)(i - (long)m * k8) * 8;
+  const size_t rowwise = (size_t)m * ld + k, tiled = tiled_index(m, k, tiles);
+  *reinterpret_cast<uint4*>(out + (to_tiled ? tiled : rowwise)) =
+      *reinterpret_cast<const uint4*>(in + (to_tiled ? rowwise : tiled));
+}
+
+// rows (M, K) with row stride ld <-> tiled rows of (K / 32) * ceil(M / 16) * 512 elements; bfloat16.
+// Rows beyond M inside the last row tile are left as they are.
+extern "C" int gs_retile_rows(const void* in, void* out, int M, int K, int ld, int to_tiled, hipStream_t stream) {
+  GS_REQUIRE(M >= 0 && K > 0 && K % 32 == 0 && ld >= K && ld % 8 == 0, "retile_rows: K=%d must be a multiple of 32, the row stride %d one of 8", K, ld);
+  GS_REQUIRE(((uintptr_t)in & 15) == 0 && ((uintptr_t)out & 15) == 0, "retile_rows: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  const long n = (long)M * (K / 8);
+  retile_rows_kernel<<<gs_ceil_div(n, 256), 256, 0, stream>>>((const bf16*)in, (bf16*)out, M, K, ld, gs_ceil_div(M, 16), to_tiled);
+  GS_LAUNCH_CHECK("retile_rows");
   return 0;
 }
 

@@ -15,9 +15,10 @@ void gs_skinny_parts_tiles(const SkinnyCall& c, int parts);
 void gs_skinny_conv_half_tiles(const SkinnyCall& c);
 void gs_skinny_qkv_tiles(const SkinnyCall& c, int d);
 
-static SkinnyCall base(const void* X, int ldx, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M,
+static SkinnyCall base(const void* X, int ldx, int x_tiled, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M,
                        int N, int K, int epilogue, hipStream_t stream) {
   SkinnyCall c = {};
+  c.ex.x_tiled = x_tiled;
   c.x = (const bf16*)X; c.ldx = ldx; c.w = (const bf16*)(Wt ? Wt : W); c.Y = Y; c.y_dtype = y_dtype; c.ldy = ldy;
   c.M = M; c.N = N; c.K = K; c.epilogue = epilogue; c.stream = stream;
   return c;
@@ -27,10 +28,11 @@ static void lazy(SkinnyCall& c, const float* res, const float* ssq, int nb, cons
   c.ex.res = res; c.ex.ssq = ssq; c.ex.nb = nb; c.ex.norm_w = norm_w; c.ex.eps = eps;
 }
 
-void gs_skinny_run_plain(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w,
+void gs_skinny_run_plain(const void* X, int ldx, int x_tiled, const float* res, const float* ssq, int nb, const float* norm_w,
                          float eps, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M, int N, int K,
-                         int epilogue, hipStream_t stream) {
-  SkinnyCall c = base(X, ldx, W, Wt, Y, y_dtype, ldy, M, N, K, epilogue, stream);
+                         int epilogue, int y_tiled, hipStream_t stream) {
+  SkinnyCall c = base(X, ldx, x_tiled, W, Wt, Y, y_dtype, ldy, M, N, K, epilogue, stream);
+  c.ex.y_tiled = y_tiled;
   if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   Wt ? gs_skinny_plain_tiles(c) : gs_skinny_plain_rows(c);
 }
@@ -38,18 +40,20 @@ void gs_skinny_run_plain(const void* X, int ldx, const float* res, const float* 
 // A weight of few rows is shared out in half tiles, so that twice as many blocks stream it.
 bool gs_skinny_halves(int N) { return N % 16 == 0 && N / 16 <= 160; }
 
-void gs_skinny_run_residual(const void* X, int ldx, const void* W, const void* Wt, float* res, float* ssq_out,
-                            const float* next_w, void* xs_out, int M, int N, int K, hipStream_t stream) {
-  SkinnyCall c = base(X, ldx, W, Wt, nullptr, GS_F32, N, M, N, K, 2, stream);
+void gs_skinny_run_residual(const void* X, int ldx, int x_tiled, const void* W, const void* Wt, float* res, float* ssq_out,
+                            const float* next_w, void* xs_out, int xs_tiled, int M, int N, int K, hipStream_t stream) {
+  SkinnyCall c = base(X, ldx, x_tiled, W, Wt, nullptr, GS_F32, N, M, N, K, 2, stream);
+  c.ex.y_tiled = xs_tiled;
   c.ex.res_out = res; c.ex.ssq_out = ssq_out; c.ex.next_w = next_w; c.ex.xs_out = (bf16*)xs_out;
   if (Wt && gs_skinny_halves(N)) gs_skinny_residual_half_tiles(c);
   else Wt ? gs_skinny_residual_tiles(c) : gs_skinny_residual_rows(c);
 }
 
-void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
+void gs_skinny_run_conv(const void* X, int ldx, int x_tiled, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
                         const void* Wt, const float* taps, const float* conv_bias, float* state, const int* slots,
-                        int conv_w, void* Y, int M, int H, int K, hipStream_t stream) {
-  SkinnyCall c = base(X, ldx, W, Wt, Y, GS_BF16, H, M, 3 * H, K, 3, stream);
+                        int conv_w, void* Y, int y_tiled, int M, int H, int K, hipStream_t stream) {
+  SkinnyCall c = base(X, ldx, x_tiled, W, Wt, Y, GS_BF16, H, M, 3 * H, K, 3, stream);
+  c.ex.y_tiled = y_tiled;
   if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.taps = taps; c.ex.conv_bias = conv_bias; c.ex.state = state; c.ex.slots = slots; c.ex.conv_w = conv_w;
   // c.N / 3 channels, as few as a narrow weight's rows; with many rows of X the blocks' reading of X outweighs that
@@ -57,12 +61,12 @@ void gs_skinny_run_conv(const void* X, int ldx, const float* res, const float* s
   else Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);
 }
 
-void gs_skinny_run_qkv(const void* X, int ldx, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
+void gs_skinny_run_qkv(const void* X, int ldx, int x_tiled, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
                        const void* Wt, const float* qw, const float* kw, float head_eps, const float* cos_t,
                        const float* sin_t, const int* positions, const int* block_table, int max_blocks,
                        int page_size, void* kcache, void* vcache, int write_kv, void* Q, int M, int nh, int nkv, int d,
                        int K, hipStream_t stream) {
-  SkinnyCall c = base(X, ldx, W, Wt, Q, GS_BF16, nh * d, M, (nh + 2 * nkv) * d, K, 4, stream);
+  SkinnyCall c = base(X, ldx, x_tiled, W, Wt, Q, GS_BF16, nh * d, M, (nh + 2 * nkv) * d, K, 4, stream);
   if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.qw = qw; c.ex.kw = kw; c.ex.head_eps = head_eps; c.ex.cos_t = cos_t; c.ex.sin_t = sin_t;
   c.ex.positions = positions; c.ex.block_table = block_table; c.ex.max_blocks = max_blocks; c.ex.page_size = page_size;
@@ -70,8 +74,8 @@ void gs_skinny_run_qkv(const void* X, int ldx, const float* res, const float* ss
   Wt ? gs_skinny_qkv_tiles(c, d) : gs_skinny_qkv_rows(c, d);
 }
 
-void gs_skinny_run_parts(const void* X, int ldx, const void* W, const void* Wt, float* part, int parts, int M, int N,
+void gs_skinny_run_parts(const void* X, int ldx, int x_tiled, const void* W, const void* Wt, float* part, int parts, int M, int N,
                          int K, hipStream_t stream) {
-  SkinnyCall c = base(X, ldx, W, Wt, part, GS_F32, N, M, N, K, 5, stream);
+  SkinnyCall c = base(X, ldx, x_tiled, W, Wt, part, GS_F32, N, M, N, K, 5, stream);
   Wt ? gs_skinny_parts_tiles(c, parts) : gs_skinny_parts_rows(c, parts);
 }

@@ -18,6 +18,12 @@
 // contiguous kilobyte and a wavefront streams a contiguous range, which HBM serves faster than
 // sixteen rows 2 K bytes apart.
 //
+// X is read either as rows of ldx elements or, with x_tiled, in the order the MFMA takes it ("tiled rows",
+// tiled_index in common.h: the 16 x 32 tile of (k step, row tile) as 64 lanes x 16 bytes): then every load of X is one
+// contiguous kilobyte instead of sixteen pieces of rows, which is what the products of many rows are bound by.  With
+// y_tiled the epilogues that write rows for a following product (SwiGLU, convolution, pre-weighted rows) write them
+// in that order.
+//
 // What feeds X (PRO):
 //   0  X is given, bfloat16.
 //   1  X is the RMSNorm of the float32 residual stream: x = res * inv_rms(row) * norm_weight, rounded to
@@ -106,6 +112,9 @@ struct SkinnyExtra {
   int max_blocks, page_size, nh, nkv, write_kv;
   bf16* kcache;
   bf16* vcache;
+  // layouts
+  int x_tiled;           // X comes as tiled rows (PRO 0 only; K a multiple of 32)
+  int y_tiled;           // EPI 1, 3: Y, EPI 2: xs_out are written as tiled rows (their width a multiple of 32)
 };
 
 template <int R, int MT, int WAVES, int PRO, int EPI, int SHUF, typename TOut>
@@ -163,7 +172,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     rrow[mt] = nullptr;
     inv[mt] = 0.f;
     if (PRO == 0) {
-      xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * ldx;
+      xrow[mt] = ex.x_tiled ? X + (size_t)(mt * 64 + lane) * 8 : X + (size_t)(xok[mt] ? m : 0) * ldx + kg * 8;
     } else {
       rrow[mt] = ex.res + (size_t)(xok[mt] ? m : 0) * K;
     }
@@ -276,10 +285,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  auto load_x = [&](int mt, int k) -> bf16x8_t {
+  const int xstep = ex.x_tiled ? MT * 512 : 32;   // elements between a row tile's consecutive k steps
+  auto load_x = [&](int mt, int s) -> bf16x8_t {
     if (PRO == 0) {
-      return load8(xrow[mt] + k);
+      return load8(xrow[mt] + (size_t)s * xstep);
     } else {
+      const int k = (s << 5) + kg * 8;
       const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(rrow[mt] + k);
       const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(rrow[mt] + k + 4);
       const f32x4_t w0 = *reinterpret_cast<const f32x4_t*>(ex.norm_w + k);
@@ -319,11 +330,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       bf16x8_t a[U][R], b[U][MT];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int k = ((s + u) << 5) + kg * 8;
 #pragma unroll
         for (int r = 0; r < R; ++r) a[u][r] = wact ? load8(wrow[r] + (size_t)(s + u) * WSTEP) : zero8();
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) b[u][mt] = xok[mt] ? load_x(mt, k) : zero8();
+        for (int mt = 0; mt < MT; ++mt) b[u][mt] = xok[mt] ? load_x(mt, s + u) : zero8();
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
@@ -339,7 +349,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     const bool kin = k < K;
     bf16x8_t b[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) b[mt] = (kin && xok[mt]) ? load_x(mt, k) : zero8();
+    for (int mt = 0; mt < MT; ++mt) b[mt] = (kin && xok[mt]) ? load_x(mt, s) : zero8();
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       bf16x8_t a = ((kin || SHUF) && wact) ? load8(wrow[r] + (size_t)s * WSTEP) : zero8();
@@ -414,7 +424,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         f32x4_t g = acc[r][mt], u = acc[r + 1][mt], o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = g[i] / (1.0f + expf(-g[i])) * u[i];
-        if (half - n > 0) store4<TOut>(Y + (size_t)m * ldy + n, o, half - n);
+        if (half - n > 0) store4<TOut>(Y + (ex.y_tiled ? tiled_index(m, n, MT) : (size_t)m * ldy + n), o, half - n);
       }
     } else if (EPI == 2) {
       // every lane takes part in the shuffles, live or not
@@ -436,7 +446,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
           else
             for (int i = 0; i < 4; ++i)
               if (n + i < N) p[i] = nv[i];
-          if (ex.xs_out) store4<bf16>(ex.xs_out + (size_t)m * N + n, xv, N - n);
+          if (ex.xs_out) store4<bf16>(ex.xs_out + (ex.y_tiled ? tiled_index(m, n, MT) : (size_t)m * N + n), xv, N - n);
         }
       }
       ss += __shfl_xor(ss, 16, 64);
@@ -464,7 +474,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
           for (int p = 0; p < PRE_TAPS; ++p)
             if (p == Wd - 1) y += ctap[i][p] * u;
           if (ex.conv_bias) y += cbias[i];
-          Y[(size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
+          Y[ex.y_tiled ? tiled_index(m, c, MT) : (size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
 #pragma unroll
           for (int p = 0; p < PRE_TAPS - 2; ++p)
             if (p < Wd - 2) hist[p] = chist[mt][i][p + 1];
@@ -475,7 +485,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
           for (int p = 0; p < Wd - 1; ++p) y += wt[p] * hist[p];
           y += wt[Wd - 1] * u;
           if (ex.conv_bias) y += ex.conv_bias[c];
-          Y[(size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
+          Y[ex.y_tiled ? tiled_index(m, c, MT) : (size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
           for (int p = 0; p < Wd - 2; ++p) hist[p] = hist[p + 1];
           hist[Wd - 2] = u;
         }

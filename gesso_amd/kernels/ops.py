@@ -71,13 +71,68 @@ def _i32(t, n=None, what="index"):
         _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} needed")
 
 
+# ---------------------------------------------------------------------- tiled rows
+
+class TiledRows:
+    """Rows of bfloat16 that feed a weight-streaming product, kept in the order the matrix cores take them.
+
+    ``(M, K)`` with K a multiple of 32; the buffer holds, for each step of 32 columns and each tile of 16 rows,
+    64 lanes x 16 bytes: lane ``l`` has row ``l % 16``, columns ``8 (l / 16) ... + 7`` of the step.  A product reads
+    such a tile with one contiguous kilobyte per wavefront instead of sixteen pieces of rows.  Kernels that write
+    rows for a product (embedding, the SwiGLU, convolution and residual epilogues, decode attention) write this
+    order when handed one of these; the products read it.  ``rows()`` gives the ordinary tensor.
+    """
+
+    __slots__ = ("buf", "shape", "dtype", "device")
+
+    def __init__(self, M: int, K: int, device):
+        _need(K % 32 == 0, f"tiled rows are a multiple of 32 wide, not {K}")
+        self.buf = torch.empty(((M + 15) // 16) * 16 * K, dtype=torch.bfloat16, device=device)
+        self.shape = (M, K)
+        self.dtype = torch.bfloat16
+        self.device = self.buf.device
+
+    @staticmethod
+    def fits(K: int) -> bool:
+        return K % 32 == 0
+
+    @classmethod
+    def of(cls, x: torch.Tensor) -> "TiledRows":
+        """The tiled copy of a bfloat16 tensor ``(M, K)``."""
+        _need(x.dim() == 2 and x.dtype == torch.bfloat16 and x.stride(1) == 1, "tiled rows are made from bfloat16 (M, K)")
+        M, K = x.shape
+        t = cls(M, K, x.device)
+        t.buf.zero_()
+        _check(lib().gs_retile_rows(_p(x), _p(t.buf), c_int(M), c_int(K), c_int(x.stride(0) if M > 1 else K), c_int(1),
+                                    _stream()))
+        return t
+
+    def rows(self) -> torch.Tensor:
+        M, K = self.shape
+        out = torch.empty((M, K), dtype=torch.bfloat16, device=self.device)
+        _check(lib().gs_retile_rows(_p(self.buf), _p(out), c_int(M), c_int(K), c_int(K), c_int(0), _stream()))
+        return out
+
+
+def _rows_out(out, M, N, device, dtype=torch.bfloat16):
+    """An output of rows ``(M, N)``: a tensor, or tiled rows when ``out`` is True (made here) or a TiledRows."""
+    if out is True:
+        out = TiledRows(M, N, device)
+    if isinstance(out, TiledRows):
+        _need(out.shape == (M, N), f"tiled rows of shape {out.shape}, expected {(M, N)}")
+        return out, out.buf, 1
+    if out is None or out is False:
+        out = torch.empty((M, N), dtype=dtype, device=device)
+    return out, out, 0
+
+
 # ---------------------------------------------------------------------- elementwise
 
 def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq: torch.Tensor = None,
           next_weight: torch.Tensor = None, xs: torch.Tensor = None) -> torch.Tensor:
     """``out[t] = table[ids[t]]`` as float32 ``(T, H)``; with ``ssq (T, 1)`` also each row's sum of squares;
     with ``next_weight (H,)`` and ``xs (T, H)`` bfloat16 also ``xs = out * next_weight``."""
-    _dev(ids, table, out, ssq, next_weight, xs)
+    _dev(ids, table, out, ssq, next_weight, None if isinstance(xs, TiledRows) else xs)
     _i32(ids, what="token ids")
     V, H = table.shape
     T = ids.numel()
@@ -86,11 +141,14 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq:
     _need(out.dtype == torch.float32 and out.shape == (T, H), "embed: out must be float32 (T, H)")
     _need(ssq is None or (ssq.dtype == torch.float32 and ssq.numel() == T), "embed: ssq must be float32 (T, 1)")
     _need((next_weight is None) == (xs is None), "embed: next_weight and xs come together")
+    xs_buf, xs_tiled = xs, 0
     if xs is not None:
+        if isinstance(xs, TiledRows):
+            xs_buf, xs_tiled = xs.buf, 1
         _need(next_weight.dtype == torch.float32 and next_weight.shape == (H,) and xs.dtype == torch.bfloat16
-              and xs.shape == (T, H) and xs.is_contiguous(), "embed: next_weight float32 (H,), xs bfloat16 (T, H)")
-    _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), _p(ssq), _p(next_weight), _p(xs), c_int(T), c_int(H),
-                          c_int(V), _stream()))
+              and tuple(xs.shape) == (T, H) and xs_buf.is_contiguous(), "embed: next_weight float32 (H,), xs bfloat16 (T, H)")
+    _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), _p(ssq), _p(next_weight), _p(xs_buf), c_int(xs_tiled),
+                          c_int(T), c_int(H), c_int(V), _stream()))
     return out
 
 
@@ -304,6 +362,9 @@ SKINNY_MAX_ROWS = 64
 
 def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the weight-streaming kernel takes this product (few rows, bfloat16, aligned rows)."""
+    if isinstance(x, TiledRows):
+        return (w.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and w.is_contiguous()
+                and w.data_ptr() % 16 == 0)
     return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[0] <= SKINNY_MAX_ROWS
             and x.shape[1] % 8 == 0 and x.stride(1) == 1 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0)
             and x.data_ptr() % 16 == 0 and w.is_contiguous() and w.data_ptr() % 16 == 0)
@@ -348,10 +409,18 @@ def lazy_ok(x, w: torch.Tensor) -> bool:
 def _lazy_args(x):
     if isinstance(x, LazyNorm):
         if x.xs is not None:
-            return (_p(x.xs), c_int(x.res.shape[1]), None, _p(x.ssq), c_int(x.ssq.shape[1]), None, c_float(x.eps))
-        return (None, c_int(x.res.shape[1]), _p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight), c_float(x.eps))
+            return _x_args(x.xs) + (None, _p(x.ssq), c_int(x.ssq.shape[1]), None, c_float(x.eps))
+        return (None, c_int(x.res.shape[1]), c_int(0), _p(x.res), _p(x.ssq), c_int(x.ssq.shape[1]), _p(x.weight),
+                c_float(x.eps))
+    return _x_args(x) + (None, None, c_int(0), None, c_float(0.0))
+
+
+def _x_args(x):
+    """Pointer, row stride and layout flag of a product's rows."""
     M, K = x.shape
-    return (_p(x), c_int(x.stride(0) if M > 1 else K), None, None, c_int(0), None, c_float(0.0))
+    if isinstance(x, TiledRows):
+        return (_p(x.buf), c_int(K), c_int(1))
+    return (_p(x), c_int(x.stride(0) if M > 1 else K), c_int(0))
 
 
 def tile_major(w: torch.Tensor) -> torch.Tensor:
@@ -365,13 +434,13 @@ def tile_major(w: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, swiglu: bool = False, wt=None):
+def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out=None, swiglu: bool = False, wt=None):
     """``x @ w.T`` for at most 64 rows, streaming the weights once; optionally ``silu(gate) * up`` of the result.
 
-    ``x`` is a bfloat16 tensor or a :class:`LazyNorm`.  With ``swiglu`` the weight holds gate rows then up
-    rows and the output is half as wide.
+    ``x`` is a bfloat16 tensor, :class:`TiledRows` or a :class:`LazyNorm`.  With ``swiglu`` the weight holds gate
+    rows then up rows and the output is half as wide, and ``out`` may be True or a :class:`TiledRows` for tiled rows.
     """
-    _dev(w, out)
+    _dev(w, out if isinstance(out, torch.Tensor) else None)
     lazy = isinstance(x, LazyNorm)
     _need(lazy_ok(x, w) if lazy else skinny_ok(x, w),
           "gemm_skinny: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
@@ -379,12 +448,12 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, sw
     N = w.shape[0]
     _need(w.shape == (N, K), f"gemm_skinny: weight is {tuple(w.shape)}, expected ({N}, {K})")
     cols = N // 2 if swiglu else N
-    if out is None:
-        out = torch.empty((M, cols), dtype=out_dtype or torch.bfloat16, device=w.device)
-    _need(out.shape == (M, cols) and out.stride(1) == 1, "gemm_skinny: out has the wrong shape")
-    _check(lib().gs_gemm_skinny(*_lazy_args(x), _p(w), _p(wt), _p(out), c_int(_dt(out)),
-                                c_int(out.stride(0) if M > 1 else cols), c_int(M), c_int(N), c_int(K),
-                                c_int(1 if swiglu else 0), _stream()))
+    out, buf, tiled = _rows_out(out, M, cols, w.device, out_dtype or torch.bfloat16)
+    _need(not tiled or swiglu, "gemm_skinny: only the SwiGLU epilogue writes tiled rows")
+    _need(tiled or (out.shape == (M, cols) and out.stride(1) == 1), "gemm_skinny: out has the wrong shape")
+    _check(lib().gs_gemm_skinny(*_lazy_args(x), _p(w), _p(wt), _p(buf), c_int(_dt(out)),
+                                c_int(cols if tiled or M <= 1 else out.stride(0)), c_int(M), c_int(N), c_int(K),
+                                c_int(1 if swiglu else 0), c_int(tiled), _stream()))
     return out
 
 
@@ -392,7 +461,7 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt
                          xs: torch.Tensor = None) -> torch.Tensor:
     """``res += x @ w.T`` in place (float32); returns the new rows' sums of squares as partial sums ``(M, nb)``.
     With ``next_weight (N,)`` and ``xs (M, N)`` bfloat16 also ``xs = res * next_weight``."""
-    _dev(w, res, next_weight, xs)
+    _dev(w, res, next_weight, None if isinstance(xs, TiledRows) else xs)
     _need(skinny_ok(x, w), "gemm_skinny_residual: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
     M, K = x.shape
     N = w.shape[0]
@@ -400,19 +469,22 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, wt
     nb = lib().gs_gemm_skinny_residual_blocks(c_int(N), c_int(0 if wt is None else 1))
     ssq = torch.empty((M, nb), dtype=torch.float32, device=res.device)
     _need((next_weight is None) == (xs is None), "gemm_skinny_residual: next_weight and xs come together")
+    xs_buf, xs_tiled = xs, 0
     if xs is not None:
+        if isinstance(xs, TiledRows):
+            xs_buf, xs_tiled = xs.buf, 1
         _need(next_weight.dtype == torch.float32 and next_weight.shape == (N,) and xs.dtype == torch.bfloat16
-              and xs.shape == (M, N) and xs.is_contiguous(), "gemm_skinny_residual: next_weight float32 (N,), xs bfloat16 (M, N)")
-    _check(lib().gs_gemm_skinny_residual(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(wt), _p(res), _p(ssq),
-                                         _p(next_weight), _p(xs), c_int(M), c_int(N), c_int(K), _stream()))
+              and tuple(xs.shape) == (M, N) and xs_buf.is_contiguous(), "gemm_skinny_residual: next_weight float32 (N,), xs bfloat16 (M, N)")
+    _check(lib().gs_gemm_skinny_residual(*_x_args(x), _p(w), _p(wt), _p(res), _p(ssq), _p(next_weight), _p(xs_buf),
+                                         c_int(xs_tiled), c_int(M), c_int(N), c_int(K), _stream()))
     return ssq
 
 
-def gemm_skinny_residual_parts(x: torch.Tensor, w: torch.Tensor, res: torch.Tensor, parts: int, wt=None,
-                               next_weight=None, eps: float = 0.0, out_dtype=None):
+def gemm_skinny_residual_parts(x, w: torch.Tensor, res: torch.Tensor, parts: int, wt=None,
+                               next_weight=None, eps: float = 0.0, out_dtype=None, tiled: bool = False):
     """``res += x @ w.T`` for up to 64 rows in two kernels: partial sums over ``parts`` parts of K from many blocks,
     then one pass that adds them to the stream.  Returns ``(ssq (M, 1), normed)``: the new rows' sums of squares and,
-    with ``next_weight``, the rows normed with that weight and ``eps`` (else None)."""
+    with ``next_weight``, the rows normed with that weight and ``eps`` (else None; as :class:`TiledRows` with ``tiled``)."""
     _dev(w, res, next_weight)
     _need(skinny_ok(x, w), "gemm_skinny_residual_parts: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
     M, K = x.shape
@@ -421,21 +493,24 @@ def gemm_skinny_residual_parts(x: torch.Tensor, w: torch.Tensor, res: torch.Tens
           "gemm_skinny_residual_parts: shapes")
     _need(1 <= parts <= 64, "gemm_skinny_residual_parts: 1 to 64 parts")
     part = torch.empty((parts, M, N), dtype=torch.float32, device=res.device)
-    _check(lib().gs_gemm_skinny_parts(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(wt), _p(part), c_int(parts),
-                                      c_int(M), c_int(N), c_int(K), _stream()))
+    _check(lib().gs_gemm_skinny_parts(*_x_args(x), _p(w), _p(wt), _p(part), c_int(parts), c_int(M), c_int(N), c_int(K),
+                                      _stream()))
     ssq = torch.empty((M, 1), dtype=torch.float32, device=res.device)
     normed = None
     if next_weight is not None:
         _need(next_weight.dtype == torch.float32 and next_weight.shape == (N,), "next_weight must be float32 (N,)")
-        normed = torch.empty((M, N), dtype=out_dtype or torch.bfloat16, device=res.device)
+        normed, nbuf, ntiled = _rows_out(bool(tiled), M, N, res.device, out_dtype or torch.bfloat16)
+    else:
+        nbuf, ntiled = None, 0
     _check(lib().gs_residual_from_parts(_p(part), c_int(parts), _p(res), _p(ssq), _p(next_weight), c_float(eps),
-                                        _p(normed), c_int(_dt(normed) if normed is not None else 1), c_int(M), c_int(N),
-                                        _stream()))
+                                        _p(nbuf), c_int(_dt(normed) if normed is not None else 1), c_int(ntiled),
+                                        c_int(M), c_int(N), _stream()))
     return ssq, normed
 
 
-def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None) -> torch.Tensor:
-    """A decode step's gated short convolution fused into its input product; ``state`` is advanced."""
+def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None, tiled: bool = False):
+    """A decode step's gated short convolution fused into its input product; ``state`` is advanced.
+    With ``tiled`` the mixed rows come as :class:`TiledRows`."""
     _dev(w_in, taps, bias, state, slots)
     _need(lazy_ok(x, w_in) if isinstance(x, LazyNorm) else skinny_ok(x, w_in),
           "gemm_skinny_conv: needs bfloat16 rows or a lazy norm, and a bfloat16 weight")
@@ -446,9 +521,9 @@ def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None) -> torch.Tensor
           "gemm_skinny_conv: taps float32 (H, W), state float32 (slots, H, W-1)")
     _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (H,)), "gemm_skinny_conv: bias float32 (H,)")
     _i32(slots, M, "slots")
-    out = torch.empty((M, H), dtype=torch.bfloat16, device=w_in.device)
-    _check(lib().gs_gemm_skinny_conv(*_lazy_args(x), _p(w_in), _p(wt), _p(taps), _p(bias), _p(state), _p(slots), c_int(W), _p(out), c_int(M),
-                                     c_int(H), c_int(K), _stream()))
+    out, buf, otiled = _rows_out(bool(tiled), M, H, w_in.device)
+    _check(lib().gs_gemm_skinny_conv(*_lazy_args(x), _p(w_in), _p(wt), _p(taps), _p(bias), _p(state), _p(slots), c_int(W),
+                                     _p(buf), c_int(otiled), c_int(M), c_int(H), c_int(K), _stream()))
     return out
 
 
@@ -516,9 +591,10 @@ def _decode_workspace(device, nseq, nh, nkv, d, nsplit):
 
 
 def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_size, window, scale, nh, nkv, d, nseq,
-                     nsplit: int, out: torch.Tensor = None) -> torch.Tensor:
-    """One query per sequence over its paged keys (bfloat16), keys split over ``nsplit`` blocks per key head."""
-    _dev(q, kcache, vcache, positions, block_table, out)
+                     nsplit: int, out=None):
+    """One query per sequence over its paged keys (bfloat16), keys split over ``nsplit`` blocks per key head.
+    ``out``: a tensor, or True / a :class:`TiledRows` for tiled rows."""
+    _dev(q, kcache, vcache, positions, block_table, out if isinstance(out, torch.Tensor) else None)
     _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
           "attention_decode takes bfloat16")
     _need(q.numel() >= (nseq - 1) * q_stride + nh * d if nseq else True, "attention_decode: q is too small")
@@ -528,13 +604,12 @@ def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_s
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= nseq,
           "block_table must be int32 (nseq, max_blocks)")
     ws = _decode_workspace(q.device, nseq, nh, nkv, d, nsplit)
-    if out is None:
-        out = torch.empty((nseq, nh * d), dtype=q.dtype, device=q.device)
-    _need(out.shape == (nseq, nh * d) and out.dtype == q.dtype, "attention_decode: out has the wrong shape or type")
+    out, buf, tiled = _rows_out(out, nseq, nh * d, q.device, q.dtype)
+    _need(tuple(out.shape) == (nseq, nh * d) and out.dtype == q.dtype, "attention_decode: out has the wrong shape or type")
     _check(lib().gs_attention_decode(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
                                      c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
-                                     _p(out), _p(ws), c_int(nseq), c_int(nh), c_int(nkv), c_int(d), c_int(nsplit),
-                                     _stream()))
+                                     _p(buf), c_int(tiled), _p(ws), c_int(nseq), c_int(nh), c_int(nkv), c_int(d),
+                                     c_int(nsplit), _stream()))
     return out
 
 
@@ -544,10 +619,11 @@ def attention_decode_raw_supports(nh: int, nkv: int, d: int, rotary_dim: int) ->
 
 def attention_decode_raw(qkv, q_stride, kcache, vcache, positions, block_table, page_size, window, scale, q_weight,
                          k_weight, head_eps, cos, sin, nh, nkv, d, nseq, nsplit: int, write_kv: bool = True,
-                         out: torch.Tensor = None) -> torch.Tensor:
+                         out=None):
     """Decode attention straight from the rows of q|k|v as their product left them: the kernel norms and rotates
     the queries and the new key, writes the new key and value into their pages, and attends."""
-    _dev(qkv, kcache, vcache, positions, block_table, q_weight, k_weight, cos, sin, out)
+    _dev(qkv, kcache, vcache, positions, block_table, q_weight, k_weight, cos, sin,
+         out if isinstance(out, torch.Tensor) else None)
     _need(qkv.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
           "attention_decode_raw takes bfloat16")
     _need(qkv.numel() >= (nseq - 1) * q_stride + (nh + 2 * nkv) * d if nseq else True, "attention_decode_raw: qkv is too small")
@@ -561,14 +637,13 @@ def attention_decode_raw(qkv, q_stride, kcache, vcache, positions, block_table, 
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= nseq,
           "block_table must be int32 (nseq, max_blocks)")
     ws = _decode_workspace(qkv.device, nseq, nh, nkv, d, nsplit)
-    if out is None:
-        out = torch.empty((nseq, nh * d), dtype=qkv.dtype, device=qkv.device)
-    _need(out.shape == (nseq, nh * d) and out.dtype == qkv.dtype, "attention_decode_raw: out has the wrong shape or type")
+    out, buf, tiled = _rows_out(out, nseq, nh * d, qkv.device, qkv.dtype)
+    _need(tuple(out.shape) == (nseq, nh * d) and out.dtype == qkv.dtype, "attention_decode_raw: out has the wrong shape or type")
     _check(lib().gs_attention_decode_raw(_p(qkv), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
                                          c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0),
                                          c_float(scale), _p(q_weight), _p(k_weight), c_float(head_eps), _p(cos), _p(sin),
-                                         c_int(d), c_int(1 if write_kv else 0), _p(out), _p(ws), c_int(nseq), c_int(nh),
-                                         c_int(nkv), c_int(d), c_int(nsplit), _stream()))
+                                         c_int(d), c_int(1 if write_kv else 0), _p(buf), c_int(tiled), _p(ws), c_int(nseq),
+                                         c_int(nh), c_int(nkv), c_int(d), c_int(nsplit), _stream()))
     return out
 
 

@@ -91,7 +91,7 @@ class Model:
             first = getattr(order[0], "first_norm", None) if order else None
             res = torch.empty((ctx.T, self.embed.shape[1]), dtype=torch.float32, device=rt.device)
             w = row_weight_of(first, res, rt)
-            xs = torch.empty(res.shape, dtype=torch.bfloat16, device=rt.device) if w is not None else None
+            xs = rt.new_rows(*res.shape) if w is not None else None
             ops.embed(ctx.token_ids, self.embed, out=res, ssq=ssq, next_weight=w, xs=xs)
             stream = ResidualStream(res, ssq=ssq, xs=xs, xs_for=first if xs is not None else None)
         else:

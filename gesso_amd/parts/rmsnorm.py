@@ -47,12 +47,13 @@ class ResidualStream:
                 w = None
             eps = eps if w is not None else 0.0
             self.ssq, self.normed = rt.ops.gemm_skinny_residual_parts(
-                out.x, out.w, self.res, rt.split_parts(out.w), wt=rt._wt(out.w), next_weight=w, eps=eps, out_dtype=rt.dtype)
+                out.x, out.w, self.res, rt.split_parts(out.w), wt=rt._wt(out.w), next_weight=w, eps=eps, out_dtype=rt.dtype,
+                tiled=w is not None and rt.rows_tiled(self.res.shape[1]))
             self.xs_for = next_norm if self.normed is not None else None
         elif isinstance(out, DeferredLinear):
             w = row_weight_of(next_norm, self.res, rt)
             if w is not None:
-                self.xs = torch.empty(self.res.shape, dtype=torch.bfloat16, device=self.res.device)
+                self.xs = rt.new_rows(*self.res.shape)
                 self.xs_for = next_norm
             self.ssq = rt.ops.gemm_skinny_residual(out.x, out.w, self.res, wt=rt._wt(out.w), next_weight=w, xs=self.xs)
         else:

@@ -64,6 +64,9 @@ class Runtime:
         # 48 blocks for LFM2-1.2B, and a block streams weights no faster than about 45 GB/s.  The plain product over
         # the whole chip plus the small kernel for norm, rotation and cache write measured half a percent faster.
         self.fuse_qkv = os.environ.get("GESSO_FUSE_QKV", "0") != "0"
+        # rows handed from one fused kernel to the next product travel in the order the matrix cores take them
+        # (ops.TiledRows): a product then loads them a contiguous kilobyte at a time
+        self.tiled_rows = dtype == torch.bfloat16 and os.environ.get("GESSO_TILED_ROWS", "1") != "0"
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""
@@ -89,8 +92,21 @@ class Runtime:
     def _wt(self, w):
         return self._tiles.get(w.data_ptr())
 
+    def rows_tiled(self, width: int) -> bool:
+        """Whether rows of this width, written by one fused kernel for the next product, are kept as tiled rows."""
+        return self.fused and self.tiled_rows and self.ops.TiledRows.fits(width)
+
+    def new_rows(self, M: int, width: int):
+        """Room for bfloat16 rows that a fused kernel writes for the product that follows."""
+        if self.rows_tiled(width):
+            return self.ops.TiledRows(M, width, self.device)
+        return torch.empty((M, width), dtype=torch.bfloat16, device=self.device)
+
     def _dense(self, x):
-        return x.materialize() if isinstance(x, self.ops.LazyNorm) else x
+        """``x`` as an ordinary tensor, whatever handle it came as."""
+        if isinstance(x, self.ops.LazyNorm):
+            x = x.materialize()
+        return x.rows() if isinstance(x, self.ops.TiledRows) else x
 
     def linear(self, x, w: torch.Tensor, bias=None, out_dtype=None, out=None) -> torch.Tensor:
         """``x @ w.T (+ bias)``; ``w (out, in)``; ``x`` a tensor or a lazy norm."""
@@ -100,6 +116,8 @@ class Runtime:
             if bias is None and self._keep_lazy(x) and ops.lazy_ok(x, w):
                 return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self._wt(w))
             x = x.materialize()
+        if isinstance(x, ops.TiledRows) and not (bias is None and ops.skinny_ok(x, w)):
+            x = x.rows()
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
             if ops.skinny_ok(x, w):
                 return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self._wt(w))
@@ -110,12 +128,13 @@ class Runtime:
     def linear_swiglu(self, x, w13: torch.Tensor) -> torch.Tensor:
         """``silu(x @ w1.T) * (x @ w3.T)`` with ``w13`` holding w1's rows, then w3's."""
         ops = self.ops
+        tiled = self.rows_tiled(w13.shape[0] // 2)
         if isinstance(x, ops.LazyNorm):
             if self._keep_lazy(x) and ops.lazy_ok(x, w13):
-                return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13))
+                return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13), out=tiled)
             x = x.materialize()
         if ops.skinny_ok(x, w13):
-            return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13))
+            return ops.gemm_skinny(x, w13, swiglu=True, wt=self._wt(w13), out=tiled)
         return ops.swiglu(self.linear(x, w13))
 
     def project(self, x: torch.Tensor, w: torch.Tensor, bias=None):
@@ -150,7 +169,8 @@ class Runtime:
         if self.fused and b_in is None and ctx.all_single and taps.shape[1] <= 16:
             x = self._rows(x)
             if ops.lazy_ok(x, w_in) or (not isinstance(x, ops.LazyNorm) and ops.skinny_ok(x, w_in)):
-                return ops.gemm_skinny_conv(x, w_in, taps, b_conv, state, ctx.slots, wt=self._wt(w_in))
+                return ops.gemm_skinny_conv(x, w_in, taps, b_conv, state, ctx.slots, wt=self._wt(w_in),
+                                            tiled=self.rows_tiled(taps.shape[0]))
         x = self._dense(x)
         bcx = self.linear(x, w_in, b_in)
         return ops.short_conv(bcx, taps, b_conv, state, ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq,
@@ -203,11 +223,12 @@ class Runtime:
         shapes they are written for.
         """
         ops = self.ops
+        out = True if self.rows_tiled(nh * d) else None
         if isinstance(q, RawQKV):
-            return self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, ctx.nseq, None)
+            return self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, ctx.nseq, out)
         fast = q.dtype == torch.bfloat16 and cache.page_size >= 2
         if ctx.all_single and fast and ops.attention_decode_supports(nh, nkv, d):
-            return self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, ctx.nseq, None)
+            return self._attention_single(q, q_stride, cache, ctx, window, scale, nh, nkv, d, ctx.nseq, out)
         if (not ctx.all_single and fast and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d)):
             # prompts: queries in tiles per sequence, both products on the matrix cores; tiles of 32 share
             # every key and value fragment between two products, which pays when portions are long

@@ -811,3 +811,126 @@ def test_attention_prefill_far_key_and_supports(ops):
                                 torch.arange(prefix, K, dtype=torch.int32, device=DEV), tiles.to(DEV), table.to(DEV), ps,
                                 None, 1.0 / math.sqrt(d), nh, nkv, d, new)
     close(got, P.causal_attention(q.double(), k.double(), v.double()).reshape(new, -1), torch.bfloat16)
+
+
+# ------------------------------------------------------------------ rows in the matrix cores' order (tiled rows)
+
+
+
+@pytest.mark.parametrize("M,K", [(1, 32), (5, 96), (16, 2048), (33, 64), (64, 8192)])
+def test_tiled_rows_hold_the_same_values(ops, M, K):
+    x = torch.randn(M, K, generator=gen(M + K)).bfloat16().to(DEV)
+    t = ops.TiledRows.of(x)
+    assert t.shape == (M, K) and t.buf.numel() == -(-M // 16) * 16 * K
+    # element (m, k): step k // 32, row tile m // 16, lane 16 ((k % 32) // 8) + m % 16, element k % 8
+    for m, k in ((0, 0), (M - 1, K - 1), (M // 2, K // 3), (M - 1, 17)):
+        at = (((k // 32) * (-(-M // 16)) + m // 16) * 64 + ((k % 32) // 8) * 16 + m % 16) * 8 + k % 8
+        assert t.buf[at] == x[m, k]
+    assert torch.equal(t.rows(), x)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(2048, 2048), (128, 64), (6144, 2048), (192, 8192)])
+def test_products_of_tiled_rows_equal_those_of_rows_bit_for_bit(ops, M, N, K):
+    g = gen(M + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    xt = ops.TiledRows.of(x)
+    for wt in (None, ops.tile_major(w)):
+        for kw in ({}, {"out_dtype": torch.float32}, {"swiglu": True}):
+            assert torch.equal(ops.gemm_skinny(xt, w, wt=wt, **kw), ops.gemm_skinny(x, w, wt=wt, **kw))
+        # the SwiGLU epilogue writing tiled rows
+        a = ops.gemm_skinny(xt, w, wt=wt, swiglu=True, out=True)
+        assert isinstance(a, ops.TiledRows) and torch.equal(a.rows(), ops.gemm_skinny(x, w, wt=wt, swiglu=True))
+        # into the residual stream, the rows for the next norm tiled as well
+        res = torch.randn(M, N, generator=g)
+        nw = (1 + 0.3 * torch.randn(N, generator=g)).to(DEV)
+        r1, r2 = res.clone().to(DEV), res.clone().to(DEV)
+        xs1, xs2 = ops.TiledRows(M, N, DEV), torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        s1 = ops.gemm_skinny_residual(xt, w, r1, wt=wt, next_weight=nw, xs=xs1)
+        s2 = ops.gemm_skinny_residual(x, w, r2, wt=wt, next_weight=nw, xs=xs2)
+        assert torch.equal(r1, r2) and torch.equal(s1, s2) and torch.equal(xs1.rows(), xs2)
+        # a product of the pre-weighted tiled rows, scaled by the rows' inverse root mean squares
+        w2 = (torch.randn(64, N, generator=g) / math.sqrt(N)).bfloat16().to(DEV)
+        l1 = ops.LazyNorm(r1, s1, nw, 1e-5, torch.bfloat16, xs=xs1)
+        l2 = ops.LazyNorm(r2, s2, nw, 1e-5, torch.bfloat16, xs=xs2)
+        assert torch.equal(ops.gemm_skinny(l1, w2), ops.gemm_skinny(l2, w2))
+        # in parts, the normed rows tiled
+        for parts in (1, 4):
+            r1, r2 = res.clone().to(DEV), res.clone().to(DEV)
+            q1, n1 = ops.gemm_skinny_residual_parts(xt, w, r1, parts, wt=wt, next_weight=nw, eps=1e-5, tiled=True)
+            q2, n2 = ops.gemm_skinny_residual_parts(x, w, r2, parts, wt=wt, next_weight=nw, eps=1e-5)
+            assert isinstance(n1, ops.TiledRows)
+            assert torch.equal(r1, r2) and torch.equal(q1, q2) and torch.equal(n1.rows(), n2)
+
+
+@pytest.mark.parametrize("M,H,W,bias", [(1, 64, 3, False), (8, 2048, 3, False), (20, 96, 4, True), (64, 160, 2, False),
+                                         (40, 2048, 3, False)])
+def test_convolution_product_of_tiled_rows(ops, M, H, W, bias):
+    g = gen(M + H + W)
+    x = torch.randn(M, H, generator=g).bfloat16().to(DEV)
+    w_in = (torch.randn(3 * H, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
+    taps = torch.randn(H, W, generator=g).to(DEV)
+    b = torch.randn(H, generator=g).to(DEV) if bias else None
+    state0 = torch.randn(M + 2, H, W - 1, generator=g)
+    slots = torch.randperm(M + 2, generator=g)[:M].to(torch.int32).to(DEV)
+    for wt in (None, ops.tile_major(w_in)):
+        s1, s2 = state0.clone().to(DEV), state0.clone().to(DEV)
+        got = ops.gemm_skinny_conv(ops.TiledRows.of(x), w_in, taps, b, s1, slots, wt=wt, tiled=True)
+        want = ops.gemm_skinny_conv(x, w_in, taps, b, s2, slots, wt=wt)
+        assert isinstance(got, ops.TiledRows) and torch.equal(got.rows(), want) and torch.equal(s1, s2)
+
+
+@pytest.mark.parametrize("T,H,V", [(1, 2048, 1000), (9, 96, 301), (40, 64, 50)])
+def test_embed_writes_tiled_rows(ops, T, H, V):
+    g = gen(T + H)
+    table = torch.randn(V, H, generator=g).bfloat16().to(DEV)
+    ids = torch.randint(0, V, (T,), generator=g).to(torch.int32).to(DEV)
+    nw = (1 + 0.3 * torch.randn(H, generator=g)).to(DEV)
+    xs1, xs2 = ops.TiledRows(T, H, DEV), torch.empty(T, H, dtype=torch.bfloat16, device=DEV)
+    o1 = ops.embed(ids, table, next_weight=nw, xs=xs1)
+    o2 = ops.embed(ids, table, next_weight=nw, xs=xs2)
+    assert torch.equal(o1, o2) and torch.equal(xs1.rows(), xs2)
+
+
+@pytest.mark.parametrize("nh,nkv,d,nsplit,raw", [(32, 8, 64, 1, True), (32, 8, 64, 4, True), (4, 2, 16, 1, False),
+                                                 (3, 1, 32, 3, False), (8, 1, 128, 2, True)])
+def test_attention_decode_writes_tiled_rows(ops, nh, nkv, d, nsplit, raw):
+    g = gen(nh + d + nsplit)
+    ps, lens = 16, [1, 64, 65, 300, 17, 129] * 4          # 24 sequences: two row tiles
+    nseq = len(lens)
+    nblk = [-(-n // ps) for n in lens]
+    kc = torch.randn(sum(nblk) + 1, nkv, ps, d, generator=g).bfloat16().to(DEV)
+    vc = torch.randn(sum(nblk) + 1, nkv, ps, d, generator=g).bfloat16().to(DEV)
+    table = torch.zeros(nseq, max(nblk), dtype=torch.int32)
+    at = 0
+    for i in range(nseq):
+        table[i, :nblk[i]] = torch.arange(at, at + nblk[i], dtype=torch.int32)
+        at += nblk[i]
+    table = table.to(DEV)
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32).to(DEV)
+    scale = 1.0 / math.sqrt(d)
+    if raw:
+        stride = (nh + 2 * nkv) * d
+        qkv = torch.randn(nseq, stride, generator=g).bfloat16().to(DEV)
+        qw = (1 + 0.2 * torch.randn(d, generator=g)).to(DEV)
+        kw = (1 + 0.2 * torch.randn(d, generator=g)).to(DEV)
+        cos, sin = rope_tables(d, 1e4, 512)
+        run = lambda out: ops.attention_decode_raw(qkv, stride, kc.clone(), vc.clone(), positions, table, ps, None, scale,
+                                                   qw, kw, 1e-5, cos, sin, nh, nkv, d, nseq, nsplit, out=out)
+    else:
+        q = torch.randn(nseq, nh * d, generator=g).bfloat16().to(DEV)
+        run = lambda out: ops.attention_decode(q, nh * d, kc, vc, positions, table, ps, None, scale, nh, nkv, d, nseq,
+                                               nsplit, out=out)
+    got, want = run(True), run(None)
+    assert isinstance(got, ops.TiledRows) and torch.equal(got.rows(), want)
+
+
+def test_tiled_rows_refuse_widths_that_are_no_multiple_of_32(ops):
+    from gesso_amd.errors import KernelError
+    with pytest.raises(KernelError):
+        ops.TiledRows(4, 40, DEV)
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(80, 64, dtype=torch.bfloat16, device=DEV)      # SwiGLU output 40 wide
+    with pytest.raises(KernelError):
+        ops.gemm_skinny(x, w, swiglu=True, out=True)
