@@ -555,6 +555,13 @@ template <int R, int MT, int WAVES, int PRO, int EPI, int SHUF, typename TOut>
 static void launch_skinny(int blocks, const bf16* X, int ldx, const bf16* W, TOut* Y, int ldy, int M, int N, int K,
                           const SkinnyExtra& ex, hipStream_t stream) {
   const size_t lds = (size_t)(WAVES - 1) * R * MT * 256 * sizeof(float);
+  if (lds > 64 * 1024) {
+    // more than the default limit of dynamic LDS: asked for once per kernel
+    static const hipError_t asked = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&gemm_skinny_kernel<R, MT, WAVES, PRO, EPI, SHUF, TOut>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    (void)asked;
+  }
   gemm_skinny_kernel<R, MT, WAVES, PRO, EPI, SHUF, TOut>
       <<<blocks, WAVES * 64, lds, stream>>>(X, ldx, W, Y, ldy, M, N, K, ex);
 }
@@ -600,11 +607,7 @@ static void skinny_plain(const SkinnyCall& c) {
   const int cols = c.epilogue == 1 ? N / 2 : N;
   const bool narrow = cols <= 8192;
   // few output columns: more wavefronts per block split K further, so that the whole chip streams
-  if (c.epilogue == 1 && M > 32 && !pro && cols % 32 == 0 && cols >= 8192) {
-    // many rows: a block that takes four weight tiles reads X half as often per weight byte
-    const int blocks = cols / 32;
-    if (f32) { GS_BY_MT4(4, 4, 4, 4, 4, 0, 1, float, blocks) } else { GS_BY_MT4(4, 4, 4, 4, 4, 0, 1, bf16, blocks) }
-  } else if (c.epilogue == 1) {
+  if (c.epilogue == 1) {
     const int blocks = gs_ceil_div(cols, 16);
     if (pro) { if (f32) { GS_BY_MT4(2, 8, 8, 4, 4, 1, 1, float, blocks) } else { GS_BY_MT4(2, 8, 8, 4, 4, 1, 1, bf16, blocks) } }
     else     { if (f32) { GS_BY_MT4(2, 8, 8, 4, 4, 0, 1, float, blocks) } else { GS_BY_MT4(2, 8, 8, 4, 4, 0, 1, bf16, blocks) } }
@@ -651,7 +654,7 @@ static void skinny_conv(const SkinnyCall& c) {
   const SkinnyExtra& ex = c.ex;
   hipStream_t stream = c.stream;
   const int blocks = gs_ceil_div(N / 3, SHUF == 2 ? 8 : 16);
-  if (ex.res) { GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks) } else { GS_BY_MT4(3, 8, 8, 8, 4, 0, 3, bf16, blocks) }
+  if (ex.res) { GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks) } else { GS_BY_MT4(3, 8, 8, 8, 8, 0, 3, bf16, blocks) }
 }
 
 template <int SHUF>
