@@ -201,13 +201,16 @@ class Runtime:
 
     def _attention_single(self, q, q_stride, cache, ctx, window, scale, nh, nkv, d, nseq, out):
         """The first ``nseq`` sequences, one query each (their rows are the first ``nseq`` rows).  A block of eight
-        wavefronts takes a tile of 64 keys per wavefront and pass; up to two passes stay in one block (no merge
-        kernel), longer key streams are split over blocks."""
+        wavefronts takes a tile of 64 keys per wavefront and pass; key streams are split over blocks (and a merge
+        kernel) only when the batch alone does not fill the chip."""
         longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
         if window:
             longest = min(longest, window)
         tiles = max(1, -(-longest // 64))
-        nsplit = max(1, min(-(-tiles // 16), 64, max(1, 2048 // max(1, nseq * nkv))))
+        # (sequence, key head) pairs fill the chip by themselves from about 256 on; fewer pairs share their keys out
+        # over blocks, each split at least 1,024 keys long (measured at 8 sequences of 32,768 keys: 4 splits 107 us,
+        # 32 splits 145 us; at 64 sequences any split is slower than none)
+        nsplit = max(1, min(tiles // 16, 64, 256 // max(1, nseq * nkv)))
         if isinstance(q, RawQKV):
             return self.ops.attention_decode_raw(q.qkv, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                                  cache.page_size, window, scale, q.q_norm, q.k_norm, q.eps,
