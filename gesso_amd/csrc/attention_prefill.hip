@@ -16,7 +16,7 @@ extern "C" int gs_attention_prefill(const void* q, int q_stride, const void* kca
                                     int page_size, int window, float scale, void* out, int nh, int nkv, int d,
                                     int tile_rows, hipStream_t stream) {
   GS_REQUIRE(gs_attention_prefill_supports(nh, nkv, d), "attention_prefill: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
-  GS_REQUIRE(ntiles >= 0 && nkv <= 65535, "attention_prefill: bad grid");
+  GS_REQUIRE(ntiles >= 0 && nkv > 0 && (long)ntiles * nkv < (1L << 31), "attention_prefill: %d tiles x %d key heads are too many blocks", ntiles, nkv);
   GS_REQUIRE(tile_rows == 16 || tile_rows == 32, "attention_prefill: tiles hold 16 or 32 queries, not %d", tile_rows);
   GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill: bad page_size/max_blocks/window");
   GS_REQUIRE(q_stride >= nh * d && q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_prefill: q rows must be 16-byte aligned");

@@ -47,7 +47,10 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
   constexpr int GT = G * 64;       // threads of a set of wavefronts
   __shared__ uint16_t vt[KSPLIT][D][PF_KSTEP + PF_PAD];
   __shared__ int pages[PF_MAXPAGES];
-  const int tile = gridDim.x - 1 - blockIdx.x, kvh = blockIdx.y;   // late tiles walk the most keys: they start first
+  // Blocks in launch order: key head fastest, tiles from the last one back.  Late tiles walk the most keys, so the
+  // longest walks all start first whatever their head; and consecutive blocks go to consecutive dies, so a die sees
+  // few key heads and their pages stay in its L2.
+  const int kvh = blockIdx.x % nkv, tile = (int)(gridDim.x / nkv) - 1 - (int)(blockIdx.x / nkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int grp = wave / G, gtid = tid - grp * GT;                 // the set, and the thread within it
@@ -333,7 +336,7 @@ static int launch_prefill(int G, dim3 grid, hipStream_t stream, const bf16* q, i
 // All the kernels of one head width (a translation unit each, so that they compile side by side).
 template <int D>
 static int prefill_for_width(const PrefillCall& c) {
-  dim3 grid(c.ntiles, c.nkv);
+  dim3 grid((unsigned)c.ntiles * (unsigned)c.nkv);
   const int G = c.nh / c.nkv;
   // groups of up to four heads share a tile's keys between two sets of wavefronts
   const bool split = G <= 4;
