@@ -313,6 +313,34 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, bias=None, out_dtype=None, out:
     return out
 
 
+def mfma_ok(x, w: torch.Tensor) -> bool:
+    """Whether the matrix-core product for many rows takes these operands (bfloat16, K a multiple of 8, aligned)."""
+    return (isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
+            and x.shape[0] > 0 and x.shape[1] % 8 == 0 and x.stride(1) == 1
+            and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0 and w.is_contiguous()
+            and w.data_ptr() % 16 == 0)
+
+
+def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, out: torch.Tensor = None, swiglu: bool = False):
+    """``x @ w.T`` for many rows on the matrix cores (bfloat16 in, float32 sums, bfloat16 or float32 out); with
+    ``swiglu`` the weight holds gate rows then up rows and the result is ``silu(gate) * up``, half as wide."""
+    _dev(w, out)
+    _need(mfma_ok(x, w), "gemm_mfma: operands must be bfloat16, K a multiple of 8, 16-byte aligned")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape == (N, K), f"gemm_mfma: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    _need(not swiglu or N % 2 == 0, "gemm_mfma: SwiGLU needs gate and up rows")
+    cols = N // 2 if swiglu else N
+    if out is None:
+        out = torch.empty((M, cols), dtype=out_dtype or torch.bfloat16, device=w.device)
+    _need(out.shape == (M, cols) and out.stride(1) == 1, "gemm_mfma: out has the wrong shape")
+    _need(not swiglu or out.dtype == torch.bfloat16, "gemm_mfma: the SwiGLU epilogue stores bfloat16")
+    _check(lib().gs_gemm_mfma(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(out), c_int(_dt(out)),
+                              c_int(out.stride(0) if M > 1 else cols), c_int(M), c_int(N), c_int(K),
+                              c_int(1 if swiglu else 0), _stream()))
+    return out
+
+
 # ---------------------------------------------------------------------- sampling
 
 def argmax_rows(logits: torch.Tensor):

@@ -934,3 +934,59 @@ def test_tiled_rows_refuse_widths_that_are_no_multiple_of_32(ops):
     w = torch.zeros(80, 64, dtype=torch.bfloat16, device=DEV)      # SwiGLU output 40 wide
     with pytest.raises(KernelError):
         ops.gemm_skinny(x, w, swiglu=True, out=True)
+
+
+# ------------------------------------------------------------------ the matrix-core product for many rows
+
+@pytest.mark.parametrize("M,N,K", [(65, 96, 72), (200, 320, 192), (513, 1000, 264), (129, 64, 8), (2048, 6144, 2048),
+                                    (300, 16384, 512), (1, 40, 64), (256, 256, 64)])
+def test_gemm_mfma(ops, M, N, K):
+    g = gen(M + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    want = x.double() @ w.double().T
+    close(ops.gemm_mfma(x.to(DEV), w.to(DEV)), want, torch.bfloat16)
+    got32 = ops.gemm_mfma(x.to(DEV), w.to(DEV), out_dtype=torch.float32)
+    assert got32.dtype == torch.float32
+    # float32 sums of exact products: only the order of the sums differs from the float64 reference
+    assert float((got32.double().cpu() - want).abs().max()) <= 2e-5 * math.sqrt(K) * max(1.0, float(want.abs().max()))
+    # rows of a wider buffer (a row stride beyond K)
+    wide = torch.zeros(M, K + 16, dtype=torch.bfloat16)
+    wide[:, :K] = x
+    assert torch.equal(ops.gemm_mfma(wide.to(DEV)[:, :K], w.to(DEV)), ops.gemm_mfma(x.to(DEV), w.to(DEV)))
+
+
+@pytest.mark.parametrize("M,F,K", [(65, 24, 64), (200, 100, 96), (130, 8192, 256), (700, 1000, 136), (2048, 4608, 1024)])
+def test_gemm_mfma_swiglu(ops, M, F, K):
+    g = gen(M + F + K)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(2 * F, K, generator=g) / math.sqrt(K) * 2).bfloat16()
+    got = ops.gemm_mfma(x.to(DEV), w.to(DEV), swiglu=True)
+    assert got.shape == (M, F)
+    y = x.double() @ w.double().T
+    close(got, P.swiglu(y[:, :F], y[:, F:]), torch.bfloat16, scale=2)
+    # and it is the plain product followed by the SwiGLU kernel, value for value (both round gate and up to bfloat16)
+    two = ops.swiglu(ops.gemm_mfma(x.to(DEV), w.to(DEV)))
+    assert float((got.float() - two.float()).abs().max()) <= 1e-2 * max(1.0, float(two.float().abs().max()))
+
+
+def test_gemm_mfma_stands_out_where_one_weight_row_matters(ops):
+    """A product whose every output is zero but one: a wrong pairing of rows and columns anywhere shows."""
+    M, N, K = 300, 520, 200
+    x = torch.zeros(M, K, dtype=torch.bfloat16)
+    w = torch.zeros(N, K, dtype=torch.bfloat16)
+    for (m, n, k) in ((0, 0, 0), (299, 519, 199), (37, 301, 65), (256, 255, 64), (128, 256, 127)):
+        x[m, k] = 2.0
+        w[n, k] = 3.0
+    got = ops.gemm_mfma(x.to(DEV), w.to(DEV), out_dtype=torch.float32).cpu()
+    want = x.float() @ w.float().T
+    assert torch.equal(got, want) and int((want != 0).sum()) == 5
+
+
+def test_gemm_mfma_refuses(ops):
+    from gesso_amd.errors import KernelError
+    x = torch.zeros(70, 60, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(16, 60, dtype=torch.bfloat16, device=DEV)
+    assert not ops.mfma_ok(x, w)                           # K no multiple of 8
+    with pytest.raises(KernelError):
+        ops.gemm_mfma(x, w)

@@ -121,3 +121,21 @@ def test_replay_of_configurations_drawn_at_random(seed, dtype, tmp_path):
         print(f"seed {seed} ({cfg.num_attention_heads}/{cfg.num_key_value_heads} heads of {cfg.head_dim}) {dtype} {way}: "
               f"worst |diff| {w:.3e} at {where}")
         assert w <= TOL[dtype] * scale, f"{way}: first look at {where}"
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_replay_with_the_hand_written_product_for_many_rows(name, folders, tmp_path, monkeypatch):
+    """Prompts of more than 64 tokens through the hand-written matrix-core product (with its SwiGLU epilogue) instead of
+    the vendor library's: whole, and in portions that change between that kernel and the weight-streaming one."""
+    monkeypatch.setenv("GESSO_GEMM", "own")          # read by the replay program's runtime
+    cfg, _ = CONFIGS[name]
+    model_dir = write_tiny(folders, name, torch.bfloat16)
+    seqs = sequences(name)
+    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
+    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    for way, make in (("whole", R.trace_whole), ("portions", lambda s: R.trace_portions(s, sizes=(70, 3, 66, 2, 90)))):
+        got, rc = R.run_trace(model_dir, "bfloat16", str(tmp_path / way), make(seqs), cfg.vocab_size)
+        assert rc == 0
+        w, where = R.worst(got, ref)
+        print(f"{name} own product, {way}: worst |diff| {w:.3e} at {where}")
+        assert w <= TOL["bfloat16"] * scale, f"{way}: first look at {where}"
