@@ -212,8 +212,44 @@ class DecaySpec:
     kind: str = "toy_decay"
 
 
+@dataclasses.dataclass(frozen=True)
+class RoutedSpec:
+    hidden: int
+    experts: int
+    inner: int
+    kind: str = "toy_routed"
+
+
 def register_toys():
     from gesso_amd.parts import MATRIX, Part, SlotState, TensorSpec, register
+
+    class RoutedFFN(Part):
+        """A feed-forward with routing: router logits in float32, the best expert per token, relu(x U^T) D^T of that
+        expert alone, weighted by the softmax weight of the choice."""
+
+        @staticmethod
+        def tensor_specs(spec):
+            out = {"router.weight": TensorSpec((spec.experts, spec.hidden), MATRIX)}
+            for e in range(spec.experts):
+                out[f"e{e}.up.weight"] = TensorSpec((spec.inner, spec.hidden), MATRIX)
+                out[f"e{e}.down.weight"] = TensorSpec((spec.hidden, spec.inner), MATRIX)
+            return out
+
+        def bind(self, tensors):
+            self.router = tensors["router.weight"]
+            self.up = [tensors[f"e{e}.up.weight"] for e in range(self.spec.experts)]
+            self.down = [tensors[f"e{e}.down.weight"] for e in range(self.spec.experts)]
+
+        def forward(self, x, ctx):
+            logits = self.rt.linear(x, self.router, out_dtype=torch.float32)
+            gate, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+            out = torch.zeros((x.shape[0], self.spec.hidden), dtype=torch.float32, device=x.device)
+            for e in range(self.spec.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    h = torch.relu(self.rt.linear(x[rows].contiguous(), self.up[e]))
+                    out[rows] = self.rt.linear(h, self.down[e]).float() * gate[rows, None]
+            return out.to(x.dtype)
 
     class DecayMixer(Part):
         """s_t = decay * s_{t-1} + x_t W^T, output s_t: a running state per request, of fixed size."""
@@ -257,6 +293,7 @@ def register_toys():
 
     register("mixer", "toy_decay", DecayMixer, replace=True)
     register("position", "toy_scaled_rope", ScaledRope, replace=True)
+    register("ffn", "toy_routed", RoutedFFN, replace=True)
 
 
 def toy_spec():
@@ -266,6 +303,8 @@ def toy_spec():
     pos = dataclasses.replace(RopeSpec(head_dim=16, rotary_dim=16, theta=1e4, max_position=64), kind="toy_scaled_rope")
     attn = AttentionSpec(hidden=H, n_heads=2, n_kv_heads=1, head_dim=16, position=pos, qk_norm=None)
     ffn = SwiGLUSpec(hidden=H, intermediate=24)
+    routed = RoutedSpec(hidden=H, experts=3, inner=16)
+    routed_names = ["router.weight"] + [f"e{e}.{k}.weight" for e in range(3) for k in ("up", "down")]
 
     def names(i, mixer_names):
         n = {"mixer_norm.weight": f"L{i}.n1", "ffn_norm.weight": f"L{i}.n2", "ffn.w1.weight": f"L{i}.w1",
@@ -274,8 +313,10 @@ def toy_spec():
         return n
 
     attn_names = ["q_proj.weight", "k_proj.weight", "v_proj.weight", "out_proj.weight"]
+    n1 = {k: v for k, v in names(1, attn_names).items() if not k.startswith("ffn.")}
+    n1.update({f"ffn.{k}": f"L1.{k}" for k in routed_names})
     blocks = (BlockSpec(DecaySpec(H, 0.5), norm, ffn, norm, names(0, ["proj.weight"])),
-              BlockSpec(attn, norm, ffn, norm, names(1, attn_names)),
+              BlockSpec(attn, norm, routed, norm, n1),
               BlockSpec(attn, norm, None, None, {k: v for k, v in names(2, attn_names).items() if not k.startswith("ffn")}))
     # block 0 runs twice (two states of its own); the last call reads the cache that call 1 wrote
     schedule = (LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(2, cache=1))
@@ -283,9 +324,11 @@ def toy_spec():
                      tie_embeddings=True, max_position=64, names={"embed": "emb", "final_norm.weight": "fn", "head": "head"})
 
 
-def toy_plain(w, ids):
-    """The toy model by hand, whole sequence, float64."""
+def toy_plain(w, ids, margins=None):
+    """The toy model by hand, whole sequence, float64.  ``margins`` collects, per routed layer, the least distance
+    between a token's best and second-best expert (a choice that near a tie may fall either way in bfloat16)."""
     T = len(ids)
+    margins = [] if margins is None else margins
     h = P.embedding(w["emb"], ids)
     eps = 1e-5
 
@@ -301,6 +344,18 @@ def toy_plain(w, ids):
         n = P.rmsnorm(h, w[f"L{i}.n2"], eps)
         return h + P.linear(P.swiglu(P.linear(n, w[f"L{i}.w1"]), P.linear(n, w[f"L{i}.w3"])), w[f"L{i}.w2"])
 
+    def routed_ffn(h, i, margins):
+        n = P.rmsnorm(h, w[f"L{i}.n2"], eps)
+        prob = torch.softmax(P.linear(n, w[f"L{i}.router.weight"]), dim=-1)
+        top = prob.sort(dim=-1, descending=True).values
+        margins.append(float((top[:, 0] - top[:, 1]).min()))
+        gate, choice = prob.max(dim=-1)
+        out = torch.zeros_like(h)
+        for t in range(T):
+            e = int(choice[t])
+            out[t] = P.linear(torch.relu(P.linear(n[t:t + 1], w[f"L{i}.e{e}.up.weight"])), w[f"L{i}.e{e}.down.weight"])[0] * gate[t]
+        return h + out
+
     def qkv(h, i):
         n = P.rmsnorm(h, w[f"L{i}.n1"], eps)
         q = P.linear(n, w[f"L{i}.q_proj.weight"]).reshape(T, 2, 16)
@@ -311,7 +366,7 @@ def toy_plain(w, ids):
 
     h = ffn(decay_block(h, 0), 0)
     q1, k1, v1 = qkv(h, 1)
-    h = ffn(h + P.linear(P.causal_attention(q1, k1, v1).reshape(T, 32), w["L1.out_proj.weight"]), 1)
+    h = routed_ffn(h + P.linear(P.causal_attention(q1, k1, v1).reshape(T, 32), w["L1.out_proj.weight"]), 1, margins)
     h = ffn(decay_block(h, 0), 0)
     q2, _, _ = qkv(h, 2)                                     # its own queries over layer 1's keys and values
     h = h + P.linear(P.causal_attention(q2, k1, v1).reshape(T, 32), w["L2.out_proj.weight"])
@@ -330,8 +385,8 @@ def test_toy_parts_register_build_and_step(fw, dtype):
     try:
         spec = toy_spec()
         table = tensor_table(spec)
-        assert "L0.proj.weight" in table and "L2.w1" not in table
-        cpu = random_tensors(table, 3, dtype, std=0.2)
+        assert "L0.proj.weight" in table and "L2.w1" not in table and "L1.e2.down.weight" in table and "L1.w1" not in table
+        cpu = random_tensors(table, 17, dtype, std=0.2)          # a seed whose routing choices are clear of ties
         eng = Engine(spec, {k: v.to(DEV, held_dtype(v.dtype, table[k].role, dtype)) for k, v in cpu.items()}, dtype,
                      DEV, page_size=4, num_pages=24, num_slots=3)
         lay = eng.manager.layout
@@ -339,7 +394,10 @@ def test_toy_parts_register_build_and_step(fw, dtype):
         assert lay.source_of_call[3] == 1
         ids = {"a": [3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7], "b": [2, 7, 1, 8, 2, 8, 1, 8, 2, 8, 4]}
         w64 = {k: v.double() for k, v in cpu.items()}
-        want = {k: toy_plain(w64, v) for k, v in ids.items()}
+        margins = []
+        want = {k: toy_plain(w64, v, margins) for k, v in ids.items()}
+        assert min(margins) > 0.02, "the fixed weights and ids keep every routing choice clear of a tie"
+
         t = (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, max(float(x.abs().max()) for x in want.values()))
         # whole
         for k, v in ids.items():
@@ -370,3 +428,4 @@ def test_toy_parts_register_build_and_step(fw, dtype):
     finally:
         unregister("mixer", "toy_decay")
         unregister("position", "toy_scaled_rope")
+        unregister("ffn", "toy_routed")
