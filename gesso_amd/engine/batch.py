@@ -35,9 +35,10 @@ def check_entries(entries: List[StepEntry], manager, vocab: int) -> None:
         n = len(e.tokens)
         if n < 1:
             raise InvalidPlan(f"request {e.rid!r} brings no tokens to this step")
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab:
-                raise InvalidPlan(f"token id {int(t)} outside the vocabulary of {vocab}", token=int(t), vocab=vocab)
+        ids = np.asarray(e.tokens, dtype=np.int64)
+        if int(ids.min()) < 0 or int(ids.max()) >= vocab:
+            t = int(ids[(ids < 0) | (ids >= vocab)][0])
+            raise InvalidPlan(f"token id {t} outside the vocabulary of {vocab}", token=t, vocab=vocab)
         for w in e.want:
             if not 0 <= int(w) < n:
                 raise InvalidPlan(f"request {e.rid!r} wants logits at place {w} of {n} tokens")

@@ -17,6 +17,8 @@ an ordinary fill before the replays.
 """
 from __future__ import annotations
 
+import gc
+
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -111,8 +113,17 @@ class DecodeRunner:
         torch.cuda.current_stream().wait_stream(side)
         self.counter.zero_()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            self._body()
+        # no collection of cyclic garbage while the stream is capturing: a finalizer that frees pinned memory or a
+        # graph of an engine long gone makes calls the capture forbids, and the process aborts
+        collecting = gc.isenabled()
+        gc.collect()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                self._body()
+        finally:
+            if collecting:
+                gc.enable()
         self.graphs[bound] = graph
 
     def run(self, rids: Sequence[Hashable], tokens: Sequence[int], n: int, samplers=None

@@ -40,7 +40,7 @@ from .batch import StepEntry
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
 
 
-@dataclass
+@dataclass(eq=False)                                 # a request is itself: compared and hashed by identity
 class Request:
     rid: Hashable
     prompt: List[int]
@@ -68,6 +68,19 @@ class Request:
     @property
     def tokens(self) -> List[int]:
         return self.prompt + self.output
+
+    @property
+    def last_token(self) -> int:
+        return self.output[-1] if self.output else self.prompt[-1]
+
+    def span(self, start: int, count: int) -> List[int]:
+        """``tokens[start:start + count]`` without building the whole list."""
+        n = len(self.prompt)
+        if start + count <= n:
+            return self.prompt[start:start + count]
+        if start >= n:
+            return self.output[start - n:start - n + count]
+        return self.prompt[start:] + self.output[:start + count - n]
 
     @property
     def pending(self) -> int:
@@ -155,8 +168,9 @@ class Scheduler:
         while True:
             budget = self.max_num_batched_tokens
             plan: List[Scheduled] = []
-            decoding = [r for r in self.running if r.pending == 1 and r.computed >= len(r.prompt)]
-            prefilling = [r for r in self.running if r not in decoding]
+            decoding, prefilling = [], []
+            for r in self.running:
+                (decoding if r.pending == 1 and r.computed >= len(r.prompt) else prefilling).append(r)
             for r in decoding:
                 if budget < 1:
                     break
@@ -232,7 +246,7 @@ class Scheduler:
             return run
         entries = []
         for s in plan:
-            toks = s.request.tokens[s.start:s.start + s.count]
+            toks = s.request.span(s.start, s.count)
             entries.append(StepEntry(s.request.rid, toks, [s.count - 1] if s.samples else []))
         try:
             logits = self.executor.step(entries)
@@ -271,7 +285,7 @@ class Scheduler:
             n = 1                     # someone waits: look at admission again after every step
         while n > 1 and self._pages_short([Scheduled(r, r.computed, n, True) for r in reqs]):
             n -= 1
-        ids, bad = ex.decode([r.rid for r in reqs], [r.tokens[-1] for r in reqs], n, [r.sampler for r in reqs])
+        ids, bad = ex.decode([r.rid for r in reqs], [r.last_token for r in reqs], n, [r.sampler for r in reqs])
         self.stats["steps"] += n
         emitted: List[Tuple[Request, int]] = []
         for i, r in enumerate(reqs):
