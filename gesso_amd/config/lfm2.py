@@ -24,6 +24,19 @@ _IGNORED = frozenset({
     "model_type", "torch_dtype", "dtype", "transformers_version", "use_cache",
     "initializer_range", "block_mlp_init_scale", "block_out_init_scale",
     "block_use_xavier_init", "conv_use_xavier_init", "_name_or_path",
+    # where random weights came from
+    "seed", "init_seed", "weights_seed", "std", "init_std", "name", "description", "comment",
+    # what a serialized configuration carries whatever the architecture: output switches, generation defaults,
+    # labels, tokenizer hints.  None of them describes the model's arithmetic.
+    "return_dict", "output_hidden_states", "output_attentions", "torchscript", "use_bfloat16", "tf_legacy_loss",
+    "pruned_heads", "chunk_size_feed_forward", "is_encoder_decoder", "is_decoder", "cross_attention_hidden_size",
+    "add_cross_attention", "tie_encoder_decoder", "max_length", "min_length", "do_sample", "early_stopping",
+    "num_beams", "num_beam_groups", "diversity_penalty", "temperature", "top_k", "top_p", "typical_p",
+    "repetition_penalty", "length_penalty", "no_repeat_ngram_size", "encoder_no_repeat_ngram_size", "bad_words_ids",
+    "num_return_sequences", "output_scores", "return_dict_in_generate", "forced_bos_token_id", "forced_eos_token_id",
+    "remove_invalid_values", "exponential_decay_length_penalty", "suppress_tokens", "begin_suppress_tokens",
+    "finetuning_task", "id2label", "label2id", "tokenizer_class", "prefix", "sep_token_id", "decoder_start_token_id",
+    "task_specific_params", "problem_type", "attn_implementation", "auto_map", "chat_template",
 })
 # Keys that repeat another key or state a fixed property; they must agree with it.
 _MUST_EQUAL = {
@@ -122,7 +135,8 @@ class Lfm2Config:
     @staticmethod
     def from_dict(raw: dict) -> "Lfm2Config":
         for key in raw:
-            if key not in _KNOWN:
+            # (keys that start with an underscore are a writer's private notes)
+            if key not in _KNOWN and not key.startswith("_"):
                 raise ConfigError(f"unsupported config.json key {key!r} (no LFM2 feature declares it)", key=key)
         for key in _REFUSED:
             if raw.get(key) not in (None, False, 0):

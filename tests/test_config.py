@@ -118,6 +118,17 @@ def test_keys_that_may_be_left_out_take_the_published_defaults():
     assert c.intermediate_size == 8192                      # 12288 -> two thirds -> up to a multiple of 256
 
 
+def test_keys_that_say_nothing_about_the_arithmetic_are_passed_over():
+    """What a serialized configuration carries whatever the architecture (output switches, generation defaults, a
+    writer's private notes) is no LFM2 feature and no error; a key nobody knows still is."""
+    c = Lfm2Config.from_dict({**BASE, "return_dict": True, "output_attentions": False, "temperature": 1.0, "top_p": 0.9,
+                              "id2label": {"0": "a"}, "_private_note": "x", "seed": 3, "init_std": 0.02})
+    assert c == Lfm2Config.from_dict(BASE)
+    for key in ("rope_thetta", "quantization_config", "num_experts"):
+        with pytest.raises(ConfigError, match=key):
+            Lfm2Config.from_dict({**BASE, key: 1})
+
+
 def test_other_spellings_of_the_same_facts():
     raw = dict(BASE)
     eps = raw.pop("norm_eps")
