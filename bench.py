@@ -7,7 +7,8 @@ model's forward from the cache, the head, and greedy choice of the token that is
 The default run: 16 layers of the 1.2B sizes, bfloat16, batch 8, 512-token random prompts,
 context 4,096 with 16-token pages.  Prints one JSON line; for more than one GPU it prints
 one line that says so and exits with 2 (this engine runs on one GPU).  ``--workload serve`` and
-``--workload long`` measure two other workloads and print a line of their own.
+``--workload long`` measure two other workloads and print a line of their own; ``--workload gemm`` times the
+products of a 2,048-token prompt one by one, the hand-written kernel beside the vendor library's.
 
 Roofline of the decode step: the bytes it has to read (every weight it uses once, the keys and
 values of the live requests, their convolution state) over its time, against 8 TB/s.  Prefill:
@@ -168,6 +169,38 @@ def serve_workload(seed: int = 5) -> dict:
             "token_budget": 1024, "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
 
 
+def gemm_workload(reps: int = 10) -> dict:
+    """The products of a 2,048-token prompt at LFM2-1.2B sizes, one by one: the hand-written matrix-core kernel (plain,
+    and gate|up with its SwiGLU epilogue) beside the vendor library's, microseconds each on random data."""
+    from gesso_amd.kernels import ops
+    ops.lib()
+    dev = "cuda:0"
+    g = torch.Generator(device="cpu").manual_seed(3)
+    out = {"metric": "products of 2,048 rows at LFM2-1.2B sizes, microseconds (ours plain / ours with SwiGLU / vendor)",
+           "unit": "us", "dtype": "bf16", "data": "synthetic: normal activations, weights N(0, 0.02)"}
+
+    def us(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return round((time.perf_counter() - t0) / reps * 1e6, 1)
+
+    for name, (n, k) in {"gate_up": (16384, 2048), "in_proj": (6144, 2048), "down": (2048, 8192),
+                         "out_proj": (2048, 2048), "qkv": (3072, 2048)}.items():
+        x = torch.randn(2048, k, generator=g).bfloat16().to(dev)
+        w = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(dev)
+        row = {"ours": us(lambda: ops.gemm_mfma(x, w)), "vendor": us(lambda: torch.mm(x, w.t()))}
+        if name == "gate_up":
+            row["ours_swiglu"] = us(lambda: ops.gemm_mfma(x, w, swiglu=True))
+            row["vendor_then_swiglu"] = us(lambda: ops.swiglu(torch.mm(x, w.t())))
+        out[name] = row
+    return out
+
+
 def long_workload(seed: int = 6) -> dict:
     """LFM2-2.6B sizes: prompts of 32,768 tokens in portions of 2,048, then 256 decode steps of 8 such requests."""
     from gesso_amd import Engine, StepEntry
@@ -220,15 +253,16 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="measure the 2,048-token prefill alone (for profiling)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
-                         "sizes at a context of 32,768")
+                         "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
         return 2
     if args.workload != "decode":
-        print(json.dumps(serve_workload() if args.workload == "serve" else long_workload()))
+        run = {"serve": serve_workload, "long": long_workload, "gemm": gemm_workload}[args.workload]
+        print(json.dumps(run()))
         return 0
 
     from gesso_amd import Engine
