@@ -177,10 +177,14 @@ __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, co
                                      const double* __restrict__ u, int* __restrict__ counter,
                                      int* __restrict__ next_ids, int* __restrict__ ring, int* __restrict__ bad_ring,
                                      int* __restrict__ positions, int* __restrict__ kv_len,
-                                     const int* __restrict__ live) {
+                                     const int* __restrict__ live, int max_steps) {
   __shared__ int sid, sbad;
   int row = blockIdx.x, rows = gridDim.x;
   int step = counter[row];
+  // a counter that the host forgot to reset must not write past the rings: such a step goes to the last ring row
+  // and marks itself bad, so the run fails loudly instead of overwriting a neighbour
+  bool over = step < 0 || step >= max_steps;
+  if (over) step = max_steps - 1;
   double T = temperature[row];
   const float* x = logits + (size_t)row * V;
   if (T > 0.0)
@@ -190,8 +194,8 @@ __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, co
   if (threadIdx.x == 0) {
     next_ids[row] = sid;
     ring[(size_t)step * rows + row] = sid;
-    bad_ring[(size_t)step * rows + row] = sbad;
-    counter[row] = step + 1;
+    bad_ring[(size_t)step * rows + row] = over ? 1 : sbad;
+    counter[row] = over ? max_steps : step + 1;
     if (live[row]) {
       positions[row] += 1;
       kv_len[row] += 1;
@@ -201,11 +205,12 @@ __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, co
 
 extern "C" int gs_decode_choose(const float* logits, int rows, int V, const double* temperature, const double* u,
                                 int* counter, int* next_ids, int* ring, int* bad_ring, int* positions, int* kv_len,
-                                const int* live, hipStream_t stream) {
+                                const int* live, int max_steps, hipStream_t stream) {
   GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
+  GS_REQUIRE(max_steps > 0, "decode_choose: the rings hold %d steps", max_steps);
   GS_REQUIRE(counter && positions && kv_len && live, "decode_choose: needs the rows' counters, positions, key counts and live flags");
   decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, counter, next_ids, ring, bad_ring,
-                                                          positions, kv_len, live);
+                                                          positions, kv_len, live, max_steps);
   GS_LAUNCH_CHECK("decode_choose");
   return 0;
 }

@@ -106,6 +106,10 @@ class DecodeRunner:
     def _record(self, bound: int) -> None:
         """One eager run on scratch rows (everything lazily initialised gets initialised), then the capture."""
         self.ctx.max_kv_len = bound
+        # the eager run reads the rows' counters and temperatures as the last run left them (a run of MAX_STEPS steps
+        # leaves the counters at MAX_STEPS, one row past the rings): both start from zero here
+        self.counter.zero_()
+        self.temperature.zero_()
         side = torch.cuda.Stream(device=self.engine.device)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):

@@ -14,7 +14,11 @@ Decisions, all tested without a GPU:
   oldest request first, each at most ``chunk_size`` and together at most the step's budget of
   ``max_num_batched_tokens``.
 * Admission: while fewer than ``max_num_seqs`` requests run, a slot is free and pages for the
-  first portion are free.
+  first portion are free, with ``watermark`` (a fraction of each pool, rounded up to whole pages) left
+  over for the requests that already run; into an idle engine a request is admitted without that margin.
+* Context: a request whose known tokens no longer fit into the context (``manager.max_length``) ends as
+  ``failed`` with :class:`~gesso_amd.errors.ResourceLimit` and keeps the tokens it has; nothing else stops
+  (the reference's ``ERR_RESOURCE_LIMIT``, ``src/Inference/kv_manager.jl:246-257``).
 * Out of pages: the request admitted last is preempted: everything it holds is given back, and
   it returns to the front of the waiting line to be computed again from its prompt and the
   tokens it has generated (its sampler state is kept, so a sampled request draws on where it
@@ -29,6 +33,7 @@ Decisions, all tested without a GPU:
 """
 from __future__ import annotations
 
+import math
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Callable, Deque, Hashable, List, Optional, Sequence, Tuple
@@ -98,13 +103,15 @@ class Scheduled:
 
 class Scheduler:
     def __init__(self, executor, choose: Callable, max_num_seqs: int = 64, max_num_batched_tokens: int = 2048,
-                 chunk_size: int = 1024, decode_run_steps: int = 8):
+                 chunk_size: int = 1024, decode_run_steps: int = 8, watermark: float = 0.01):
         """``executor``: ``add_request``, ``finish_request``, ``step(entries) -> logits`` and ``manager``.
 
         ``choose(logits, samplers) -> ids or exceptions``, one per row.
         """
         if max_num_seqs < 1 or max_num_batched_tokens < 1 or chunk_size < 1:
             raise InvalidPlan("max_num_seqs, max_num_batched_tokens and chunk_size must be positive")
+        if not 0 <= watermark < 1:
+            raise InvalidPlan(f"the admission watermark is a fraction of the pool in [0, 1), not {watermark}")
         self.executor = executor
         self.manager = executor.manager
         self.choose = choose
@@ -112,6 +119,8 @@ class Scheduler:
         self.max_num_batched_tokens = max_num_batched_tokens
         self.chunk_size = chunk_size
         self.decode_run_steps = max(1, decode_run_steps)
+        # pages per pool that an admission leaves free for the requests already running
+        self.keep_free = [int(math.ceil(watermark * p.total)) for p in self.manager.pools]
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []          # in admission order
         self.finished: List[Request] = []
@@ -149,12 +158,22 @@ class Scheduler:
     def _portion(self, r: Request, budget: int) -> int:
         return min(r.pending, self.chunk_size, budget)
 
-    def _pages_short(self, plan: List[Scheduled]) -> bool:
+    def _pages_short(self, plan: List[Scheduled], keep: Sequence[int] = ()) -> bool:
+        """Whether the pools cannot take the plan and still have ``keep[g]`` pages left."""
         need = [0] * len(self.manager.pools)
         for s in plan:
             for g, n in enumerate(self.manager.pages_needed(s.request.rid, s.count)):
                 need[g] += n
-        return any(n > pool.n_free for n, pool in zip(need, self.manager.pools))
+        keep = list(keep) or [0] * len(need)
+        return any(n + k > pool.n_free for n, k, pool in zip(need, keep, self.manager.pools))
+
+    def _outgrown(self, r: Request) -> Optional[ResourceLimit]:
+        """The error of a request whose known tokens do not fit into the context any more, else None."""
+        held = r.computed + r.pending
+        if held <= self.manager.max_length:
+            return None
+        return ResourceLimit(f"request {r.rid!r} would hold {held} tokens, the context holds {self.manager.max_length}",
+                             length=held, max_length=self.manager.max_length)
 
     def schedule(self) -> List[Scheduled]:
         """Decide the next step.  Admits, and preempts if pages run out; returns the plan (may be empty)."""
@@ -164,6 +183,11 @@ class Scheduler:
         for r in [r for r in self.waiting if r.cancelled]:
             self.waiting.remove(r)
             self._finish(r, "cancelled", live=False)
+        # and so do requests that have outgrown the context: each fails alone
+        for r in list(self.running):
+            err = self._outgrown(r)
+            if err is not None:
+                self._finish(r, "failed", error=err)
 
         while True:
             budget = self.max_num_batched_tokens
@@ -195,6 +219,11 @@ class Scheduler:
             # admission, oldest first, while the step has room
             while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
                 r = self.waiting[0]
+                err = self._outgrown(r)
+                if err is not None:
+                    self.waiting.popleft()
+                    self._finish(r, "failed", live=False, error=err)
+                    continue
                 n = self._portion(r, budget)
                 if n < 1:
                     break
@@ -205,7 +234,7 @@ class Scheduler:
                 except OutOfSlots:
                     break
                 trial = plan + [Scheduled(r, 0, n, n == r.pending)]
-                if self._pages_short(trial):
+                if self._pages_short(trial, self.keep_free if self.running else ()):
                     self.executor.finish_request(r.rid)
                     if not self.running:
                         # the pool is empty and the first portion still does not fit: try a smaller one
@@ -283,6 +312,7 @@ class Scheduler:
         n = min(self.decode_run_steps, min(r.max_new_tokens - len(r.output) for r in reqs))
         if self.waiting:
             n = 1                     # someone waits: look at admission again after every step
+        n = min(n, min(self.manager.max_length - r.computed for r in reqs))    # schedule() left each room for one
         while n > 1 and self._pages_short([Scheduled(r, r.computed, n, True) for r in reqs]):
             n -= 1
         ids, bad = ex.decode([r.rid for r in reqs], [r.last_token for r in reqs], n, [r.sampler for r in reqs])

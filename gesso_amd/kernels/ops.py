@@ -585,7 +585,8 @@ def gemm_skinny_qkv(x, wqkv, q_weight, k_weight, head_eps, cos, sin, positions, 
 
 def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live) -> None:
     """Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``; results into the loop's buffers;
-    then the row's counter counts up and a live row moves one position on."""
+    then the row's counter counts up and a live row moves one position on.  A counter at or beyond the rings' step
+    count writes into their last row and marks the step bad."""
     _dev(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "decode_choose: logits are float32 (rows, V)")
     rows, V = logits.shape
@@ -597,7 +598,8 @@ def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, pos
         _i32(t)
     _need(ring.shape == u.shape and bad_ring.shape == u.shape, "decode_choose: buffer shapes")
     _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(u), _p(counter), _p(next_ids),
-                                  _p(ring), _p(bad_ring), _p(positions), _p(kv_len), _p(live), _stream()))
+                                  _p(ring), _p(bad_ring), _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]),
+                                  _stream()))
 
 
 def attention_decode_supports(nh: int, nkv: int, d: int) -> bool:

@@ -325,3 +325,45 @@ def test_recorded_decode_across_a_bound_on_the_context(tmp_path):
             checked += 1
         tok = int(ids[0][0])
     assert checked == 5 and len(eng._runners[1].graphs) == 2
+
+
+def test_a_full_run_before_a_new_recording_leaves_the_rings_alone(tmp_path):
+    """A run of the most steps a run may have leaves every row's counter one past the rings; the recording that a
+    longer context then asks for starts with an eager step, which must not write there.  Rows beside the rings are
+    watched, and the tokens are those of the plain model."""
+    import dataclasses
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.engine.decode import DecodeRunner
+    from gesso_amd.weights import write_model_folder
+    from tiny import TINY_D, STD
+    cfg_d = dataclasses.replace(TINY_D, max_position_embeddings=1536)
+    d = write_model_folder(str(tmp_path / "long_d"), cfg_d, 12, torch.bfloat16, std=STD)
+    cfg, w = P.read_config(d), P.read_weights(d)
+    seqs = [random_ids(n, cfg["V"], 5000 + n) for n in (960, 950, 957, 941)]
+    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=4 * 1152, num_slots=5)
+    runner = eng._runners[4] = DecodeRunner(eng, 4)
+    steps = DecodeRunner.MAX_STEPS
+    guard = {}
+    for name in ("ring", "bad_ring"):                      # the rings as the middle rows of larger buffers
+        big = torch.full((steps + 2, 4), -7, dtype=torch.int32, device=eng.device)
+        guard[name] = big
+        setattr(runner, name, big[1:steps + 1])
+    toks = []
+    for i, s in enumerate(seqs):
+        eng.add_request(i)
+        toks.append(int(eng.step([StepEntry(i, s, [len(s) - 1])]).argmax()))
+    rids = list(range(4))
+    for n in (steps, steps, 8):                             # 960 -> 992 -> 1024 (first recording), then beyond it
+        ids, bad = eng.decode(rids, toks, n)
+        assert not bad.any()
+        for step in range(n):
+            for s, t in zip(seqs, toks):
+                s.append(t)
+            toks = ids[step].tolist()
+        logits = runner.logits[:4].double().cpu()          # of the run's last step
+        for i, s in enumerate(seqs):
+            ref = P.forward(cfg, w, s)[-1]
+            assert float((logits[i] - ref).abs().max()) <= 1.5e-2 * max(1.0, float(ref.abs().max()))
+    assert len(runner.graphs) == 2
+    for name, big in guard.items():
+        assert bool((big[0] == -7).all()) and bool((big[-1] == -7).all()), f"a step wrote beside {name}"

@@ -314,3 +314,46 @@ def test_runs_shrink_to_the_pages_that_are_left_and_nucleus_requests_step_singly
     c = s2.add(Request("c", [1, 2, 3], max_new_tokens=5, sampler=Sampler(0.9, 0.5, 3)))
     s2.run()
     assert c.tokens == expected([1, 2, 3], 5) and eng2.runs == []
+
+
+def test_a_request_that_outgrows_the_context_fails_alone_and_keeps_its_tokens():
+    # b's prompt of 14 tokens fits a context of 16, its 8 new tokens do not: it fails when the 17th token would be fed
+    for engine in (FakeEngine(max_length=16), FakeDecodeEngine(max_length=16)):
+        eng, s = make(engine, decode_run_steps=8)
+        a = s.add(Request("a", [1, 2, 3], max_new_tokens=6))
+        b = s.add(Request("b", list(range(14)), max_new_tokens=8))
+        c = s.add(Request("c", list(range(30)), max_new_tokens=1))            # never fits
+        s.run()
+        assert a.finish_reason == "complete" and a.tokens == expected([1, 2, 3], 6)
+        assert b.finish_reason == "failed" and isinstance(b.error, ResourceLimit)
+        # tokens at positions 14, 15, 16 were chosen from 14, 15 and 16 cached tokens; the next would need a 17th fed
+        assert b.tokens == expected(range(14), 3)
+        assert c.finish_reason == "failed" and isinstance(c.error, ResourceLimit) and c.output == []
+        assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+
+
+def test_admission_leaves_the_watermark_free_for_those_who_run():
+    # 10 pages of 4; a holds 5 after its prompt.  b's prompt needs 4: with a margin of 2 pages (0.2 of 10) it waits
+    eng, s = make(FakeEngine(num_pages=10, page_size=4), chunk_size=32, max_num_batched_tokens=64, watermark=0.2)
+    a = s.add(Request("a", list(range(20)), max_new_tokens=4))
+    s.step()
+    b = s.add(Request("b", list(range(16)), max_new_tokens=2))
+    s.step()
+    assert b.status == "waiting" and s.stats["preemptions"] == 0
+    s.run()
+    assert a.tokens == expected(range(20), 4) and b.tokens == expected(range(16), 2)
+    assert s.stats["preemptions"] == 0
+    # without a margin the same request is admitted at once
+    eng2, s2 = make(FakeEngine(num_pages=10, page_size=4), chunk_size=32, max_num_batched_tokens=64, watermark=0.0)
+    s2.add(Request("a", list(range(20)), max_new_tokens=4))
+    s2.step()
+    b2 = s2.add(Request("b", list(range(16)), max_new_tokens=2))
+    s2.step()
+    assert b2.status == "running"
+    # an idle engine admits without the margin: a request that needs every page still runs
+    eng3, s3 = make(FakeEngine(num_pages=4, page_size=4), chunk_size=32, max_num_batched_tokens=64, watermark=0.5)
+    c = s3.add(Request("c", list(range(14)), max_new_tokens=2))
+    s3.run()
+    assert c.finish_reason == "complete" and c.tokens == expected(range(14), 2)
+    with pytest.raises(InvalidPlan):
+        make(watermark=1.0)
