@@ -25,6 +25,8 @@
 // launch can be recorded into a graph.  q (T, q_stride), head h at [h D, (h+1) D); caches
 // (pages, nkv, page_size, D); out (T, nh D).  Window: keys lo..pos with lo = pos - window + 1.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 #define DEC_MAXG 8
 #define DEC_LOG2E 1.4426950408889634f
@@ -520,6 +522,50 @@ extern "C" int gs_attention_decode(const void* q, int q_stride, const void* kcac
                                    int nkv, int d, int nsplit, hipStream_t stream) {
   return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
                       scale, out, out_tiled, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream);
+}
+
+// ---- the entry point that allocates nothing (declared and described in no_alloc.h)
+//
+// `scratch` is the name of the device array as host code sees it: a stand-in, not a device address.  Its address on
+// the current GPU comes from hipGetSymbolAddress, once per device with that device current (each GPU holds its own
+// copy at its own address), and only that pointer goes to kernels.
+static __device__ __align__(256) float scratch[GS_DECODE_STATIC_FLOATS];
+
+#define GS_MAX_DEVICES 64
+static float* g_scratch_ptr[GS_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int static_workspace(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  GS_REQUIRE(e == hipSuccess, "attention_decode_static: no current device: %s", hipGetErrorString(e));
+  GS_REQUIRE(dev >= 0 && dev < GS_MAX_DEVICES, "attention_decode_static: device %d outside [0, %d)", dev, GS_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    GS_REQUIRE(e == hipSuccess && p != nullptr, "attention_decode_static: the static workspace has no address on device %d: %s",
+               dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int gs_attention_decode_static(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                          const int* positions, const int* block_table, int max_blocks, int page_size,
+                                          int window, float scale, void* out, int out_tiled, int nseq, int nh, int nkv,
+                                          int d, int nsplit, hipStream_t stream) {
+  GS_REQUIRE(nseq >= 0 && nh > 0 && nkv > 0 && d > 0 && nsplit >= 1 && nsplit <= 64,
+             "attention_decode_static: bad sizes nseq=%d nh=%d nkv=%d d=%d nsplit=%d", nseq, nh, nkv, d, nsplit);
+  const long need = gs_attention_decode_workspace(nseq, nh, nkv, d, nsplit);
+  GS_REQUIRE(need <= (long)GS_DECODE_STATIC_FLOATS,
+             "attention_decode_static: %ld floats of workspace needed (nseq=%d nh=%d d=%d nsplit=%d), the static one holds %ld",
+             need, nseq, nh, d, nsplit, (long)GS_DECODE_STATIC_FLOATS);
+  float* ws = nullptr;
+  if (static_workspace(&ws) != 0) return -1;
+  return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
+                      scale, out, out_tiled, ws, nseq, nh, nkv, d, nsplit, nullptr, stream);
 }
 
 // Whether the kernel also takes the head norms, the rotation and the cache write: heads of 64 or 128 rotated whole.
