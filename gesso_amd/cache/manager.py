@@ -96,7 +96,11 @@ class CacheManager:
         self.needs_slot = bool(layout.slots)
         self.max_length = int(max_length)
         self.requests: Dict[Hashable, RequestCache] = {}
-        self.fresh_slots: List[int] = []    # slots handed out and not yet zeroed on the device
+        self.fresh_slots: List[int] = []    # slots handed out and not yet given their initial value on the device
+        # debug poison: with track_released set, what comes back is listed here until the engine has overwritten it
+        self.track_released = False
+        self.released_pages: List[List[int]] = [[] for _ in self.pools]
+        self.released_slots: List[int] = []
 
     # ------------------------------------------------------------------ requests
 
@@ -175,6 +179,8 @@ class CacheManager:
                 for b in range(min(passed, len(table))):
                     table[b] = RELEASED
                 self.pools[g].give_back(gone)
+                if self.track_released:
+                    self.released_pages[g].extend(gone)
 
     def release(self, rid: Hashable) -> None:
         """The request is over (finished, aborted, preempted): everything it holds comes back."""
@@ -182,11 +188,22 @@ class CacheManager:
         if rc is None:
             raise InvalidPlan(f"request {rid!r} is not live")
         for g, table in enumerate(rc.tables):
-            self.pools[g].give_back([p for p in table if p != RELEASED])
+            held = [p for p in table if p != RELEASED]
+            self.pools[g].give_back(held)
+            if self.track_released:
+                self.released_pages[g].extend(held)
         if rc.slot is not None:
             self.slot_pool.give_back([rc.slot])
             if rc.slot in self.fresh_slots:
                 self.fresh_slots.remove(rc.slot)
+            if self.track_released:
+                self.released_slots.append(rc.slot)
+
+    def take_released(self):
+        """``(pages per group, slots)`` given back since the last call; the lists start anew."""
+        pages, slots = self.released_pages, self.released_slots
+        self.released_pages, self.released_slots = [[] for _ in self.pools], []
+        return pages, slots
 
     # ------------------------------------------------------------------ accounting
 

@@ -4,7 +4,8 @@ Pages of a group: one tensor ``(members, 2, num_pages + 1, n_kv_heads, page_size
 activation type; index 0/1 of the second axis is K/V, so that a page id addresses the same page
 in every layer of the group.  A head's rows of a page are contiguous (``page_size x head_dim``),
 which is what the attention kernels stream.  Slot state: per state-keeping layer and state
-name a float32 tensor ``(num_slots + 1, *shape)``.  The extra page and the extra slot at the end
+name a tensor ``(num_slots + 1, *shape)`` of the type the layer asked for (float32 or bfloat16), with the value a
+fresh slot starts from in ``state_init``.  The extra page and the extra slot at the end
 belong to no request: padded entries of a fixed-size batch write there.
 """
 from __future__ import annotations
@@ -14,9 +15,10 @@ from typing import Dict, Optional
 
 import torch
 
+from ..errors import InvalidPlan
 from .manager import CacheLayout
 
-_DTYPES = {"float32": torch.float32}
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
 @dataclass
@@ -32,7 +34,7 @@ class PagedView:
 
 @dataclass
 class SlotView:
-    state: Dict[str, torch.Tensor]   # name -> (num_slots + 1, *shape) float32
+    state: Dict[str, torch.Tensor]   # name -> (num_slots + 1, *shape)
     write: bool
 
 
@@ -50,9 +52,15 @@ class CacheStorage:
                                        dtype=dtype, device=device))
         self.member_index = {c: i for g in layout.paged for i, c in enumerate(g.members)}
         self.state: Dict[int, Dict[str, torch.Tensor]] = {}
+        self.state_init: Dict[int, Dict[str, float]] = {}
         for m in layout.slots:
-            self.state[m.call] = {name: torch.zeros((num_slots + 1,) + tuple(shape), dtype=_DTYPES[dt], device=device)
-                                  for name, shape, dt in m.need.tensors}
+            self.state[m.call], self.state_init[m.call] = {}, {}
+            for name, shape, dt, init in m.need.entries():
+                if dt not in _DTYPES:
+                    raise InvalidPlan(f"state {name!r} of schedule entry {m.call} asks for {dt!r}; slots hold "
+                                      f"{sorted(_DTYPES)}")
+                self.state[m.call][name] = torch.full((num_slots + 1,) + shape, init, dtype=_DTYPES[dt], device=device)
+                self.state_init[m.call][name] = init
 
     @property
     def scratch_page(self):
@@ -73,6 +81,32 @@ class CacheStorage:
         if src in self.state:
             return SlotView(self.state[src], write)
         return None
+
+    # ------------------------------------------------------------------ filling (initial values, debug poison)
+
+    def fill_slots(self, ops, slots, value) -> None:
+        """``value``: a number, ``"initial"`` for each state's own initial value, or None for NaN."""
+        ids = None
+        for call, states in self.state.items():
+            for name, t in states.items():
+                if ids is None:
+                    ids = torch.tensor(list(slots), dtype=torch.int32, device=t.device)
+                v = self.state_init[call][name] if value == "initial" else (float("nan") if value is None else value)
+                ops.fill_rows(t, ids, v)
+
+    def fill_pages(self, ops, group: int, pages, value: float) -> None:
+        """Every layer's keys and values of the given pages of one group."""
+        kv = self.kv[group]
+        ids = torch.tensor(list(pages), dtype=torch.int32, device=kv.device)
+        ops.fill_rows(kv, ids, value, planes=3)          # (members, 2) planes of (pages + 1) rows
+
+    def poison_all(self) -> None:
+        """NaN everywhere but in the spare page and slot (padded rows of a recorded batch compute on those)."""
+        for kv in self.kv:
+            kv[:, :, :-1].fill_(float("nan"))
+        for states in self.state.values():
+            for t in states.values():
+                t[:-1].fill_(float("nan"))
 
     def bytes(self) -> int:
         n = sum(t.numel() * t.element_size() for t in self.kv)

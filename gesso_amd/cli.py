@@ -38,6 +38,10 @@ def parse_launch(argv: List[str]) -> argparse.Namespace:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--prefill-chunk", type=int, default=None, help="largest portion of a prompt per step (GESSO_PREFILL_CHUNK)")
     ap.add_argument("--max-num-seqs", type=int, default=64)
+    ap.add_argument("--gemm", default="auto", choices=["auto", "own", "library"],
+                    help="products of more than 64 rows: the vendor library where it is faster (auto), the hand-written "
+                         "kernel everywhere (own), the library wherever it can go (library)")
+    ap.add_argument("--poison", action="store_true", help="debugging: fill pages and slots that are given back with NaN")
     ap.add_argument("--cpu", action="store_true", help="refused: there is no CPU path")
     ap.add_argument("--check", action="store_true", help="self-test on a tiny random model")
     return ap.parse_args(argv)
@@ -84,9 +88,10 @@ def main(argv=None) -> int:
         return 2
 
     from .engine.session import Session
+    from .parts.runtime import RuntimeOptions
 
     kw = dict(dtype=args.dtype, page_size=args.page_size, context_length=args.n_ctx, chunk_size=args.prefill_chunk,
-              max_num_seqs=args.max_num_seqs)
+              max_num_seqs=args.max_num_seqs, kernel_options=RuntimeOptions(many_rows=args.gemm), poison=args.poison)
     if args.model is not None:
         session = Session(args.model, **kw)
     else:

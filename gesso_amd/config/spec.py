@@ -28,12 +28,14 @@ class RMSNormSpec:
 
 @dataclass(frozen=True)
 class RopeSpec:
-    """Rotary encoding over the first ``rotary_dim`` features of a head, half-split pairs."""
+    """Rotary encoding over the first ``rotary_dim`` features of a head; ``layout``: pairs ``(i, i + rotary_dim/2)``
+    (``"half"``) or ``(2i, 2i + 1)`` (``"interleaved"``)."""
 
     head_dim: int
     rotary_dim: int
     theta: float
     max_position: int
+    layout: str = "half"
     kind: str = "rope"
 
 
@@ -114,6 +116,8 @@ class ModelSpec:
     # names: "embed" -> table, "final_norm.weight" -> ..., "head" -> untied head
     eos_token_ids: Tuple[int, ...] = ()
     ignored_tensors: Tuple[str, ...] = ()   # suffixes that a file may hold and nobody reads
+    embed_scale: Optional[float] = None     # the embedding rows are multiplied by this (None: as they are)
+    logit_softcap: Optional[float] = None   # logits = cap * tanh(logits / cap) (None: as they are)
 
     def __post_init__(self):
         n = len(self.blocks)

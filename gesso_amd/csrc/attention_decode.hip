@@ -161,7 +161,7 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
       load8f(raw.sin_t + (size_t)pos * (D / 2) + 32 * st + 8 * kg, s8[st]);
     }
     if (raw.qw) {
-      const float inv = 1.0f / sqrtf(group4_sum(ss) / (float)D + raw.eps);
+      const float inv = norm_inverse(group4_sum(ss), (float)D, raw.eps);
 #pragma unroll
       for (int st = 0; st < KS; ++st) {
         float w8[8];
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
         ks += kf[e] * kf[e];
       }
       if (raw.kw) {
-        const float inv = 1.0f / sqrtf(wave_sum_dpp(ks) / (float)D + raw.eps);
+        const float inv = norm_inverse(wave_sum_dpp(ks), (float)D, raw.eps);
 #pragma unroll
         for (int e = 0; e < E; ++e) kf[e] = kf[e] * inv * raw.kw[lane + 64 * e];
       }

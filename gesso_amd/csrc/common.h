@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <string.h>
 
 #define GS_F32 0
 #define GS_BF16 1
@@ -60,6 +61,15 @@ __device__ __forceinline__ float from_f32<float>(float v) {
 template <>
 __device__ __forceinline__ bf16 from_f32<bf16>(float v) {
   return f32_to_bf16(v);
+}
+
+// 1 / sqrt(mean + eps) of a norm, from the sum of squares ss over n values.  A denominator that is not finite or not
+// positive (the reference raises a numerical-instability error there, src/Operators/cpu.jl:260-266) gives NaN: it
+// poisons the row, so that the choice of the next token fails for this request alone, also where the row's values are
+// finite and only their sum of squares has overflowed (1 / inf would quietly give a row of zeros).
+__device__ __forceinline__ float norm_inverse(float ss, float n, float eps) {
+  const float r = sqrtf(ss / n + eps);
+  return (r > 0.f && r < INFINITY) ? 1.0f / r : __builtin_nanf("");
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -170,3 +180,16 @@ __host__ __device__ __forceinline__ size_t tiled_index(int m, int k, int tiles) 
 }
 
 static inline int gs_ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
+
+// A float as bfloat16 on the host: round to nearest, ties to even; NaN stays NaN.
+static inline bf16 host_bf16(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  bf16 r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r.x = (uint16_t)((u >> 16) | 0x40);
+  } else {
+    r.x = (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+  }
+  return r;
+}

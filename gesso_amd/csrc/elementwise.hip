@@ -19,18 +19,19 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 6; }
+extern "C" int gs_abi_version() { return 7; }
 
 // ------------------------------------------------------------------ embedding
 
-// out[t, :] = table[ids[t], :] as float32; an id outside the table gives a NaN row.
+// out[t, :] = table[ids[t], :] * scale as float32 (scale 1 for most models; some multiply the embedding by a
+// constant); an id outside the table gives a NaN row.
 // With ssq: ssq[t] = sum of squares of the row (one partial sum per row, for a norm that follows).
 // With next_w and xs: xs[t, :] = bfloat16(row * next_w), the rows pre-weighted for the first norm's consumer,
 // as rows of H or, with xs_tiles = ceil(T / 16) > 0, as tiled rows.
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
                              float* __restrict__ ssq, const float* __restrict__ next_w, bf16* __restrict__ xs,
-                             int xs_tiles, int H, int V) {
+                             int xs_tiles, int H, int V, float scale) {
   __shared__ float red[17];
   int t = blockIdx.x;
   int id = ids[t];
@@ -46,6 +47,8 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
       for (int j = threadIdx.x * 8; j < H; j += blockDim.x * 8) {
         float v[8];
         load8f(row + j, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] *= scale;
         store8f(o + j, v);
 #pragma unroll
         for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
@@ -59,7 +62,7 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
       }
     } else {
       for (int j = threadIdx.x; j < H; j += blockDim.x) {
-        float v = to_f32(row[j]);
+        float v = to_f32(row[j]) * scale;
         o[j] = v;
         ss += v * v;
         if (xs) xs[xs_tiles ? tiled_index(t, j, xs_tiles) : (size_t)t * H + j] = f32_to_bf16(v * next_w[j]);
@@ -73,15 +76,16 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
 }
 
 extern "C" int gs_embed(const int* ids, const void* table, int table_dtype, float* out, float* ssq,
-                        const float* next_w, void* xs, int xs_tiled, int T, int H, int V, hipStream_t stream) {
+                        const float* next_w, void* xs, int xs_tiled, int T, int H, int V, float scale,
+                        hipStream_t stream) {
   GS_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
   GS_REQUIRE(!xs_tiled || (xs && H % 32 == 0), "embed: tiled rows need a width that is a multiple of 32, not %d", H);
   const int xs_tiles = xs_tiled ? gs_ceil_div(T, 16) : 0;
   if (T == 0) return 0;
   if (table_dtype == GS_F32)
-    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, ssq, next_w, (bf16*)xs, xs_tiles, H, V);
+    embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, ssq, next_w, (bf16*)xs, xs_tiles, H, V, scale);
   else if (table_dtype == GS_BF16)
-    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, ssq, next_w, (bf16*)xs, xs_tiles, H, V);
+    embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, out, ssq, next_w, (bf16*)xs, xs_tiles, H, V, scale);
   else
     GS_REQUIRE(false, "embed: unknown dtype %d", table_dtype);
   GS_LAUNCH_CHECK("embed");
@@ -149,7 +153,7 @@ __global__ void residual_from_parts_kernel(const float* __restrict__ part, int p
   ss = block_sum(ss, red);
   if (threadIdx.x == 0) ssq[m] = ss;
   if (!normed) return;
-  const float inv = 1.0f / sqrtf(ss / (float)N + eps);
+  const float inv = norm_inverse(ss, (float)N, eps);
   for (int u = 0; u < turns; ++u) {
     const int j = (u * blockDim.x + threadIdx.x) * 4;
     if (j >= N) continue;
@@ -252,7 +256,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict
       }
     }
     ss = block_sum(ss, red);
-    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    const float inv = norm_inverse(ss, (float)H, eps);
     for (int u = 0; u < turns; ++u) {
       const int j = (u * blockDim.x + threadIdx.x) * 8;
       if (j >= H) break;
@@ -285,7 +289,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict
     ss += v * v;
   }
   ss = block_sum(ss, red);
-  float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  float inv = norm_inverse(ss, (float)H, eps);
   for (int j = threadIdx.x; j < H; j += blockDim.x) {
     float v = x[j];
     if (dl && rows) v += to_f32(dl[j]);
@@ -336,7 +340,7 @@ __global__ void norm_from_ssq_kernel(const float* __restrict__ res, const float*
   float s = 0.f;
   for (int b = lane; b < nb; b += 64) s += ssq[(size_t)t * nb + b];
   s = wave_sum(s);
-  const float inv = 1.0f / sqrtf(s / (float)H + eps);
+  const float inv = norm_inverse(s, (float)H, eps);
 #pragma unroll
   for (int i = 0; i < 8; ++i)
     if (j0 + i < H) out[(size_t)t * H + j0 + i] = from_f32<TO>(x[i] * inv * wv[i]);
@@ -435,6 +439,21 @@ extern "C" int gs_swiglu(const void* in, void* out, int dtype, int T, int F, hip
 
 // ------------------------------------------------------------------ fills
 
+// Soft cap of logits in place: x = cap * tanh(x / cap) (the reference's final_logit_softcap of the families that
+// have one, src/Inference/architecture_spec.jl:248; not an LFM2 feature).
+__global__ void softcap_kernel(float* p, float cap, long n) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = cap * tanhf(p[i] / cap);
+}
+
+extern "C" int gs_softcap(float* p, float cap, long n, hipStream_t stream) {
+  GS_REQUIRE(n >= 0 && cap > 0.f, "softcap: the cap must be positive");
+  if (n == 0) return 0;
+  softcap_kernel<<<gs_ceil_div(n, 256), 256, 0, stream>>>(p, cap, n);
+  GS_LAUNCH_CHECK("softcap");
+  return 0;
+}
+
 __global__ void fill_f32_kernel(float* p, float v, long n) {
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
@@ -449,18 +468,29 @@ extern "C" int gs_fill_f32(float* p, float v, long n, hipStream_t stream) {
   return 0;
 }
 
-// Zero the state rows of given slots: state (num_slots, row) float32; slots (n).
-__global__ void zero_slots_kernel(float* state, const int* slots, long row) {
-  int s = slots[blockIdx.y];
-  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (s >= 0 && i < row) state[(size_t)s * row + i] = 0.f;
+// Fill chosen rows of a pool with one value: pool (outer, num_rows, row) of float32 or bfloat16, ids (n) rows to
+// fill in every one of the `outer` planes (a negative id is skipped).  A request's state slots are rows of a pool
+// with one plane, a cache page is a row in each layer's K and V plane.  Used to give a fresh slot its initial
+// value and to poison what a request gave back.
+template <typename T>
+__global__ void fill_rows_kernel(T* pool, const int* ids, long row, long plane, T value) {
+  const int id = ids[blockIdx.y];
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= 0 && i < row) pool[(size_t)blockIdx.z * plane + (size_t)id * row + i] = value;
 }
 
-extern "C" int gs_zero_slots(float* state, const int* slots, int n, long row, hipStream_t stream) {
-  GS_REQUIRE(n >= 0 && row >= 0, "zero_slots: bad sizes");
-  if (n == 0 || row == 0) return 0;
-  dim3 grid(gs_ceil_div(row, 256), n);
-  zero_slots_kernel<<<grid, 256, 0, stream>>>(state, slots, row);
-  GS_LAUNCH_CHECK("zero_slots");
+extern "C" int gs_fill_rows(void* pool, int dtype, const int* ids, int n, long row, int outer, long num_rows, float value,
+                            hipStream_t stream) {
+  GS_REQUIRE(n >= 0 && row >= 0 && outer >= 0 && num_rows >= 0, "fill_rows: bad sizes");
+  GS_REQUIRE(n <= 65535 && outer <= 65535, "fill_rows: %d rows in %d planes are more than one launch takes", n, outer);
+  if (n == 0 || row == 0 || outer == 0) return 0;
+  dim3 grid(gs_ceil_div(row, 256), n, outer);
+  if (dtype == GS_F32)
+    fill_rows_kernel<float><<<grid, 256, 0, stream>>>((float*)pool, ids, row, num_rows * row, value);
+  else if (dtype == GS_BF16)
+    fill_rows_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)pool, ids, row, num_rows * row, host_bf16(value));
+  else
+    GS_REQUIRE(false, "fill_rows: unknown dtype %d", dtype);
+  GS_LAUNCH_CHECK("fill_rows");
   return 0;
 }

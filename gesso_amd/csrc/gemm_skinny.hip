@@ -121,30 +121,6 @@ extern "C" int gs_gemm_skinny_conv(const void* X, int ldx, int x_tiled, const fl
   return 0;
 }
 
-// Head widths whose attention input the fused kernel takes (the whole head is rotated).
-extern "C" int gs_gemm_skinny_qkv_supports(int d, int rotary_dim) {
-  return (d == 32 || d == 64 || d == 128) && rotary_dim == d;
-}
-
-// q (M, nh d) stored, k and v written to the cache, from (normed res) W_qkv^T for a decode step.
-extern "C" int gs_gemm_skinny_qkv(const void* X, int ldx, int x_tiled, const float* res, const float* ssq, int nb, const float* norm_w, float eps,
-                                  const void* W, const void* Wt, const float* qw, const float* kw, float head_eps,
-                                  const float* cos_t, const float* sin_t, const int* positions,
-                                  const int* block_table, int max_blocks, int page_size, void* kcache, void* vcache,
-                                  int write_kv, void* Q, int M, int nh, int nkv, int d, int K, hipStream_t stream) {
-  const int N = (nh + 2 * nkv) * d;
-  if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16) || check_x(X, ldx, x_tiled, res, ssq, nb, norm_w, eps, K)) return -1;
-  GS_REQUIRE(gs_gemm_skinny_qkv_supports(d, d), "gemm_skinny_qkv: head width %d is not taken", d);
-  GS_REQUIRE((qw == nullptr) == (kw == nullptr), "gemm_skinny_qkv: q and k norm weights come together");
-  GS_REQUIRE(cos_t && sin_t && positions && block_table && kcache && vcache && page_size > 0 && max_blocks > 0,
-             "gemm_skinny_qkv: missing rotation tables or cache");
-  if (M == 0) return 0;
-  gs_skinny_run_qkv(X, ldx, x_tiled, res, ssq, nb, norm_w, eps, W, Wt, qw, kw, head_eps, cos_t, sin_t, positions, block_table,
-                    max_blocks, page_size, kcache, vcache, write_kv, Q, M, nh, nkv, d, K, stream);
-  GS_LAUNCH_CHECK("gemm_skinny_qkv");
-  return 0;
-}
-
 // Tile-major copy: out[(t * ksteps + s) * 512 + lane * 8 + j] = W[16 t + lane % 16][32 s + 8 (lane / 16) + j].
 __global__ void tile_major_kernel(const bf16* __restrict__ W, bf16* __restrict__ out, int N, int K) {
   const int ksteps = K >> 5;

@@ -11,10 +11,5 @@ void gs_skinny_run_residual(const void* X, int ldx, int x_tiled, const void* W, 
 void gs_skinny_run_conv(const void* X, int ldx, int x_tiled, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
                         const void* Wt, const float* taps, const float* conv_bias, float* state, const int* slots,
                         int conv_w, void* Y, int y_tiled, int M, int H, int K, hipStream_t stream);
-void gs_skinny_run_qkv(const void* X, int ldx, int x_tiled, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
-                       const void* Wt, const float* qw, const float* kw, float head_eps, const float* cos_t,
-                       const float* sin_t, const int* positions, const int* block_table, int max_blocks,
-                       int page_size, void* kcache, void* vcache, int write_kv, void* Q, int M, int nh, int nkv, int d,
-                       int K, hipStream_t stream);
 void gs_skinny_run_parts(const void* X, int ldx, int x_tiled, const void* W, const void* Wt, float* part, int parts, int M, int N,
                          int K, hipStream_t stream);

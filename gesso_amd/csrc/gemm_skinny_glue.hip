@@ -5,7 +5,6 @@
 void gs_skinny_plain_rows(const SkinnyCall& c);
 void gs_skinny_residual_rows(const SkinnyCall& c);
 void gs_skinny_conv_rows(const SkinnyCall& c);
-void gs_skinny_qkv_rows(const SkinnyCall& c, int d);
 void gs_skinny_plain_tiles(const SkinnyCall& c);
 void gs_skinny_residual_tiles(const SkinnyCall& c);
 void gs_skinny_residual_half_tiles(const SkinnyCall& c);
@@ -13,7 +12,6 @@ void gs_skinny_conv_tiles(const SkinnyCall& c);
 void gs_skinny_parts_rows(const SkinnyCall& c, int parts);
 void gs_skinny_parts_tiles(const SkinnyCall& c, int parts);
 void gs_skinny_conv_half_tiles(const SkinnyCall& c);
-void gs_skinny_qkv_tiles(const SkinnyCall& c, int d);
 
 static SkinnyCall base(const void* X, int ldx, int x_tiled, const void* W, const void* Wt, void* Y, int y_dtype, int ldy, int M,
                        int N, int K, int epilogue, hipStream_t stream) {
@@ -59,19 +57,6 @@ void gs_skinny_run_conv(const void* X, int ldx, int x_tiled, const float* res, c
   // c.N / 3 channels, as few as a narrow weight's rows; with many rows of X the blocks' reading of X outweighs that
   if (Wt && gs_skinny_halves(c.N / 3) && M <= 32) gs_skinny_conv_half_tiles(c);
   else Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);
-}
-
-void gs_skinny_run_qkv(const void* X, int ldx, int x_tiled, const float* res, const float* ssq, int nb, const float* norm_w, float eps, const void* W,
-                       const void* Wt, const float* qw, const float* kw, float head_eps, const float* cos_t,
-                       const float* sin_t, const int* positions, const int* block_table, int max_blocks,
-                       int page_size, void* kcache, void* vcache, int write_kv, void* Q, int M, int nh, int nkv, int d,
-                       int K, hipStream_t stream) {
-  SkinnyCall c = base(X, ldx, x_tiled, W, Wt, Q, GS_BF16, nh * d, M, (nh + 2 * nkv) * d, K, 4, stream);
-  if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
-  c.ex.qw = qw; c.ex.kw = kw; c.ex.head_eps = head_eps; c.ex.cos_t = cos_t; c.ex.sin_t = sin_t;
-  c.ex.positions = positions; c.ex.block_table = block_table; c.ex.max_blocks = max_blocks; c.ex.page_size = page_size;
-  c.ex.nh = nh; c.ex.nkv = nkv; c.ex.write_kv = write_kv; c.ex.kcache = (bf16*)kcache; c.ex.vcache = (bf16*)vcache;
-  Wt ? gs_skinny_qkv_tiles(c, d) : gs_skinny_qkv_rows(c, d);
 }
 
 void gs_skinny_run_parts(const void* X, int ldx, int x_tiled, const void* W, const void* Wt, float* part, int parts, int M, int N,

@@ -43,8 +43,6 @@
 //      block's columns stored as partial sums for the next norm.
 //   3  gated short convolution of a decode step: tiles are the B, C, X rows of 16 channels; u = B X,
 //      y = taps . (history, u) + bias, out = C y, history shifted; one token per sequence.
-//   4  attention input of a decode step: the block owns one head (R = d / 16 tiles); per-head RMSNorm of
-//      q and k heads, half-split rotation, q stored, k and v written into the cache page.
 #pragma once
 #include "common.h"
 
@@ -101,17 +99,6 @@ struct SkinnyExtra {
   float* state;          // (slots, H, W - 1)
   const int* slots;      // (M)
   int conv_w;
-  // EPI 4
-  const float* qw;       // (d) or null
-  const float* kw;
-  float head_eps;
-  const float* cos_t;    // (positions, d / 2)
-  const float* sin_t;
-  const int* positions;  // (M)
-  const int* block_table;
-  int max_blocks, page_size, nh, nkv, write_kv;
-  bf16* kcache;
-  bf16* vcache;
   // layouts
   int x_tiled;           // X comes as tiled rows (PRO 0 only; K a multiple of 32)
   int y_tiled;           // EPI 1, 3: Y, EPI 2: xs_out are written as tiled rows (their width a multiple of 32)
@@ -183,7 +170,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
         for (int b = kg; b < ex.nb; b += 4) s += ex.ssq[(size_t)m * ex.nb + b];
       s += __shfl_xor(s, 16, 64);
       s += __shfl_xor(s, 32, 64);
-      inv[mt] = 1.0f / sqrtf(s / (float)K + ex.eps);
+      inv[mt] = norm_inverse(s, (float)K, ex.eps);
     }
   }
 
@@ -199,17 +186,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       if (lane + 64 * j < ex.nb) pre[j] = ex.ssq[(size_t)wave * ex.nb + lane + 64 * j];
   }
 
-  // What the epilogue reads besides the product (the stream's old rows, the convolution's history and taps, the
-  // positions and rotation factors) is loaded here, by the wavefront that runs the epilogue, so that these
+  // What the epilogue reads besides the product (the stream's old rows, the convolution's history and taps) is
+  // loaded here, by the wavefront that runs the epilogue, so that these
   // round trips pass under the product's own instead of after it.
   constexpr int PRE_TAPS = 4;                       // convolutions of up to this width are held in registers
-  constexpr bool PRE_ROT = R * MT <= 8;             // rotation factors too, while the registers allow
   const bool half_ok = SHUF != 2 || kg < 2;
   f32x4_t rold[EPI == 2 ? R : 1][EPI == 2 ? MT : 1], nextw[EPI == 2 ? R : 1];
   float chist[EPI == 3 ? MT : 1][4][PRE_TAPS - 1], ctap[4][PRE_TAPS], cbias[4];
-  int epos[EPI == 4 ? MT : 1], epage[EPI == 4 ? MT : 1];
-  float ecos[(EPI == 4 && PRE_ROT) ? MT : 1][(EPI == 4 && PRE_ROT) ? R / 2 + 1 : 1][4],
-      esin[(EPI == 4 && PRE_ROT) ? MT : 1][(EPI == 4 && PRE_ROT) ? R / 2 + 1 : 1][4];
   const bool vec4 = (N & 3) == 0;
   if (EPI == 2 && wave == 0) {
 #pragma unroll
@@ -255,30 +238,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       }
     }
   }
-  if (EPI == 4 && wave == 0) {
-    constexpr int d = 16 * R;
-    const int hh = blockIdx.x;
-    const bool is_q = hh < ex.nh, is_k = !is_q && hh < ex.nh + ex.nkv;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      epos[mt] = xok[mt] ? ex.positions[mt * 16 + r16] : 0;
-      epage[mt] = (xok[mt] && !is_q && ex.write_kv)
-                      ? ex.block_table[(size_t)(mt * 16 + r16) * ex.max_blocks + epos[mt] / ex.page_size] : 0;
-      if (PRE_ROT && (is_q || is_k)) {
-#pragma unroll
-        for (int r = 0; r < R / 2; ++r) {
-          const float* cp = ex.cos_t + (size_t)epos[mt] * (d / 2) + r * 16 + kg * 4;
-          const float* sp = ex.sin_t + (size_t)epos[mt] * (d / 2) + r * 16 + kg * 4;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            ecos[mt][r][i] = cp[i];
-            esin[mt][r][i] = sp[i];
-          }
-        }
-      }
-    }
-  }
-
   f32x4_t acc[R][MT];
 #pragma unroll
   for (int r = 0; r < R; ++r)
@@ -364,7 +323,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       if (m == wave) ssum = (pre[0] + pre[1]) + (pre[2] + pre[3]);
       for (int b = (m == wave ? 256 : 0) + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
       ssum = wave_sum_dpp(ssum);
-      if (lane == 0) inv_s[m] = 1.0f / sqrtf(ssum / (float)K + ex.eps);
+      if (lane == 0) inv_s[m] = norm_inverse(ssum, (float)K, ex.eps);
     }
     if (WAVES == 1) __syncthreads();
   }
@@ -490,63 +449,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
           hist[Wd - 2] = u;
         }
       }
-    } else if (EPI == 4) {
-      // one head of d = 16 R features; tile r and tile r + R/2 hold the two halves of each rotation pair
-      constexpr int d = 16 * R;
-      const int hh = blockIdx.x;  // head among q heads, then k heads, then v heads
-      const bool is_q = hh < ex.nh, is_k = !is_q && hh < ex.nh + ex.nkv;
-      float v[R][4];
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[r][i] = to_f32(f32_to_bf16(acc[r][mt][i]));  // as the unfused path stores qkv
-      const float* nw = is_q ? ex.qw : ex.kw;
-      if (is_q || is_k) {
-        if (nw) {
-          float ss = 0.f;
-#pragma unroll
-          for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ss += v[r][i] * v[r][i];
-          ss += __shfl_xor(ss, 16, 64);
-          ss += __shfl_xor(ss, 32, 64);
-          const float hinv = 1.0f / sqrtf(ss / (float)d + ex.head_eps);
-#pragma unroll
-          for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) v[r][i] = v[r][i] * hinv * nw[r * 16 + kg * 4 + i];
-        }
-        if (live) {
-          const int pos = epos[mt];
-#pragma unroll
-          for (int r = 0; r < R / 2; ++r)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int j = r * 16 + kg * 4 + i;  // pair (j, j + d/2)
-              const float c = PRE_ROT ? ecos[mt][r][i] : ex.cos_t[(size_t)pos * (d / 2) + j];
-              const float sn = PRE_ROT ? esin[mt][r][i] : ex.sin_t[(size_t)pos * (d / 2) + j];
-              const float a = v[r][i], b = v[r + R / 2][i];
-              v[r][i] = a * c - b * sn;
-              v[r + R / 2][i] = a * sn + b * c;
-            }
-        }
-      }
-      if (!live) continue;
-      bf16* dst;
-      if (is_q) {
-        dst = (bf16*)Y + (size_t)m * ldy + (size_t)hh * d;
-      } else {
-        if (!ex.write_kv) continue;
-        const int pos = epos[mt];
-        const int kvh = is_k ? hh - ex.nh : hh - ex.nh - ex.nkv;
-        const int page = epage[mt];
-        dst = (is_k ? ex.kcache : ex.vcache) + (((size_t)page * ex.nkv + kvh) * ex.page_size + pos % ex.page_size) * d;
-      }
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        f32x4_t o = {v[r][0], v[r][1], v[r][2], v[r][3]};
-        store4<bf16>(dst + r * 16 + kg * 4, o, 4);
-      }
     }
   }
 }
@@ -655,23 +557,4 @@ static void skinny_conv(const SkinnyCall& c) {
   hipStream_t stream = c.stream;
   const int blocks = gs_ceil_div(N / 3, SHUF == 2 ? 8 : 16);
   if (ex.res) { GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks) } else { GS_BY_MT4(3, 8, 8, 8, 8, 0, 3, bf16, blocks) }
-}
-
-template <int SHUF>
-static void skinny_qkv(const SkinnyCall& c, int d) {
-  const bf16 *x = c.x, *w = c.w;
-  void* Y = c.Y;
-  const int ldx = c.ldx, ldy = c.ldy, M = c.M, N = c.N, K = c.K;
-  const SkinnyExtra& ex = c.ex;
-  hipStream_t stream = c.stream;
-  const int blocks = N / d;
-  if (ex.res) {
-    if (d == 32) { GS_BY_MT4(2, 16, 16, 8, 8, 1, 4, bf16, blocks) }
-    else if (d == 64) { GS_BY_MT4(4, 16, 8, 4, 4, 1, 4, bf16, blocks) }
-    else { GS_BY_MT4(8, 8, 4, 2, 2, 1, 4, bf16, blocks) }
-  } else {
-    if (d == 32) { GS_BY_MT4(2, 16, 16, 8, 8, 0, 4, bf16, blocks) }
-    else if (d == 64) { GS_BY_MT4(4, 16, 8, 4, 4, 0, 4, bf16, blocks) }
-    else { GS_BY_MT4(8, 8, 4, 2, 2, 0, 4, bf16, blocks) }
-  }
 }

@@ -4,5 +4,4 @@
 void gs_skinny_plain_rows(const SkinnyCall& c) { skinny_plain<0>(c); }
 void gs_skinny_residual_rows(const SkinnyCall& c) { skinny_residual<0>(c); }
 void gs_skinny_conv_rows(const SkinnyCall& c) { skinny_conv<0>(c); }
-void gs_skinny_qkv_rows(const SkinnyCall& c, int d) { skinny_qkv<0>(c, d); }
 void gs_skinny_parts_rows(const SkinnyCall& c, int parts) { skinny_parts<0>(c, parts); }

@@ -6,5 +6,4 @@ void gs_skinny_residual_tiles(const SkinnyCall& c) { skinny_residual<1>(c); }
 void gs_skinny_residual_half_tiles(const SkinnyCall& c) { skinny_residual<2>(c); }
 void gs_skinny_conv_tiles(const SkinnyCall& c) { skinny_conv<1>(c); }
 void gs_skinny_conv_half_tiles(const SkinnyCall& c) { skinny_conv<2>(c); }
-void gs_skinny_qkv_tiles(const SkinnyCall& c, int d) { skinny_qkv<1>(c, d); }
 void gs_skinny_parts_tiles(const SkinnyCall& c, int parts) { skinny_parts<1>(c, parts); }

@@ -2,9 +2,10 @@
 //
 // qkv (T, (nh + 2 nkv) d): q heads, then k heads, then v heads, each head d wide.
 //   q, k: x = x / sqrt(mean(x^2) + eps) * w  over the head (when a weight is given), then for the
-//         first rotary_dim features, pairs (i, i + rotary_dim/2):
-//           x_i' = x_i cos - x_j sin,  x_j' = x_i sin + x_j cos,  angle = pos * theta^(-2i/rotary_dim)
-//         with cos/sin from a table (max_position, rotary_dim/2) made on the host in float64.
+//         first rotary_dim features, pairs (a, b) = (i, i + rotary_dim/2) ("half-split") or, with `interleaved`,
+//         (2i, 2i + 1) (reference src/Operators/cpu.jl:357-371):
+//           x_a' = x_a cos - x_b sin,  x_b' = x_a sin + x_b cos,  angle = pos * theta^(-2i/rotary_dim)
+//         with cos/sin row i from a table (max_position, rotary_dim/2) made on the host in float64.
 //   q is written back in place; k (after norm and rotation) and v (as it is) go to the cache:
 //   page = block_table[seq, pos / page_size], row = pos % page_size,
 //   cache (num_pages, nkv, page_size, d).
@@ -14,7 +15,7 @@
 template <typename T>
 __global__ void qknorm_rope_kv_kernel(T* __restrict__ qkv, const float* __restrict__ qw, const float* __restrict__ kw,
                                       float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                                      int rotary_dim, const int* __restrict__ positions,
+                                      int rotary_dim, int interleaved, const int* __restrict__ positions,
                                       const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                       int max_blocks, int page_size, T* __restrict__ kcache, T* __restrict__ vcache,
                                       int ntok, int nh, int nkv, int d, int write_kv) {
@@ -49,22 +50,22 @@ __global__ void qknorm_rope_kv_kernel(T* __restrict__ qkv, const float* __restri
       ss += v * v;
     }
     ss = wave_sum(ss);
-    inv = 1.0f / sqrtf(ss / (float)d + eps);
+    inv = norm_inverse(ss, (float)d, eps);
   }
   T* o = hh < nh ? x : dst;
   int half = rotary_dim >> 1;
   const float* cr = cos_t ? cos_t + (size_t)pos * half : nullptr;
   const float* sr = sin_t ? sin_t + (size_t)pos * half : nullptr;
   for (int i = lane; i < half; i += 64) {
-    int j = i + half;
-    float a = to_f32(x[i]) * inv, b = to_f32(x[j]) * inv;
+    const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+    float a = to_f32(x[ia]) * inv, b = to_f32(x[ib]) * inv;
     if (w) {
-      a *= w[i];
-      b *= w[j];
+      a *= w[ia];
+      b *= w[ib];
     }
     float c = cr[i], s = sr[i];
-    o[i] = from_f32<T>(a * c - b * s);
-    o[j] = from_f32<T>(a * s + b * c);
+    o[ia] = from_f32<T>(a * c - b * s);
+    o[ib] = from_f32<T>(a * s + b * c);
   }
   for (int j = rotary_dim + lane; j < d; j += 64) {  // features beyond the rotary part
     float a = to_f32(x[j]) * inv;
@@ -109,7 +110,7 @@ __global__ void qknorm_rope_kv_vec_kernel(T* __restrict__ qkv, const float* __re
       for (int k = 0; k < 8; ++k) ss += v[k] * v[k];
 #pragma unroll
       for (int m = 1; m < L; m <<= 1) ss += __shfl_xor(ss, m, 64);
-      const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+      const float inv = norm_inverse(ss, (float)d, eps);
       float w8[8];
       load8f(w + sub * 8, w8);
 #pragma unroll
@@ -131,8 +132,8 @@ __global__ void qknorm_rope_kv_vec_kernel(T* __restrict__ qkv, const float* __re
 }
 
 extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const float* kw, float eps,
-                                 const float* cos_t, const float* sin_t, int rotary_dim, int max_position,
-                                 const int* positions, const int* seq_of_token, const int* block_table,
+                                 const float* cos_t, const float* sin_t, int rotary_dim, int interleaved,
+                                 int max_position, const int* positions, const int* seq_of_token, const int* block_table,
                                  int max_blocks, int page_size, void* kcache, void* vcache, int ntok, int nh, int nkv,
                                  int d, int write_kv, hipStream_t stream) {
   GS_REQUIRE(ntok >= 0 && nh > 0 && nkv > 0 && d > 0, "qknorm_rope_kv: bad sizes T=%d nh=%d nkv=%d d=%d", ntok, nh,
@@ -145,7 +146,7 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
   GS_REQUIRE((qw == nullptr) == (kw == nullptr), "qknorm_rope_kv: q and k norm weights come together");
   if (ntok == 0) return 0;
   long units = (long)ntok * (nh + 2 * nkv);
-  const bool vec = rotary_dim == d && (d == 16 || d == 32 || d == 64 || d == 128) && (dtype == GS_F32 || dtype == GS_BF16) &&
+  const bool vec = !interleaved && rotary_dim == d && (d == 16 || d == 32 || d == 64 || d == 128) && (dtype == GS_F32 || dtype == GS_BF16) &&
                    ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0 &&
                    ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0 && ((uintptr_t)qw & 15) == 0 &&
                    ((uintptr_t)kw & 15) == 0;
@@ -171,7 +172,7 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
   }
   int blocks = gs_ceil_div(units, 4);
 #define GS_RUN(T)                                                                                               \
-  qknorm_rope_kv_kernel<T><<<blocks, 256, 0, stream>>>((T*)qkv, qw, kw, eps, cos_t, sin_t, rotary_dim, positions, \
+  qknorm_rope_kv_kernel<T><<<blocks, 256, 0, stream>>>((T*)qkv, qw, kw, eps, cos_t, sin_t, rotary_dim, interleaved, positions, \
                                                        seq_of_token, block_table, max_blocks, page_size,        \
                                                        (T*)kcache, (T*)vcache, ntok, nh, nkv, d, write_kv)
   if (dtype == GS_F32)

@@ -44,64 +44,30 @@ def check_entries(entries: List[StepEntry], manager, vocab: int) -> None:
                 raise InvalidPlan(f"request {e.rid!r} wants logits at place {w} of {n} tokens")
 
 
-class StepContext:
-    """The flattened batch on the device, plus the host-side facts kernels are chosen by."""
+# What parts may read of a step.  Host-side facts kernels are chosen by: T (tokens), nseq, n_want, q_lens, all_single,
+# max_q_len, max_kv_len (None: unknown here, kernels read kv_len on the device), decode_only (every sequence brings
+# one token and wants its logits, in order).  Device tensors, int32: token_ids, positions, seq_of_token (T each),
+# q_start (nseq + 1), kv_len, slots (nseq each), want_rows (n_want), block_tables (per paged group (nseq, blocks)).
+CONTEXT_FIELDS = ("T", "nseq", "n_want", "q_lens", "all_single", "max_q_len", "max_kv_len", "decode_only",
+                  "token_ids", "positions", "seq_of_token", "q_start", "kv_len", "slots", "want_rows", "block_tables")
 
-    def __init__(self, entries: List[StepEntry], manager, storage, vocab: int, device, pad_to: int = 0):
-        ps = manager.page_size
-        nseq = len(entries)
-        lens = []
-        for e in entries:
-            lens.append(len(e.tokens))
-        T = sum(lens)
-        self.T, self.nseq = T, nseq
-        self.q_lens = lens
-        self.all_single = all(n == 1 for n in lens)
-        self.max_q_len = max(lens)
 
-        rcs = [manager.get(e.rid) for e in entries]
-        starts = np.zeros(nseq + 1, dtype=np.int32)
-        starts[1:] = np.cumsum(lens)
-        tokens = np.empty(T, dtype=np.int64)
-        positions = np.empty(T, dtype=np.int32)
-        seq_of = np.empty(T, dtype=np.int32)
-        want_rows: List[int] = []
-        for i, (e, rc) in enumerate(zip(entries, rcs)):
-            a, b = starts[i], starts[i + 1]
-            tokens[a:b] = np.asarray(e.tokens, dtype=np.int64)
-            positions[a:b] = np.arange(rc.length, rc.length + lens[i], dtype=np.int32)
-            seq_of[a:b] = i
-            want_rows.extend(int(a) + int(w) for w in e.want)
-        kv_len = np.asarray([rc.length + n for rc, n in zip(rcs, lens)], dtype=np.int32)
-        self.max_kv_len = int(kv_len.max()) if nseq else 0
-        slots = np.asarray([storage.scratch_slot if rc.slot is None else rc.slot for rc in rcs], dtype=np.int32)
-        self.n_want = len(want_rows)
+class BatchContext:
+    """A step as the parts see it: the fields of ``CONTEXT_FIELDS``, the cache views, the tiling of queries.
 
-        n_groups = len(manager.pools)
-        max_blocks = max(1, -(-self.max_kv_len // ps))
-        tables = np.empty((n_groups, nseq, max_blocks), dtype=np.int32)
-        for g in range(n_groups):
-            tables[g, :, :] = storage.num_pages[g]            # the scratch page: never read
-            for i, rc in enumerate(rcs):
-                t = rc.tables[g]
-                n = min(len(t), max_blocks)
-                row = np.asarray(t[:n], dtype=np.int32)
-                row[row < 0] = storage.num_pages[g]
-                tables[g, i, :n] = row
-        self.max_blocks = max_blocks
+    Whoever builds a context (a step from entries, the recorded decode step from its static buffers) hands all
+    fields to :meth:`_set`, which refuses a missing or an unknown one: a field added to the list must be served
+    by every builder before anything runs."""
 
-        parts = [tokens.astype(np.int32), positions, seq_of, starts, kv_len, slots,
-                 np.asarray(want_rows, dtype=np.int32), tables.reshape(-1)]
-        sizes = [p.size for p in parts]
-        host = torch.from_numpy(np.concatenate(parts)).pin_memory() if device.type == "cuda" else torch.from_numpy(np.concatenate(parts))
-        dev = host.to(device, non_blocking=True)
-        views = torch.split(dev, sizes)
-        (self.token_ids, self.positions, self.seq_of_token, self.q_start, self.kv_len, self.slots,
-         self.want_rows, flat_tables) = views
-        self.block_tables = [flat_tables.view(n_groups, nseq, max_blocks)[g] for g in range(n_groups)] if n_groups else []
-        self._tiles = None
-        self._host = host          # keeps the pinned buffer alive until the copy has run
+    def _set(self, storage, **fields) -> None:
+        if set(fields) != set(CONTEXT_FIELDS):
+            missing, unknown = set(CONTEXT_FIELDS) - set(fields), set(fields) - set(CONTEXT_FIELDS)
+            raise InvalidPlan(f"{type(self).__name__} must set the context's fields exactly",
+                              missing=sorted(missing), unknown=sorted(unknown))
+        for k, v in fields.items():
+            setattr(self, k, v)
         self._storage = storage
+        self._tiles = None
 
     def cache_view(self, call: int):
         return self._storage.view(call, self.block_tables)
@@ -130,3 +96,57 @@ class StepContext:
             t = torch.tensor([seq, row, cnt], dtype=torch.int32).pin_memory().to(self.token_ids.device, non_blocking=True)
             self._tiles = ((rows, skip), t)
         return self._tiles[1]
+
+
+class StepContext(BatchContext):
+    """The flattened batch of one step on the device."""
+
+    def __init__(self, entries: List[StepEntry], manager, storage, vocab: int, device):
+        ps = manager.page_size
+        nseq = len(entries)
+        lens = []
+        for e in entries:
+            lens.append(len(e.tokens))
+        T = sum(lens)
+        rcs = [manager.get(e.rid) for e in entries]
+        starts = np.zeros(nseq + 1, dtype=np.int32)
+        starts[1:] = np.cumsum(lens)
+        tokens = np.empty(T, dtype=np.int64)
+        positions = np.empty(T, dtype=np.int32)
+        seq_of = np.empty(T, dtype=np.int32)
+        want_rows: List[int] = []
+        for i, (e, rc) in enumerate(zip(entries, rcs)):
+            a, b = starts[i], starts[i + 1]
+            tokens[a:b] = np.asarray(e.tokens, dtype=np.int64)
+            positions[a:b] = np.arange(rc.length, rc.length + lens[i], dtype=np.int32)
+            seq_of[a:b] = i
+            want_rows.extend(int(a) + int(w) for w in e.want)
+        kv_len = np.asarray([rc.length + n for rc, n in zip(rcs, lens)], dtype=np.int32)
+        max_kv_len = int(kv_len.max()) if nseq else 0
+        slots = np.asarray([storage.scratch_slot if rc.slot is None else rc.slot for rc in rcs], dtype=np.int32)
+        n_groups = len(manager.pools)
+        max_blocks = max(1, -(-max_kv_len // ps))
+        tables = np.empty((n_groups, nseq, max_blocks), dtype=np.int32)
+        for g in range(n_groups):
+            tables[g, :, :] = storage.num_pages[g]            # the scratch page: never read
+            for i, rc in enumerate(rcs):
+                t = rc.tables[g]
+                n = min(len(t), max_blocks)
+                row = np.asarray(t[:n], dtype=np.int32)
+                row[row < 0] = storage.num_pages[g]
+                tables[g, i, :n] = row
+        self.max_blocks = max_blocks
+
+        parts = [tokens.astype(np.int32), positions, seq_of, starts, kv_len, slots,
+                 np.asarray(want_rows, dtype=np.int32), tables.reshape(-1)]
+        sizes = [p.size for p in parts]
+        host = torch.from_numpy(np.concatenate(parts)).pin_memory() if device.type == "cuda" else torch.from_numpy(np.concatenate(parts))
+        dev = host.to(device, non_blocking=True)
+        views = torch.split(dev, sizes)
+        token_ids, positions_d, seq_of_d, q_start, kv_len_d, slots_d, want_d, flat_tables = views
+        tables_d = [flat_tables.view(n_groups, nseq, max_blocks)[g] for g in range(n_groups)] if n_groups else []
+        self._set(storage, T=T, nseq=nseq, n_want=len(want_rows), q_lens=lens, all_single=all(n == 1 for n in lens),
+                  max_q_len=max(lens), max_kv_len=max_kv_len, decode_only=False, token_ids=token_ids,
+                  positions=positions_d, seq_of_token=seq_of_d, q_start=q_start, kv_len=kv_len_d, slots=slots_d,
+                  want_rows=want_d, block_tables=tables_d)
+        self._host = host          # keeps the pinned buffer alive until the copy has run

@@ -25,6 +25,7 @@ import numpy as np
 import torch
 
 from ..errors import InvalidPlan
+from .batch import BatchContext
 from ..sampling.sampler import Sampler
 
 
@@ -35,24 +36,16 @@ def _capacity(n: int) -> int:
     return c
 
 
-class _DecodeContext:
-    """What the parts read of a step, all of it static device buffers (see StepContext for the fields)."""
+class DecodeContext(BatchContext):
+    """The recorded decode step as the parts see it: every field a static device buffer of the runner, or a fact
+    that holds for every replay (one token per sequence, every row wanted, in order)."""
 
     def __init__(self, runner):
         r = runner
-        self.T = self.nseq = self.n_want = r.cap
-        self.q_lens = [1] * r.cap
-        self.all_single = True
-        self.max_q_len = 1
-        self.max_kv_len = None            # an upper bound, set per recording; kernels read kv_len on the device
-        self.decode_only = True
-        self.token_ids, self.positions, self.kv_len, self.slots = r.tok, r.pos, r.kv_len, r.slots
-        self.seq_of_token, self.q_start, self.want_rows = r.seq_of_token, r.q_start, r.seq_of_token
-        self.block_tables = r.block_tables
-        self._storage = r.engine.storage
-
-    def cache_view(self, call: int):
-        return self._storage.view(call, self.block_tables)
+        self._set(r.engine.storage, T=r.cap, nseq=r.cap, n_want=r.cap, q_lens=[1] * r.cap, all_single=True,
+                  max_q_len=1, max_kv_len=None, decode_only=True, token_ids=r.tok, positions=r.pos,
+                  seq_of_token=r.seq_of_token, q_start=r.q_start, kv_len=r.kv_len, slots=r.slots,
+                  want_rows=r.seq_of_token, block_tables=r.block_tables)
 
 
 class DecodeRunner:
@@ -79,7 +72,7 @@ class DecodeRunner:
         self.counter = torch.zeros(cap, **i32)          # steps made since the host last looked, per row
         self.ring = torch.zeros((self.MAX_STEPS, cap), **i32)
         self.bad_ring = torch.zeros((self.MAX_STEPS, cap), **i32)
-        self.ctx = _DecodeContext(self)
+        self.ctx = DecodeContext(self)
         # one recording per bound on the context length: launch shapes (how attention splits its keys) depend on it
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
 
@@ -157,7 +150,20 @@ class DecodeRunner:
             if not 0 <= int(t) < eng.spec.vocab:
                 raise InvalidPlan(f"token id {int(t)} outside the vocabulary of {eng.spec.vocab}")
         mgr.reserve_many([(r, n) for r in rids])
-        eng._zero_fresh_slots()
+        # from here on the cache is written: an error leaves these requests without a usable state
+        try:
+            ids, bad = self._run(rids, rcs, tokens, n, samplers, graph)
+        except Exception as err:
+            raise eng.fail_requests(rids, err) from err
+        for r in rids:
+            mgr.commit(r, n)
+        eng.steps += n
+        return ids, bad
+
+    def _run(self, rids, rcs, tokens, n, samplers, graph):
+        eng, cap, B = self.engine, self.cap, len(rids)
+        st = eng.storage
+        eng.prepare_cache()
         # one int32 buffer for the per-row facts, one copy
         host = np.zeros((5, cap), dtype=np.int32)
         host[0, :B] = tokens
@@ -179,6 +185,7 @@ class DecodeRunner:
                 tab[i, :len(row)] = row
             bt[:, :width].copy_(torch.from_numpy(tab).pin_memory().to(eng.device, non_blocking=True))
         temp = np.zeros(cap, dtype=np.float64)
+        before = {}               # row -> the sampler's state before each of its draws
         if samplers is not None and any(s is not None for s in samplers):
             u = np.zeros((n, cap), dtype=np.float64)
             for i, s in enumerate(samplers):
@@ -186,7 +193,10 @@ class DecodeRunner:
                     if s.top_p < 1:
                         raise InvalidPlan("nucleus sampling does not run in the recorded decode loop")
                     temp[i] = s.temperature
-                    u[:, i] = [s.unit() for _ in range(n)]
+                    before[i] = []
+                    for k in range(n):
+                        before[i].append(s.state)
+                        u[k, i] = s.unit()
             self.u[:n].copy_(torch.from_numpy(u).pin_memory().to(eng.device, non_blocking=True))
         self.temperature.copy_(torch.from_numpy(temp).pin_memory().to(eng.device, non_blocking=True))
         self.counter.zero_()
@@ -194,9 +204,12 @@ class DecodeRunner:
             graph.replay()
         ids = self.ring[:n, :B].cpu().numpy()
         bad = self.bad_ring[:n, :B].cpu().numpy()
-        for r in rids:
-            mgr.commit(r, n)
-        eng.steps += n
+        # a step whose logits were not finite emits no token and makes no draw (as the step-by-step choice does):
+        # the draws were made up front, so the sampler goes back to where it stood before that step
+        for i, states in before.items():
+            hit = np.flatnonzero(bad[:, i])
+            if hit.size:
+                samplers[i].state = states[int(hit[0])]
         return ids, bad
 
 

@@ -19,9 +19,9 @@ from ..cache.manager import CacheLayout, CacheManager
 from ..cache.storage import CacheStorage
 from ..config.registry import load_config
 from ..config.spec import ModelSpec
-from ..errors import InvalidPlan
+from ..errors import GessoError, InvalidPlan, StepFailed
 from ..models.model import Model, tensor_table, tied_aliases
-from ..parts.runtime import Runtime
+from ..parts.runtime import Runtime, RuntimeOptions
 from ..weights.loader import load_tensors, random_tensors
 from .batch import StepContext, StepEntry, check_entries
 
@@ -39,15 +39,18 @@ def parse_dtype(dtype) -> torch.dtype:
 class Engine:
     def __init__(self, spec: ModelSpec, tensors, dtype, device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, num_slots: int = 8,
-                 max_context: Optional[int] = None):
+                 max_context: Optional[int] = None, options: Optional[RuntimeOptions] = None, poison: bool = False):
         """``tensors``: ``file name -> tensor`` on the device, in the widths the loader chose.
 
         The page pool holds ``num_pages`` pages per group, or enough for ``max_tokens`` tokens.
+        ``options``: how kernels are chosen (:class:`~gesso_amd.parts.runtime.RuntimeOptions`).
+        ``poison``: a debugging aid: every page and slot that is given back is filled with NaN before the next
+        step runs, so that a kernel that reads a row it has no business with shows in the logits.
         """
         self.spec = spec
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
-        self.rt = Runtime(self.device, self.dtype)
+        self.rt = Runtime(self.device, self.dtype, options)
         self.model = Model(spec, self.rt)
         self.model.bind(tensors)
         self.page_size = int(page_size)
@@ -60,6 +63,10 @@ class Engine:
         layout = CacheLayout.plan(needs, [c.cache for c in spec.schedule])
         self.manager = CacheManager(layout, self.page_size, int(num_pages), int(num_slots), self.max_context)
         self.storage = CacheStorage(layout, self.page_size, int(num_pages), int(num_slots), self.dtype, self.device)
+        self.poison = bool(poison)
+        self.manager.track_released = self.poison
+        if self.poison:
+            self.storage.poison_all()
         self.steps = 0
         self._runners = {}
 
@@ -103,15 +110,32 @@ class Engine:
 
     # ------------------------------------------------------------------ the step
 
-    def _zero_fresh_slots(self) -> None:
+    def prepare_cache(self) -> None:
+        """Before a step's kernels run: with poisoning on, NaN into what was given back since the last step; then the
+        initial value into every slot handed out since."""
+        ops = self.rt.ops
+        if self.poison:
+            pages, slots = self.manager.take_released()
+            for g, ids in enumerate(pages):
+                if ids:
+                    self.storage.fill_pages(ops, g, ids, float("nan"))
+            if slots:
+                self.storage.fill_slots(ops, slots, None)
         fresh = self.manager.fresh_slots
-        if not fresh:
-            return
-        slots = torch.tensor(fresh, dtype=torch.int32, device=self.device)
-        for states in self.storage.state.values():
-            for t in states.values():
-                self.rt.ops.zero_slots(t, slots)
-        fresh.clear()
+        if fresh:
+            self.storage.fill_slots(ops, fresh, "initial")
+            fresh.clear()
+
+    def fail_requests(self, rids, err: Exception) -> StepFailed:
+        """A step broke off in the middle: the state of its requests (pages partly written, histories partly
+        advanced) is worth nothing, so they are released; the reference invalidates the state of a generation that
+        fails (``src/Inference/Inference.jl:2730-2736``)."""
+        gone = []
+        for rid in rids:
+            if rid in self.manager.requests:
+                self.manager.release(rid)
+                gone.append(rid)
+        return StepFailed(f"a step failed and its requests were released: {err}", requests=gone)
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
@@ -119,9 +143,13 @@ class Engine:
             return None
         check_entries(entries, self.manager, self.spec.vocab)
         self.manager.reserve_many([(e.rid, len(e.tokens)) for e in entries])
-        self._zero_fresh_slots()
-        ctx = StepContext(entries, self.manager, self.storage, self.spec.vocab, self.device)
-        logits = self.model.forward(ctx)
+        # from here on the cache is written: an error leaves the requests of this step without a usable state
+        try:
+            self.prepare_cache()
+            ctx = StepContext(entries, self.manager, self.storage, self.spec.vocab, self.device)
+            logits = self.model.forward(ctx)
+        except Exception as err:
+            raise self.fail_requests([e.rid for e in entries], err) from err
         for e in entries:
             self.manager.commit(e.rid, len(e.tokens))
         self.steps += 1

@@ -19,7 +19,7 @@ from typing import Callable, List, Optional, Sequence, Union
 
 import torch
 
-from ..errors import InvalidPlan
+from ..errors import GessoError, InvalidPlan
 from ..sampling.sampler import Sampler, choose
 from .batch import StepEntry
 from .engine import Engine
@@ -49,14 +49,19 @@ class Session:
                  max_num_seqs: int = 64, max_num_batched_tokens: Optional[int] = None,
                  chunk_size: Optional[int] = None, num_pages: Optional[int] = None,
                  max_tokens: Optional[int] = None, random_weights_seed: Optional[int] = None,
-                 random_weights_std: float = 0.02):
+                 random_weights_std: float = 0.02, watermark: float = 0.01, kernel_options=None,
+                 poison: bool = False):
         """``model``: a folder with config.json and model.safetensors, or a typed configuration
         together with ``random_weights_seed``.  ``context_length``: most tokens one request may hold.
-        The cache holds ``num_pages`` pages, or ``max_tokens`` tokens (default: four contexts)."""
+        The cache holds ``num_pages`` pages, or ``max_tokens`` tokens (default: four contexts).
+        ``watermark``: the fraction of the pages that an admission leaves free for those who run.
+        ``kernel_options``: a :class:`~gesso_amd.parts.runtime.RuntimeOptions`; ``poison``: fill what is
+        given back with NaN (a debugging aid, see :class:`Engine`)."""
         self.chunk_size = chunk_size or default_prefill_chunk()
         self.max_num_seqs = max_num_seqs
         self.max_num_batched_tokens = max_num_batched_tokens or max(self.chunk_size, max_num_seqs)
-        kw = dict(page_size=page_size, num_slots=max_num_seqs)
+        self.watermark = watermark
+        kw = dict(page_size=page_size, num_slots=max_num_seqs, options=kernel_options, poison=poison)
         if isinstance(model, (str, os.PathLike)):
             from ..config.registry import load_config
             _, cfg = load_config(os.fspath(model))
@@ -77,6 +82,7 @@ class Session:
         spec = self.engine.spec
         self.eos_ids = (int(eos_token_id),) if eos_token_id is not None else tuple(spec.eos_token_ids)
         self.last_stats = {}
+        self.last_results = []
         self._next_id = 0
         self._closed = False
 
@@ -101,7 +107,8 @@ class Session:
         return choose(self.engine.rt.ops, logits, samplers)
 
     def scheduler(self) -> Scheduler:
-        return Scheduler(self.engine, self._choose, self.max_num_seqs, self.max_num_batched_tokens, self.chunk_size)
+        return Scheduler(self.engine, self._choose, self.max_num_seqs, self.max_num_batched_tokens, self.chunk_size,
+                         watermark=self.watermark)
 
     def generate(self, prompts, max_new_tokens: int = 8, sampler=None, temperature: float = 0.0, top_p: float = 1.0,
                  seed: int = 0, eos_ids=None, stop_ids=(), on_token: Optional[Callable] = None):
@@ -111,6 +118,10 @@ class Session:
         ``sampler`` (one :class:`Sampler`, or one per prompt) or ``temperature > 0`` is given; with one
         sampler and several prompts, prompt ``i`` draws from seed ``seed + i``.  ``on_token(id)`` (one
         prompt) or ``on_token(i, id)`` (several) may return False to stop that request.
+
+        A request that fails (non-finite logits, a prompt that fits no cache) stops alone; the others run to
+        their end, ``last_results`` holds every request's :class:`BatchResult`, and then the first failure is
+        raised, with ``detail["results"]`` = ``last_results``.
         """
         if self._closed:
             raise InvalidPlan("the session is closed")
@@ -143,9 +154,13 @@ class Session:
             self._next_id += 1
             requests.append(sched.add(r))
         self._run(sched, requests)
+        self.last_results = [BatchResult(r.tokens, r.finish_reason, r.error) for r in requests]
         for r in requests:
             if r.finish_reason == "failed":
-                raise r.error
+                err = r.error
+                if isinstance(err, GessoError):
+                    err.detail.setdefault("results", self.last_results)
+                raise err
         out = [r.tokens for r in requests]
         return out[0] if single else out
 

@@ -20,8 +20,8 @@ class GessoError(Exception):
         base = super().__str__()
         if not self.detail:
             return base
-        facts = ", ".join(f"{k}={v!r}" for k, v in self.detail.items())
-        return f"{base} ({facts})"
+        facts = ", ".join(f"{k}={v!r}" for k, v in self.detail.items() if k != "results")   # results: whole outputs
+        return f"{base} ({facts})" if facts else base
 
 
 class ConfigError(GessoError, ValueError):
@@ -60,6 +60,13 @@ class NumericalInstability(GessoError):
     """Non-finite logits where a token was to be chosen (``session.jl:444-458``)."""
 
     code = "ERR_NUMERICAL_INSTABILITY"
+
+
+class StepFailed(GessoError):
+    """A step broke off after it had begun to write the cache; ``detail["requests"]`` lists the requests whose
+    state was dropped with it (they are no longer live).  The cause is chained (``__cause__``)."""
+
+    code = "ERR_STEP_FAILED"
 
 
 class KernelError(GessoError):

@@ -129,8 +129,8 @@ def _rows_out(out, M, N, device, dtype=torch.bfloat16):
 # ---------------------------------------------------------------------- elementwise
 
 def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq: torch.Tensor = None,
-          next_weight: torch.Tensor = None, xs: torch.Tensor = None) -> torch.Tensor:
-    """``out[t] = table[ids[t]]`` as float32 ``(T, H)``; with ``ssq (T, 1)`` also each row's sum of squares;
+          next_weight: torch.Tensor = None, xs: torch.Tensor = None, scale: float = 1.0) -> torch.Tensor:
+    """``out[t] = table[ids[t]] * scale`` as float32 ``(T, H)``; with ``ssq (T, 1)`` also each row's sum of squares;
     with ``next_weight (H,)`` and ``xs (T, H)`` bfloat16 also ``xs = out * next_weight``."""
     _dev(ids, table, out, ssq, next_weight, None if isinstance(xs, TiledRows) else xs)
     _i32(ids, what="token ids")
@@ -148,7 +148,7 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor = None, ssq:
         _need(next_weight.dtype == torch.float32 and next_weight.shape == (H,) and xs.dtype == torch.bfloat16
               and tuple(xs.shape) == (T, H) and xs_buf.is_contiguous(), "embed: next_weight float32 (H,), xs bfloat16 (T, H)")
     _check(lib().gs_embed(_p(ids), _p(table), _dt(table), _p(out), _p(ssq), _p(next_weight), _p(xs_buf), c_int(xs_tiled),
-                          c_int(T), c_int(H), c_int(V), _stream()))
+                          c_int(T), c_int(H), c_int(V), c_float(scale), _stream()))
     return out
 
 
@@ -196,6 +196,14 @@ def swiglu(x: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     return out
 
 
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """``cap * tanh(logits / cap)`` in place (float32)."""
+    _dev(logits)
+    _need(logits.dtype == torch.float32, "softcap takes float32 logits")
+    _check(lib().gs_softcap(_p(logits), c_float(cap), c_long(logits.numel()), _stream()))
+    return logits
+
+
 def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
     _dev(t)
     _need(t.dtype == torch.float32, "fill_f32 takes float32")
@@ -203,13 +211,20 @@ def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
     return t
 
 
-def zero_slots(state: torch.Tensor, slots: torch.Tensor) -> None:
-    """Zero ``state[slot]`` for each slot in ``slots`` (int32); ``state (num_slots, ...)`` float32."""
-    _dev(state, slots)
-    _i32(slots, what="slots")
-    _need(state.dtype == torch.float32, "state is float32")
-    row = state[0].numel()
-    _check(lib().gs_zero_slots(_p(state), _p(slots), c_int(slots.numel()), c_long(row), _stream()))
+def fill_rows(pool: torch.Tensor, ids: torch.Tensor, value: float, planes: int = 1) -> None:
+    """``pool[..., id, ...] = value`` for each id in ``ids`` (int32): ``pool`` is ``(planes..., rows, *row shape)`` with
+    ``planes`` leading axes flattened into one (1: ``(rows, ...)``), float32 or bfloat16.  A fresh state slot gets its
+    initial value this way; with poisoning on, so do the pages and slots a request gave back (NaN)."""
+    _dev(pool, ids)
+    _i32(ids, what="row ids")
+    lead = pool.shape[:planes - 1] if planes > 1 else ()
+    outer = 1
+    for n in lead:
+        outer *= n
+    rows = pool.shape[len(lead)]
+    row = pool[(0,) * (len(lead) + 1)].numel() if pool.numel() else 0
+    _check(lib().gs_fill_rows(_p(pool), c_int(_dt(pool)), _p(ids), c_int(ids.numel()), c_long(row), c_int(outer),
+                              c_long(rows), c_float(value), _stream()))
 
 
 # ---------------------------------------------------------------------- short convolution
@@ -240,9 +255,14 @@ def short_conv(bcx, taps, bias, state, seq_of_token, q_start, slots, nseq: int, 
 
 # ---------------------------------------------------------------------- attention
 
+ROPE_LAYOUTS = ("half", "interleaved")
+
+
 def qknorm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, positions, seq_of_token, block_table,
-                   page_size, kcache, vcache, nh, nkv, d, write_kv=True) -> None:
-    """Head norm and rotation of q (in place) and k; k and v written into the pages."""
+                   page_size, kcache, vcache, nh, nkv, d, write_kv=True, layout: str = "half") -> None:
+    """Head norm and rotation of q (in place) and k; k and v written into the pages.  ``layout``: which features
+    form a rotation pair, ``"half"`` (i, i + rotary_dim/2) or ``"interleaved"`` (2i, 2i + 1)."""
+    _need(layout in ROPE_LAYOUTS, f"qknorm_rope_kv: pairs are laid out 'half' or 'interleaved', not {layout!r}")
     _dev(qkv, q_weight, k_weight, cos, sin, positions, seq_of_token, block_table, kcache, vcache)
     T = qkv.shape[0]
     _need(qkv.shape == (T, (nh + 2 * nkv) * d), "qknorm_rope_kv: qkv must be (T, (nh + 2 nkv) d)")
@@ -260,7 +280,8 @@ def qknorm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, positions
     _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
           "cache must be (pages, nkv, page_size, d)")
     _check(lib().gs_qknorm_rope_kv(_p(qkv), c_int(_dt(qkv)), _p(q_weight), _p(k_weight), c_float(eps), _p(cos),
-                                   _p(sin), c_int(rotary_dim), c_int(max_pos), _p(positions), _p(seq_of_token),
+                                   _p(sin), c_int(rotary_dim), c_int(1 if layout == "interleaved" else 0), c_int(max_pos),
+                                   _p(positions), _p(seq_of_token),
                                    _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
                                    _p(vcache), c_int(T), c_int(nh), c_int(nkv), c_int(d),
                                    c_int(1 if write_kv else 0), _stream()))
@@ -553,34 +574,6 @@ def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None, tiled: bool = F
     _check(lib().gs_gemm_skinny_conv(*_lazy_args(x), _p(w_in), _p(wt), _p(taps), _p(bias), _p(state), _p(slots), c_int(W),
                                      _p(buf), c_int(otiled), c_int(M), c_int(H), c_int(K), _stream()))
     return out
-
-
-def gemm_skinny_qkv_supports(d: int, rotary_dim: int) -> bool:
-    return bool(lib().gs_gemm_skinny_qkv_supports(c_int(d), c_int(rotary_dim)))
-
-
-def gemm_skinny_qkv(x, wqkv, q_weight, k_weight, head_eps, cos, sin, positions, block_table, page_size,
-                    kcache, vcache, nh, nkv, d, write_kv=True, wt=None) -> torch.Tensor:
-    """A decode step's q, k, v: product, head norms, rotation and cache write in one kernel; returns q ``(M, nh d)``."""
-    _dev(wqkv, q_weight, k_weight, cos, sin, positions, block_table, kcache, vcache)
-    _need(lazy_ok(x, wqkv) if isinstance(x, LazyNorm) else skinny_ok(x, wqkv),
-          "gemm_skinny_qkv: needs bfloat16 rows or a lazy norm, and a bfloat16 weight")
-    M, K = x.shape
-    _need(wqkv.shape == ((nh + 2 * nkv) * d, K), "gemm_skinny_qkv: the weight must be ((nh + 2 nkv) d, K)")
-    for w in (q_weight, k_weight):
-        _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "gemm_skinny_qkv: head norm weight float32 (d,)")
-    _need(cos.dtype == torch.float32 and cos.shape == sin.shape and cos.shape[1] == d // 2, "gemm_skinny_qkv: tables (P, d/2)")
-    _i32(positions, M, "positions")
-    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] >= M, "block_table int32 (M, blocks)")
-    _need(kcache.dtype == torch.bfloat16 and kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d)
-          and vcache.shape == kcache.shape, "cache must be bfloat16 (pages, nkv, page_size, d)")
-    q = torch.empty((M, nh * d), dtype=torch.bfloat16, device=wqkv.device)
-    _check(lib().gs_gemm_skinny_qkv(*_lazy_args(x), _p(wqkv),
-                                    _p(wt), _p(q_weight), _p(k_weight), c_float(head_eps), _p(cos), _p(sin), _p(positions),
-                                    _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
-                                    _p(vcache), c_int(1 if write_kv else 0), _p(q), c_int(M), c_int(nh), c_int(nkv),
-                                    c_int(d), c_int(K), _stream()))
-    return q
 
 
 def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live) -> None:

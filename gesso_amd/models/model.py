@@ -82,20 +82,22 @@ class Model:
     def forward(self, ctx) -> Optional[torch.Tensor]:
         """Run the tokens of ``ctx`` through every scheduled block; float32 logits at ``ctx.want_rows``."""
         ops, rt = self.rt.ops, self.rt
-        decode_only = getattr(ctx, "decode_only", False)
+        decode_only = ctx.decode_only
         # the norm that reads the stream after the i-th scheduled block: the next block's first, then the final one
+        # (``first_norm`` and ``row_weight`` are the optional hints of blocks and norms, see parts/base.py)
         order = [self.blocks[call.layer] for call in self.spec.schedule]
         readers = [getattr(b, "first_norm", None) for b in order[1:]] + [self.final_norm if decode_only else None]
+        scale = 1.0 if self.spec.embed_scale is None else float(self.spec.embed_scale)
         if rt.fused:
             ssq = torch.empty((ctx.T, 1), dtype=torch.float32, device=rt.device)
             first = getattr(order[0], "first_norm", None) if order else None
             res = torch.empty((ctx.T, self.embed.shape[1]), dtype=torch.float32, device=rt.device)
             w = row_weight_of(first, res, rt)
             xs = rt.new_rows(*res.shape) if w is not None else None
-            ops.embed(ctx.token_ids, self.embed, out=res, ssq=ssq, next_weight=w, xs=xs)
+            ops.embed(ctx.token_ids, self.embed, out=res, ssq=ssq, next_weight=w, xs=xs, scale=scale)
             stream = ResidualStream(res, ssq=ssq, xs=xs, xs_for=first if xs is not None else None)
         else:
-            stream = ResidualStream(ops.embed(ctx.token_ids, self.embed))
+            stream = ResidualStream(ops.embed(ctx.token_ids, self.embed, scale=scale))
         for i, call in enumerate(self.spec.schedule):
             stream.following = readers[i]
             order[i].forward(stream, ctx, ctx.cache_view(i))
@@ -104,4 +106,7 @@ class Model:
         # every row wanted, in order (a decode step): no gather, and the norm may stay lazy
         rows = None if decode_only else ctx.want_rows
         normed = self.final_norm.add_norm(stream, rows=rows)
-        return self.rt.linear(normed, self.head, out_dtype=torch.float32)
+        logits = self.rt.linear(normed, self.head, out_dtype=torch.float32)
+        if self.spec.logit_softcap is not None:
+            ops.softcap(logits, float(self.spec.logit_softcap))
+        return logits

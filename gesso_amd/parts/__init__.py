@@ -2,4 +2,4 @@ from . import attention, block, rmsnorm, rope, shortconv, swiglu  # noqa: F401  
 from .base import MATRIX, TABLE, VECTOR, PagedKV, Part, SlotState, TensorSpec
 from .registry import build, part_class, register, unregister
 from .rmsnorm import ResidualStream
-from .runtime import Runtime
+from .runtime import DeferredLinear, Runtime, RuntimeOptions

@@ -17,6 +17,17 @@ from .base import MATRIX, VECTOR, PagedKV, Part, TensorSpec
 from .registry import build, register
 
 
+class RawQKV:
+    """Rows of q|k|v as their product left them, with what the decode kernel needs to finish them itself
+    (head norms, rotation, cache write)."""
+
+    __slots__ = ("qkv", "q_norm", "k_norm", "eps", "position", "dtype")
+
+    def __init__(self, qkv, q_norm, k_norm, eps, position):
+        self.qkv, self.q_norm, self.k_norm, self.eps, self.position = qkv, q_norm, k_norm, eps, position
+        self.dtype = qkv.dtype
+
+
 class Attention(Part):
     graph_safe = True
 
@@ -58,13 +69,85 @@ class Attention(Part):
         self.k_norm = tensors.get("k_norm.weight")
 
     def forward(self, x, ctx, cache):
-        s = self.spec
-        nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
-        q, q_stride = self.rt.attention_in(x, self.wqkv, self.bqkv, self.q_norm, self.k_norm,
-                                           s.qk_norm.eps if s.qk_norm is not None else 1.0, self.position, ctx,
-                                           cache, nh, nkv, d)
-        o = self.rt.attention(q, q_stride, cache, ctx, s.window, self.scale, nh, nkv, d)
+        q, q_stride = self.project_in(x, ctx, cache)
+        o = self.attend(q, q_stride, ctx, cache)
         return self.rt.project(o, self.wo, self.bo)
+
+    # ------------------------------------------------------------------ the mixer's inner steps
+
+    def project_in(self, x, ctx, cache):
+        """q, k, v products, head norms, position encoding, cache write.  Returns ``(q, q_stride)``: the queries
+        as rows of a buffer, ``q_stride`` apart, head h at ``[h d, (h+1) d)``; or a :class:`RawQKV` for the decode
+        kernel that norms, rotates and writes the cache itself."""
+        s, rt, ops, pos = self.spec, self.rt, self.rt.ops, self.position
+        nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
+        eps = s.qk_norm.eps if s.qk_norm is not None else 1.0
+        layout = getattr(pos, "layout", "half")
+        qkv = rt.linear(x, self.wqkv, self.bqkv)          # a lazy norm goes through as it is where the product takes it
+        stride = (nh + 2 * nkv) * d
+        if (rt.fused and ctx.all_single and cache.k.dtype == torch.bfloat16 and qkv.dtype == torch.bfloat16
+                and cache.page_size >= 2 and (self.q_norm is None) == (self.k_norm is None) and layout == "half"
+                and ops.attention_decode_raw_supports(nh, nkv, d, pos.rotary_dim)):
+            return RawQKV(qkv, self.q_norm, self.k_norm, eps, pos), stride
+        ops.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, eps, pos.cos, pos.sin, pos.rotary_dim, ctx.positions,
+                           ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
+                           write_kv=cache.write, layout=layout)
+        return qkv, stride
+
+    def _single(self, q, q_stride, cache, ctx, nseq, out):
+        """The first ``nseq`` sequences, one query each (their rows are the first ``nseq`` rows).  A block of eight
+        wavefronts takes a tile of 64 keys per wavefront and pass; key streams are split over blocks (and a merge
+        kernel) only when the batch alone does not fill the chip."""
+        s, ops = self.spec, self.rt.ops
+        nh, nkv, d, window = s.n_heads, s.n_kv_heads, s.head_dim, s.window
+        longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
+        if window:
+            longest = min(longest, window)
+        tiles = max(1, -(-longest // 64))
+        # (sequence, key head) pairs fill the chip by themselves from about 256 on; fewer pairs share their keys out
+        # over blocks, each split at least 1,024 keys long (measured at 8 sequences of 32,768 keys: 4 splits 107 us,
+        # 32 splits 145 us; at 64 sequences any split is slower than none)
+        nsplit = max(1, min(tiles // 16, 64, 256 // max(1, nseq * nkv)))
+        if isinstance(q, RawQKV):
+            return ops.attention_decode_raw(q.qkv, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
+                                            cache.page_size, window, self.scale, q.q_norm, q.k_norm, q.eps,
+                                            q.position.cos, q.position.sin, nh, nkv, d, nseq, nsplit,
+                                            write_kv=cache.write, out=out)
+        return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
+                                    cache.page_size, window, self.scale, nh, nkv, d, nseq, nsplit, out=out)
+
+    def attend(self, q, q_stride, ctx, cache) -> torch.Tensor:
+        """Causal attention of this step's queries over the paged cache; ``(T, nh * d)``.
+
+        The generic kernel takes every size; faster kernels take over for the sizes and batch
+        shapes they are written for.
+        """
+        s, rt, ops = self.spec, self.rt, self.rt.ops
+        nh, nkv, d, window = s.n_heads, s.n_kv_heads, s.head_dim, s.window
+        out = True if rt.rows_tiled(nh * d) else None
+        if isinstance(q, RawQKV):
+            return self._single(q, q_stride, cache, ctx, ctx.nseq, out)
+        fast = q.dtype == torch.bfloat16 and cache.page_size >= 2
+        if ctx.all_single and fast and ops.attention_decode_supports(nh, nkv, d):
+            return self._single(q, q_stride, cache, ctx, ctx.nseq, out)
+        if (not ctx.all_single and fast and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d)):
+            # prompts: queries in tiles per sequence, both products on the matrix cores; tiles of 32 share
+            # every key and value fragment between two products, which pays when portions are long
+            # (groups of more than four heads have no registers for tiles of 32)
+            rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16
+            # decoded tokens at the batch's head go to the kernel for single queries: as tiles of one query they
+            # would each hold a whole block that walks all the keys alone
+            lead = getattr(ctx, "lead_single", 0)
+            if not ops.attention_decode_supports(nh, nkv, d):
+                lead = 0
+            out = torch.empty((ctx.T, nh * d), dtype=q.dtype, device=q.device)
+            if lead:
+                self._single(q, q_stride, cache, ctx, lead, out[:lead])
+            return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows, lead),
+                                         cache.block_table, cache.page_size, window, self.scale, nh, nkv, d, ctx.T,
+                                         out=out, tile_rows=rows)
+        return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token,
+                                     cache.block_table, cache.page_size, window, self.scale, nh, nkv, d, ctx.T)
 
 
 register("mixer", "attention", Attention)

@@ -7,16 +7,21 @@ in the weight file.
 
 Interfaces (duck-typed; the classes below are convenient bases):
 
-* norm            ``tensor_specs(spec)``, ``bind(tensors)``,
-                  ``add_norm(residual, delta, out=None, rows=None) -> normed``
+* norm            ``tensor_specs(spec)``, ``bind(tensors)``, ``add_norm(stream, rows=None, out=None) -> normed``;
+                  optional hint ``row_weight``: a float32 vector ``w`` with ``norm(x) = inv_rms(x) * (x * w)``, which
+                  lets whatever writes the stream before the norm leave the rows pre-weighted (None: no such form)
 * position        ``tensor_specs(spec)`` (usually none), ``bind``, attributes
-                  ``cos``, ``sin`` (``(max_position, rotary_dim/2)`` float32) and ``rotary_dim``;
+                  ``cos``, ``sin`` (``(max_position, rotary_dim/2)`` float32), ``rotary_dim`` and ``layout``
+                  (``"half"``: pairs ``(i, i + rotary_dim/2)``, ``"interleaved"``: ``(2i, 2i + 1)``);
                   or ``rotary_dim == 0`` for none
 * mixer           ``tensor_specs(spec)``, ``cache_need(spec) -> PagedKV | SlotState | None``,
                   ``bind(tensors)``, ``forward(x, ctx, cache) -> (T, hidden)``
 * feed-forward    ``tensor_specs(spec)``, ``bind(tensors)``, ``forward(x, ctx) -> (T, hidden)``
 * block           ``tensor_specs(spec)``, ``cache_need(spec)``, ``bind``,
-                  ``forward(stream, ctx, cache)`` on a :class:`ResidualStream`
+                  ``forward(stream, ctx, cache)`` on a :class:`ResidualStream`; optional hint ``first_norm``: the
+                  norm that reads the stream first when the block runs (None: unknown)
+
+``Part`` below carries the optional hints with their defaults, so a part derived from it need not mention them.
 """
 from __future__ import annotations
 
@@ -49,13 +54,29 @@ class PagedKV:
 
 @dataclass(frozen=True)
 class SlotState:
-    """Per-request state of fixed size: ``name -> (shape, dtype name)``; zero at a request's start."""
+    """Per-request state of fixed size.  ``tensors``: ``(name, shape, dtype name)`` or ``(name, shape, dtype name,
+    initial value)`` each; ``dtype name`` is ``"float32"`` or ``"bfloat16"``; a slot handed to a request is filled
+    with the initial value (0 unless given)."""
 
-    tensors: Tuple[Tuple[str, Tuple[int, ...], str], ...]
+    tensors: Tuple[tuple, ...]
+
+    def entries(self):
+        """``(name, shape, dtype name, initial value)`` of every tensor."""
+        out = []
+        for t in self.tensors:
+            if len(t) not in (3, 4):
+                raise ValueError(f"a state tensor is (name, shape, dtype[, initial value]), not {t!r}")
+            name, shape, dtype = t[:3]
+            out.append((name, tuple(int(n) for n in shape), dtype, float(t[3]) if len(t) == 4 else 0.0))
+        return out
 
 
 class Part:
     """Base of parts: keeps spec and runtime; subclasses fill the rest."""
+
+    graph_safe = False      # True: forward makes no host round trip, so a decode step through it may be recorded
+    row_weight = None       # norms: see the module's text
+    first_norm = None       # blocks: see the module's text
 
     def __init__(self, spec, rt):
         self.spec = spec

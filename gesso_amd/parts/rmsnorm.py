@@ -47,7 +47,7 @@ class ResidualStream:
                 w = None
             eps = eps if w is not None else 0.0
             self.ssq, self.normed = rt.ops.gemm_skinny_residual_parts(
-                out.x, out.w, self.res, rt.split_parts(out.w), wt=rt._wt(out.w), next_weight=w, eps=eps, out_dtype=rt.dtype,
+                out.x, out.w, self.res, rt.split_parts(out.w), wt=rt.tiles_of(out.w), next_weight=w, eps=eps, out_dtype=rt.dtype,
                 tiled=w is not None and rt.rows_tiled(self.res.shape[1]))
             self.xs_for = next_norm if self.normed is not None else None
         elif isinstance(out, DeferredLinear):
@@ -55,7 +55,7 @@ class ResidualStream:
             if w is not None:
                 self.xs = rt.new_rows(*self.res.shape)
                 self.xs_for = next_norm
-            self.ssq = rt.ops.gemm_skinny_residual(out.x, out.w, self.res, wt=rt._wt(out.w), next_weight=w, xs=self.xs)
+            self.ssq = rt.ops.gemm_skinny_residual(out.x, out.w, self.res, wt=rt.tiles_of(out.w), next_weight=w, xs=self.xs)
         else:
             self.pending, self.ssq = out, None
 

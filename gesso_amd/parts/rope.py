@@ -1,7 +1,9 @@
-"""Position encodings as tables: what the attention kernels need is ``cos``, ``sin`` and ``rotary_dim``.
+"""Position encodings as tables: what the attention kernels need is ``cos``, ``sin``, ``rotary_dim`` and ``layout``.
 
-Rotary, half-split pairs ``(i, i + rotary_dim/2)``, angle ``pos * theta^(-2i/rotary_dim)``
-(reference ``src/Operators/cpu.jl:357-371``, ``interleaved=false``).  Angles, cosines and
+Rotary; pair ``i`` is ``(i, i + rotary_dim/2)`` (``layout = "half"``) or ``(2i, 2i + 1)`` (``"interleaved"``), its
+angle ``pos * theta^(-2i/rotary_dim)`` (reference ``src/Operators/cpu.jl:357-371``; LFM2 has ``interleaved=false``,
+``src/Inference/architecture_spec.jl:66``).  A kernel that is written for one layout is not used for the other: the
+mixer asks ``layout`` before it takes a fused route.  Angles, cosines and
 sines are computed on the host in float64 and stored as float32, one table per distinct spec.
 Another encoding (scaled frequencies, another theta per layer) is another class that fills
 the same three attributes; ``rotary_dim = 0`` means none.
@@ -29,6 +31,9 @@ class Rope(Part):
         if spec.rotary_dim % 2 or not 0 < spec.rotary_dim <= spec.head_dim:
             raise ValueError(f"rotary_dim {spec.rotary_dim} must be even and within the head width {spec.head_dim}")
         self.rotary_dim = spec.rotary_dim
+        self.layout = getattr(spec, "layout", "half")
+        if self.layout not in rt.ops.ROPE_LAYOUTS:
+            raise ValueError(f"rotation pairs are laid out 'half' or 'interleaved', not {self.layout!r}")
 
         def make():
             cos, sin = rope_tables(spec.rotary_dim, spec.theta, spec.max_position)
@@ -40,6 +45,7 @@ class Rope(Part):
 class NoPosition(Part):
     graph_safe = True
     rotary_dim = 0
+    layout = "half"
     cos = None
     sin = None
 

@@ -40,8 +40,23 @@ class ShortConv(Part):
         self.b_out = tensors.get("out_proj.bias")
 
     def forward(self, x, ctx, cache):
-        mixed = self.rt.conv_in(x, self.w_in, self.b_in, self.taps, self.b_conv, cache.state["history"], ctx)
+        mixed = self.mix(x, ctx, cache.state["history"])
         return self.rt.project(mixed, self.w_out, self.b_out)
+
+    def mix(self, x, ctx, state):
+        """Input product and gated short convolution: ``(T, H)`` mixed rows; ``state`` is advanced.
+
+        While a decode step is recorded the convolution runs as the epilogue of its input product
+        (one token per sequence, taps in registers); otherwise the product, then the kernel over segments."""
+        rt, ops = self.rt, self.rt.ops
+        if rt.fused and self.b_in is None and ctx.all_single and self.taps.shape[1] <= 16:
+            x = rt.lazy_rows(x)
+            if rt.streams(x, self.w_in):
+                return ops.gemm_skinny_conv(x, self.w_in, self.taps, self.b_conv, state, ctx.slots,
+                                            wt=rt.tiles_of(self.w_in), tiled=rt.rows_tiled(self.taps.shape[0]))
+        bcx = rt.linear(rt.dense(x), self.w_in, self.b_in)
+        return ops.short_conv(bcx, self.taps, self.b_conv, state, ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq,
+                              ctx.all_single)
 
 
 register("mixer", "short_conv", ShortConv)

@@ -143,9 +143,10 @@ class TraceRun:
         return rc
 
 
-def run_trace(model_dir, dtype, out_dir, trace: Trace, vocab: int, max_tokens=None):
+def run_trace(model_dir, dtype, out_dir, trace: Trace, vocab: int, max_tokens=None, page_size=None, extra=()):
     """Replay `trace`; returns {name: {position: logits row}} and the exit status."""
-    tr = TraceRun(model_dir, dtype, out_dir, max_tokens or trace.max_tokens)
+    extra = list(extra) + (["--page-size", str(page_size)] if page_size is not None else [])
+    tr = TraceRun(model_dir, dtype, out_dir, max_tokens or trace.max_tokens, extra=extra)
     got = {}
     try:
         for rec, rows in zip(trace.steps, trace.rows):
@@ -171,3 +172,26 @@ def worst(got, ref):
             if d > w:
                 w, where = d, (name, pos)
     return w, where
+
+
+def compare_trace(model_dir, dtype, out_dir, trace: Trace, vocab: int, ref, max_tokens=None, extra=()):
+    """Replay `trace` and compare every wanted row with `ref[name][position]` as it comes (nothing is kept: for
+    vocabularies of tens of thousands).  Returns (worst |difference|, where, exit status)."""
+    tr = TraceRun(model_dir, dtype, out_dir, max_tokens or trace.max_tokens, extra=extra)
+    w, where = 0.0, None
+    try:
+        for rec, rows in zip(trace.steps, trace.rows):
+            tr.step(rec)
+            if rows:
+                lg = tr.logits(rec["step"], vocab)
+                os.remove(os.path.join(out_dir, f"{rec['step']}.f32"))
+                assert lg.shape[0] == len(rows), (lg.shape, len(rows))
+                for (name, pos), row in zip(rows, lg):
+                    d = float(np.abs(row.astype(np.float64) - ref[name.split(".", 1)[-1]][pos]).max())
+                    if not np.isfinite(d):
+                        d = float("inf")
+                    if d > w:
+                        w, where = d, (name, pos)
+    finally:
+        rc = tr.close()
+    return w, where, rc

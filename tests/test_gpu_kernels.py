@@ -88,13 +88,22 @@ def test_swiglu(ops, dtype):
     close(got, P.swiglu(x[:, :100].double(), x[:, 100:].double()), dtype)
 
 
-def test_residual_add_and_zero_slots(ops):
+def test_residual_add_and_fill_rows(ops):
     res = torch.randn(3, 10, generator=gen(3))
     d = torch.randn(3, 10, generator=gen(4)).bfloat16()
     assert torch.equal(ops.residual_add(res.clone().to(DEV), d.to(DEV)).cpu(), res + d.float())
+    ids = torch.tensor([3, 1, -1], dtype=torch.int32, device=DEV)     # a negative id is skipped
     state = torch.ones(5, 4, 2, device=DEV)
-    ops.zero_slots(state, torch.tensor([3, 1], dtype=torch.int32, device=DEV))
+    ops.fill_rows(state, ids, 0.0)
     assert state.sum(dim=(1, 2)).tolist() == [8, 0, 8, 0, 8]
+    half = torch.ones(5, 301, dtype=torch.bfloat16, device=DEV)       # a row that is no multiple of the block
+    ops.fill_rows(half, ids, 0.25)
+    assert half.float().sum(dim=1).tolist() == [301, 75.25, 301, 75.25, 301]
+    # pages: rows 3 and 1 in every one of 2 x 2 planes of 5 rows, NaN, nothing else touched
+    pool = torch.ones(2, 2, 5, 3, 4, 6, dtype=torch.bfloat16, device=DEV)
+    ops.fill_rows(pool, ids, float("nan"), planes=3)
+    bad = torch.isnan(pool.float()).flatten(3).all(dim=3)
+    assert bad[:, :, [1, 3]].all() and not torch.isnan(pool[:, :, [0, 2, 4]].float()).any()
 
 
 # ------------------------------------------------------------------ short convolution
@@ -112,7 +121,7 @@ def test_short_conv_segments_and_history(ops, H, W, bias, dtype):
     data = {s: torch.randn(total[s], 3 * H, generator=g).to(dtype) for s in lens}
     want = {s: P.short_conv(data[s].double(), taps.double(), None if b is None else b.double()) for s in lens}
     state = torch.full((5, H, W - 1), 7.0, device=DEV)
-    ops.zero_slots(state, torch.tensor(list(lens), dtype=torch.int32, device=DEV))
+    ops.fill_rows(state, torch.tensor(list(lens), dtype=torch.int32, device=DEV), 0.0)
     at = {s: 0 for s in lens}
     got = {s: [] for s in lens}
     for step in range(4):
@@ -180,8 +189,9 @@ def rope_tables(rd, theta, n):
 @pytest.mark.parametrize("nh,nkv,d,rd,norm", [(4, 2, 16, 16, True), (3, 1, 48, 48, True), (2, 2, 128, 64, False),
                                                (5, 5, 80, 80, True), (8, 2, 256, 256, True), (32, 8, 64, 64, True),
                                                (3, 1, 32, 32, False), (2, 1, 128, 128, True)])
+@pytest.mark.parametrize("layout", ["half", "interleaved"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_qknorm_rope_kv(ops, nh, nkv, d, rd, norm, dtype):
+def test_qknorm_rope_kv(ops, nh, nkv, d, rd, norm, dtype, layout):
     g = gen(nh * 100 + d)
     ps, theta, eps = 8, 1e4, 1e-5
     # two sequences: one continues at position 13 with 5 tokens (crossing a page edge at 16), one starts with 3
@@ -198,7 +208,7 @@ def test_qknorm_rope_kv(ops, nh, nkv, d, rd, norm, dtype):
     x = qkv.clone().to(DEV)
     ops.qknorm_rope_kv(x, None if qw is None else qw.to(DEV), None if kw is None else kw.to(DEV), eps, cos, sin, rd,
                        torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(seq, dtype=torch.int32, device=DEV),
-                       table.to(DEV), ps, kc, vc, nh, nkv, d)
+                       table.to(DEV), ps, kc, vc, nh, nkv, d, layout=layout)
     src = qkv.double()
     q = src[:, :nh * d].reshape(T, nh, d)
     k = src[:, nh * d:(nh + nkv) * d].reshape(T, nkv, d)
@@ -208,7 +218,13 @@ def test_qknorm_rope_kv(ops, nh, nkv, d, rd, norm, dtype):
 
     def rot(t):
         out = t.clone()
-        out[..., :rd] = P.rope(t[..., :rd], pos, theta)
+        if layout == "half":
+            out[..., :rd] = P.rope(t[..., :rd], pos, theta)
+        else:
+            # pairs (2i, 2i + 1) (reference src/Operators/cpu.jl:357-371, interleaved): the half-split rotation of the
+            # features put in the order evens, odds, and put back
+            order = list(range(0, rd, 2)) + list(range(1, rd, 2))
+            out[..., order] = P.rope(t[..., order], pos, theta)
         return out
 
     q, k = rot(q), rot(k)
@@ -658,34 +674,6 @@ def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias, weight
     assert float((s1 - s2).abs().max()) <= 1e-2 * max(1.0, float(s2.abs().max()))
     untouched = [i for i in range(M + 2) if i not in slots.tolist()]
     assert torch.equal(s1[untouched].cpu(), state0[untouched])
-
-
-@pytest.mark.parametrize("weighted", [False, True])
-@pytest.mark.parametrize("M,nh,nkv,d,norm", [(1, 32, 8, 64, True), (8, 4, 2, 32, True), (33, 2, 1, 128, False), (64, 3, 3, 64, True)])
-def test_gemm_skinny_qkv_equals_the_separate_kernels(ops, M, nh, nkv, d, norm, weighted):
-    H = nh * d
-    res, nw, lazy = lazy_case(ops, M, H, M + H, weighted)
-    g = gen(nh + d)
-    wqkv = (torch.randn((nh + 2 * nkv) * d, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
-    qw = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV) if norm else None
-    kw = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV) if norm else None
-    ps = 16
-    cos, sin = rope_tables(d, 1e4, 256)
-    positions = torch.randint(0, 200, (M,), generator=g).to(torch.int32)
-    table = torch.zeros(M, 13, dtype=torch.int32)
-    for m in range(M):
-        table[m] = torch.arange(13, dtype=torch.int32) + 13 * m
-    kc1 = torch.zeros(13 * M, nkv, ps, d, dtype=torch.bfloat16, device=DEV)
-    vc1, kc2, vc2 = torch.zeros_like(kc1), torch.zeros_like(kc1), torch.zeros_like(kc1)
-    q = ops.gemm_skinny_qkv(lazy, wqkv, qw, kw, 1e-5, cos, sin, positions.to(DEV), table.to(DEV), ps, kc1, vc1, nh, nkv, d)
-    qkv = ops.gemm_skinny(lazy, wqkv)
-    ops.qknorm_rope_kv(qkv, qw, kw, 1e-5, cos, sin, d, positions.to(DEV), torch.arange(M, dtype=torch.int32, device=DEV),
-                       table.to(DEV), ps, kc2, vc2, nh, nkv, d)
-    ref_q = qkv[:, :nh * d].float()
-    assert float((q.float() - ref_q).abs().max()) <= 2e-2 * max(1.0, float(ref_q.abs().max()))
-    assert float((kc1.float() - kc2.float()).abs().max()) <= 2e-2 * max(1.0, float(kc2.float().abs().max()))
-    assert float((vc1.float() - vc2.float()).abs().max()) <= 2e-2 * max(1.0, float(vc2.float().abs().max()))
-    assert int((kc1.float().abs().sum(dim=(1, 3)) > 0).sum()) == M      # one row per token, nothing else
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 16384, 2048), (24, 96, 64), (64, 2048, 8192)])

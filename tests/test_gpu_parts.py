@@ -2,9 +2,10 @@
 
 A harness builds one part from its spec with random tensors, a cache for it and step contexts,
 and runs it whole and in portions.  The toy parts at the end (a mixer with a running state of
-its own, a position encoding with another table, a schedule that runs a block twice and lets a
-layer read another layer's cache) are defined here, registered here and stepped through the
-unchanged engine.
+its own, in float32 and in bfloat16, that starts from a value other than zero; a feed-forward with routing; a
+position encoding with another table and interleaved pairs; a schedule that runs a block twice and lets a
+layer read another layer's cache; a scaled embedding and capped logits) are defined here, registered here and
+stepped through the unchanged engine.
 """
 import dataclasses
 import math
@@ -60,10 +61,7 @@ class Harness:
             if e.rid not in self.manager.requests:
                 self.manager.admit(e.rid)
         if self.manager.fresh_slots:
-            slots = torch.tensor(self.manager.fresh_slots, dtype=torch.int32, device=DEV)
-            for states in self.storage.state.values():
-                for t in states.values():
-                    self.rt.ops.zero_slots(t, slots)
+            self.storage.fill_slots(self.rt.ops, self.manager.fresh_slots, "initial")
             self.manager.fresh_slots.clear()
         self.manager.reserve_many([(e.rid, len(e.tokens)) for e in es])
         c = StepContext(es, self.manager, self.storage, 1, DEV)
@@ -252,7 +250,9 @@ def register_toys():
             return out.to(x.dtype)
 
     class DecayMixer(Part):
-        """s_t = decay * s_{t-1} + x_t W^T, output s_t: a running state per request, of fixed size."""
+        """s_t = decay * s_{t-1} + x_t W^T from s_{-1} = 0.25, output s_t (1 + t / 64): a running state per request in
+        float32 that starts from a value other than zero, and a count of the tokens seen, kept in bfloat16 (whole
+        numbers up to 256 are exact there)."""
 
         @staticmethod
         def tensor_specs(spec):
@@ -260,35 +260,40 @@ def register_toys():
 
         @staticmethod
         def cache_need(spec):
-            return SlotState((("running", (spec.hidden,), "float32"),))
+            return SlotState((("running", (spec.hidden,), "float32", 0.25), ("seen", (1,), "bfloat16")))
 
         def bind(self, tensors):
             self.w = tensors["proj.weight"]
 
         def forward(self, x, ctx, cache):
             y = self.rt.linear(x, self.w).float()
-            state = cache.state["running"]
+            state, seen = cache.state["running"], cache.state["seen"]
+            assert state.dtype == torch.float32 and seen.dtype == torch.bfloat16
             out = torch.empty_like(y)
             slots = ctx.slots.tolist()
             at = 0
             for slot, n in zip(slots, ctx.q_lens):
-                s = state[slot]
+                s, c = state[slot], float(seen[slot, 0])
                 for t in range(at, at + n):
                     s = self.spec.decay * s + y[t]
-                    out[t] = s
+                    out[t] = s * (1.0 + c / 64.0)
+                    c += 1.0
                 state[slot] = s
+                seen[slot, 0] = c
                 at += n
             return out.to(x.dtype)
 
     class ScaledRope(Part):
-        """Another position encoding: angles divided by a factor; the same three attributes."""
+        """Another position encoding: position p rotates by the angle of 4 p, and the pairs are (2i, 2i + 1)."""
+
+        layout = "interleaved"
 
         def __init__(self, spec, rt):
             super().__init__(spec, rt)
             from gesso_amd.parts.rope import rope_tables
             cos, sin = rope_tables(spec.rotary_dim, spec.theta, spec.max_position * 4)
             self.rotary_dim = spec.rotary_dim
-            self.cos = cos[::4].contiguous().to(rt.device)      # position p rotates by the angle of p / ... 4 p
+            self.cos = cos[::4].contiguous().to(rt.device)
             self.sin = sin[::4].contiguous().to(rt.device)
 
     register("mixer", "toy_decay", DecayMixer, replace=True)
@@ -321,7 +326,23 @@ def toy_spec():
     # block 0 runs twice (two states of its own); the last call reads the cache that call 1 wrote
     schedule = (LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(2, cache=1))
     return ModelSpec(architecture="ToyForTests", hidden=H, vocab=V, blocks=blocks, schedule=schedule, final_norm=norm,
-                     tie_embeddings=True, max_position=64, names={"embed": "emb", "final_norm.weight": "fn", "head": "head"})
+                     tie_embeddings=True, max_position=64, names={"embed": "emb", "final_norm.weight": "fn", "head": "head"},
+                     embed_scale=1.5, logit_softcap=3.0)
+
+
+def rope_interleaved(x, positions, theta):
+    """Pairs ``(2i, 2i + 1)`` at angle ``pos * theta^(-2i/d)``: the reference's ``interleaved=true``
+    (``src/Operators/cpu.jl:357-371``)."""
+    T, _, d = x.shape
+    out = x.clone()
+    for t in range(T):
+        for i in range(d // 2):
+            ang = float(positions[t]) * float(theta) ** (-2.0 * i / d)
+            c, s = math.cos(ang), math.sin(ang)
+            a, b = x[t, :, 2 * i], x[t, :, 2 * i + 1]
+            out[t, :, 2 * i] = a * c - b * s
+            out[t, :, 2 * i + 1] = a * s + b * c
+    return out
 
 
 def toy_plain(w, ids, margins=None):
@@ -329,15 +350,15 @@ def toy_plain(w, ids, margins=None):
     between a token's best and second-best expert (a choice that near a tie may fall either way in bfloat16)."""
     T = len(ids)
     margins = [] if margins is None else margins
-    h = P.embedding(w["emb"], ids)
+    h = P.embedding(w["emb"], ids) * 1.5
     eps = 1e-5
 
     def decay_block(h, i):
         y = P.linear(P.rmsnorm(h, w[f"L{i}.n1"], eps), w[f"L{i}.proj.weight"])
-        s, out = torch.zeros(h.shape[1], dtype=h.dtype), []
+        s, out = torch.full((h.shape[1],), 0.25, dtype=h.dtype), []
         for t in range(T):
             s = 0.5 * s + y[t]
-            out.append(s)
+            out.append(s * (1.0 + t / 64.0))
         return h + torch.stack(out)
 
     def ffn(h, i):
@@ -362,7 +383,7 @@ def toy_plain(w, ids, margins=None):
         k = P.linear(n, w[f"L{i}.k_proj.weight"]).reshape(T, 1, 16)
         v = P.linear(n, w[f"L{i}.v_proj.weight"]).reshape(T, 1, 16)
         pos = [4 * t for t in range(T)]                      # the scaled encoding: table row p is angle of 4 p
-        return P.rope(q, pos, 1e4), P.rope(k, pos, 1e4), v
+        return rope_interleaved(q, pos, 1e4), rope_interleaved(k, pos, 1e4), v
 
     h = ffn(decay_block(h, 0), 0)
     q1, k1, v1 = qkv(h, 1)
@@ -370,7 +391,7 @@ def toy_plain(w, ids, margins=None):
     h = ffn(decay_block(h, 0), 0)
     q2, _, _ = qkv(h, 2)                                     # its own queries over layer 1's keys and values
     h = h + P.linear(P.causal_attention(q2, k1, v1).reshape(T, 32), w["L2.out_proj.weight"])
-    return P.linear(P.rmsnorm(h, w["fn"], eps), w["emb"])
+    return 3.0 * torch.tanh(P.linear(P.rmsnorm(h, w["fn"], eps), w["emb"]) / 3.0)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -124,17 +124,17 @@ def test_replay_of_configurations_drawn_at_random(seed, dtype, tmp_path):
 
 
 @pytest.mark.parametrize("name", ["B", "D"])
-def test_replay_with_the_hand_written_product_for_many_rows(name, folders, tmp_path, monkeypatch):
+def test_replay_with_the_hand_written_product_for_many_rows(name, folders, tmp_path):
     """Prompts of more than 64 tokens through the hand-written matrix-core product (with its SwiGLU epilogue) instead of
     the vendor library's: whole, and in portions that change between that kernel and the weight-streaming one."""
-    monkeypatch.setenv("GESSO_GEMM", "own")          # read by the replay program's runtime
     cfg, _ = CONFIGS[name]
     model_dir = write_tiny(folders, name, torch.bfloat16)
     seqs = sequences(name)
     ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
     scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
     for way, make in (("whole", R.trace_whole), ("portions", lambda s: R.trace_portions(s, sizes=(70, 3, 66, 2, 90)))):
-        got, rc = R.run_trace(model_dir, "bfloat16", str(tmp_path / way), make(seqs), cfg.vocab_size)
+        got, rc = R.run_trace(model_dir, "bfloat16", str(tmp_path / way), make(seqs), cfg.vocab_size,
+                              extra=["--gemm", "own"])
         assert rc == 0
         w, where = R.worst(got, ref)
         print(f"{name} own product, {way}: worst |diff| {w:.3e} at {where}")
