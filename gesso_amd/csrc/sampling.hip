@@ -236,6 +236,11 @@ extern "C" int gs_sample_temperature(const float* logits, int rows, int V, const
 // are then counted off in id order.  Done twice: for the nucleus' edge, and for the draw.
 // Sums run in another order than a sequential walk, so results differ from it by rounding only.
 //
+// The same row, temperature, top_p and draw give the same id in every run: the histogram's masses are summed as
+// 64-bit integers (each weight scaled so that the largest weight a pass can meet, times V, still fits), and integer
+// addition does not care in which order the threads' atomic adds arrive.  A weight more than about 2^-45 below the
+// largest of its pass counts as zero mass there; it keeps its count, and the pass that narrows down to it scales anew.
+//
 // wbuf (rows, V) float64 is scratch for the weights.
 
 struct Crossing {
@@ -244,23 +249,28 @@ struct Crossing {
 };
 
 // strict = 0: first running sum >= target; strict = 1: first running sum > target.
-__device__ Crossing radix_descend(const double* __restrict__ w, int V, double target, int strict, double* hmass,
-                                  int* hcount, Crossing* shared_out) {
+__device__ Crossing radix_descend(const double* __restrict__ w, int V, double target, int strict,
+                                  unsigned long long* hmass, int* hcount, Crossing* shared_out) {
   unsigned long long prefix = 0;
   double above = 0.0;
+  int lv = 1;                                   // V <= 2^lv
+  while ((1 << lv) < V && lv < 30) ++lv;
   for (int pass = 0; pass < 8; ++pass) {
     int shift = 56 - 8 * pass;
     for (int b = threadIdx.x; b < 256; b += blockDim.x) {
-      hmass[b] = 0.0;
+      hmass[b] = 0ull;
       hcount[b] = 0;
     }
     __syncthreads();
     unsigned long long himask = pass == 0 ? 0ull : (~0ull) << (shift + 8);
+    // the largest weight this pass can meet: 1 (the row's maximum has weight exp(0)) or the largest pattern under the prefix
+    const double wmax = pass == 0 ? 1.0 : __longlong_as_double((long long)(prefix | ((1ull << (shift + 8)) - 1ull)));
+    const double scale = exp2((double)(62 - lv)) / wmax, unscale = 1.0 / scale;
     for (int j = threadIdx.x; j < V; j += blockDim.x) {
       unsigned long long bits = (unsigned long long)__double_as_longlong(w[j]);
       if ((bits & himask) == prefix) {
         int b = (int)((bits >> shift) & 0xff);
-        atomicAdd(&hmass[b], w[j]);
+        atomicAdd(&hmass[b], (unsigned long long)__double2ll_rn(w[j] * scale));
         atomicAdd(&hcount[b], 1);
       }
     }
@@ -271,7 +281,7 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
       for (int b = 255; b >= 0; --b) {
         if (hcount[b] == 0) continue;
         lowest = b;
-        double next = acc + hmass[b];
+        double next = acc + (double)hmass[b] * unscale;
         if (strict ? (target < next) : (next >= target)) {
           pick = b;
           break;
@@ -280,7 +290,7 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
       }
       if (pick < 0) {  // rounding left the target just above the whole mass: the last weight it is
         pick = lowest;
-        acc -= hmass[lowest];
+        acc -= (double)hmass[lowest] * unscale;
       }
       shared_out->bits = prefix | ((unsigned long long)pick << shift);
       shared_out->above = acc;
@@ -299,7 +309,7 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
 __global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
                                     const double* __restrict__ top_p, const double* __restrict__ u,
                                     double* __restrict__ wbuf, int* __restrict__ ids, int* __restrict__ bad) {
-  __shared__ double hmass[256];
+  __shared__ unsigned long long hmass[256];
   __shared__ int hcount[256];
   __shared__ Crossing cross;
   __shared__ float redf[SAMP_THREADS / 64];

@@ -129,6 +129,13 @@ class Scheduler:
     # ------------------------------------------------------------------ requests
 
     def add(self, request: Request) -> Request:
+        vocab = getattr(getattr(self.executor, "spec", None), "vocab", None)
+        if vocab is not None:
+            bad = next((t for t in request.prompt if not 0 <= t < vocab), None)
+            if bad is not None:              # refused here, alone, before it could stop a step that others share
+                err = InvalidPlan(f"token id {bad} outside the vocabulary of {vocab}", token=bad, vocab=vocab)
+                self._finish(request, "failed", live=False, error=err)
+                return request
         if request.max_new_tokens == 0:
             self._finish(request, "complete", live=False)
             return request

@@ -140,22 +140,38 @@ def linear(x: torch.Tensor, w: torch.Tensor, b=None) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- blocks
+#
+# ``store`` (default: nothing) is applied wherever an implementation that keeps activations in a narrower type than it
+# computes in would store one: the rows a norm hands to a product, a product's result, the mixed rows of the
+# convolution, rotated queries and keys, attention's output, the SwiGLU's output.  The residual stream and everything
+# inside a function above stay in the type of the inputs.  With ``store = to_bfloat16`` the model shows how far any
+# pipeline with bfloat16 activations must stand from the plain one; the reference has no such mode (its device path
+# is float32, ``ext/GessoAMDGPUExt.jl:25``).
 
-def conv_block(h, w, prefix, eps, hist=None):
+def _keep(x):
+    return x
+
+
+def to_bfloat16(x: torch.Tensor) -> torch.Tensor:
+    """Round to bfloat16 (nearest, ties to even) and widen again."""
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
+def conv_block(h, w, prefix, eps, hist=None, store=_keep):
     """norm -> in_proj -> gated conv -> out_proj, added to the stream.
 
     Reference: ``src/Inference/lfm2.jl:192-204`` and the add at ``src/Inference/Inference.jl:282``.
     """
-    n = rmsnorm(h, w[prefix + "operator_norm.weight"], eps)
-    bcx = linear(n, w[prefix + "conv.in_proj.weight"], w.get(prefix + "conv.in_proj.bias"))
+    n = store(rmsnorm(h, w[prefix + "operator_norm.weight"], eps))
+    bcx = store(linear(n, w[prefix + "conv.in_proj.weight"], w.get(prefix + "conv.in_proj.bias")))
     taps = w[prefix + "conv.conv.weight"]
     taps = taps.reshape(taps.shape[0], taps.shape[-1])
     mixed, hist = short_conv(bcx, taps, w.get(prefix + "conv.conv.bias"), hist)
-    sub = linear(mixed, w[prefix + "conv.out_proj.weight"], w.get(prefix + "conv.out_proj.bias"))
+    sub = store(linear(store(mixed), w[prefix + "conv.out_proj.weight"], w.get(prefix + "conv.out_proj.bias")))
     return h + sub, hist
 
 
-def attention_block(h, w, prefix, cfg, positions):
+def attention_block(h, w, prefix, cfg, positions, store=_keep):
     """norm -> q,k,v -> per-head q/k norm -> rope -> causal GQA -> out_proj, added to the stream.
 
     Reference: ``src/Inference/Inference.jl:296-357`` (head norm before the rotation at
@@ -163,26 +179,28 @@ def attention_block(h, w, prefix, cfg, positions):
     """
     T = h.shape[0]
     nh, nkv, d, eps = cfg["nh"], cfg["nkv"], cfg["d"], cfg["eps"]
-    n = rmsnorm(h, w[prefix + "operator_norm.weight"], eps)
-    q = linear(n, w[prefix + "self_attn.q_proj.weight"]).reshape(T, nh, d)
-    k = linear(n, w[prefix + "self_attn.k_proj.weight"]).reshape(T, nkv, d)
-    v = linear(n, w[prefix + "self_attn.v_proj.weight"]).reshape(T, nkv, d)
+    n = store(rmsnorm(h, w[prefix + "operator_norm.weight"], eps))
+    q = store(linear(n, w[prefix + "self_attn.q_proj.weight"])).reshape(T, nh, d)
+    k = store(linear(n, w[prefix + "self_attn.k_proj.weight"])).reshape(T, nkv, d)
+    v = store(linear(n, w[prefix + "self_attn.v_proj.weight"])).reshape(T, nkv, d)
     q = rmsnorm(q, w[prefix + "self_attn.q_layernorm.weight"], eps)
     k = rmsnorm(k, w[prefix + "self_attn.k_layernorm.weight"], eps)
-    q = rope(q, positions, cfg["theta"])
-    k = rope(k, positions, cfg["theta"])
-    o = causal_attention(q, k, v).reshape(T, nh * d)
-    return h + linear(o, w[prefix + "self_attn.out_proj.weight"])
+    q = store(rope(q, positions, cfg["theta"]))
+    k = store(rope(k, positions, cfg["theta"]))
+    o = store(causal_attention(q, k, v).reshape(T, nh * d))
+    return h + store(linear(o, w[prefix + "self_attn.out_proj.weight"]))
 
 
-def feed_forward_block(h, w, prefix, eps):
+def feed_forward_block(h, w, prefix, eps, store=_keep):
     """norm -> w1 (gate), w3 (up) -> swiglu -> w2 (down), added to the stream.
 
     Reference: ``src/Inference/Inference.jl:360-363`` and ``:843-884``.
     """
-    n = rmsnorm(h, w[prefix + "ffn_norm.weight"], eps)
-    a = swiglu(linear(n, w[prefix + "feed_forward.w1.weight"]), linear(n, w[prefix + "feed_forward.w3.weight"]))
-    return h + linear(a, w[prefix + "feed_forward.w2.weight"])
+    n = store(rmsnorm(h, w[prefix + "ffn_norm.weight"], eps))
+    gate = store(linear(n, w[prefix + "feed_forward.w1.weight"]))
+    up = store(linear(n, w[prefix + "feed_forward.w3.weight"]))
+    a = store(swiglu(gate, up))
+    return h + store(linear(a, w[prefix + "feed_forward.w2.weight"]))
 
 
 # --------------------------------------------------------------------------- model
@@ -219,7 +237,7 @@ def read_weights(model_dir: str, dtype=torch.float64) -> dict:
     return out
 
 
-def forward(cfg: dict, w: dict, ids, start_pos: int = 0) -> torch.Tensor:
+def forward(cfg: dict, w: dict, ids, start_pos: int = 0, store=_keep) -> torch.Tensor:
     """Logits ``(T, V)`` of a whole sequence, positions ``start_pos .. start_pos+T-1``.
 
     Reference: ``reference_prefill``, ``src/Inference/Inference.jl:179-391`` (embedding,
@@ -231,11 +249,11 @@ def forward(cfg: dict, w: dict, ids, start_pos: int = 0) -> torch.Tensor:
     for i, kind in enumerate(cfg["layers"]):
         prefix = f"model.layers.{i}."
         if kind == "conv":
-            h, _ = conv_block(h, w, prefix, cfg["eps"])
+            h, _ = conv_block(h, w, prefix, cfg["eps"], store=store)
         else:
-            h = attention_block(h, w, prefix, cfg, positions)
-        h = feed_forward_block(h, w, prefix, cfg["eps"])
-    n = rmsnorm(h, w["model.embedding_norm.weight"], cfg["eps"])
+            h = attention_block(h, w, prefix, cfg, positions, store=store)
+        h = feed_forward_block(h, w, prefix, cfg["eps"], store=store)
+    n = store(rmsnorm(h, w["model.embedding_norm.weight"], cfg["eps"]))
     head = w["model.embed_tokens.weight"] if cfg["tied"] else w["lm_head.weight"]
     return linear(n, head)
 

@@ -174,11 +174,10 @@ def worst(got, ref):
     return w, where
 
 
-def compare_trace(model_dir, dtype, out_dir, trace: Trace, vocab: int, ref, max_tokens=None, extra=()):
-    """Replay `trace` and compare every wanted row with `ref[name][position]` as it comes (nothing is kept: for
-    vocabularies of tens of thousands).  Returns (worst |difference|, where, exit status)."""
+def visit_trace(model_dir, dtype, out_dir, trace: Trace, vocab: int, visit, max_tokens=None, extra=()):
+    """Replay `trace` and hand every wanted row to `visit(name, position, row)` as it comes (nothing is kept: for
+    vocabularies of tens of thousands).  Returns the exit status."""
     tr = TraceRun(model_dir, dtype, out_dir, max_tokens or trace.max_tokens, extra=extra)
-    w, where = 0.0, None
     try:
         for rec, rows in zip(trace.steps, trace.rows):
             tr.step(rec)
@@ -187,11 +186,28 @@ def compare_trace(model_dir, dtype, out_dir, trace: Trace, vocab: int, ref, max_
                 os.remove(os.path.join(out_dir, f"{rec['step']}.f32"))
                 assert lg.shape[0] == len(rows), (lg.shape, len(rows))
                 for (name, pos), row in zip(rows, lg):
-                    d = float(np.abs(row.astype(np.float64) - ref[name.split(".", 1)[-1]][pos]).max())
-                    if not np.isfinite(d):
-                        d = float("inf")
-                    if d > w:
-                        w, where = d, (name, pos)
+                    visit(name, pos, row.astype(np.float64))
     finally:
         rc = tr.close()
-    return w, where, rc
+    return rc
+
+
+class Distance:
+    """Running largest and root-mean-square difference between rows, with the place of the largest."""
+
+    def __init__(self):
+        self.worst, self.where, self.sq, self.n = 0.0, None, 0.0, 0
+
+    def add(self, a, b, where):
+        d = np.abs(a - b)
+        m = float(d.max())
+        if not np.isfinite(m):
+            m = float("inf")
+        if m > self.worst:
+            self.worst, self.where = m, where
+        self.sq += float((d * d).sum())
+        self.n += d.size
+
+    @property
+    def rms(self):
+        return (self.sq / max(1, self.n)) ** 0.5

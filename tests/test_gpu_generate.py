@@ -138,12 +138,138 @@ def test_preemption_on_the_gpu_changes_no_output(plain):
     prompts = [random_ids(n, cfg["V"], 50 + n) for n in (20, 33, 9, 41, 15)]
     roomy = Session(d, dtype="float32", context_length=128, max_tokens=1024)
     want = roomy.generate(prompts, max_new_tokens=20, eos_ids=())
-    tight = Session(d, dtype="float32", context_length=128, num_pages=7, page_size=16, chunk_size=16, max_num_seqs=3)
+    # with the margin at admission switched off, so that the pool runs dry in the middle of decoding; pages and slots
+    # that come back are filled with NaN before they are used again: a request computed again must not see them
+    tight = Session(d, dtype="float32", context_length=128, num_pages=7, page_size=16, chunk_size=16, max_num_seqs=3,
+                    watermark=0.0, poison=True)
     got = tight.generate(prompts, max_new_tokens=20, eos_ids=())
     assert got == want
     assert tight.last_stats["preemptions"] > 0
     st = tight.engine.manager.stats()
     assert st["pages_free"] == [7] and st["slots_free"] == st["slots_total"]
+
+
+def test_a_sampled_request_that_is_preempted_draws_on_where_it_stopped(plain):
+    """Requests that draw at a temperature, in a pool so small that some are preempted and computed again: each must
+    come out as in a roomy pool, token for token (the sampler's state is kept across the preemption, and a draw is made
+    once per token, never again for a token that is already there)."""
+    from gesso_amd import Sampler, Session
+    d, cfg, w = plain["A"]
+    prompts = [random_ids(n, cfg["V"], 90 + n) for n in (20, 33, 9, 41, 15)]
+    roomy = Session(d, dtype="float32", context_length=128, max_tokens=1024)
+    want = roomy.generate(prompts, max_new_tokens=20, sampler=Sampler(0.8, seed=7), eos_ids=())
+    tight = Session(d, dtype="float32", context_length=128, num_pages=7, page_size=16, chunk_size=16, max_num_seqs=3,
+                    watermark=0.0)
+    got = tight.generate(prompts, max_new_tokens=20, sampler=Sampler(0.8, seed=7), eos_ids=())
+    assert tight.last_stats["preemptions"] > 0
+    assert got == want
+    ids, state = list(prompts[0]), 7                       # and the roomy run is the plain sampler's
+    for _ in range(20):
+        tok, state = P.sample_id(P.forward(cfg, w, ids)[-1].tolist(), 0.8, 1.0, state)
+        ids.append(tok)
+    assert want[0] == ids
+
+
+def test_poison_fills_what_is_given_back_and_a_read_past_the_end_shows_it(plain):
+    from gesso_amd import Engine, StepEntry
+    d, cfg, w = plain["A"]
+    eng = Engine.from_folder(d, dtype="float32", page_size=8, num_pages=6, num_slots=2, poison=True)
+    kv = eng.storage.kv[0]
+    assert bool(torch.isnan(kv[:, :, :-1]).all())                    # nothing holds a stale value from the start
+    ids = random_ids(13, cfg["V"], 31)
+    eng.add_request("a")
+    logits = eng.step([StepEntry("a", ids, [12])])
+    ref = P.forward(cfg, w, ids)[-1]
+    assert float((logits[0].double().cpu() - ref).abs().max()) <= 1e-4 * max(1.0, float(ref.abs().max()))
+    pages = list(eng.manager.get("a").tables[0])
+    slot = eng.manager.get("a").slot
+    assert len(pages) == 2 and not torch.isnan(kv[:, :, pages[0]]).any()
+    # the second page holds rows 8..12; its last three rows belong to nobody yet
+    assert not torch.isnan(kv[:, :, pages[1], :, :5]).any() and bool(torch.isnan(kv[:, :, pages[1], :, 5:]).all())
+    # a read one row past the end, through the generic attention kernel: the NaN arrives on the host
+    ops = eng.rt.ops
+    m = eng.model.blocks[1].mixer.spec
+    q = torch.ones((1, m.n_heads * m.head_dim), device=eng.device)
+    table = torch.tensor([pages], dtype=torch.int32, device=eng.device)
+    zero = torch.zeros(1, dtype=torch.int32, device=eng.device)
+
+    def attend(last_key):
+        pos = torch.tensor([last_key], dtype=torch.int32, device=eng.device)
+        return ops.attention_generic(q, q.shape[1], kv[0, 0], kv[0, 1], pos, zero, table, 8, None, 0.25, m.n_heads,
+                                     m.n_kv_heads, m.head_dim, 1)
+
+    assert bool(torch.isfinite(attend(12)).all()) and bool(torch.isnan(attend(13)).any())
+    eng.finish_request("a")
+    eng.add_request("b")                                              # the next step poisons what "a" gave back
+    eng.step([StepEntry("b", ids[:3], [])])
+    held = eng.manager.get("b").tables[0]
+    for p in pages:
+        if p not in held:
+            assert bool(torch.isnan(kv[:, :, p]).all())
+    state = eng.storage.state[0]["history"]
+    if eng.manager.get("b").slot != slot:
+        assert bool(torch.isnan(state[slot]).all())
+    assert not torch.isnan(state[eng.manager.get("b").slot]).any()
+
+
+def test_a_step_that_fails_in_the_middle_releases_its_requests(plain):
+    """A kernel refuses in the middle of the model (here: a feed-forward that raises at its second call): histories
+    are partly advanced and pages partly written, so the step's requests are dropped whole; others are untouched."""
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.errors import InvalidPlan, KernelError, StepFailed
+    d, cfg, w = plain["A"]
+    eng = Engine.from_folder(d, dtype="float32", page_size=8, max_tokens=256, num_slots=4)
+    ids = random_ids(20, cfg["V"], 8)
+    eng.add_request("bystander")
+    eng.step([StepEntry("bystander", ids[:9], [])])
+    ffn = eng.model.blocks[2].ffn
+    real, calls = ffn.forward, []
+
+    def failing(x, ctx):
+        calls.append(1)
+        raise KernelError("refused, for the test")
+
+    eng.add_request("a"); eng.add_request("b")
+    ffn.forward = failing
+    with pytest.raises(StepFailed) as info:
+        eng.step([StepEntry("a", ids[:5], [4]), StepEntry("b", ids[:2], [])])
+    ffn.forward = real
+    assert calls and sorted(info.value.detail["requests"]) == ["a", "b"] and isinstance(info.value.__cause__, KernelError)
+    assert not eng.has_request("a") and not eng.has_request("b") and eng.has_request("bystander")
+    eng.manager.check()
+    with pytest.raises(InvalidPlan, match="not live"):
+        eng.step([StepEntry("a", ids[5:7], [])])
+    # the bystander goes on as if nothing had happened, and a new request under the old name starts from nothing
+    got = eng.step([StepEntry("bystander", ids[9:], [len(ids) - 10])])[0].double().cpu()
+    ref = P.forward(cfg, w, ids)
+    assert float((got - ref[-1]).abs().max()) <= 1e-4 * max(1.0, float(ref.abs().max()))
+    eng.add_request("a")
+    got = eng.step([StepEntry("a", ids[:5], [4])])[0].double().cpu()
+    assert float((got - ref[4]).abs().max()) <= 1e-4 * max(1.0, float(ref.abs().max()))
+
+
+def test_one_requests_failure_leaves_the_others_their_results(plain):
+    from gesso_amd import BatchRequest, Session, run_batch
+    from gesso_amd.errors import InvalidPlan, ResourceLimit
+    d, cfg, w = plain["A"]
+    s = Session(d, dtype="float32", context_length=48, max_tokens=256)
+    p = random_ids(6, cfg["V"], 9)
+    long = random_ids(40, cfg["V"], 10)
+    # run_batch: a request whose new tokens outgrow the context fails when it gets there; the others complete
+    res = run_batch([BatchRequest(s, p, max_new_tokens=5), BatchRequest(s, long, max_new_tokens=20),
+                     BatchRequest(s, p[:3], max_new_tokens=4), BatchRequest(s, [1, 999999], max_new_tokens=2)])
+    assert [r.status for r in res] == ["complete", "failed", "complete", "failed"]
+    assert isinstance(res[1].error, ResourceLimit) and isinstance(res[3].error, InvalidPlan)
+    assert res[0].ids == P.greedy(cfg, w, p, 5) and res[2].ids == P.greedy(cfg, w, p[:3], 4)
+    assert res[1].ids == P.greedy(cfg, w, long, 9)            # 48 tokens in the cache, and the token chosen from them
+    # generate: the failure is raised after all have run; what the others made is at hand
+    with pytest.raises(InvalidPlan, match="outside the vocabulary") as info:
+        s.generate([p, [1, 999999], p[:3]], max_new_tokens=4)
+    results = info.value.detail["results"]
+    assert [r.status for r in results] == ["complete", "failed", "complete"] and results is s.last_results
+    assert results[0].ids == P.greedy(cfg, w, p, 4) and results[2].ids == P.greedy(cfg, w, p[:3], 4)
+    st = s.engine.manager.stats()
+    assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
 
 
 def test_run_batch_statuses_and_cancel(plain):
@@ -230,7 +356,9 @@ def test_recorded_decode_loop_equals_single_steps(folders, name, dtype):
     d = write_tiny(folders, name, torch.float32 if dtype == "float32" else torch.bfloat16)
     cfg, _ = CONFIGS[name]
     prompts = [random_ids(n, cfg.vocab_size, 300 + n) for n in (7, 19, 33)]
-    samplers = lambda: [None, Sampler(0.8, 1.0, 5), None]
+    # float32: one request draws at a temperature; bfloat16: all greedy, so that each token can be held against the
+    # plain logits (a draw has no such check: where it falls depends on every logit's rounding)
+    samplers = lambda: [None, Sampler(0.8, 1.0, 5) if dtype == "float32" else None, None]
 
     def prefill(eng):
         firsts = []
@@ -249,7 +377,8 @@ def test_recorded_decode_loop_equals_single_steps(folders, name, dtype):
         ref.append(list(toks))
     # the recorded loop: runs of 1, 8, 5 and 7 steps, with unrelated work between the runs
     eng2 = Engine.from_folder(d, dtype=dtype, page_size=8, max_tokens=512)
-    toks, sm, got = prefill(eng2), samplers(), []
+    first = prefill(eng2)
+    toks, sm, got = list(first), samplers(), []
     for n in (1, 8, 5, 7):
         ids, bad = eng2.decode([0, 1, 2], toks, n, sm)
         assert not bad.any()
@@ -262,9 +391,15 @@ def test_recorded_decode_loop_equals_single_steps(folders, name, dtype):
     if dtype == "float32":
         assert got == ref
     else:
-        # bfloat16: the recorded loop uses the weight-streaming products throughout; near-ties may fall the other way
-        agree = sum(a == b for ra, rb in zip(got, ref) for a, b in zip(ra, rb))
-        assert agree >= 0.9 * 21 * 3
+        # bfloat16: the recorded loop's fused kernels round elsewhere than the step-by-step ones, so a near-tie may fall
+        # the other way; every token it chose must be the plain model's best, or as good within the logits' tolerance
+        cfgp, w = P.read_config(d), P.read_weights(d)
+        for i, p in enumerate(prompts):
+            seq = list(p) + [first[i]] + [row[i] for row in got]
+            plain_rows = P.forward(cfgp, w, seq[:-1])
+            for at in range(len(p) + 1, len(seq)):
+                row = plain_rows[at - 1]
+                assert float(row.max() - row[seq[at]]) <= 1.5e-2 * max(1.0, float(row.abs().max())), (i, at)
     assert [eng2.length(i) for i in range(3)] == [len(p) + 21 for p in prompts]
 
 

@@ -72,6 +72,18 @@ def test_add_rmsnorm(ops, H, dtype):
     assert torch.equal(r3.cpu(), res)
 
 
+def test_a_norm_whose_sum_of_squares_overflows_poisons_the_row(ops):
+    """Values that are finite with a sum of squares that is not: dividing by an infinite root would quietly give a row
+    of zeros; the row comes out NaN instead, so that the request fails where its next token is chosen (the reference
+    raises at the norm, ``src/Operators/cpu.jl:260-266``).  Other rows are untouched."""
+    res = torch.randn(3, 64, generator=gen(12))
+    res[1] *= 1e30
+    w = torch.ones(64)
+    out = ops.add_rmsnorm(res.to(DEV), None, w.to(DEV), 1e-5, torch.float32).cpu()
+    assert bool(torch.isnan(out[1]).all()) and bool(torch.isfinite(out[[0, 2]]).all())
+    close(out[[0, 2]], P.rmsnorm(res[[0, 2]].double(), w.double(), 1e-5), torch.float32)
+
+
 def test_rmsnorm_does_not_depend_on_the_batch(ops):
     g = gen(1)
     res = torch.randn(9, 200, generator=g)
@@ -418,6 +430,26 @@ def test_sample_top_p_follows_the_plain_sampler(ops, V, temp, top_p):
                                 torch.full((rows,), top_p, dtype=torch.float64, device=DEV),
                                 torch.tensor(us, dtype=torch.float64, device=DEV))
     assert ids.tolist() == want and not any(bad.tolist())
+
+
+def test_sample_top_p_gives_the_same_id_every_time_and_at_the_models_vocabulary(ops):
+    """The histogram's masses are integer sums, so no order of the threads' additions can move an edge; a row of
+    65,536 logits with thousands of weights that differ in their last bits, drawn many times with the same draw."""
+    V, rows = 65536, 6
+    logits = torch.randn(rows, V, generator=gen(91)) * 1.5
+    logits[1] = (logits[1] * 4096).round() / 4096 * 1e-3          # near-ties everywhere
+    logits[2, 1000:3000] = 5.0                                      # two thousand exact ties inside the nucleus
+    t = torch.full((rows,), 0.9, dtype=torch.float64, device=DEV)
+    p = torch.full((rows,), 0.73, dtype=torch.float64, device=DEV)
+    us = [P.splitmix64_unit(40 + r)[1] for r in range(rows)]
+    u = torch.tensor(us, dtype=torch.float64, device=DEV)
+    x = logits.to(DEV)
+    first, _ = ops.sample_top_p(x, t, p, u)
+    for _ in range(30):
+        again, bad = ops.sample_top_p(x, t, p, u)
+        assert again.tolist() == first.tolist() and not any(bad.tolist())
+    for r in (0, 2, 5):                                              # and they are the plain sampler's ids
+        assert first[r].item() == P.sample_id(logits[r].tolist(), 0.9, 0.73, 40 + r)[0], r
 
 
 # ------------------------------------------------------------------ the weight-streaming product

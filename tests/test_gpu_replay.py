@@ -139,3 +139,35 @@ def test_replay_with_the_hand_written_product_for_many_rows(name, folders, tmp_p
         w, where = R.worst(got, ref)
         print(f"{name} own product, {way}: worst |diff| {w:.3e} at {where}")
         assert w <= TOL["bfloat16"] * scale, f"{way}: first look at {where}"
+
+
+@pytest.mark.parametrize("poison", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_with_pages_of_eight_and_portions_of_thirteen(dtype, poison, folders, tmp_path):
+    """The second tiny configuration as its workload is described: pages of 8 tokens, prompts of 1, 9, 40 and 100 tokens
+    plus 24 more, portions of 13.  With ``poison`` every page and slot that is given back is filled with NaN before the
+    next step: a kernel that reads a row of a page that is not its sequence's (the rest of a last page, a page of
+    someone who has finished) would carry the NaN into the logits."""
+    cfg, _ = CONFIGS["B"]
+    model_dir = write_tiny(folders, "B", torch.float32 if dtype == "float32" else torch.bfloat16)
+    seqs = sequences("B")
+    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
+    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    ways = {"whole": R.trace_whole, "tail": R.trace_tail, "portions": lambda s: R.trace_portions(s, sizes=(13,)),
+            "mixed": lambda s: R.trace_mixed(s, seed=3)}
+    big = R.Trace()
+    for way, make in ways.items():
+        t = make({f"{way}.{k}": v for k, v in seqs.items()})
+        for rec, rows in zip(t.steps, t.rows):
+            big.steps.append(dict(rec, step=len(big.steps)))
+            big.rows.append(rows)
+        big.max_tokens = max(big.max_tokens, t.max_tokens)
+    got, rc = R.run_trace(model_dir, dtype, str(tmp_path / "out"), big, cfg.vocab_size, page_size=8,
+                          extra=["--poison"] if poison else [])
+    assert rc == 0
+    for way in ways:
+        mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
+        assert {k: len(v) for k, v in mine.items()} == {k: len(v) for k, v in seqs.items()}, way
+        w, where = R.worst(mine, ref)
+        print(f"B, pages of 8, {dtype}, poison {poison}, {way}: worst |diff| {w:.3e} at {where}")
+        assert w <= TOL[dtype] * scale, f"{way}: first look at {where}"
