@@ -1,0 +1,333 @@
+// Prompt attention for long portions: 32 queries a wavefront, keys and values shared by a block through LDS.
+//
+// The kernel of attention_prefill_impl.h gives a wavefront 16 or 32 queries, loads keys straight into registers
+// and meets at two barriers per 64 keys; its wavefronts move in step, so the matrix cores wait while the softmax's
+// arithmetic runs and the other way round.  Here a block's wavefronts meet once per 64 keys, and two blocks
+// share a compute unit, so that one block's products run under the other's softmax:
+//
+//   * A block owns one key head and 32 WQ consecutive queries of one sequence; wavefront w takes query head
+//     w % G of the group and queries 32 (w / G) .. + 31.  (WQ = 8, 4, 2, 2, 1 for groups of 1, 2, 3, 4 and more
+//     heads: up to eight wavefronts share what is staged.)
+//   * Keys are walked in steps of 64.  A step's key rows (as they lie in the pages) and value rows (transposed:
+//     features x keys) are staged in LDS, two buffers: the loads of step s + 1 are issued before step s is
+//     computed and written to the other buffer after it; one barrier a step.  Where each key's row starts in the
+//     caches (a division by the page size, a look into the block table, a product) is worked out once per key and
+//     block, by one wavefront, three steps ahead, and lies in LDS: a thread that loads a row reads one word.
+//   * v_mfma_f32_32x32x16_bf16, both products transposed so that everything a lane holds concerns one query
+//     (lane % 32):  S^T = K Q^T  (A: 32 keys x 16 features from LDS, B: the query fragment, in registers; the
+//     lane gets keys 8 (i / 4) + 4 (lane / 32) + i % 4, i = 0 .. 15, of each 32-key half),  O^T = V^T P^T  (A: 32
+//     features x 16 keys from the transposed values in LDS, B: the lane's own probabilities as they are).  No
+//     probability crosses lanes; the maximum and the sum of a row are exchanged between lanes l and l ^ 32.
+//   * Online softmax in float32, base-2 exponentials of scores scaled by log2 e; the reference point moves only
+//     when the maximum has grown by more than 2^6 (see attention_prefill_impl.h).  Steps that every query of the
+//     wavefront sees whole carry no masks.
+//
+// Bank conflicts: key rows are 16 bytes longer than the head; the transposed values put key k of feature f at
+// column k ^ 8 ((f / 8) % 8), which spreads the sixteen-byte chunks that one wavefront writes (eight features of two
+// keys a lane) over all banks and keeps every group of four keys that a product reads in one piece.
+//
+// Causal rule, window, tiles, q, caches and out as in attention_prefill_impl.h.  Heads 64 wide.
+#include <type_traits>
+
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 pw_bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float pw_f32x16_t;
+
+#define PW_KS 64
+#define PW_SLACK 6.0f
+#define PW_LOG2E 1.4426950408889634f
+
+// maximum and sum over the lanes l and l ^ 32, by a row swap (a VALU move, no trip through LDS)
+__device__ __forceinline__ float pair_max(float x) {
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+template <int D, int G, int WQ>
+__global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
+    const int* __restrict__ positions, const int* __restrict__ tile_seq, const int* __restrict__ tile_row,
+    const int* __restrict__ tile_n, const int* __restrict__ block_table, int max_blocks, int page_size,
+    unsigned page_magic, int window, float scale, bf16* __restrict__ out, int nh, int nkv) {
+  constexpr int NT = G * WQ * 64;
+  constexpr int KK = D / 16;                  // feature steps of a score product
+  constexpr int FT = D / 32;                  // feature tiles of the output
+  constexpr int DC = D / 8;                   // 16-byte chunks of a row
+  constexpr int KROW = D + 8, VROW = PW_KS + 4;
+  constexpr int NKC = PW_KS * DC;             // key chunks of a step
+  constexpr int NVU = (PW_KS / 2) * DC;       // value units of a step: two keys x one chunk
+  constexpr int CK = (NKC + NT - 1) / NT, CV = (NVU + NT - 1) / NT;
+  static_assert(D == 64, "the swizzle of the transposed values is written for heads of 64");
+  __shared__ __align__(16) uint16_t ks[2][PW_KS][KROW];
+  __shared__ __align__(16) uint16_t vt[2][D][VROW];
+  __shared__ uint32_t rowoff[3][PW_KS];       // where a step's key rows start in the caches, in units of 16 bytes
+
+  // blocks in launch order: key head fastest, tiles from the last one back (late tiles walk the most keys)
+  const int kvh = blockIdx.x % nkv, tile = (int)(gridDim.x / nkv) - 1 - (int)(blockIdx.x / nkv);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hf = lane >> 5;
+  const int h = kvh * G + wave % G, qsub = wave / G;
+  const int seq = tile_seq[tile], row0 = tile_row[tile], nq = tile_n[tile];
+  const int* bt = block_table + (size_t)seq * max_blocks;
+  const int pos0 = positions[row0];                       // positions of a tile are consecutive
+  const int last_key = pos0 + nq - 1;
+  const int first_key = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
+  const int kbeg = (first_key / PW_KS) * PW_KS;
+  const int nsteps = (last_key - kbeg) / PW_KS + 1;
+  const int blk_lo = (int)__umulhi((unsigned)first_key, page_magic), blk_hi = (int)__umulhi((unsigned)last_key, page_magic);
+  const float sc = scale * PW_LOG2E;
+
+  // this wavefront's queries
+  const int nqs = nq - qsub * 32 < 0 ? 0 : (nq - qsub * 32 > 32 ? 32 : nq - qsub * 32);
+  const bool has_rows = nqs > 0;
+  const int r0 = row0 + qsub * 32;
+  const int pfirst = pos0 + qsub * 32, plast = pfirst + (has_rows ? nqs : 1) - 1;
+  const bool live = l32 < nqs;
+  const int my_pos = pfirst + (live ? l32 : (has_rows ? nqs - 1 : 0));
+  const int my_lo = window > 0 ? (my_pos - window + 1 > 0 ? my_pos - window + 1 : 0) : 0;
+  pw_bf16x8_t qf[KK];
+  {
+    const bf16* qrow = q + (size_t)(has_rows ? r0 + (live ? l32 : nqs - 1) : row0) * q_stride + (size_t)h * D + hf * 8;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const pw_bf16x8_t*>(qrow + kk * 16);
+  }
+  float m = -INFINITY, l = 0.f;
+  pw_f32x16_t acc[FT];
+#pragma unroll
+  for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[ft][e] = 0.f;
+
+  // ---- staging: row starts of a step into rowoff, rows of a step into registers, registers into LDS
+  // Key u of step s is looked up by thread u - (first key of the step) of the first wavefront: its page is loaded
+  // early (page_of), its row start put into LDS late (put_rows).  u is clamped to the keys of this tile: rows
+  // beyond are masked, and every load is of a row the sequence holds.
+  auto key_of = [&](int s) -> int {
+    const int u = kbeg + s * PW_KS + tid;
+    return u < first_key ? first_key : (u > last_key ? last_key : u);
+  };
+  auto page_of = [&](int s) -> int {
+    if (tid >= PW_KS) return 0;
+    return bt[(int)__umulhi((unsigned)key_of(s), page_magic)];
+  };
+  auto put_rows = [&](int s, int page) {
+    if (tid < PW_KS) {
+      const int u = key_of(s);
+      const int offs = u - (int)__umulhi((unsigned)u, page_magic) * page_size;
+      rowoff[s % 3][tid] = (((uint32_t)page * (uint32_t)nkv + (uint32_t)kvh) * (uint32_t)page_size + (uint32_t)offs) * DC;
+    }
+  };
+  const uint4* k16 = reinterpret_cast<const uint4*>(kcache);
+  const uint4* v16 = reinterpret_cast<const uint4*>(vcache);
+  uint4 kreg[CK], vreg[CV][2];
+  auto issue = [&](int s) {
+#pragma unroll
+    for (int x = 0; x < CK; ++x) {
+      const int i = tid + x * NT;
+      if (NKC % NT == 0 || i < NKC) kreg[x] = k16[(size_t)rowoff[s % 3][i / DC] + (i % DC)];
+    }
+#pragma unroll
+    for (int x = 0; x < CV; ++x) {
+      const int i = tid + x * NT;
+      if (NVU % NT == 0 || i < NVU) {
+        const int kp = i / DC, c = i % DC;
+        const uint2 two = *reinterpret_cast<const uint2*>(&rowoff[s % 3][2 * kp]);
+        vreg[x][0] = v16[(size_t)two.x + c];
+        vreg[x][1] = v16[(size_t)two.y + c];
+      }
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int x = 0; x < CK; ++x) {
+      const int i = tid + x * NT;
+      if (NKC % NT == 0 || i < NKC) *reinterpret_cast<uint4*>(&ks[buf][i / DC][(i % DC) * 8]) = kreg[x];
+    }
+#pragma unroll
+    for (int x = 0; x < CV; ++x) {
+      const int i = tid + x * NT;
+      if (NVU % NT == 0 || i < NVU) {
+        const int kp = i / DC, c = i % DC;
+        const int col = (2 * kp) ^ (8 * (c & 7));         // features 8 c .. 8 c + 7 share the swizzle
+        const uint32_t a[4] = {vreg[x][0].x, vreg[x][0].y, vreg[x][0].z, vreg[x][0].w};
+        const uint32_t b[4] = {vreg[x][1].x, vreg[x][1].y, vreg[x][1].z, vreg[x][1].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e][col]) = (a[e] & 0xffffu) | (b[e] << 16);
+          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e + 1][col]) = (a[e] >> 16) | (b[e] & 0xffff0000u);
+        }
+      }
+    }
+  };
+
+  // ---- one step of this wavefront's queries over the 64 keys in buffer `buf`
+  auto compute = [&](int buf, int k0, auto masked) {
+    constexpr bool MASK = decltype(masked)::value;
+    pw_f32x16_t st[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) st[kt][e] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const pw_bf16x8_t a = *reinterpret_cast<const pw_bf16x8_t*>(&ks[buf][kt * 32 + l32][kk * 16 + hf * 8]);
+        st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], st[kt], 0, 0, 0);
+      }
+    }
+    if (MASK) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = k0 + kt * 32 + 8 * (e >> 2) + 4 * hf + (e & 3);
+          if (key > my_pos || key < my_lo) st[kt][e] = -INFINITY;
+        }
+    }
+    float mloc = st[0][0];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) mloc = fmaxf(mloc, st[kt][e]);
+    mloc = pair_max(mloc) * sc;                 // sc > 0: the scaled maximum is the maximum of the scaled scores
+    if (mloc > m + PW_SLACK || m == -INFINITY) {
+      if (mloc > -INFINITY) {
+        const float a = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mloc);
+        l *= a;
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[ft][e] *= a;
+        m = mloc;
+      }
+    }
+    const bool none = MASK && m == -INFINITY;   // nothing seen yet: every key so far was masked
+    const float nm = none ? 0.f : -m;
+    float lsum = 0.f;
+    pw_bf16x8_t pf[4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float pj = none ? 0.f : __builtin_amdgcn_exp2f(fmaf(st[kt][e], sc, nm));
+        lsum += pj;
+        pf[kt * 2 + (e >> 3)][e & 7] = (__bf16)pj;
+      }
+    l += pair_sum(lsum);
+    // O^T += V^T P^T: chunk c holds, for the lanes of half hf, the keys kb .. kb + 3 and kb + 8 .. kb + 11
+#pragma unroll
+    for (int ft = 0; ft < FT; ++ft) {
+      const int f = ft * 32 + l32;
+      const int swz = 8 * ((f >> 3) & 7);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int kb = (c >> 1) * 32 + (c & 1) * 16 + hf * 4;
+        union {
+          pw_bf16x8_t v;
+          uint2 u2[2];
+        } a;
+        a.u2[0] = *reinterpret_cast<const uint2*>(&vt[buf][f][kb ^ swz]);
+        a.u2[1] = *reinterpret_cast<const uint2*>(&vt[buf][f][(kb + 8) ^ swz]);
+        acc[ft] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[c], acc[ft], 0, 0, 0);
+      }
+    }
+  };
+
+  put_rows(0, page_of(0));
+  if (nsteps > 1) put_rows(1, page_of(1));
+  if (nsteps > 2) put_rows(2, page_of(2));
+  __syncthreads();
+  issue(0);
+  stash(0);
+  __syncthreads();
+  for (int s = 0; s < nsteps; ++s) {
+    const int k0 = kbeg + s * PW_KS;
+    const int page_ahead = s + 3 < nsteps ? page_of(s + 3) : 0;
+    if (s + 1 < nsteps) issue(s + 1);
+    // the wavefront computes where its queries see any of the step's keys
+    if (has_rows && k0 <= plast && (window == 0 || k0 + PW_KS - 1 >= pfirst - window + 1)) {
+      const bool inner = k0 + PW_KS - 1 <= pfirst && (window == 0 || k0 >= plast - window + 1);
+      if (inner) compute(s & 1, k0, std::false_type{});
+      else compute(s & 1, k0, std::true_type{});
+    }
+    if (s + 1 < nsteps) stash((s + 1) & 1);
+    if (s + 3 < nsteps) put_rows(s + 3, page_ahead);     // rowoff[s % 3] was read for the last time when step s was issued
+    __syncthreads();
+  }
+
+  if (!live) return;
+  const float inv = 1.0f / l;
+  bf16* orow = out + (size_t)(r0 + l32) * nh * D + (size_t)h * D;
+#pragma unroll
+  for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      uint2 o;
+      o.x = (uint32_t)f32_to_bf16(acc[ft][g4 * 4 + 0] * inv).x | ((uint32_t)f32_to_bf16(acc[ft][g4 * 4 + 1] * inv).x << 16);
+      o.y = (uint32_t)f32_to_bf16(acc[ft][g4 * 4 + 2] * inv).x | ((uint32_t)f32_to_bf16(acc[ft][g4 * 4 + 3] * inv).x << 16);
+      *reinterpret_cast<uint2*>(orow + ft * 32 + g4 * 8 + hf * 4) = o;
+    }
+}
+
+// Queries a tile of this kernel holds for a group of g query heads to a key head: 32 per wavefront, and as many
+// wavefronts per head as make eight to a block (`full`) or four (for steps with few tiles: twice the blocks, two to a
+// compute unit, which spreads a short prompt's uneven walks better).
+static int wide_rows(int g, int full) {
+  const int wq = g == 1 ? 8 : (g == 2 ? 4 : (g <= 4 ? 2 : 1));
+  return 32 * (full || wq == 1 ? wq : wq / 2);
+}
+
+extern "C" int gs_attention_prefill_wide_supports(int nh, int nkv, int d) {
+  if (nkv <= 0 || nh % nkv) return 0;
+  const int g = nh / nkv;
+  return d == 64 && g >= 1 && g <= 8;
+}
+
+// The most queries a tile may hold (the host cuts each sequence's queries into tiles of at most this many).
+extern "C" int gs_attention_prefill_wide_rows(int nh, int nkv, int full) { return nkv > 0 ? wide_rows(nh / nkv, full) : 0; }
+
+extern "C" int gs_attention_prefill_wide(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                         const int* positions, const int* tile_seq, const int* tile_row,
+                                         const int* tile_n, int ntiles, const int* block_table, int max_blocks,
+                                         int page_size, long cache_pages, int window, float scale, void* out, int nh,
+                                         int nkv, int d, int tile_rows, hipStream_t stream) {
+  GS_REQUIRE(gs_attention_prefill_wide_supports(nh, nkv, d), "attention_prefill_wide: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
+  const int G = nh / nkv;
+  GS_REQUIRE(tile_rows == wide_rows(G, 1) || tile_rows == wide_rows(G, 0),
+             "attention_prefill_wide: tiles of a group of %d heads hold up to %d or %d queries, not %d", G, wide_rows(G, 1), wide_rows(G, 0), tile_rows);
+  const bool full = tile_rows == wide_rows(G, 1);
+  GS_REQUIRE(ntiles >= 0 && (long)ntiles * nkv < (1L << 31), "attention_prefill_wide: %d tiles x %d key heads are too many blocks", ntiles, nkv);
+  GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill_wide: bad page_size/max_blocks/window");
+  GS_REQUIRE(q_stride >= nh * d && q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_prefill_wide: q rows must be 16-byte aligned");
+  GS_REQUIRE(((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0 && ((uintptr_t)out & 7) == 0,
+             "attention_prefill_wide: cache and output must be aligned");
+  GS_REQUIRE(page_size >= 2 && (long)max_blocks * page_size * page_size < (1L << 32),
+             "attention_prefill_wide: page_size %d with %d blocks a sequence is outside what the kernel's division takes", page_size, max_blocks);
+  // row starts are kept as 32-bit counts of 16 bytes
+  GS_REQUIRE(cache_pages > 0 && (double)cache_pages * nkv * page_size * (d / 8) < 4294967296.0,
+             "attention_prefill_wide: a cache of %ld pages is beyond the 64 GB a layer that the kernel's row index takes", cache_pages);
+  if (ntiles == 0) return 0;
+  const unsigned page_magic = (unsigned)((1ull << 32) / (unsigned)page_size + 1);
+  dim3 grid((unsigned)ntiles * (unsigned)nkv);
+#define GS_RUN(GG, WQ)                                                                                                \
+  attention_prefill_wide_kernel<64, GG, WQ><<<grid, GG * WQ * 64, 0, stream>>>(                                       \
+      (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions, tile_seq, tile_row, tile_n,       \
+      block_table, max_blocks, page_size, page_magic, window, scale, (bf16*)out, nh, nkv)
+  switch (G) {
+    case 1: if (full) GS_RUN(1, 8); else GS_RUN(1, 4); break;
+    case 2: if (full) GS_RUN(2, 4); else GS_RUN(2, 2); break;
+    case 3: if (full) GS_RUN(3, 2); else GS_RUN(3, 1); break;
+    case 4: if (full) GS_RUN(4, 2); else GS_RUN(4, 1); break;
+    case 5: GS_RUN(5, 1); break;
+    case 6: GS_RUN(6, 1); break;
+    case 7: GS_RUN(7, 1); break;
+    default: GS_RUN(8, 1); break;
+  }
+#undef GS_RUN
+  GS_LAUNCH_CHECK("attention_prefill_wide");
+  return 0;
+}

@@ -454,6 +454,50 @@ extern "C" int gs_softcap(float* p, float cap, long n, hipStream_t stream) {
   return 0;
 }
 
+// Reads a buffer once with 16-byte loads, eight in flight per lane, and folds what it read into one word per block:
+// a measurement of what the memory system delivers to kernels of this library's kind (the ceiling that the decode
+// step's weight streams are held against), nothing the model uses.  A block walks a contiguous share of the buffer,
+// 32 KB a turn, as a weight-streaming product walks its rows (contiguous = 1), or the whole grid sweeps the buffer
+// together, neighbours in the grid reading neighbours in memory (contiguous = 0).
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ p, long n16, int contiguous,
+                                                          unsigned* __restrict__ sink) {
+  unsigned acc = 0;
+  long i, end, step, lane_step;
+  if (contiguous) {
+    const long per = ((n16 + gridDim.x - 1) / gridDim.x + 2047) / 2048 * 2048;   // whole turns of 8 x 256 words
+    i = (long)blockIdx.x * per + threadIdx.x;
+    end = (long)(blockIdx.x + 1) * per < n16 ? (long)(blockIdx.x + 1) * per : n16;
+    lane_step = blockDim.x;
+    step = 8 * lane_step;
+  } else {
+    lane_step = (long)gridDim.x * blockDim.x;
+    i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    end = n16;
+    step = 8 * lane_step;
+  }
+  for (; i + 7 * lane_step < end; i += step) {
+    uint4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = p[i + u * lane_step];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (; i < end; i += lane_step) {
+    const uint4 v = p[i];
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == 0x9e3779b9u) sink[blockIdx.x] = acc;     // practically never: the store only keeps the loads alive
+}
+
+extern "C" int gs_stream_read(const void* p, long bytes, unsigned* sink, int blocks, int contiguous, hipStream_t stream) {
+  GS_REQUIRE(bytes >= 0 && bytes % 16 == 0 && ((uintptr_t)p & 15) == 0, "stream_read: a 16-byte aligned buffer of whole 16-byte words");
+  GS_REQUIRE(blocks > 0 && blocks <= 65535 && sink, "stream_read: 1 to 65535 blocks and a word per block to write to");
+  if (bytes == 0) return 0;
+  stream_read_kernel<<<blocks, 256, 0, stream>>>((const uint4*)p, bytes / 16, contiguous, sink);
+  GS_LAUNCH_CHECK("stream_read");
+  return 0;
+}
+
 __global__ void fill_f32_kernel(float* p, float v, long n) {
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;

@@ -204,6 +204,17 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
     return logits
 
 
+def stream_read(buf: torch.Tensor, blocks: int = 2048, contiguous: bool = True, sink: torch.Tensor = None) -> None:
+    """Read ``buf`` once from memory with a plain streaming kernel (a measurement, see ``bench.py``): each block its
+    own contiguous share, or the grid sweeping the buffer together."""
+    _dev(buf, sink)
+    nbytes = buf.numel() * buf.element_size()
+    if sink is None:
+        sink = torch.zeros(blocks, dtype=torch.int32, device=buf.device)
+    _need(sink.dtype == torch.int32 and sink.numel() >= blocks, "stream_read: sink holds an int32 per block")
+    _check(lib().gs_stream_read(_p(buf), c_long(nbytes), _p(sink), c_int(blocks), c_int(1 if contiguous else 0), _stream()))
+
+
 def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
     _dev(t)
     _need(t.dtype == torch.float32, "fill_f32 takes float32")
@@ -698,4 +709,40 @@ def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table
                                       _p(tiles[1]), _p(tiles[2]), c_int(nt), _p(block_table),
                                       c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
                                       _p(out), c_int(nh), c_int(nkv), c_int(d), c_int(tile_rows), _stream()))
+    return out
+
+
+def attention_prefill_wide_supports(nh: int, nkv: int, d: int) -> bool:
+    return bool(lib().gs_attention_prefill_wide_supports(c_int(nh), c_int(nkv), c_int(d)))
+
+
+def attention_prefill_wide_rows(nh: int, nkv: int, full: bool = True) -> int:
+    """The most queries a tile of :func:`attention_prefill_wide` holds for these head counts: blocks of eight
+    wavefronts (``full``), or of four for steps with few tiles."""
+    return int(lib().gs_attention_prefill_wide_rows(c_int(nh), c_int(nkv), c_int(1 if full else 0)))
+
+
+def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv,
+                           d, ntok, out: torch.Tensor = None, full: bool = True) -> torch.Tensor:
+    """Causal GQA of long prompt portions (bfloat16, heads of 64): 32 queries a wavefront, keys and values shared by a
+    block through LDS.  ``tiles`` as for :func:`attention_prefill`, of at most ``attention_prefill_wide_rows(nh, nkv,
+    full)`` rows."""
+    _dev(q, kcache, vcache, positions, tiles, block_table, out)
+    _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
+          "attention_prefill_wide takes bfloat16")
+    _need(q.numel() >= (ntok - 1) * q_stride + nh * d if ntok else True, "attention_prefill_wide: q is too small")
+    _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
+          "cache must be (pages, nkv, page_size, d)")
+    _i32(positions, ntok, "positions")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[0] == 3, "tiles must be int32 (3, ntiles)")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
+    if out is None:
+        out = torch.empty((ntok, nh * d), dtype=q.dtype, device=q.device)
+    _need(out.shape == (ntok, nh * d) and out.dtype == q.dtype, "attention_prefill_wide: out has the wrong shape or type")
+    nt = tiles.shape[1]
+    _check(lib().gs_attention_prefill_wide(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(tiles[0]),
+                                           _p(tiles[1]), _p(tiles[2]), c_int(nt), _p(block_table),
+                                           c_int(block_table.shape[1]), c_int(page_size), c_long(kcache.shape[0]),
+                                           c_int(window or 0), c_float(scale), _p(out), c_int(nh), c_int(nkv), c_int(d),
+                                           c_int(attention_prefill_wide_rows(nh, nkv, full)), _stream()))
     return out

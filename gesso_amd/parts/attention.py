@@ -131,18 +131,24 @@ class Attention(Part):
         if ctx.all_single and fast and ops.attention_decode_supports(nh, nkv, d):
             return self._single(q, q_stride, cache, ctx, ctx.nseq, out)
         if (not ctx.all_single and fast and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d)):
-            # prompts: queries in tiles per sequence, both products on the matrix cores; tiles of 32 share
-            # every key and value fragment between two products, which pays when portions are long
-            # (groups of more than four heads have no registers for tiles of 32)
-            rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16
+            # prompts: queries in tiles per sequence, both products on the matrix cores
             # decoded tokens at the batch's head go to the kernel for single queries: as tiles of one query they
             # would each hold a whole block that walks all the keys alone
-            lead = getattr(ctx, "lead_single", 0)
-            if not ops.attention_decode_supports(nh, nkv, d):
-                lead = 0
+            lead = ctx.lead_single if ops.attention_decode_supports(nh, nkv, d) else 0
             out = torch.empty((ctx.T, nh * d), dtype=q.dtype, device=q.device)
             if lead:
                 self._single(q, q_stride, cache, ctx, lead, out[:lead])
+            choice = rt.options.prompt_attention
+            if (choice != "tiles" and ops.attention_prefill_wide_supports(nh, nkv, d)
+                    and (choice == "wide" or ctx.max_q_len >= 64)):
+                # long portions: 32 queries a wavefront, keys and values shared by the block through LDS
+                rows = ops.attention_prefill_wide_rows(nh, nkv)
+                return ops.attention_prefill_wide(q, q_stride, cache.k, cache.v, ctx.positions,
+                                                  ctx.query_tiles(rows, lead), cache.block_table, cache.page_size,
+                                                  window, self.scale, nh, nkv, d, ctx.T, out=out)
+            # tiles of 32 share every key and value fragment between two products, which pays when portions are
+            # long (groups of more than four heads have no registers for tiles of 32)
+            rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16
             return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows, lead),
                                          cache.block_table, cache.page_size, window, self.scale, nh, nkv, d, ctx.T,
                                          out=out, tile_rows=rows)

@@ -32,6 +32,9 @@ class RuntimeOptions:
     vendor's for bfloat16 results (measured on random data at 2,048 rows: 109 us against our 161 for gate|up, 124
     against 162 with the SwiGLU pass counted in; 50 against 75 for 6144 x 2048), ours where the result is float32 and
     inside a recorded graph.
+    ``prompt_attention``: attention of prompt portions in bfloat16: ``"wide"`` = the kernel for long portions wherever it
+    takes the sizes (heads of 64), ``"tiles"`` = the kernel with tiles of 16 or 32 queries always, ``"auto"`` = the
+    first for steps with a portion of at least 64 tokens, else the second.
     ``tiled_rows``: rows handed from one fused kernel to the next product travel in the order the matrix cores
     take them (``ops.TiledRows``): a product then loads them a contiguous kilobyte at a time.
     ``tile_weights``: keep a tile-major copy of each bfloat16 weight for the streaming kernels.
@@ -43,6 +46,7 @@ class RuntimeOptions:
     """
 
     many_rows: str = "auto"
+    prompt_attention: str = "auto"
     tiled_rows: bool = True
     tile_weights: bool = True
     fold_norm_rows: int = 0
@@ -51,6 +55,8 @@ class RuntimeOptions:
     def __post_init__(self):
         if self.many_rows not in ("auto", "own", "library"):
             raise KernelError(f"many_rows is 'auto', 'own' or 'library', not {self.many_rows!r}")
+        if self.prompt_attention not in ("auto", "wide", "tiles"):
+            raise KernelError(f"prompt_attention is 'auto', 'wide' or 'tiles', not {self.prompt_attention!r}")
         if self.fold_norm_rows < 0 or self.weighted_rows_max < 0:
             raise KernelError("row limits are nonnegative")
 

@@ -833,6 +833,89 @@ def test_attention_prefill_far_key_and_supports(ops):
     close(got, P.causal_attention(q.double(), k.double(), v.double()).reshape(new, -1), torch.bfloat16)
 
 
+def paged(k, v, ps, g):
+    """Keys and values (K, nkv, d) laid into pages of ps in a random order; returns caches and the block table row."""
+    K, nkv, d = k.shape
+    nblk = -(-K // ps)
+    pad = nblk * ps - K
+    kp = torch.cat([k, torch.full((pad, nkv, d), float("nan"), dtype=k.dtype)])      # rows past the end: never read
+    vp = torch.cat([v, torch.full((pad, nkv, d), float("nan"), dtype=v.dtype)])
+    perm = torch.randperm(nblk + 2, generator=g)[:nblk]
+    kc = torch.full((nblk + 2, nkv, ps, d), float("nan"), dtype=k.dtype)
+    vc = torch.full_like(kc, float("nan"))
+    kc[perm] = kp.reshape(nblk, ps, nkv, d).permute(0, 2, 1, 3)
+    vc[perm] = vp.reshape(nblk, ps, nkv, d).permute(0, 2, 1, 3)
+    return kc, vc, perm.to(torch.int32)
+
+
+@pytest.mark.parametrize("nh,nkv,ps", [(32, 8, 16), (3, 1, 16), (5, 5, 4), (4, 2, 8), (16, 2, 16), (6, 2, 6)])
+@pytest.mark.parametrize("window", [None, 37, 200])
+def test_attention_prefill_wide(ops, nh, nkv, ps, window):
+    """The kernel for long portions, heads of 64: four sequences in one launch (a long chunk over a cached prefix that
+    ends inside a page, a fresh prompt of some hundred tokens, a single token, a chunk that starts at a step's edge).
+    Rows of pages past a sequence's end hold NaN: a value read from there, even with weight zero, would show."""
+    d = 64
+    assert ops.attention_prefill_wide_supports(nh, nkv, d) and not ops.attention_prefill_wide_supports(nh, nkv, 128)
+    rows = ops.attention_prefill_wide_rows(nh, nkv)
+    assert rows == {1: 256, 2: 128, 3: 64, 4: 64}.get(nh // nkv, 32)
+    g = gen(nh + ps + (window or 0))
+    prefix, new = [75, 0, 45, 128], [141, 333, 1, 70]
+    kcs, vcs, tables, qs, want = [], [], [], [], []
+    base = 0
+    for i, (p0, n) in enumerate(zip(prefix, new)):
+        K = p0 + n
+        k, v = torch.randn(K, nkv, d, generator=g).bfloat16(), torch.randn(K, nkv, d, generator=g).bfloat16()
+        q = torch.randn(n, nh, d, generator=g)
+        if i == 1:
+            q[-1] *= 3.0                                   # sharper weights on one row
+            k[7] = (q[-1, ::nh // nkv] * 0.5).bfloat16()   # and a far key that carries weight for it
+        q = q.bfloat16()
+        kc, vc, tab = paged(k, v, ps, g)
+        kcs.append(kc); vcs.append(vc); tables.append(tab + base)
+        base += kc.shape[0]
+        qs.append(q.reshape(n, -1))
+        want.append(P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(n, -1))
+    kc, vc = torch.cat(kcs), torch.cat(vcs)
+    table = torch.zeros(len(new), max(t.numel() for t in tables), dtype=torch.int32)
+    for i, t in enumerate(tables):
+        table[i, :t.numel()] = t
+    qall, want = torch.cat(qs), torch.cat(want)
+    positions = torch.tensor([p + j for p, n in zip(prefix, new) for j in range(n)], dtype=torch.int32)
+    tiles, row = [[], [], []], 0
+    for i, n in enumerate(new):
+        for a in range(0, n, rows):
+            tiles[0].append(i); tiles[1].append(row + a); tiles[2].append(min(rows, n - a))
+        row += n
+    tiles = torch.tensor(tiles, dtype=torch.int32)
+    stride = (nh + 2 * nkv) * d
+    wide = torch.zeros(sum(new), stride, dtype=torch.bfloat16)
+    wide[:, :nh * d] = qall
+    got = ops.attention_prefill_wide(wide.to(DEV), stride, kc.to(DEV), vc.to(DEV), positions.to(DEV), tiles.to(DEV),
+                                     table.to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, sum(new))
+    close(got, want, torch.bfloat16)
+
+
+def test_attention_prefill_wide_over_thousands_of_keys(ops):
+    """A chunk of 200 queries over a prefix of 5,000 keys in pages of two (the most pages a step can touch), with and
+    without a window; one key far back carries weight for the last query."""
+    g = gen(6)
+    nh, nkv, d, ps, prefix, new = 8, 2, 64, 2, 5000, 200
+    K = prefix + new
+    for window in (None, 3000):
+        k, v, q = torch.randn(K, nkv, d, generator=g), torch.randn(K, nkv, d, generator=g), torch.randn(new, nh, d, generator=g)
+        far = 1999 if window is None else K - 2990
+        k[far, 0] = q[-1, 0] * 1.5
+        q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+        kc, vc, tab = paged(k, v, ps, g)
+        rows = ops.attention_prefill_wide_rows(nh, nkv)
+        tiles = torch.tensor([[0] * -(-new // rows), list(range(0, new, rows)),
+                              [min(rows, new - a) for a in range(0, new, rows)]], dtype=torch.int32)
+        got = ops.attention_prefill_wide(q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV),
+                                         torch.arange(prefix, K, dtype=torch.int32, device=DEV), tiles.to(DEV),
+                                         tab[None].contiguous().to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, new)
+        close(got, P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(new, -1), torch.bfloat16)
+
+
 # ------------------------------------------------------------------ rows in the matrix cores' order (tiled rows)
 
 
