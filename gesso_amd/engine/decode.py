@@ -86,8 +86,9 @@ class DecodeRunner:
         finally:
             rt.no_library = rt.fused = False
         self.logits = logits
-        ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring,
-                          self.pos, self.kv_len, self.live)
+        with rt.stage("sample"):
+            ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring,
+                              self.pos, self.kv_len, self.live)
 
     def _bound(self, longest: int) -> int:
         """The recording that serves contexts of up to ``longest`` tokens: 1024, 2048, 4096, ... tokens."""
@@ -200,8 +201,20 @@ class DecodeRunner:
             self.u[:n].copy_(torch.from_numpy(u).pin_memory().to(eng.device, non_blocking=True))
         self.temperature.copy_(torch.from_numpy(temp).pin_memory().to(eng.device, non_blocking=True))
         self.counter.zero_()
-        for _ in range(n):
-            graph.replay()
+        profile = eng.rt.profile
+        if profile is None:
+            for _ in range(n):
+                graph.replay()
+        else:
+            # profiled: the same step, launched kernel by kernel, with a pair of events around every stage
+            self.ctx.max_kv_len = self._bound(max(rc.length for rc in rcs) + n)
+            profile.window = True
+            try:
+                for _ in range(n):
+                    with profile.bracket("__step__"):
+                        self._body()
+            finally:
+                profile.window = False
         ids = self.ring[:n, :B].cpu().numpy()
         bad = self.bad_ring[:n, :B].cpu().numpy()
         # a step whose logits were not finite emits no token and makes no draw (as the step-by-step choice does):

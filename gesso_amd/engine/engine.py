@@ -155,6 +155,15 @@ class Engine:
         self.steps += 1
         return logits
 
+    # ------------------------------------------------------------------ profiling
+
+    def profile_decode(self, on: bool = True):
+        """Switch the decode stage profiler on (returns it) or off.  While it is on, decode runs launch their step
+        kernel by kernel with HIP events around every stage (:mod:`gesso_amd.engine.profile`)."""
+        from .profile import StageProfile
+        self.rt.profile = StageProfile() if on else None
+        return self.rt.profile
+
     # ------------------------------------------------------------------ decoding, recorded
 
     DECODE_MAX_BATCH = 64

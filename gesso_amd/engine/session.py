@@ -7,7 +7,8 @@ max_new_tokens=8, on_token)`` returning the prompt followed by the new ids (``:1
 ``reference_generate`` (``sampler``, ``eos_ids``, ``stop_ids``, ``on_token``;
 ``src/Inference/Inference.jl:2081-2102``), ``BatchRequest``/``run_batch``/``cancel``
 (``src/Runtime/Runtime.jl:33-51``, ``:98-182``), the pass size ``GESSO_PREFILL_CHUNK`` (default 1024,
-``Inference.jl:1765-1773``) and the timing line of ``GESSO_PROFILE=timing`` (``:2538-2544``).
+``Inference.jl:1765-1773``), the timing line of ``GESSO_PROFILE=timing`` (``:2538-2544``) and the stage table of
+``GESSO_PROFILE=decode`` (``src/Inference/decode_profile.jl``; also ``Engine.profile_decode``).
 Unlike the reference, one session serves many requests at once.
 """
 from __future__ import annotations
@@ -79,6 +80,8 @@ class Session:
         else:
             self.engine = Engine.from_config(cfg, random_weights_seed, dtype=dtype, device=device,
                                              std=random_weights_std, **kw)
+        if "decode" in _env_list("GESSO_PROFILE"):
+            self.engine.profile_decode(True)
         spec = self.engine.spec
         self.eos_ids = (int(eos_token_id),) if eos_token_id is not None else tuple(spec.eos_token_ids)
         self.last_stats = {}
@@ -185,6 +188,12 @@ class Session:
         st = dict(sched.stats)
         st.update(prefill_ms=(first - t0) * 1e3, decode_ms=(t1 - first) * 1e3,
                   new_tokens=sum(len(r.output) for r in requests), cache=self.engine.manager.stats())
+        profile = self.engine.rt.profile
+        if profile is not None:
+            st["decode_profile"] = profile.report()
+            for line in profile.lines():
+                print(line, flush=True)
+            self.engine.profile_decode(True)              # a fresh one for the next call
         self.last_stats = st
         if "timing" in _env_list("GESSO_PROFILE"):
             print(f"gesso_timing prefill_ms={st['prefill_ms']:.3f} decode_ms={st['decode_ms']:.3f} "

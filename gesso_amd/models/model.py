@@ -88,6 +88,25 @@ class Model:
         order = [self.blocks[call.layer] for call in self.spec.schedule]
         readers = [getattr(b, "first_norm", None) for b in order[1:]] + [self.final_norm if decode_only else None]
         scale = 1.0 if self.spec.embed_scale is None else float(self.spec.embed_scale)
+        with rt.stage("embed"):
+            stream = self._embed(ctx, order, scale)
+        for i, call in enumerate(self.spec.schedule):
+            stream.following = readers[i]
+            order[i].forward(stream, ctx, ctx.cache_view(i))
+        if ctx.n_want == 0:
+            return None
+        # every row wanted, in order (a decode step): no gather, and the norm may stay lazy
+        rows = None if decode_only else ctx.want_rows
+        with rt.stage("norm"):
+            normed = self.final_norm.add_norm(stream, rows=rows)
+        with rt.stage("lm_head"):
+            logits = self.rt.linear(normed, self.head, out_dtype=torch.float32)
+            if self.spec.logit_softcap is not None:
+                ops.softcap(logits, float(self.spec.logit_softcap))
+        return logits
+
+    def _embed(self, ctx, order, scale):
+        ops, rt = self.rt.ops, self.rt
         if rt.fused:
             ssq = torch.empty((ctx.T, 1), dtype=torch.float32, device=rt.device)
             first = getattr(order[0], "first_norm", None) if order else None
@@ -98,15 +117,5 @@ class Model:
             stream = ResidualStream(res, ssq=ssq, xs=xs, xs_for=first if xs is not None else None)
         else:
             stream = ResidualStream(ops.embed(ctx.token_ids, self.embed, scale=scale))
-        for i, call in enumerate(self.spec.schedule):
-            stream.following = readers[i]
-            order[i].forward(stream, ctx, ctx.cache_view(i))
-        if ctx.n_want == 0:
-            return None
-        # every row wanted, in order (a decode step): no gather, and the norm may stay lazy
-        rows = None if decode_only else ctx.want_rows
-        normed = self.final_norm.add_norm(stream, rows=rows)
-        logits = self.rt.linear(normed, self.head, out_dtype=torch.float32)
-        if self.spec.logit_softcap is not None:
-            ops.softcap(logits, float(self.spec.logit_softcap))
-        return logits
+        return stream
+

@@ -30,6 +30,7 @@ class RawQKV:
 
 class Attention(Part):
     graph_safe = True
+    stage, out_stage = "attn_mixer", "attn_outproj"   # the decode profiler's names
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
@@ -70,7 +71,8 @@ class Attention(Part):
 
     def forward(self, x, ctx, cache):
         q, q_stride = self.project_in(x, ctx, cache)
-        o = self.attend(q, q_stride, ctx, cache)
+        with self.rt.stage("attn_core"):
+            o = self.attend(q, q_stride, ctx, cache)
         return self.rt.project(o, self.wo, self.bo)
 
     # ------------------------------------------------------------------ the mixer's inner steps
@@ -83,15 +85,17 @@ class Attention(Part):
         nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
         eps = s.qk_norm.eps if s.qk_norm is not None else 1.0
         layout = getattr(pos, "layout", "half")
-        qkv = rt.linear(x, self.wqkv, self.bqkv)          # a lazy norm goes through as it is where the product takes it
+        with rt.stage("attn_proj"):
+            qkv = rt.linear(x, self.wqkv, self.bqkv)      # a lazy norm goes through as it is where the product takes it
         stride = (nh + 2 * nkv) * d
         if (rt.fused and ctx.all_single and cache.k.dtype == torch.bfloat16 and qkv.dtype == torch.bfloat16
                 and cache.page_size >= 2 and (self.q_norm is None) == (self.k_norm is None) and layout == "half"
                 and ops.attention_decode_raw_supports(nh, nkv, d, pos.rotary_dim)):
             return RawQKV(qkv, self.q_norm, self.k_norm, eps, pos), stride
-        ops.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, eps, pos.cos, pos.sin, pos.rotary_dim, ctx.positions,
-                           ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
-                           write_kv=cache.write, layout=layout)
+        with rt.stage("attn_headnorm_rope"):
+            ops.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, eps, pos.cos, pos.sin, pos.rotary_dim, ctx.positions,
+                               ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
+                               write_kv=cache.write, layout=layout)
         return qkv, stride
 
     def _single(self, q, q_stride, cache, ctx, nseq, out):

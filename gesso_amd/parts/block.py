@@ -51,12 +51,22 @@ class PreNormBlock(Part):
         return self.mixer_norm
 
     def forward(self, stream, ctx, cache):
-        after = stream.following
-        x = self.mixer_norm.add_norm(stream)
-        stream.push(self.mixer.forward(x, ctx, cache), self.rt, next_norm=self.ffn_norm if self.ffn is not None else after)
+        after, rt = stream.following, self.rt
+        with rt.stage("norm"):
+            x = self.mixer_norm.add_norm(stream)
+        # a stage per kind of mixer (the profiler's names: conv_mixer, attn_mixer, ...); a sub-layer's last product
+        # runs inside push, straight into the stream, and belongs to its stage
+        with rt.stage(getattr(self.mixer, "stage", "mixer")):
+            out = self.mixer.forward(x, ctx, cache)
+            with rt.stage(getattr(self.mixer, "out_stage", "mixer_out")):
+                stream.push(out, rt, next_norm=self.ffn_norm if self.ffn is not None else after)
         if self.ffn is not None:
-            x = self.ffn_norm.add_norm(stream)
-            stream.push(self.ffn.forward(x, ctx), self.rt, next_norm=after)
+            with rt.stage("norm"):
+                x = self.ffn_norm.add_norm(stream)
+            with rt.stage(getattr(self.ffn, "stage", "ffn")):
+                out = self.ffn.forward(x, ctx)
+                with rt.stage(getattr(self.ffn, "out_stage", "ffn_out")):
+                    stream.push(out, rt, next_norm=after)
 
     @property
     def graph_safe(self) -> bool:

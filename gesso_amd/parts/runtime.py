@@ -61,6 +61,17 @@ class RuntimeOptions:
             raise KernelError("row limits are nonnegative")
 
 
+class _NoStage:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_STAGE = _NoStage()
+
+
 class DeferredLinear:
     """A sub-layer's last product, not yet computed: ``x @ w.T`` to be added to the residual stream."""
 
@@ -91,6 +102,11 @@ class Runtime:
         self.weighted_rows_max = options.weighted_rows_max
         self.tiled_rows = dtype == torch.bfloat16 and options.tiled_rows
         self.many_rows = options.many_rows
+        self.profile = None            # a StageProfile while decode steps are profiled (engine/profile.py)
+
+    def stage(self, name: str):
+        """A context manager that brackets a named stage of the decode step when the profiler is on; else nothing."""
+        return _NO_STAGE if self.profile is None else self.profile.bracket(name)
 
     def shared(self, key, make):
         """One object per key for all parts (rotary tables and the like)."""

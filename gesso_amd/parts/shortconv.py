@@ -15,6 +15,7 @@ from .registry import register
 
 class ShortConv(Part):
     graph_safe = True
+    stage, out_stage = "conv_mixer", "conv_out"       # the decode profiler's names
 
     @staticmethod
     def tensor_specs(spec):
@@ -52,11 +53,14 @@ class ShortConv(Part):
         if rt.fused and self.b_in is None and ctx.all_single and self.taps.shape[1] <= 16:
             x = rt.lazy_rows(x)
             if rt.streams(x, self.w_in):
-                return ops.gemm_skinny_conv(x, self.w_in, self.taps, self.b_conv, state, ctx.slots,
-                                            wt=rt.tiles_of(self.w_in), tiled=rt.rows_tiled(self.taps.shape[0]))
-        bcx = rt.linear(rt.dense(x), self.w_in, self.b_in)
-        return ops.short_conv(bcx, self.taps, self.b_conv, state, ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq,
-                              ctx.all_single)
+                with rt.stage("conv_in"):          # product and convolution are one kernel here
+                    return ops.gemm_skinny_conv(x, self.w_in, self.taps, self.b_conv, state, ctx.slots,
+                                                wt=rt.tiles_of(self.w_in), tiled=rt.rows_tiled(self.taps.shape[0]))
+        with rt.stage("conv_in"):
+            bcx = rt.linear(rt.dense(x), self.w_in, self.b_in)
+        with rt.stage("conv_mix"):
+            return ops.short_conv(bcx, self.taps, self.b_conv, state, ctx.seq_of_token, ctx.q_start, ctx.slots,
+                                  ctx.nseq, ctx.all_single)
 
 
 register("mixer", "short_conv", ShortConv)

@@ -14,6 +14,7 @@ from .registry import register
 
 class SwiGLU(Part):
     graph_safe = True
+    stage, out_stage = "dense_ffn", "ffn_down"        # the decode profiler's names
 
     @staticmethod
     def tensor_specs(spec):
@@ -29,7 +30,8 @@ class SwiGLU(Part):
         self.w2 = self.rt.prepare(tensors["w2.weight"])
 
     def forward(self, x, ctx):
-        a = self.rt.linear_swiglu(x, self.w13)
+        with self.rt.stage("ffn_gateup"):                # with its activation where the kernel fuses them
+            a = self.rt.linear_swiglu(x, self.w13)
         return self.rt.project(a, self.w2)
 
 

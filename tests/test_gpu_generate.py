@@ -502,3 +502,28 @@ def test_a_full_run_before_a_new_recording_leaves_the_rings_alone(tmp_path):
     assert len(runner.graphs) == 2
     for name, big in guard.items():
         assert bool((big[0] == -7).all()) and bool((big[-1] == -7).all()), f"a step wrote beside {name}"
+
+
+def test_decode_stage_profiler(folders):
+    """Stages of a decode step, timed by HIP events: disjoint, named as the reference names them, summing to less than
+    the step; sub-stages beside them; the tokens are those of the unprofiled run; prompts are not counted."""
+    from gesso_amd import Session
+    d = write_tiny(folders, "B", torch.bfloat16)
+    s = Session(d, dtype="bfloat16", context_length=96)
+    prompts = [[3, 141, 59, 26, 500], [7, 8, 9]]
+    want = s.generate(prompts, max_new_tokens=10, eos_ids=())
+    prof = s.engine.profile_decode(True)
+    got = s.generate(prompts, max_new_tokens=10, eos_ids=())
+    assert got == want
+    r = s.last_stats["decode_profile"]
+    # the first token of each request comes from its prompt's step; the other nine from decode steps
+    assert r["steps"] == 9 and r["step_ms"] > 0
+    assert set(r["stages_ms"]) == {"embed", "conv_mixer", "attn_mixer", "norm", "dense_ffn", "lm_head", "sample"} - \
+        ({"norm"} if r["stages_ms"].get("norm") is None else set())
+    assert sum(r["stages_ms"].values()) <= r["step_ms"] * 1.001 and r["other_ms"] >= 0
+    calls = r["calls_per_step"]
+    assert calls["conv_mixer"] == 3 and calls["attn_mixer"] == 3 and calls["dense_ffn"] == 6 and calls["lm_head"] == 1
+    assert {"conv_in", "conv_out", "attn_proj", "attn_core", "attn_outproj", "ffn_gateup", "ffn_down"} <= set(r["substages_ms"])
+    assert r["substages_ms"]["ffn_gateup"] + r["substages_ms"]["ffn_down"] <= r["stages_ms"]["dense_ffn"] * 1.001
+    s.engine.profile_decode(False)
+    assert s.generate(prompts, max_new_tokens=10, eos_ids=()) == want and "decode_profile" not in s.last_stats
