@@ -239,6 +239,32 @@ def gemm_workload(reps: int = 10) -> dict:
     return out
 
 
+def stages_workload(batch: int = 8, steps: int = 32) -> dict:
+    """The decode step of LFM2-1.2B sizes stage by stage (the decode stage profiler: HIP events around each stage of
+    an eagerly launched step; the recorded step itself is faster by what the launches cost)."""
+    from gesso_amd import Engine, StepEntry
+    cfg = model_config()
+    engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=16, max_context=4096,
+                                max_tokens=batch * 1024, num_slots=batch + 1)
+    g = torch.Generator().manual_seed(2)
+    rids, first = [("st", i) for i in range(batch)], []
+    for rid in rids:
+        engine.add_request(rid)
+        ids = torch.randint(0, cfg.vocab_size, (512,), generator=g).tolist()
+        first.append(int(engine.step([StepEntry(rid, ids, [511])]).argmax(1)[0]))
+    ids, _ = engine.decode(rids, first, 8)                      # records the graph, warms everything
+    prof = engine.profile_decode(True)
+    engine.decode(rids, ids[-1].tolist(), 4)                    # eager warm-up of the profiled path
+    prof = engine.profile_decode(True)
+    engine.decode(rids, ids[-1].tolist(), steps)
+    r = prof.report()
+    out = {"metric": "decode step of LFM2-1.2B sizes by stage, milliseconds a step (eager launches)", "batch": batch,
+           "steps": r["steps"], "step_ms": round(r["step_ms"], 4), "other_ms": round(r["other_ms"], 4)}
+    out.update({f"stage_{k}": round(v, 4) for k, v in r["stages_ms"].items()})
+    out.update({f"sub_{k}": round(v, 4) for k, v in r["substages_ms"].items()})
+    return out
+
+
 def long_workload(seed: int = 6) -> dict:
     """LFM2-2.6B sizes: prompts of 32,768 tokens in portions of 2,048, then 256 decode steps of 8 such requests."""
     from gesso_amd import Engine, StepEntry
@@ -292,14 +318,18 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="measure the 2,048-token prefill alone (for profiling)")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the measurement of what the machine delivers")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
-                         "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's")
+                         "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
+                         "stages: the decode step stage by stage")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
         return 2
     if args.workload != "decode":
+        if args.workload == "stages":
+            print(json.dumps(stages_workload(args.batch, min(args.steps, 32))))
+            return 0
         run = {"serve": serve_workload, "long": long_workload, "gemm": gemm_workload}[args.workload]
         print(json.dumps(run()))
         return 0
