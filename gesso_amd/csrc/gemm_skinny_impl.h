@@ -284,24 +284,66 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   constexpr int UQ = (WAVES >= 16 ? 12 : 24) / (R + MT);   // sixteen wavefronts leave a lane 128 registers
   constexpr int U = UQ >= 8 ? 8 : (UQ >= 4 ? 4 : (UQ >= 2 ? 2 : 1));
   constexpr int WSTEP = SHUF ? 512 : 32;  // elements between a row tile's consecutive k steps
-  if ((K & 31) == 0 || SHUF) {
-    for (; s + U <= s1; s += U) {
-      bf16x8_t a[U][R], b[U][MT];
+  if (MT < 3) {
+    // few rows: the steps' loads are issued U at a time, then multiplied (the ring below costs registers, and with
+    // them a resident wavefront per SIMD, which these shapes need more)
+    if ((K & 31) == 0 || SHUF) {
+      for (; s + U <= s1; s += U) {
+        bf16x8_t a[U][R], b[U][MT];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int r = 0; r < R; ++r) a[u][r] = wact ? load8(wrow[r] + (size_t)(s + u) * WSTEP) : zero8();
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) b[u][mt] = xok[mt] ? load_x(mt, s + u) : zero8();
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r], b[u][mt], acc[r][mt], 0, 0, 0);
+      }
+    }
+  } else if (((K & 31) == 0 || SHUF) && s1 - s0 >= U) {
+    // many rows: a ring of U steps in registers: a step is multiplied as soon as it has arrived and its place is
+    // asked for again at once, U steps ahead, so that loads are in flight the whole time (loads return in order;
+    // 19.6 against 20.4 us for gate|up at 64 rows).
+    bf16x8_t a[U][R], b[U][MT];
+    auto fetch = [&](int u, int step) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        // every lane loads (its address is a valid one): a load under a lane mask would hide from the
+        // compiler how many loads are in flight, and it would wait for all of them
+        const bf16x8_t v = load8(wrow[r] + (size_t)step * WSTEP);
+        a[u][r] = (SHUF != 2 || wact) ? v : zero8();
+      }
+      // rows past M read row 0 or the padding of the last tile; their columns of the result are never stored
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b[u][mt] = load_x(mt, step);
+    };
+    auto multiply = [&](int u) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r], b[u][mt], acc[r][mt], 0, 0, 0);
+    };
+#pragma unroll
+    for (int u = 0; u < U; ++u) fetch(u, s0 + u);
+    const int groups = (s1 - s0) / U;
+    for (int g = 1; g < groups; ++g) {
+      const int base = s0 + g * U;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) a[u][r] = wact ? load8(wrow[r] + (size_t)(s + u) * WSTEP) : zero8();
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) b[u][mt] = xok[mt] ? load_x(mt, s + u) : zero8();
+        multiply(u);
+        fetch(u, base + u);
       }
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r], b[u][mt], acc[r][mt], 0, 0, 0);
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u) multiply(u);
+    s = s0 + groups * U;
   }
   for (; s < s1; ++s) {
     const int k = (s << 5) + kg * 8;
