@@ -429,13 +429,16 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
 
 #define DEC_WAVES 8
 
-template <int D, int RAW>
-static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, bf16* kc, bf16* vc,
+// Wavefronts a block: eight, so that one block covers about a thousand keys in a pass or two; four where the grid
+// alone holds two blocks and more for every compute unit (many sequences): blocks of four leave a lane's registers
+// to two blocks a compute unit, whose chains of round trips then overlap.
+template <int D, int RAW, int WV>
+static int launch_decode_w(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, bf16* kc, bf16* vc,
                          const int* positions, const int* bt, int max_blocks, int page_size, unsigned page_magic,
                          int window, float scale, bf16* out, float* part_o, float* part_ml, int nh, int nkv,
                          int out_tiles, DecodeRaw raw) {
 #define GS_RUN(GG)                                                                                                     \
-  attention_decode_kernel<D, GG, DEC_WAVES, RAW><<<grid, DEC_WAVES * 64, 0, stream>>>(                                 \
+  attention_decode_kernel<D, GG, WV, RAW><<<grid, WV * 64, 0, stream>>>(                                 \
       q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_magic, window, scale, out, part_o, part_ml, nh, \
       nkv, out_tiles, raw)
   switch (G) {
@@ -451,6 +454,27 @@ static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, in
   }
 #undef GS_RUN
   return 0;
+}
+
+static int g_decode_cus = 0;   // compute units of the device, asked for once
+
+template <int D, int RAW>
+static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, bf16* kc, bf16* vc,
+                         const int* positions, const int* bt, int max_blocks, int page_size, unsigned page_magic,
+                         int window, float scale, bf16* out, float* part_o, float* part_ml, int nh, int nkv,
+                         int out_tiles, DecodeRaw raw) {
+  if (g_decode_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    g_decode_cus = n;
+  }
+  const long blocks = (long)grid.x * grid.y * grid.z;
+  if (D <= 64 && blocks >= 2L * g_decode_cus)
+    return launch_decode_w<D, RAW, 4>(G, grid, stream, q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_magic,
+                                      window, scale, out, part_o, part_ml, nh, nkv, out_tiles, raw);
+  return launch_decode_w<D, RAW, DEC_WAVES>(G, grid, stream, q, q_stride, kc, vc, positions, bt, max_blocks, page_size,
+                                            page_magic, window, scale, out, part_o, part_ml, nh, nkv, out_tiles, raw);
 }
 
 // Whether this kernel takes the sizes: head widths 16, 32, 64, 128 and groups of up to 8 heads.

@@ -141,9 +141,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
     if (n >= N) n = N - 1;                                // clamped: loaded, never stored
     if (SHUF == 2)
       wrow[r] = W + ((size_t)(rowbase[r] >> 4) * ((K + 31) >> 5)) * 512 + (kg * 16 + (rowbase[r] & 8) + (r16 & 7)) * 8;
-    else if (SHUF)
+    else if (SHUF) {
       // tile-major: the 16 x 32 tile of (row tile, k step) is 64 lanes x 16 bytes in the operand's own order
-      wrow[r] = W + ((size_t)(rowbase[r] >> 4) * ((K + 31) >> 5)) * 512 + lane * 8;
+      // (a tile past the weight's last, where a block's tiles outnumber what is left, reads the last: loaded, never stored)
+      const int tile = (rowbase[r] >> 4) < ((N + 15) >> 4) ? (rowbase[r] >> 4) : ((N + 15) >> 4) - 1;
+      wrow[r] = W + ((size_t)tile * ((K + 31) >> 5)) * 512 + lane * 8;
+    }
     else
       wrow[r] = W + (size_t)n * K + kg * 8;
   }

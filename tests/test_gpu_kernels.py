@@ -652,7 +652,7 @@ def test_gemm_skinny_residual_leaves_rows_weighted_for_the_next_norm(ops, M, N, 
 
 
 @pytest.mark.parametrize("M,N,K,parts", [(64, 2048, 8192, 8), (40, 96, 320, 3), (33, 144, 104, 1), (17, 2048, 2048, 16),
-                                          (5, 100, 64, 4)])
+                                          (5, 100, 64, 4), (33, 144, 128, 2)])   # the last: an odd number of weight tiles, tile-major
 def test_gemm_skinny_residual_in_parts(ops, M, N, K, parts):
     g = gen(M + N + K + parts)
     x = torch.randn(M, K, generator=g).bfloat16()
