@@ -531,12 +531,15 @@ def test_attention_decode(ops, nh, nkv, d, ps, nsplit, window):
     close(got, same.double().cpu(), torch.bfloat16)
 
 
-@pytest.mark.parametrize("nh,nkv,d,norm,nsplit,write", [(32, 8, 64, True, 1, True), (2, 1, 64, False, 3, True),
-                                                        (8, 1, 128, True, 2, True), (5, 5, 64, True, 1, False)])
-def test_attention_decode_from_raw_rows_equals_the_separate_kernels(ops, nh, nkv, d, norm, nsplit, write):
-    """Head norms, rotation and cache write inside the attention kernel against the kernel that does them alone."""
+@pytest.mark.parametrize("nh,nkv,d,norm,nsplit,write,copies", [(32, 8, 64, True, 1, True, 1), (2, 1, 64, False, 3, True, 1),
+                                                               (8, 1, 128, True, 2, True, 1), (5, 5, 64, True, 1, False, 1),
+                                                               (32, 8, 64, True, 1, True, 12), (4, 2, 64, True, 2, True, 24)])
+def test_attention_decode_from_raw_rows_equals_the_separate_kernels(ops, nh, nkv, d, norm, nsplit, write, copies):
+    """Head norms, rotation and cache write inside the attention kernel against the kernel that does them alone.
+    With many sequences (`copies` of the six lengths) the grid holds two blocks and more a compute unit, and the
+    kernel runs in blocks of four wavefronts."""
     g = gen(nh * 7 + d + nsplit)
-    ps, lens = 16, [1, 64, 65, 300, 17, 129]
+    ps, lens = 16, [1, 64, 65, 300, 17, 129] * copies
     nseq = len(lens)
     nblk = [-(-n // ps) for n in lens]
     total = sum(nblk)
