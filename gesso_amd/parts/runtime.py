@@ -32,6 +32,12 @@ class RuntimeOptions:
     vendor's for bfloat16 results (measured on random data at 2,048 rows: 109 us against our 161 for gate|up, 124
     against 162 with the SwiGLU pass counted in; 50 against 75 for 6144 x 2048), ours where the result is float32 and
     inside a recorded graph.
+    ``tune_library``: where the vendor library computes a product of many rows, let it measure its own candidate
+    kernels the first time a shape with a whole number of 256 rows comes (a prompt portion of the usual sizes) and
+    keep the fastest (``torch.cuda.tunable``; at 2,048 rows of LFM2-1.2B's layers 43.9 against 49.9 us for 6144 x 2048,
+    65.5 against 76.0 for 2048 x 8192, 100 against 108 for 16384 x 2048).  A shape costs about a second once; the
+    choices are kept in a file in the user's temporary folder for later runs.  The switch is the process's, not this
+    runtime's: ``torch``'s own products in the same process are tuned by the same rule.
     ``prompt_attention``: attention of prompt portions in bfloat16: ``"wide"`` = the kernel for long portions wherever it
     takes the sizes (heads of 64), ``"tiles"`` = the kernel with tiles of 16 or 32 queries always, ``"auto"`` = the
     first for steps with a portion of at least 64 tokens, else the second.
@@ -46,6 +52,7 @@ class RuntimeOptions:
     """
 
     many_rows: str = "auto"
+    tune_library: bool = True
     prompt_attention: str = "auto"
     tiled_rows: bool = True
     tile_weights: bool = True
@@ -59,6 +66,29 @@ class RuntimeOptions:
             raise KernelError(f"prompt_attention is 'auto', 'wide' or 'tiles', not {self.prompt_attention!r}")
         if self.fold_norm_rows < 0 or self.weighted_rows_max < 0:
             raise KernelError("row limits are nonnegative")
+
+
+_TUNED_SHAPES = None
+
+
+def _enable_library_tuning():
+    """Switch the vendor library's tunable products on for this process (results are used, nothing is tuned until a
+    product asks for it) and return the set of shapes already asked for, shared by every runtime of the process."""
+    global _TUNED_SHAPES
+    if _TUNED_SHAPES is None:
+        import os
+        import tempfile
+        from torch.cuda import tunable
+        folder = os.path.join(tempfile.gettempdir(), f"gesso_amd_{os.getuid()}")
+        try:
+            os.makedirs(folder, exist_ok=True)
+            tunable.set_filename(os.path.join(folder, "library_products.csv"), insert_device_ordinal=True)
+        except OSError:
+            pass                          # no folder to keep the choices in: they are measured again next time
+        tunable.enable(True)
+        tunable.tuning_enable(False)
+        _TUNED_SHAPES = set()
+    return _TUNED_SHAPES
 
 
 class _NoStage:
@@ -102,6 +132,9 @@ class Runtime:
         self.weighted_rows_max = options.weighted_rows_max
         self.tiled_rows = dtype == torch.bfloat16 and options.tiled_rows
         self.many_rows = options.many_rows
+        self._tuned = None             # shapes the vendor library has been asked to tune, or None: no tuning
+        if options.tune_library and dtype == torch.bfloat16 and options.many_rows != "own":
+            self._tuned = _enable_library_tuning()
         self.profile = None            # a StageProfile while decode steps are profiled (engine/profile.py)
 
     def stage(self, name: str):
@@ -164,10 +197,27 @@ class Runtime:
                 return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self.tiles_of(w))
             library = out_dtype == torch.bfloat16 and not self.no_library and self.many_rows != "own"
             if library:
-                return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
+                return self._library_product(x, w, out)
             if self.many_rows != "library" and ops.mfma_ok(x, w) and (out is None or out.is_contiguous()):
                 return ops.gemm_mfma(x, w, out_dtype=out_dtype, out=out)
         return ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
+
+    TUNED_ROWS, TUNED_SHAPES = 256, 64    # shapes with whole multiples of so many rows are tuned, up to so many shapes
+
+    def _library_product(self, x, w, out):
+        """``x @ w.T`` by the vendor library; the first product of a shape worth it is also the library's tuning run."""
+        tuned = self._tuned
+        if tuned is not None:
+            key = (x.shape[0], w.shape[0], w.shape[1])
+            if key not in tuned and x.shape[0] % self.TUNED_ROWS == 0 and len(tuned) < self.TUNED_SHAPES:
+                tuned.add(key)
+                from torch.cuda import tunable
+                tunable.tuning_enable(True)
+                try:
+                    return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
+                finally:
+                    tunable.tuning_enable(False)
+        return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
 
     def linear_swiglu(self, x, w13: torch.Tensor) -> torch.Tensor:
         """``silu(x @ w1.T) * (x @ w3.T)`` with ``w13`` holding w1's rows, then w3's."""

@@ -109,6 +109,28 @@ def test_rope_part_tables(fw):
         build("position", RopeSpec(head_dim=16, rotary_dim=18, theta=1e4, max_position=8), rt)
 
 
+def test_library_products_of_many_rows_are_tuned_once_per_shape_and_stay_right(fw):
+    """A product of a whole number of 256 rows is the vendor library's tuning run the first time its shape comes; what
+    it computes equals the plain product, before and after, and with tuning switched off."""
+    from gesso_amd.parts import Runtime, RuntimeOptions
+    g = gen(11)
+    x = torch.randn(512, 384, generator=g).bfloat16()
+    w = (torch.randn(320, 384, generator=g) / math.sqrt(384)).bfloat16()
+    want = x.double() @ w.double().T
+    rt = Runtime(DEV, torch.bfloat16)
+    assert rt._tuned is not None
+    for _ in range(2):
+        got = rt.linear(x.to(DEV), w.to(DEV)).double().cpu()
+        assert float((got - want).abs().max()) <= tol(torch.bfloat16, want)
+        assert (512, 320, 384) in rt._tuned
+    y = rt.linear(x[:300].to(DEV), w.to(DEV)).double().cpu()          # 300 rows: not a shape that is tuned
+    assert (300, 320, 384) not in rt._tuned and float((y - want[:300]).abs().max()) <= tol(torch.bfloat16, want)
+    plain = Runtime(DEV, torch.bfloat16, RuntimeOptions(tune_library=False))
+    assert plain._tuned is None
+    got = plain.linear(x.to(DEV), w.to(DEV)).double().cpu()
+    assert float((got - want).abs().max()) <= tol(torch.bfloat16, want)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_part(fw, dtype):
     from gesso_amd.config import SwiGLUSpec
