@@ -33,11 +33,12 @@ class RuntimeOptions:
     against 162 with the SwiGLU pass counted in; 50 against 75 for 6144 x 2048), ours where the result is float32 and
     inside a recorded graph.
     ``tune_library``: where the vendor library computes a product of many rows, let it measure its own candidate
-    kernels the first time a shape with a whole number of 256 rows comes (a prompt portion of the usual sizes) and
+    kernels the first time a shape of 512, 1024, 2048, ... rows comes (a whole prompt portion of the usual sizes) and
     keep the fastest (``torch.cuda.tunable``; at 2,048 rows of LFM2-1.2B's layers 43.9 against 49.9 us for 6144 x 2048,
-    65.5 against 76.0 for 2048 x 8192, 100 against 108 for 16384 x 2048).  A shape costs about a second once; the
-    choices are kept in a file in the user's temporary folder for later runs.  The switch is the process's, not this
-    runtime's: ``torch``'s own products in the same process are tuned by the same rule.
+    65.5 against 76.0 for 2048 x 8192, 100 against 108 for 16384 x 2048).  A shape costs about a second once (two at
+    8,192 rows); the choices are kept in a file in the user's temporary folder for later runs.  Other row counts take
+    the library's own first choice, so that a server's steps of ever new sizes do not stall.  The switch is the
+    process's, not this runtime's: ``torch``'s own products in the same process use what was tuned.
     ``prompt_attention``: attention of prompt portions in bfloat16: ``"wide"`` = the kernel for long portions wherever it
     takes the sizes (heads of 64), ``"tiles"`` = the kernel with tiles of 16 or 32 queries always, ``"auto"`` = the
     first for steps with a portion of at least 64 tokens, else the second.
@@ -86,7 +87,8 @@ def _enable_library_tuning():
         except OSError:
             pass                          # no folder to keep the choices in: they are measured again next time
         tunable.enable(True)
-        tunable.tuning_enable(False)
+        tunable.tuning_enable(False)    # (with less time for each candidate than the library's default the choices got no better than untuned)
+
         _TUNED_SHAPES = set()
     return _TUNED_SHAPES
 
@@ -202,14 +204,15 @@ class Runtime:
                 return ops.gemm_mfma(x, w, out_dtype=out_dtype, out=out)
         return ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
 
-    TUNED_ROWS, TUNED_SHAPES = 256, 64    # shapes with whole multiples of so many rows are tuned, up to so many shapes
+    TUNED_ROWS, TUNED_SHAPES = 512, 64    # shapes of a power of two of rows from so many on are tuned, up to so many shapes
 
     def _library_product(self, x, w, out):
         """``x @ w.T`` by the vendor library; the first product of a shape worth it is also the library's tuning run."""
         tuned = self._tuned
         if tuned is not None:
             key = (x.shape[0], w.shape[0], w.shape[1])
-            if key not in tuned and x.shape[0] % self.TUNED_ROWS == 0 and len(tuned) < self.TUNED_SHAPES:
+            M = x.shape[0]
+            if key not in tuned and M >= self.TUNED_ROWS and M & (M - 1) == 0 and len(tuned) < self.TUNED_SHAPES:
                 tuned.add(key)
                 from torch.cuda import tunable
                 tunable.tuning_enable(True)
