@@ -29,6 +29,9 @@ LIB_NAME = "libgesso_hip.so"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
+# the vendor's matrix product library (products of many rows, library_gemm.hip)
+LINK = ["-lhipblaslt"]
+
 _lock = threading.Lock()
 _lib = None
 
@@ -39,7 +42,7 @@ def sources():
 
 def _digest() -> str:
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + LINK).encode())
     for name in sorted(os.listdir(CSRC)):
         if name.endswith((".hip", ".h")):
             h.update(name.encode())
@@ -113,7 +116,7 @@ def build(force: bool = True, verbose: bool = True) -> str:
     with ThreadPoolExecutor(workers) as pool:
         objs = list(pool.map(compile_one, srcs))
     tmp = lib + f".tmp{os.getpid()}"
-    p = subprocess.run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs,
+    p = subprocess.run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs + LINK,
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
     if p.returncode != 0:
         raise KernelError(f"linking the HIP extension failed:\n{p.stdout[-4000:]}")

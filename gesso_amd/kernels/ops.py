@@ -373,6 +373,41 @@ def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, out: torch.Tenso
     return out
 
 
+def library_gemm(x: torch.Tensor, w: torch.Tensor, workspace: torch.Tensor, out: torch.Tensor = None, tune: bool = True):
+    """``x @ w.T`` for many rows by the vendor's library, called directly (bfloat16 in and out, float32 sums).  The
+    first call of a shape makes its plan, with ``tune`` by measuring the library's two dozen best guesses on these
+    operands (a few milliseconds), else by taking its first choice.
+    ``workspace``: device bytes the library's kernels may use.  Not to be recorded into a graph."""
+    _dev(w, workspace, out if out is not None and out.is_contiguous() else None)
+    _need(x.is_cuda and x.dim() == 2 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.stride(1) == 1,
+          "library_gemm: bfloat16 (M, K) rows and a bfloat16 weight")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(w.shape == (N, K), f"library_gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _need(out.shape == (M, N) and out.dtype == torch.bfloat16 and out.stride(1) == 1, "library_gemm: out is bfloat16 (M, N)")
+    _check(lib().gs_library_gemm(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(out),
+                                 c_int(out.stride(0) if M > 1 else N), c_int(M), c_int(N), c_int(K), _p(workspace),
+                                 c_long(workspace.numel() * workspace.element_size()), c_int(1 if tune else 0), _stream()))
+    return out
+
+
+def library_gemm_ok(x, w: torch.Tensor) -> bool:
+    """Whether :func:`library_gemm` takes these operands (bfloat16, K and the row stride multiples of 8, aligned)."""
+    return (isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
+            and x.shape[0] > 0 and x.shape[1] % 8 == 0 and x.stride(1) == 1
+            and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0 and w.is_contiguous()
+            and w.data_ptr() % 16 == 0 and w.shape[0] % 8 == 0)
+
+
+def library_gemm_plan(M: int, N: int, K: int):
+    """``(plans kept in all, candidates measured for this shape, the best one's microseconds)``."""
+    cand, best = c_int(0), c_float(0.0)
+    n = lib().gs_library_gemm_plans(c_int(M), c_int(N), c_int(K), ctypes.byref(cand), ctypes.byref(best))
+    return n, cand.value, best.value
+
+
 # ---------------------------------------------------------------------- sampling
 
 def argmax_rows(logits: torch.Tensor):

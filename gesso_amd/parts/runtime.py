@@ -32,13 +32,9 @@ class RuntimeOptions:
     vendor's for bfloat16 results (measured on random data at 2,048 rows: 109 us against our 161 for gate|up, 124
     against 162 with the SwiGLU pass counted in; 50 against 75 for 6144 x 2048), ours where the result is float32 and
     inside a recorded graph.
-    ``tune_library``: where the vendor library computes a product of many rows, let it measure its own candidate
-    kernels the first time a shape of 512, 1024, 2048, ... rows comes (a whole prompt portion of the usual sizes) and
-    keep the fastest (``torch.cuda.tunable``; at 2,048 rows of LFM2-1.2B's layers 43.9 against 49.9 us for 6144 x 2048,
-    65.5 against 76.0 for 2048 x 8192, 100 against 108 for 16384 x 2048).  A shape costs about a second once (two at
-    8,192 rows); the choices are kept in a file in the user's temporary folder for later runs.  Other row counts take
-    the library's own first choice, so that a server's steps of ever new sizes do not stall.  The switch is the
-    process's, not this runtime's: ``torch``'s own products in the same process use what was tuned.
+    ``tune_library``: where the vendor library computes a product of many rows, the first product of a shape measures
+    the library's two dozen best guesses on the operands at hand, cold, and keeps the library's first choice unless
+    another is clearly faster (a few tens of milliseconds a shape).  Off: the library's first choice.
     ``prompt_attention``: attention of prompt portions in bfloat16: ``"wide"`` = the kernel for long portions wherever it
     takes the sizes (heads of 64), ``"tiles"`` = the kernel with tiles of 16 or 32 queries always, ``"auto"`` = the
     first for steps with a portion of at least 64 tokens, else the second.
@@ -67,30 +63,6 @@ class RuntimeOptions:
             raise KernelError(f"prompt_attention is 'auto', 'wide' or 'tiles', not {self.prompt_attention!r}")
         if self.fold_norm_rows < 0 or self.weighted_rows_max < 0:
             raise KernelError("row limits are nonnegative")
-
-
-_TUNED_SHAPES = None
-
-
-def _enable_library_tuning():
-    """Switch the vendor library's tunable products on for this process (results are used, nothing is tuned until a
-    product asks for it) and return the set of shapes already asked for, shared by every runtime of the process."""
-    global _TUNED_SHAPES
-    if _TUNED_SHAPES is None:
-        import os
-        import tempfile
-        from torch.cuda import tunable
-        folder = os.path.join(tempfile.gettempdir(), f"gesso_amd_{os.getuid()}")
-        try:
-            os.makedirs(folder, exist_ok=True)
-            tunable.set_filename(os.path.join(folder, "library_products.csv"), insert_device_ordinal=True)
-        except OSError:
-            pass                          # no folder to keep the choices in: they are measured again next time
-        tunable.enable(True)
-        tunable.tuning_enable(False)    # (with less time for each candidate than the library's default the choices got no better than untuned)
-
-        _TUNED_SHAPES = set()
-    return _TUNED_SHAPES
 
 
 class _NoStage:
@@ -134,9 +106,8 @@ class Runtime:
         self.weighted_rows_max = options.weighted_rows_max
         self.tiled_rows = dtype == torch.bfloat16 and options.tiled_rows
         self.many_rows = options.many_rows
-        self._tuned = None             # shapes the vendor library has been asked to tune, or None: no tuning
-        if options.tune_library and dtype == torch.bfloat16 and options.many_rows != "own":
-            self._tuned = _enable_library_tuning()
+        self.tune_library = options.tune_library
+        self._library_ws = None        # device bytes for the vendor library's kernels, made at the first such product
         self.profile = None            # a StageProfile while decode steps are profiled (engine/profile.py)
 
     def stage(self, name: str):
@@ -204,22 +175,18 @@ class Runtime:
                 return ops.gemm_mfma(x, w, out_dtype=out_dtype, out=out)
         return ops.gemm_tiled(x, w, bias, out_dtype=out_dtype, out=out)
 
-    TUNED_ROWS, TUNED_SHAPES = 512, 64    # shapes of a power of two of rows from so many on are tuned, up to so many shapes
+    LIBRARY_WORKSPACE = 64 << 20
 
     def _library_product(self, x, w, out):
-        """``x @ w.T`` by the vendor library; the first product of a shape worth it is also the library's tuning run."""
-        tuned = self._tuned
-        if tuned is not None:
-            key = (x.shape[0], w.shape[0], w.shape[1])
-            M = x.shape[0]
-            if key not in tuned and M >= self.TUNED_ROWS and M & (M - 1) == 0 and len(tuned) < self.TUNED_SHAPES:
-                tuned.add(key)
-                from torch.cuda import tunable
-                tunable.tuning_enable(True)
-                try:
-                    return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
-                finally:
-                    tunable.tuning_enable(False)
+        """``x @ w.T`` by the vendor library: called directly where it takes the operands (``ops.library_gemm``: a plan
+        per shape, a few microseconds of host time a call), else through ``torch.mm``."""
+        ops = self.ops
+        if ops.library_gemm_ok(x, w) and (out is None or (out.dtype == torch.bfloat16 and out.stride(1) == 1
+                                                          and out.data_ptr() % 16 == 0
+                                                          and (out.shape[0] <= 1 or out.stride(0) % 8 == 0))):
+            if self._library_ws is None:
+                self._library_ws = torch.empty(self.LIBRARY_WORKSPACE, dtype=torch.uint8, device=self.device)
+            return ops.library_gemm(x, w, self._library_ws, out=out, tune=self.tune_library)
         return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
 
     def linear_swiglu(self, x, w13: torch.Tensor) -> torch.Tensor:

@@ -109,26 +109,34 @@ def test_rope_part_tables(fw):
         build("position", RopeSpec(head_dim=16, rotary_dim=18, theta=1e4, max_position=8), rt)
 
 
-def test_library_products_of_many_rows_are_tuned_once_per_shape_and_stay_right(fw):
-    """A product of 512, 1024, ... rows is the vendor library's tuning run the first time its shape comes; what
-    it computes equals the plain product, before and after, and with tuning switched off."""
+def test_library_products_of_many_rows_are_planned_once_per_shape_and_stay_right(fw):
+    """A product of many rows goes to the vendor library directly; the first product of a shape measures the library's
+    candidates (with tuning on) and keeps a plan; what it computes equals the plain product before and after."""
+    from gesso_amd.kernels import ops
     from gesso_amd.parts import Runtime, RuntimeOptions
     g = gen(11)
-    x = torch.randn(512, 384, generator=g).bfloat16()
+    x = torch.randn(520, 384, generator=g).bfloat16()
     w = (torch.randn(320, 384, generator=g) / math.sqrt(384)).bfloat16()
     want = x.double() @ w.double().T
     rt = Runtime(DEV, torch.bfloat16)
-    assert rt._tuned is not None
-    for _ in range(2):
+    before = ops.library_gemm_plan(520, 320, 384)[0]
+    for _ in range(3):
         got = rt.linear(x.to(DEV), w.to(DEV)).double().cpu()
         assert float((got - want).abs().max()) <= tol(torch.bfloat16, want)
-        assert (512, 320, 384) in rt._tuned
-    y = rt.linear(x[:384].to(DEV), w.to(DEV)).double().cpu()          # 384 rows: not a shape that is tuned
-    assert (384, 320, 384) not in rt._tuned and float((y - want[:384]).abs().max()) <= tol(torch.bfloat16, want)
+    plans, candidates, best_us = ops.library_gemm_plan(520, 320, 384)
+    assert plans == before + 1 and candidates >= 1 and best_us > 0
+    # rows of another stride (a slice of a wider buffer), an output given, and tuning off
+    wide = torch.randn(200, 768, generator=g).bfloat16().to(DEV)
+    out = torch.full((200, 320), float("nan"), dtype=torch.bfloat16, device=DEV)
     plain = Runtime(DEV, torch.bfloat16, RuntimeOptions(tune_library=False))
-    assert plain._tuned is None
-    got = plain.linear(x.to(DEV), w.to(DEV)).double().cpu()
-    assert float((got - want).abs().max()) <= tol(torch.bfloat16, want)
+    got = plain.linear(wide[:, :384], w.to(DEV), out=out)
+    assert got is out
+    ref = wide[:, :384].double().cpu() @ w.double().T
+    assert float((out.double().cpu() - ref).abs().max()) <= tol(torch.bfloat16, ref)
+    # a width the direct call does not take (no multiple of 8) still goes to the library, through torch
+    w5 = (torch.randn(77, 384, generator=g) / math.sqrt(384)).bfloat16()
+    y = rt.linear(x.to(DEV), w5.to(DEV)).double().cpu()
+    assert float((y - x.double() @ w5.double().T).abs().max()) <= tol(torch.bfloat16, want)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
