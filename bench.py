@@ -318,6 +318,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="measure the 2,048-token prefill alone (for profiling)")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the measurement of what the machine delivers")
+    ap.add_argument("--no-tune", action="store_true", help="the vendor library's first choice for every product of many "
+                    "rows (for profiles: no tuning runs among the kernels)")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
@@ -344,9 +346,10 @@ def main() -> int:
     prompt_len, context = 512, 4096
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     max_batch = max(args.batch, 1 if args.no_points else 64)
+    from gesso_amd.parts import RuntimeOptions
     engine = Engine.from_config(cfg, seed=0, dtype=dtype, page_size=16, max_context=context,
                                 max_tokens=max_batch * (prompt_len + args.steps + args.warmup + 32) + 4096,
-                                num_slots=max_batch + 1)
+                                num_slots=max_batch + 1, options=RuntimeOptions(tune_library=not args.no_tune))
     wbytes = weight_bytes(engine)
     if args.only_prefill:
         sec = prefill_run(engine, cfg, 2048)
