@@ -54,6 +54,8 @@ void gs_skinny_run_conv(const void* X, int ldx, int x_tiled, const float* res, c
   c.ex.y_tiled = y_tiled;
   if (res || ssq) lazy(c, res, ssq, nb, norm_w, eps);
   c.ex.taps = taps; c.ex.conv_bias = conv_bias; c.ex.state = state; c.ex.slots = slots; c.ex.conv_w = conv_w;
+  c.ex.conv_vec = conv_w >= 2 && conv_w <= 4 && H % 4 == 0 && H >= 4 &&
+                  (((uintptr_t)taps | (uintptr_t)conv_bias | (uintptr_t)state) & 15) == 0;
   // c.N / 3 channels, as few as a narrow weight's rows; with many rows of X the blocks' reading of X outweighs that
   if (Wt && gs_skinny_halves(c.N / 3) && M <= 32) gs_skinny_conv_half_tiles(c);
   else Wt ? gs_skinny_conv_tiles(c) : gs_skinny_conv_rows(c);

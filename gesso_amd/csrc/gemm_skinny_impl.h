@@ -45,6 +45,7 @@
 //      y = taps . (history, u) + bias, out = C y, history shifted; one token per sequence.
 #pragma once
 #include "common.h"
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
@@ -99,6 +100,8 @@ struct SkinnyExtra {
   float* state;          // (slots, H, W - 1)
   const int* slots;      // (M)
   int conv_w;
+  int conv_vec;          // widths 2..4, H a multiple of 4, taps, bias and state 16-byte aligned: the epilogue keeps taps
+                         // and history in registers and moves them sixteen bytes at a time
   // layouts
   int x_tiled;           // X comes as tiled rows (PRO 0 only; K a multiple of 32)
   int y_tiled;           // EPI 1, 3: Y, EPI 2: xs_out are written as tiled rows (their width a multiple of 32)
@@ -243,26 +246,47 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       }
     }
   }
-  const bool pre_conv = EPI == 3 && ex.conv_w <= PRE_TAPS;
+  const bool pre_conv = EPI == 3 && ex.conv_vec != 0;
+  // A lane's four channels are neighbours, so their taps (4 x width floats), their bias and, per row, their history
+  // (4 x (width - 1) floats) are each one run of memory: moved sixteen bytes at a time, the width a compile-time
+  // number in each of the three forms.  A block's channels past H read the last four (loaded, never used), a row
+  // past M its row 0's slot.
+  auto conv_width = [&](auto&& body) {
+    switch (ex.conv_w) {
+      case 2: body(std::integral_constant<int, 2>{}); break;
+      case 3: body(std::integral_constant<int, 3>{}); break;
+      default: body(std::integral_constant<int, 4>{}); break;
+    }
+  };
   auto preload_conv = [&]() {
     if (EPI == 3 && wave == 0 && pre_conv) {
-      const int H = N / 3, Wd = ex.conv_w;
-      // (a channel past H reads channel H - 1, a tap past the width tap 0, a row past M its row 0's slot)
-      const float* bias_p = ex.conv_bias ? ex.conv_bias : ex.taps;
+      const int H = N / 3;
+      const int c0 = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4;
+      const int cc0 = c0 + 3 < H ? c0 : H - 4;
+      const f32x4_t bv = *reinterpret_cast<const f32x4_t*>((ex.conv_bias ? ex.conv_bias : ex.taps) + cc0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int c = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4 + i;
-        const int cc = c < H ? c : H - 1;
-        cbias[i] = bias_p[cc];
+      for (int i = 0; i < 4; ++i) cbias[i] = bv[i];
+      conv_width([&](auto wc) {
+        constexpr int WD = decltype(wc)::value;
+        f32x4_t tq[WD];
 #pragma unroll
-        for (int p = 0; p < PRE_TAPS; ++p) ctap[i][p] = ex.taps[(size_t)cc * Wd + (p < Wd ? p : 0)];
+        for (int q = 0; q < WD; ++q) tq[q] = *reinterpret_cast<const f32x4_t*>(ex.taps + (size_t)cc0 * WD + 4 * q);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int p = 0; p < WD; ++p) ctap[i][p] = tq[(i * WD + p) / 4][(i * WD + p) % 4];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
+          f32x4_t hq[WD - 1];
+          const float* hp = ex.state + ((size_t)cslot[mt] * H + cc0) * (WD - 1);
 #pragma unroll
-          for (int p = 0; p < PRE_TAPS - 1; ++p)
-            chist[mt][i][p] = ex.state[((size_t)cslot[mt] * H + cc) * (Wd - 1) + (p < Wd - 1 ? p : 0)];
+          for (int q = 0; q < WD - 1; ++q) hq[q] = *reinterpret_cast<const f32x4_t*>(hp + 4 * q);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int p = 0; p < WD - 1; ++p) chist[mt][i][p] = hq[(i * (WD - 1) + p) / 4][(i * (WD - 1) + p) % 4];
         }
-      }
+      });
     }
   };
   if (EPI == 3 && MT >= 3) preload_conv();   // the loop of many row tiles keeps its order
@@ -509,39 +533,51 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       if (!live) continue;
       const int H = N / 3, Wd = ex.conv_w;
       const int slot = cslot[mt];
+      const int c0 = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4;
+      if (pre_conv) {
+        if (c0 >= H || !half_ok) continue;
+        conv_width([&](auto wc) {
+          constexpr int WD = decltype(wc)::value;
+          f32x4_t out, nh[WD - 1];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            // the products run on the values as the unfused path stores them: rounded to bfloat16
+            const float Bv = to_f32(f32_to_bf16(acc[0][mt][i])), Cv = to_f32(f32_to_bf16(acc[R > 1 ? 1 : 0][mt][i])),
+                        Xv = to_f32(f32_to_bf16(acc[R > 2 ? 2 : 0][mt][i]));
+            const float u = Bv * Xv;
+            float y = 0.f;
+#pragma unroll
+            for (int p = 0; p < WD - 1; ++p) y += ctap[i][p] * chist[mt][i][p];
+            y += ctap[i][WD - 1] * u;
+            if (ex.conv_bias) y += cbias[i];
+            out[i] = Cv * y;
+#pragma unroll
+            for (int p = 0; p < WD - 1; ++p)
+              nh[(i * (WD - 1) + p) / 4][(i * (WD - 1) + p) % 4] = p < WD - 2 ? chist[mt][i][p + 1] : u;
+          }
+          store4<TOut>(Y + (ex.y_tiled ? tiled_index(m, c0, MT) : (size_t)m * ldy + c0), out, 4);
+          float* hp = ex.state + ((size_t)slot * H + c0) * (WD - 1);
+#pragma unroll
+          for (int q = 0; q < WD - 1; ++q) *reinterpret_cast<f32x4_t*>(hp + 4 * q) = nh[q];
+        });
+        continue;
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int c = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4 + i;
+        const int c = c0 + i;
         if (c >= H || !half_ok) break;
-        // the products run on the values as the unfused path stores them: rounded to bfloat16
-        const float Bv = to_f32(f32_to_bf16(acc[0][mt][i])), Cv = to_f32(f32_to_bf16(acc[1][mt][i])),
-                    Xv = to_f32(f32_to_bf16(acc[2][mt][i]));
+        const float Bv = to_f32(f32_to_bf16(acc[0][mt][i])), Cv = to_f32(f32_to_bf16(acc[R > 1 ? 1 : 0][mt][i])),
+                    Xv = to_f32(f32_to_bf16(acc[R > 2 ? 2 : 0][mt][i]));
         const float u = Bv * Xv;
         float* hist = ex.state + ((size_t)slot * H + c) * (Wd - 1);
-        if (pre_conv) {
-          float y = 0.f;
-#pragma unroll
-          for (int p = 0; p < PRE_TAPS - 1; ++p)
-            if (p < Wd - 1) y += ctap[i][p] * chist[mt][i][p];
-#pragma unroll
-          for (int p = 0; p < PRE_TAPS; ++p)
-            if (p == Wd - 1) y += ctap[i][p] * u;
-          if (ex.conv_bias) y += cbias[i];
-          Y[ex.y_tiled ? tiled_index(m, c, MT) : (size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
-#pragma unroll
-          for (int p = 0; p < PRE_TAPS - 2; ++p)
-            if (p < Wd - 2) hist[p] = chist[mt][i][p + 1];
-          if (Wd >= 2) hist[Wd - 2] = u;
-        } else {
-          const float* wt = ex.taps + (size_t)c * Wd;
-          float y = 0.f;
-          for (int p = 0; p < Wd - 1; ++p) y += wt[p] * hist[p];
-          y += wt[Wd - 1] * u;
-          if (ex.conv_bias) y += ex.conv_bias[c];
-          Y[ex.y_tiled ? tiled_index(m, c, MT) : (size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
-          for (int p = 0; p < Wd - 2; ++p) hist[p] = hist[p + 1];
-          hist[Wd - 2] = u;
-        }
+        const float* wt = ex.taps + (size_t)c * Wd;
+        float y = 0.f;
+        for (int p = 0; p < Wd - 1; ++p) y += wt[p] * hist[p];
+        y += wt[Wd - 1] * u;
+        if (ex.conv_bias) y += ex.conv_bias[c];
+        Y[ex.y_tiled ? tiled_index(m, c, MT) : (size_t)m * ldy + c] = from_f32<TOut>(Cv * y);
+        for (int p = 0; p < Wd - 2; ++p) hist[p] = hist[p + 1];
+        hist[Wd - 2] = u;
       }
     }
   }
@@ -650,5 +686,5 @@ static void skinny_conv(const SkinnyCall& c) {
   const SkinnyExtra& ex = c.ex;
   hipStream_t stream = c.stream;
   const int blocks = gs_ceil_div(N / 3, SHUF == 2 ? 8 : 16);
-  if (ex.res) { GS_BY_MT4(3, 8, 8, 8, 4, 1, 3, bf16, blocks) } else { GS_BY_MT4(3, 8, 8, 8, 8, 0, 3, bf16, blocks) }
+  if (ex.res) { GS_BY_MT4(3, 8, 8, 4, 4, 1, 3, bf16, blocks) } else { GS_BY_MT4(3, 8, 8, 8, 8, 0, 3, bf16, blocks) }
 }
