@@ -32,9 +32,10 @@ class RuntimeOptions:
     vendor's for bfloat16 results (measured on random data at 2,048 rows: 109 us against our 161 for gate|up, 124
     against 162 with the SwiGLU pass counted in; 50 against 75 for 6144 x 2048), ours where the result is float32 and
     inside a recorded graph.
-    ``tune_library``: where the vendor library computes a product of many rows, the first product of a shape measures
-    the library's two dozen best guesses on the operands at hand, cold, and keeps the library's first choice unless
-    another is clearly faster (a few tens of milliseconds a shape).  Off: the library's first choice.
+    ``tune_library``: where the vendor library computes a product of 512, 1024, 2048, ... rows (whole prompt portions),
+    the first product of a shape measures the library's two dozen best guesses on the operands at hand, cold, and
+    keeps the library's first choice unless another is clearly faster (some ten milliseconds a shape).  Other row
+    counts, and all with this off, take the library's first choice.
     ``prompt_attention``: attention of prompt portions in bfloat16: ``"wide"`` = the kernel for long portions wherever it
     takes the sizes (heads of 64), ``"tiles"`` = the kernel with tiles of 16 or 32 queries always, ``"auto"`` = the
     first for steps with a portion of at least 64 tokens, else the second.
@@ -186,7 +187,11 @@ class Runtime:
                                                           and (out.shape[0] <= 1 or out.stride(0) % 8 == 0))):
             if self._library_ws is None:
                 self._library_ws = torch.empty(self.LIBRARY_WORKSPACE, dtype=torch.uint8, device=self.device)
-            return ops.library_gemm(x, w, self._library_ws, out=out, tune=self.tune_library)
+            # measured only for the row counts that come again and again (whole prompt portions: a power of two from
+            # 512 on): a measurement takes some ten milliseconds a shape, and a server's steps bring ever new row counts
+            M = x.shape[0]
+            return ops.library_gemm(x, w, self._library_ws, out=out,
+                                    tune=self.tune_library and M >= 512 and M & (M - 1) == 0)
         return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
 
     def linear_swiglu(self, x, w13: torch.Tensor) -> torch.Tensor:
