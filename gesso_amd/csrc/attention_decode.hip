@@ -124,22 +124,60 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
     for (int i = 0; i < NI; ++i) vreg[i] = *reinterpret_cast<const uint4*>(vcache + vo[i]);
   };
 
-  bf16x8_t kn[4][KS];
-  uint4 vn[NI];
-  int t = t0 + wave;
-  if (t < t1) issue(t, kn, vn);
-
+  // Loads in the order of what they wait for: the queries, the norm weights and the step's own key and value
+  // (they wait for nothing), the rotation factors and the page numbers (for the position), the key and value rows
+  // (for the page numbers).  Loads return in order, so the queries are normed and rotated while the rows are on
+  // their way.
   // the queries as the second operand: lane (r16, kg) holds head r16's features 32 s + 8 kg .. + 8
+  // (lanes past the group load head 0's: every lane loads, no branch hides a load from the compiler's count)
   bf16x8_t qreg[KS];
 #pragma unroll
   for (int st = 0; st < KS; ++st) {
-    if (r16 < G && 32 * st + 8 * kg < D)
-      qreg[st] = *reinterpret_cast<const bf16x8_t*>(q + (size_t)seq * q_stride + (size_t)(kvh * G + r16) * D + 32 * st + 8 * kg);
+    if (32 * st + 8 * kg < D)
+      qreg[st] = *reinterpret_cast<const bf16x8_t*>(q + (size_t)seq * q_stride + (size_t)(kvh * G + (r16 < G ? r16 : 0)) * D + 32 * st + 8 * kg);
     else
       qreg[st] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (!RAW && r16 >= G) qreg[st] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
   }
-  __shared__ __align__(16) uint16_t knew[RAW ? D : 8], vnew[RAW ? D : 8];
+  // Every wavefront keeps a copy of its own of the step's key and value in LDS (the wavefront whose tile holds the
+  // new key reads them there: the cache's rows were loaded before they were written), so no wavefront waits for
+  // another; wavefront 0 of the block whose keys end with the new one also writes them to the cache.
+  __shared__ __align__(16) uint16_t knew[RAW ? W : 1][RAW ? D : 8], vnew[RAW ? W : 1][RAW ? D : 8];
   const bool has_new = RAW && raw.write_kv && t0 < t1 && t1 == tiles;   // this block's keys end with the new one
+  constexpr int E = D >= 64 ? D / 64 : 1;
+  float qw8[RAW ? KS : 1][8], c8[RAW ? KS / 2 : 1][8], s8[RAW ? KS / 2 : 1][8];
+  float kraw_f[E], kw_f[E], kc_f = 1.f, ks_f = 0.f;
+  bf16 vraw_b[E];
+  if constexpr (RAW != 0) {
+    if (raw.qw) {
+#pragma unroll
+      for (int st = 0; st < KS; ++st) load8f(raw.qw + 32 * st + 8 * kg, qw8[st]);
+    }
+    const bf16* kraw = q + (size_t)seq * q_stride + (size_t)(nh + kvh) * D;
+    const bf16* vraw = q + (size_t)seq * q_stride + (size_t)(nh + nkv + kvh) * D;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      kraw_f[e] = to_f32(kraw[lane + 64 * e]);
+      vraw_b[e] = vraw[lane + 64 * e];
+      kw_f[e] = raw.kw ? raw.kw[lane + 64 * e] : 1.f;
+    }
+    // (weights and rotation factors in 16-byte loads: the tables' rows and this lane's offsets are multiples of 8)
+#pragma unroll
+    for (int st = 0; st < KS / 2; ++st) {
+      load8f(raw.cos_t + (size_t)pos * (D / 2) + 32 * st + 8 * kg, c8[st]);
+      load8f(raw.sin_t + (size_t)pos * (D / 2) + 32 * st + 8 * kg, s8[st]);
+    }
+    const int pi = E == 2 ? lane : (lane & 31);          // index of this lane's pair of the key
+    kc_f = raw.cos_t[(size_t)pos * (D / 2) + pi];
+    ks_f = raw.sin_t[(size_t)pos * (D / 2) + pi];
+  }
+  bf16x8_t kn[4][KS];
+  uint4 vn[NI];
+  int t = t0 + wave;
+  // (a wavefront without a tile asks for the block's first one: its address is a valid one, and a load behind a
+  // branch would make the compiler wait for every load in flight where it needs the queries)
+  issue(t < t1 ? t : (t0 < tiles ? t0 : 0), kn, vn);
+
   if constexpr (RAW != 0) {
     // head norm and rotation of this lane's part of its query: float32 arithmetic on the product's bfloat16
     // values, rounded to bfloat16 again, as the separate kernel does.  The halves of a rotation pair (i, i + D/2)
@@ -153,22 +191,12 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
         qf[st][j] = (float)qreg[st][j];
         ss += qf[st][j] * qf[st][j];
       }
-    // (weights and rotation factors in 16-byte loads: the tables' rows and this lane's offsets are multiples of 8)
-    float c8[KS / 2][8], s8[KS / 2][8];
-#pragma unroll
-    for (int st = 0; st < KS / 2; ++st) {
-      load8f(raw.cos_t + (size_t)pos * (D / 2) + 32 * st + 8 * kg, c8[st]);
-      load8f(raw.sin_t + (size_t)pos * (D / 2) + 32 * st + 8 * kg, s8[st]);
-    }
     if (raw.qw) {
       const float inv = norm_inverse(group4_sum(ss), (float)D, raw.eps);
 #pragma unroll
-      for (int st = 0; st < KS; ++st) {
-        float w8[8];
-        load8f(raw.qw + 32 * st + 8 * kg, w8);
+      for (int st = 0; st < KS; ++st)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) qf[st][j] = qf[st][j] * inv * w8[j];
-      }
+        for (int j = 0; j < 8; ++j) qf[st][j] = qf[st][j] * inv * qw8[st][j];
     }
 #pragma unroll
     for (int st = 0; st < KS / 2; ++st)
@@ -182,44 +210,42 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
     for (int st = 0; st < KS; ++st)
 #pragma unroll
       for (int j = 0; j < 8; ++j) qreg[st][j] = (r16 < G) ? (__bf16)qf[st][j] : (__bf16)0.f;
-    // the new key and value: wavefront 0, lane = feature (and feature + 64 for heads of 128)
-    if (has_new && wave == 0) {
-      constexpr int E = D >= 64 ? D / 64 : 1;
-      const bf16* kraw = q + (size_t)seq * q_stride + (size_t)(nh + kvh) * D;
-      const bf16* vraw = q + (size_t)seq * q_stride + (size_t)(nh + nkv + kvh) * D;
+    // the new key and value: lane = feature (and feature + 64 for heads of 128)
+    if (raw.write_kv) {
       float kf[E];
       float ks = 0.f;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        kf[e] = to_f32(kraw[lane + 64 * e]);
+        kf[e] = kraw_f[e];
         ks += kf[e] * kf[e];
       }
       if (raw.kw) {
         const float inv = norm_inverse(wave_sum_dpp(ks), (float)D, raw.eps);
 #pragma unroll
-        for (int e = 0; e < E; ++e) kf[e] = kf[e] * inv * raw.kw[lane + 64 * e];
+        for (int e = 0; e < E; ++e) kf[e] = kf[e] * inv * kw_f[e];
       }
-      const int i = E == 2 ? lane : (lane & 31);          // index of this lane's pair
-      const float c = raw.cos_t[(size_t)pos * (D / 2) + i], sn = raw.sin_t[(size_t)pos * (D / 2) + i];
       if (E == 2) {
         const float a = kf[0], b = kf[E - 1];
-        kf[0] = a * c - b * sn;
-        kf[E - 1] = a * sn + b * c;
+        kf[0] = a * kc_f - b * ks_f;
+        kf[E - 1] = a * ks_f + b * kc_f;
       } else {
         const float other = __shfl_xor(kf[0], 32, 64);
-        kf[0] = lane < 32 ? kf[0] * c - other * sn : other * sn + kf[0] * c;
+        kf[0] = lane < 32 ? kf[0] * kc_f - other * ks_f : other * ks_f + kf[0] * kc_f;
       }
       const long row = row_off(pos);
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        const bf16 kb = f32_to_bf16(kf[e]), vb = vraw[lane + 64 * e];
-        knew[lane + 64 * e] = kb.x;
-        vnew[lane + 64 * e] = vb.x;
-        kcache[row + lane + 64 * e] = kb;
-        vcache[row + lane + 64 * e] = vb;
+        const bf16 kb = f32_to_bf16(kf[e]);
+        knew[wave][lane + 64 * e] = kb.x;
+        vnew[wave][lane + 64 * e] = vraw_b[e].x;
+        if (has_new && wave == 0) {
+          kcache[row + lane + 64 * e] = kb;
+          vcache[row + lane + 64 * e] = vraw_b[e];
+        }
       }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // LDS writes of this wavefront are visible to its own lanes
     }
-    __syncthreads();
   }
   const float qscale = scale * DEC_LOG2E;   // scores are scaled after the product, in float32
 
@@ -241,11 +267,11 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
       for (int kt = 0; kt < 4; ++kt)
         if (4 * r16 + kt == rel) {
 #pragma unroll
-          for (int st = 0; st < KS; ++st) kc[kt][st] = *reinterpret_cast<const bf16x8_t*>(&knew[32 * st + 8 * kg]);
+          for (int st = 0; st < KS; ++st) kc[kt][st] = *reinterpret_cast<const bf16x8_t*>(&knew[wave][32 * st + 8 * kg]);
         }
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        if (kq + i * KG == rel) vc[i] = *reinterpret_cast<const uint4*>(&vnew[dc * 8]);
+        if (kq + i * KG == rel) vc[i] = *reinterpret_cast<const uint4*>(&vnew[wave][dc * 8]);
     }
     // sc[kt][i]: head r16, key base + 4 (4 kg + i) + kt
     f32x4_t sc[4];
