@@ -165,7 +165,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(const bf16* __r
         if (EPI == 1) {
           // on the values as the unfused path stores them: rounded to bfloat16
           const float g = to_f32(f32_to_bf16(v)), u = to_f32(f32_to_bf16(acc[i][j + (EPI == 1 ? TN / 2 : 0)][e]));
-          v = g / (1.0f + expf(-g)) * u;
+          // (the hardware's exponential and reciprocal: a block has 32,768 of these to do, and the library's expf and
+          // a float division, some eighty instructions an element, took a fifth of the kernel's time)
+          v = g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)) * u;
         }
         Y[(size_t)m * ldy + n] = from_f32<TOut>(v);
       }
@@ -210,10 +212,10 @@ extern "C" int gs_gemm_mfma(const void* X, int ldx, const void* W, void* Y, int 
     if (use_big) launch_mfma<256, 256, 4, 2, 1, bf16>(x, ldx, w, (bf16*)Y, ldy, M, N, K, stream);
     else launch_mfma<128, 256, 2, 2, 1, bf16>(x, ldx, w, (bf16*)Y, ldy, M, N, K, stream);
   } else if (y_dtype == GS_BF16) {
-    if (use_big) launch_mfma<256, 256, 4, 2, 0, bf16>(x, ldx, w, (bf16*)Y, ldy, M, N, K, stream);
+    if (use_big) launch_mfma<256, 256, 2, 4, 0, bf16>(x, ldx, w, (bf16*)Y, ldy, M, N, K, stream);
     else launch_mfma<128, 128, 2, 2, 0, bf16>(x, ldx, w, (bf16*)Y, ldy, M, N, K, stream);
   } else {
-    if (use_big) launch_mfma<256, 256, 4, 2, 0, float>(x, ldx, w, (float*)Y, ldy, M, N, K, stream);
+    if (use_big) launch_mfma<256, 256, 2, 4, 0, float>(x, ldx, w, (float*)Y, ldy, M, N, K, stream);
     else launch_mfma<128, 128, 2, 2, 0, float>(x, ldx, w, (float*)Y, ldy, M, N, K, stream);
   }
   GS_LAUNCH_CHECK("gemm_mfma");
