@@ -531,6 +531,55 @@ def test_attention_decode(ops, nh, nkv, d, ps, nsplit, window):
     close(got, same.double().cpu(), torch.bfloat16)
 
 
+@pytest.mark.parametrize("nsplit", [1, 3])
+@pytest.mark.parametrize("window", [None, 70])
+def test_attention_decode_sees_the_far_key_and_not_the_keys_outside(ops, nsplit, window):
+    """A key far back that carries most of the weight must count in full; a key one place past the sequence's end (on
+    the last page) and, with a window, the key one place before the window's start are made to stand out ten times
+    more and must count for nothing: a mask off by one moves the result by far more than the tolerance."""
+    g = gen(31 + nsplit)
+    nh, nkv, d, ps = 8, 2, 64, 16
+    lens = [17, 63, 64, 65, 300, 700, 129, 1030]
+    nseq = len(lens)
+    nblk = [-(-(n + 1) // ps) for n in lens]                 # room for the key past the end
+    total = sum(nblk)
+    perm = torch.randperm(total + 2, generator=g)[:total] + 1
+    kc = torch.randn(total + 3, nkv, ps, d, generator=g)
+    vc = torch.randn(total + 3, nkv, ps, d, generator=g)
+    table = torch.zeros(nseq, max(nblk), dtype=torch.int32)
+    q = torch.randn(nseq, nh, d, generator=g)
+    want, moved, at = [], [], 0
+    G = nh // nkv
+    for i, n in enumerate(lens):
+        pages = perm[at:at + nblk[i]]
+        at += nblk[i]
+        table[i, :nblk[i]] = pages.to(torch.int32)
+
+        def put(u, row):                                     # key u of this sequence, for every key head
+            kc[pages[u // ps], :, u % ps] = row
+
+        lo = max(0, n - window) if window else 0
+        far = lo + min(3, n - 1 - lo)                        # a visible key near the far end of what is seen
+        qdir = q[i, ::G]                                     # one query per key head: (nkv, d)
+        put(far, qdir * 2.0)
+        put(n, qdir * 20.0)                                  # one past the end: must not be seen
+        if window and lo > 0:
+            put(lo - 1, qdir * 20.0)                         # one before the window: must not be seen
+        k = kc[pages].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:n].bfloat16().double()
+        v = vc[pages].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:n].bfloat16().double()
+        qi = q[i].bfloat16().double().reshape(1, nh, d)
+        want.append(P.causal_attention(qi, k, v, window or 0).reshape(-1))
+        k2 = k.clone()
+        k2[far] = 0.0                                        # without the far key the result is another one
+        moved.append(float((P.causal_attention(qi, k2, v, window or 0).reshape(-1) - want[-1]).abs().max()))
+    want = torch.stack(want)
+    assert min(moved) > 0.1
+    positions = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    got = ops.attention_decode(q.reshape(nseq, -1).bfloat16().to(DEV), nh * d, kc.bfloat16().to(DEV), vc.bfloat16().to(DEV),
+                               positions.to(DEV), table.to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, nseq, nsplit)
+    close(got, want, torch.bfloat16)
+
+
 @pytest.mark.parametrize("nh,nkv,d,norm,nsplit,write,copies", [(32, 8, 64, True, 1, True, 1), (2, 1, 64, False, 3, True, 1),
                                                                (8, 1, 128, True, 2, True, 1), (5, 5, 64, True, 1, False, 1),
                                                                (32, 8, 64, True, 1, True, 12), (4, 2, 64, True, 2, True, 24)])
@@ -895,6 +944,42 @@ def test_attention_prefill_wide(ops, nh, nkv, ps, window):
     wide[:, :nh * d] = qall
     got = ops.attention_prefill_wide(wide.to(DEV), stride, kc.to(DEV), vc.to(DEV), positions.to(DEV), tiles.to(DEV),
                                      table.to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, sum(new))
+    close(got, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("kernel", ["wide", "tiles16", "tiles32"])
+@pytest.mark.parametrize("window", [None, 50])
+def test_prompt_attention_never_sees_the_next_key_nor_the_one_before_its_window(ops, kernel, window):
+    """Every key stands out for the query one place before it (and, with a window, for the query `window` places after
+    it): a causal mask or a window's edge that is off by one lets one such key in, and it then carries nearly all of
+    that query's weight.  One chunk of 150 queries over a prefix of 83 keys, heads of 64 in groups of two."""
+    g = gen(9 + (window or 0))
+    nh, nkv, d, ps, prefix, new = 4, 2, 64, 16, 83, 150
+    K = prefix + new
+    G = nh // nkv
+    v = torch.randn(K, nkv, d, generator=g)
+    q = torch.randn(new, nh, d, generator=g)
+    k = torch.randn(K, nkv, d, generator=g) * 0.3
+    for u in range(prefix + 1, K):                        # key u: for query u - 1 (the next key: never visible)
+        k[u] += q[u - 1 - prefix, ::G] * 6.0
+    if window:
+        for u in range(prefix - window, K - window):      # key u: also for query u + window (just outside its window)
+            if u >= 0:
+                k[u] += q[u + window - prefix, ::G] * 6.0
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    want = P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(new, -1)
+    # the control: with the mask one place too wide the result is another one altogether
+    if not window:
+        loose = P.causal_attention(torch.cat([q.double()[1:], q.double()[-1:]]), k.double(), v.double(), 0).reshape(new, -1)
+        assert float((loose - want).abs().max()) > 0.5
+    kc, vc, tab = paged(k, v, ps, g)
+    positions = torch.arange(prefix, K, dtype=torch.int32)
+    rows = ops.attention_prefill_wide_rows(nh, nkv) if kernel == "wide" else int(kernel[5:])
+    tiles = torch.tensor([[0] * -(-new // rows), list(range(0, new, rows)), [min(rows, new - a) for a in range(0, new, rows)]],
+                         dtype=torch.int32)
+    args = (q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV), positions.to(DEV), tiles.to(DEV), tab[None].to(DEV), ps,
+            window, 1.0 / math.sqrt(d), nh, nkv, d, new)
+    got = ops.attention_prefill_wide(*args) if kernel == "wide" else ops.attention_prefill(*args, tile_rows=rows)
     close(got, want, torch.bfloat16)
 
 
