@@ -8,6 +8,7 @@ layer read another layer's cache; a scaled embedding and capped logits) are defi
 stepped through the unchanged engine.
 """
 import dataclasses
+import os
 import math
 
 import pytest
@@ -480,3 +481,54 @@ def test_toy_parts_register_build_and_step(fw, dtype):
         unregister("mixer", "toy_decay")
         unregister("position", "toy_scaled_rope")
         unregister("ffn", "toy_routed")
+
+
+def test_a_toy_architecture_goes_from_its_folder_to_tokens(fw, tmp_path):
+    """Another architecture is a typed configuration, a function from it to a model spec and one call of
+    `register_architecture`: here the toy model above gets a configuration of two keys, a folder is written for it with
+    seeded weights, `Session` loads the folder by the name in its config.json and generates greedily (prompt in
+    portions, recorded decode steps or not: the toy mixer decides), and the tokens are the plain toy model's."""
+    from gesso_amd import Session
+    from gesso_amd.config import register_architecture, unregister_architecture
+    from gesso_amd.parts import unregister
+    from gesso_amd.weights import write_model_folder
+    from gesso_amd.weights.safetensors_io import SafetensorsFile
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyConfig:
+        decay: float = 0.5
+        max_position_embeddings: int = 64
+
+        def to_json(self):
+            return {"architectures": ["ToyForTests"], "decay": self.decay, "max_position_embeddings": self.max_position_embeddings}
+
+    def parse(raw):
+        assert set(raw) == {"architectures", "decay", "max_position_embeddings"}
+        return ToyConfig(float(raw["decay"]), int(raw["max_position_embeddings"]))
+
+    register_toys()
+    register_architecture("ToyForTests", parse, lambda c: toy_spec(), lambda c: c.to_json())
+    try:
+        folder = write_model_folder(str(tmp_path / "toy"), ToyConfig(), seed=17, dtype=torch.float32, std=0.2)
+        stored = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+        w64 = {k: stored.tensor(k).double() for k in stored.names()}
+        stored.close()
+        prompt = [3, 1, 4, 1, 5, 9, 2, 6, 5]
+        want, margins = list(prompt), []
+        for _ in range(5):
+            logits = toy_plain(w64, want, [])[-1]
+            top = logits.topk(2).values
+            margins.append(float(top[0] - top[1]))
+            want.append(int(logits.argmax()))
+        assert min(margins) > 1e-3, "the seed keeps the greedy choices clear of ties"
+        sess = Session(folder, dtype="float32", context_length=64, page_size=4, chunk_size=4, max_num_seqs=2)
+        assert sess.engine.spec.architecture == "ToyForTests"
+        got = sess.generate([prompt], max_new_tokens=5)[0]
+        assert got == want
+        sess.close()
+    finally:
+        unregister_architecture("ToyForTests")
+        unregister("mixer", "toy_decay")
+        unregister("position", "toy_scaled_rope")
+        unregister("ffn", "toy_routed")
+
