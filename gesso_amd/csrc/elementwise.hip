@@ -383,6 +383,39 @@ extern "C" int gs_residual_add(float* res, const void* delta, int delta_dtype, l
   return 0;
 }
 
+// out[t, j] = y[t, j] + bias[j]: the bias of a product whose float32 sums a matrix-core kernel made; one rounding,
+// after the bias.  Four columns per thread when N is a multiple of 4 and the rows are 16-byte aligned.
+template <typename TOut, int V>
+__global__ void add_bias_kernel(const float* __restrict__ y, const float* __restrict__ bias, TOut* __restrict__ out,
+                                int N, long ldo, long n) {
+  long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * V;
+  if (i >= n) return;
+  long t = i / N;
+  int j = (int)(i - t * N);
+#pragma unroll
+  for (int k = 0; k < V; ++k) out[t * ldo + j + k] = from_f32<TOut>(y[i + k] + bias[j + k]);
+}
+
+extern "C" int gs_add_bias(const float* y, const float* bias, void* out, int out_dtype, int M, int N, long ldo,
+                           hipStream_t stream) {
+  GS_REQUIRE(M >= 0 && N > 0 && ldo >= N, "add_bias: bad sizes M=%d N=%d ldo=%ld", M, N, ldo);
+  long n = (long)M * N;
+  if (n == 0) return 0;
+  const bool v4 = N % 4 == 0 && ldo % 4 == 0;
+  long threads = v4 ? n / 4 : n;
+  int blocks = (int)gs_ceil_div(threads, 256);
+  if (out_dtype == GS_F32) {
+    if (v4) add_bias_kernel<float, 4><<<blocks, 256, 0, stream>>>(y, bias, (float*)out, N, ldo, n);
+    else add_bias_kernel<float, 1><<<blocks, 256, 0, stream>>>(y, bias, (float*)out, N, ldo, n);
+  } else if (out_dtype == GS_BF16) {
+    if (v4) add_bias_kernel<bf16, 4><<<blocks, 256, 0, stream>>>(y, bias, (bf16*)out, N, ldo, n);
+    else add_bias_kernel<bf16, 1><<<blocks, 256, 0, stream>>>(y, bias, (bf16*)out, N, ldo, n);
+  } else
+    GS_REQUIRE(false, "add_bias: unknown dtype %d", out_dtype);
+  GS_LAUNCH_CHECK("add_bias");
+  return 0;
+}
+
 // ------------------------------------------------------------------ SwiGLU
 
 // in (T, 2F): gate in columns [0, F), up in [F, 2F).  out[t, j] = silu(gate) * up, silu(g) = g / (1 + exp(-g)).

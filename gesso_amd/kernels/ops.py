@@ -196,6 +196,23 @@ def swiglu(x: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     return out
 
 
+def add_bias(y: torch.Tensor, bias: torch.Tensor, out_dtype=None, out: torch.Tensor = None) -> torch.Tensor:
+    """``y + bias`` row by row: ``y`` float32 ``(M, N)`` contiguous (a product's sums), ``bias`` float32 ``(N,)``;
+    the result in ``out_dtype``, rounded once."""
+    _dev(y, bias)
+    _need(out is None or out.is_cuda, "kernel operands must live on the GPU")
+    _need(y.dtype == torch.float32 and y.dim() == 2 and y.is_contiguous(), "add_bias: y must be float32 (M, N), contiguous")
+    M, N = y.shape
+    _need(bias.dtype == torch.float32 and bias.shape == (N,) and bias.is_contiguous(), "add_bias: bias must be float32 (N,)")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or torch.float32, device=y.device)
+    _need(out.shape == (M, N) and out.stride(1) == 1 and out.dtype in (torch.float32, torch.bfloat16),
+          "add_bias: out has the wrong shape or type")
+    _check(lib().gs_add_bias(_p(y), _p(bias), _p(out), c_int(_dt(out)), c_int(M), c_int(N),
+                             c_long(out.stride(0) if M > 1 else N), _stream()))
+    return out
+
+
 def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
     """``cap * tanh(logits / cap)`` in place (float32)."""
     _dev(logits)

@@ -166,6 +166,10 @@ class Runtime:
             x = x.materialize()
         if isinstance(x, ops.TiledRows) and not (bias is None and ops.skinny_ok(x, w)):
             x = x.rows()
+        if (bias is not None and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias.dtype == torch.float32
+                and (ops.skinny_ok(x, w) or (self.many_rows != "library" and ops.mfma_ok(x, w)))):
+            # the matrix cores' float32 sums, then the bias and one rounding
+            return ops.add_bias(self.linear(x, w, out_dtype=torch.float32), bias, out_dtype, out)
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and bias is None:
             if ops.skinny_ok(x, w):
                 return ops.gemm_skinny(x, w, out_dtype=out_dtype, out=out, wt=self.tiles_of(w))

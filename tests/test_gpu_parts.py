@@ -140,6 +140,35 @@ def test_library_products_of_many_rows_are_planned_once_per_shape_and_stay_right
     assert float((y - x.double() @ w5.double().T).abs().max()) <= tol(torch.bfloat16, want)
 
 
+@pytest.mark.parametrize("rows", [1, 9, 64, 65, 300])
+@pytest.mark.parametrize("N,K", [(96, 64), (77, 40)])
+def test_a_bfloat16_product_with_bias_sums_on_the_matrix_cores_and_rounds_once(fw, rows, N, K, monkeypatch):
+    """A projection with a bias (``conv_bias: true``) takes the same matrix-core kernels as one without: float32 sums,
+    then bias and one rounding.  The FMA kernel must not be what computes it where the fast kernels take the operands
+    (K a multiple of 8), and the result is within half a bfloat16 step of the float64 one, which a product rounded
+    before the bias would not always be."""
+    from gesso_amd.kernels import ops
+    from gesso_amd.parts import Runtime
+    g = gen(rows + N)
+    x = torch.randn(rows, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    bias = torch.randn(N, generator=g) * 3
+    want = x.double() @ w.double().T + bias.double()
+    rt = Runtime(DEV, torch.bfloat16)
+    calls = []
+    real = ops.gemm_tiled
+    monkeypatch.setattr(ops, "gemm_tiled", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    out = torch.full((rows, N + 8), float("nan"), dtype=torch.bfloat16, device=DEV)
+    got = rt.linear(x.to(DEV), w.to(DEV), bias.to(DEV), out=out[:, :N])
+    assert not calls
+    assert torch.isnan(out[:, N:]).all()
+    err = (got.double().cpu() - want).abs()
+    step = 2.0 ** (torch.floor(torch.log2(want.abs().clamp_min(1e-30))) - 7)      # a bfloat16 step at each value
+    assert bool((err <= 0.5 * step + 1e-4).all()), float((err / step).max())
+    f32 = rt.linear(x.to(DEV), w.to(DEV), bias.to(DEV), out_dtype=torch.float32)
+    assert f32.dtype == torch.float32 and float((f32.double().cpu() - want).abs().max()) <= 1e-4
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_part(fw, dtype):
     from gesso_amd.config import SwiGLUSpec
