@@ -436,12 +436,48 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   }
 
   if (scaled) {
-    for (int m = wave; m < M; m += WAVES) {
-      float ssum = 0.f;
-      if (m == wave) ssum = (pre[0] + pre[1]) + (pre[2] + pre[3]);
-      for (int b = (m == wave ? 256 : 0) + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
+    // a wavefront's first row was asked for at the start; its further rows (row wave + WAVES, ...) are asked for here
+    // in batches, every load of a batch in flight before the first is added, at addresses that always exist (a row
+    // or a partial sum that does not is read from the first and counted as zero): no load sits behind a branch
+    constexpr int RPW = (MT * 16 + WAVES - 1) / WAVES;
+    constexpr int BATCH = RPW - 1 < 8 ? (RPW > 1 ? RPW - 1 : 1) : 8;
+    if (wave < M) {
+      float ssum = (pre[0] + pre[1]) + (pre[2] + pre[3]);
+      for (int b = 256 + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)wave * ex.nb + b];
       ssum = wave_sum_dpp(ssum);
-      if (lane == 0) inv_s[m] = norm_inverse(ssum, (float)K, ex.eps);
+      if (lane == 0) inv_s[wave] = norm_inverse(ssum, (float)K, ex.eps);
+    }
+    if (MT == 1) {   // at most one further row: the plain loop is the smallest code, and the step of few rows feels it
+      for (int m = wave + WAVES; m < M; m += WAVES) {
+        float ssum = 0.f;
+        for (int b = lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
+        ssum = wave_sum_dpp(ssum);
+        if (lane == 0) inv_s[m] = norm_inverse(ssum, (float)K, ex.eps);
+      }
+    }
+#pragma unroll
+    for (int i0 = 1; MT > 1 && i0 < RPW; i0 += BATCH) {
+      if (wave + i0 * WAVES < M) {
+        float q[BATCH][4];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+          const int m = wave + (i0 + i) * WAVES;
+          const float* row = ex.ssq + (size_t)(m < M ? m : wave) * ex.nb;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) q[i][j] = row[lane + 64 * j < ex.nb ? lane + 64 * j : 0];
+        }
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+          const int m = wave + (i0 + i) * WAVES;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) q[i][j] = lane + 64 * j < ex.nb ? q[i][j] : 0.f;
+          float ssum = (q[i][0] + q[i][1]) + (q[i][2] + q[i][3]);
+          if (ex.nb > 256 && m < M)
+            for (int b = 256 + lane; b < ex.nb; b += 64) ssum += ex.ssq[(size_t)m * ex.nb + b];
+          ssum = wave_sum_dpp(ssum);
+          if (lane == 0 && i0 + i < RPW && m < M) inv_s[m] = norm_inverse(ssum, (float)K, ex.eps);
+        }
+      }
     }
     if (WAVES == 1) __syncthreads();
   }
