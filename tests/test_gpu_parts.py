@@ -561,3 +561,151 @@ def test_a_toy_architecture_goes_from_its_folder_to_tokens(fw, tmp_path):
         unregister("position", "toy_scaled_rope")
         unregister("ffn", "toy_routed")
 
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_toy_norm_and_a_toy_block_arrangement_register_build_and_step(fw, dtype):
+    """The two kinds of part that the other toy tests leave out.  A norm that centres its rows and has a bias (no
+    ``row_weight``: nothing may pre-weight rows for it) serves as a block's norm, beside an RMSNorm in the same block,
+    and as the model's last norm (with ``rows``).  A block arrangement that feeds one normed input to the mixer and to
+    the feed-forward at once and adds both (no ``first_norm`` hint) runs before an ordinary block.  Registered from
+    here, built by kind, stepped whole and in portions beside another request, against the arithmetic written out."""
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.config import AttentionSpec, BlockSpec, LayerCall, ModelSpec, RMSNormSpec, RopeSpec, ShortConvSpec, SwiGLUSpec
+    from gesso_amd.models.model import tensor_table
+    from gesso_amd.parts import VECTOR, Part, TensorSpec, register, unregister
+    from gesso_amd.parts.registry import build, part_class
+    from gesso_amd.weights import random_tensors
+    from gesso_amd.weights.loader import held_dtype
+
+    @dataclasses.dataclass(frozen=True)
+    class CenteredSpec:
+        size: int
+        eps: float
+        kind: str = "toy_centered"
+
+    @dataclasses.dataclass(frozen=True)
+    class ParallelSpec:
+        mixer: object
+        norm: object
+        ffn: object
+        names: dict = dataclasses.field(compare=False, hash=False, default_factory=dict)
+        kind: str = "toy_parallel"
+
+    class CenteredNorm(Part):
+        @staticmethod
+        def tensor_specs(spec):
+            return {"weight": TensorSpec((spec.size,), VECTOR, "one_plus_normal"), "bias": TensorSpec((spec.size,), VECTOR)}
+
+        def bind(self, tensors):
+            self.weight, self.bias = tensors["weight"], tensors["bias"]
+
+        def add_norm(self, stream, rows=None, out=None):
+            stream.flush(self.rt)
+            x = stream.res if rows is None else stream.res[rows.long()]
+            x = x - x.mean(-1, keepdim=True)
+            y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.spec.eps) * self.weight + self.bias
+            return y.to(self.rt.dtype)
+
+    class ParallelBlock(Part):
+        def __init__(self, spec, rt):
+            super().__init__(spec, rt)
+            self.norm, self.mixer, self.ffn = build("norm", spec.norm, rt), build("mixer", spec.mixer, rt), build("ffn", spec.ffn, rt)
+
+        @staticmethod
+        def tensor_specs(spec):
+            return {f"{role}.{k}": ts for role, cat, sub in (("norm", "norm", spec.norm), ("mixer", "mixer", spec.mixer),
+                                                             ("ffn", "ffn", spec.ffn))
+                    for k, ts in part_class(cat, sub).tensor_specs(sub).items()}
+
+        @staticmethod
+        def cache_need(spec):
+            return part_class("mixer", spec.mixer).cache_need(spec.mixer)
+
+        def bind(self, tensors):
+            from gesso_amd.parts.base import sub_tensors
+            for role in ("norm", "mixer", "ffn"):
+                getattr(self, role).bind(sub_tensors(tensors, role))
+
+        def forward(self, stream, ctx, cache):
+            x = self.norm.add_norm(stream)
+            stream.push(self.mixer.forward(x, ctx, cache), self.rt)
+            stream.push(self.ffn.forward(x, ctx), self.rt)
+
+    H, V, eps = 48, 56, 1e-4
+    centered = CenteredSpec(H, eps)
+    attn = AttentionSpec(hidden=H, n_heads=3, n_kv_heads=1, head_dim=16, qk_norm=None,
+                         position=RopeSpec(head_dim=16, rotary_dim=16, theta=1e4, max_position=64))
+    b0 = ParallelSpec(attn, centered, SwiGLUSpec(hidden=H, intermediate=40),
+                      {**{f"mixer.{k}_proj.weight": f"A.{k}" for k in ("q", "k", "v", "out")}, "norm.weight": "A.nw",
+                       "norm.bias": "A.nb", "ffn.w1.weight": "A.w1", "ffn.w3.weight": "A.w3", "ffn.w2.weight": "A.w2"})
+    b1 = BlockSpec(ShortConvSpec(hidden=H, width=3), centered, SwiGLUSpec(hidden=H, intermediate=24), RMSNormSpec(H, 1e-5),
+                   {"mixer.in_proj.weight": "B.in", "mixer.conv.weight": "B.taps", "mixer.out_proj.weight": "B.out",
+                    "mixer_norm.weight": "B.nw", "mixer_norm.bias": "B.nb", "ffn_norm.weight": "B.n2",
+                    "ffn.w1.weight": "B.w1", "ffn.w3.weight": "B.w3", "ffn.w2.weight": "B.w2"})
+    spec = ModelSpec(architecture="ToyNormsAndBlocks", hidden=H, vocab=V, blocks=(b0, b1), schedule=(LayerCall(0), LayerCall(1)),
+                     final_norm=centered, tie_embeddings=False, max_position=64,
+                     names={"embed": "emb", "head": "head", "final_norm.weight": "fw", "final_norm.bias": "fb"})
+
+    def centered_norm(x, w, b):
+        x = x - x.mean(-1, keepdim=True)
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w + b
+
+    def plain(w, ids):
+        T = len(ids)
+        h = P.embedding(w["emb"], ids)
+        n = centered_norm(h, w["A.nw"], w["A.nb"])
+        pos = list(range(T))
+        q = P.rope(P.linear(n, w["A.q"]).reshape(T, 3, 16), pos, 1e4)
+        k = P.rope(P.linear(n, w["A.k"]).reshape(T, 1, 16), pos, 1e4)
+        v = P.linear(n, w["A.v"]).reshape(T, 1, 16)
+        mixed = P.linear(P.causal_attention(q, k, v).reshape(T, 48), w["A.out"])
+        fed = P.linear(P.swiglu(P.linear(n, w["A.w1"]), P.linear(n, w["A.w3"])), w["A.w2"])
+        h = h + mixed + fed
+        n = centered_norm(h, w["B.nw"], w["B.nb"])
+        u, _ = P.short_conv(P.linear(n, w["B.in"]), w["B.taps"].reshape(H, 3))
+        h = h + P.linear(u, w["B.out"])
+        n = P.rmsnorm(h, w["B.n2"], 1e-5)
+        h = h + P.linear(P.swiglu(P.linear(n, w["B.w1"]), P.linear(n, w["B.w3"])), w["B.w2"])
+        return P.linear(centered_norm(h, w["fw"], w["fb"]), w["head"])
+
+    register("norm", "toy_centered", CenteredNorm, replace=True)
+    register("block", "toy_parallel", ParallelBlock, replace=True)
+    try:
+        table = tensor_table(spec)
+        assert {"A.nb", "B.nb", "fb", "A.q", "B.taps", "head"} <= set(table) and "A.n2" not in table
+        cpu = random_tensors(table, 5, dtype, std=0.2)
+        eng = Engine(spec, {k: v.to(DEV, held_dtype(v.dtype, table[k].role, dtype)) for k, v in cpu.items()}, dtype,
+                     DEV, page_size=4, num_pages=16, num_slots=3)
+        assert not eng.model.graph_safe          # the toy parts do not say that they may be recorded
+        w64 = {k: v.double() for k, v in cpu.items()}
+        ids = {"a": [3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9], "b": [2, 7, 1, 8, 2, 8, 1, 8, 2]}
+        want = {k: plain(w64, v) for k, v in ids.items()}
+        # the bias and the centring matter: the same rows through an RMSNorm in their place are far off
+        off = P.linear(P.rmsnorm(P.embedding(w64["emb"], ids["a"]), w64["fw"], eps), w64["head"])
+        t = (2e-5 if dtype == torch.float32 else 3e-2) * max(1.0, max(float(x.abs().max()) for x in want.values()))
+        assert float((off - want["a"]).abs().max()) > 20 * t
+        eng.add_request("a")
+        got = eng.step([StepEntry("a", ids["a"], list(range(13)))]).double().cpu()
+        eng.finish_request("a")
+        assert float((got - want["a"]).abs().max()) <= t
+        # a in portions 6, 1, 6 beside b in 2, 6, 1; only some places wanted (the last norm gets ``rows``)
+        eng.add_request("a"); eng.add_request("b")
+        at = {"a": 0, "b": 0}
+        for na, nb in ((6, 2), (1, 6), (6, 1)):
+            ea = StepEntry("a", ids["a"][at["a"]:at["a"] + na], [na - 1])
+            eb = StepEntry("b", ids["b"][at["b"]:at["b"] + nb], [0, nb - 1])
+            lg = eng.step([ea, eb]).double().cpu()
+            rows = torch.stack([want["a"][at["a"] + na - 1], want["b"][at["b"]], want["b"][at["b"] + nb - 1]])
+            assert float((lg - rows).abs().max()) <= t, (na, nb)
+            at["a"] += na; at["b"] += nb
+        # decoding goes step by step where a part cannot be recorded, through the same entry point
+        out, bad = eng.decode(["a", "b"], [7, 11], 2)
+        assert not bad.any()
+        lg = plain(w64, ids["a"] + [7])[-1]
+        assert int(out[0, 0]) == int(lg.argmax()) or float(lg.topk(2).values.diff().abs()) < 2 * t
+        eng.finish_request("a"); eng.finish_request("b")
+        assert eng.manager.stats()["pages_free"] == [16] and eng.manager.stats()["slots_free"] == 3
+    finally:
+        unregister("norm", "toy_centered")
+        unregister("block", "toy_parallel")
