@@ -261,17 +261,19 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
   auto compute = [&](int t, bf16x8_t (*kc)[KS], uint4* vc) {
     const int base = lo + (t << 6);
     if (RAW && has_new && t == tiles - 1) {
-      // the new key's row and the new value's row come from LDS: the cache's rows were loaded before they were written
+      // the new key's row and the new value's row come from LDS: the cache's rows were loaded before they were written.
+      // So do the places past it, which were loaded from the same row of the cache: their probabilities are zero, but
+      // what that row held before this step (anything: the page may have been another request's) must not meet them
       const int rel = pos - base;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
-        if (4 * r16 + kt == rel) {
+        if (4 * r16 + kt >= rel) {
 #pragma unroll
           for (int st = 0; st < KS; ++st) kc[kt][st] = *reinterpret_cast<const bf16x8_t*>(&knew[wave][32 * st + 8 * kg]);
         }
 #pragma unroll
       for (int i = 0; i < NI; ++i)
-        if (kq + i * KG == rel) vc[i] = *reinterpret_cast<const uint4*>(&vnew[wave][dc * 8]);
+        if (kq + i * KG >= rel) vc[i] = *reinterpret_cast<const uint4*>(&vnew[wave][dc * 8]);
     }
     // sc[kt][i]: head r16, key base + 4 (4 kg + i) + kt
     f32x4_t sc[4];

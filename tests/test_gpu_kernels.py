@@ -611,8 +611,14 @@ def test_attention_decode_from_raw_rows_equals_the_separate_kernels(ops, nh, nkv
     k1, v1, q1 = kc.clone().to(DEV), vc.clone().to(DEV), qkv.clone().to(DEV)
     ops.qknorm_rope_kv(q1, qw, kw, 1e-5, cos, sin, d, positions, seq_of, table.to(DEV), ps, k1, v1, nh, nkv, d, write_kv=write)
     want = ops.attention_decode(q1, stride, k1, v1, positions, table.to(DEV), ps, None, scale, nh, nkv, d, nseq, nsplit)
-    # all in one
+    # all in one; what the rows of the new keys and values held before (a page that was another request's, anything)
+    # must not reach the result: the kernel loads those rows before it writes them, for the places past the end too
     k2, v2 = kc.clone().to(DEV), vc.clone().to(DEV)
+    if write:
+        for i, n in enumerate(lens):
+            page, row = int(table[i, (n - 1) // ps]), (n - 1) % ps
+            k2[page, :, row] = float("nan")
+            v2[page, :, row] = float("nan")
     got = ops.attention_decode_raw(qkv.to(DEV), stride, k2, v2, positions, table.to(DEV), ps, None, scale, qw, kw, 1e-5,
                                    cos, sin, nh, nkv, d, nseq, nsplit, write_kv=write)
     assert float((got.float() - want.float()).abs().max()) <= 2e-2 * max(1.0, float(want.float().abs().max()))

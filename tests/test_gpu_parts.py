@@ -709,3 +709,118 @@ def test_a_toy_norm_and_a_toy_block_arrangement_register_build_and_step(fw, dtyp
     finally:
         unregister("norm", "toy_centered")
         unregister("block", "toy_parallel")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_model_with_a_full_and_a_windowed_attention_layer_runs_on_two_page_groups(fw, dtype):
+    """Layers with different needs keep pages of their own: one attention layer sees all keys, one only the last 10,
+    a short convolution keeps a slot.  With pages of 4 the windowed group gives pages back as the window passes them,
+    to the other request among others; what is given back is filled with NaN (``poison``), so a kernel that read a key
+    before the window, through a stale table entry or a page that now belongs to someone else, shows in the logits.
+    Whole, in portions beside another request, and through the recorded decode loop (heads of 64: the fast kernels in
+    bfloat16), against the arithmetic written out."""
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.config import AttentionSpec, BlockSpec, LayerCall, ModelSpec, RMSNormSpec, RopeSpec, ShortConvSpec, SwiGLUSpec
+    from gesso_amd.models.model import tensor_table
+    from gesso_amd.weights import random_tensors
+    from gesso_amd.weights.loader import held_dtype
+
+    H, V, eps, W = 128, 72, 1e-5, 10
+    norm = RMSNormSpec(H, eps)
+    rope = RopeSpec(head_dim=64, rotary_dim=64, theta=1e4, max_position=128)
+    full = AttentionSpec(hidden=H, n_heads=2, n_kv_heads=1, head_dim=64, position=rope, qk_norm=RMSNormSpec(64, eps))
+    near = AttentionSpec(hidden=H, n_heads=2, n_kv_heads=2, head_dim=64, position=rope, qk_norm=None, window=W)
+
+    def names(i, mixer_names, ffn=True):
+        n = {f"mixer.{k}": f"L{i}.{k}" for k in mixer_names}
+        n["mixer_norm.weight"] = f"L{i}.n1"
+        if ffn:
+            n.update({"ffn_norm.weight": f"L{i}.n2", "ffn.w1.weight": f"L{i}.w1", "ffn.w3.weight": f"L{i}.w3", "ffn.w2.weight": f"L{i}.w2"})
+        return n
+
+    proj = ["q_proj.weight", "k_proj.weight", "v_proj.weight", "out_proj.weight"]
+    blocks = (BlockSpec(full, norm, SwiGLUSpec(H, 96), norm, names(0, proj + ["q_norm.weight", "k_norm.weight"])),
+              BlockSpec(near, norm, SwiGLUSpec(H, 64), norm, names(1, proj)),
+              BlockSpec(ShortConvSpec(H, 3), norm, None, None, names(2, ["in_proj.weight", "conv.weight", "out_proj.weight"], False)))
+    spec = ModelSpec(architecture="ToyTwoGroups", hidden=H, vocab=V, blocks=blocks,
+                     schedule=(LayerCall(0), LayerCall(1), LayerCall(2)), final_norm=norm, tie_embeddings=True,
+                     max_position=128, names={"embed": "emb", "final_norm.weight": "fn"})
+
+    def attention(h, w, i, nkv, window, qk):
+        T = h.shape[0]
+        n = P.rmsnorm(h, w[f"L{i}.n1"], eps)
+        q = P.linear(n, w[f"L{i}.q_proj.weight"]).reshape(T, 2, 64)
+        k = P.linear(n, w[f"L{i}.k_proj.weight"]).reshape(T, nkv, 64)
+        v = P.linear(n, w[f"L{i}.v_proj.weight"]).reshape(T, nkv, 64)
+        if qk:
+            q, k = P.rmsnorm(q, w[f"L{i}.q_norm.weight"], eps), P.rmsnorm(k, w[f"L{i}.k_norm.weight"], eps)
+        q, k = P.rope(q, range(T), 1e4), P.rope(k, range(T), 1e4)
+        h = h + P.linear(P.causal_attention(q, k, v, window).reshape(T, H), w[f"L{i}.out_proj.weight"])
+        n = P.rmsnorm(h, w[f"L{i}.n2"], eps)
+        return h + P.linear(P.swiglu(P.linear(n, w[f"L{i}.w1"]), P.linear(n, w[f"L{i}.w3"])), w[f"L{i}.w2"])
+
+    def plain(w, ids):
+        h = attention(attention(P.embedding(w["emb"], ids), w, 0, 1, 0, True), w, 1, 2, W, False)
+        n = P.rmsnorm(h, w["L2.n1"], eps)
+        u, _ = P.short_conv(P.linear(n, w["L2.in_proj.weight"]), w["L2.conv.weight"].reshape(H, 3))
+        h = h + P.linear(u, w["L2.out_proj.weight"])
+        return P.linear(P.rmsnorm(h, w["fn"], eps), w["emb"])
+
+    table = tensor_table(spec)
+    cpu = random_tensors(table, 23, dtype, std=0.15)
+    w64 = {k: v.double() for k, v in cpu.items()}
+    eng = Engine(spec, {k: v.to(DEV, held_dtype(v.dtype, table[k].role, dtype)) for k, v in cpu.items()}, dtype, DEV,
+                 page_size=4, num_pages=32, num_slots=3, max_context=96, poison=True)
+    lay = eng.manager.layout
+    assert [g.need.window for g in lay.paged] == [None, W] and len(lay.slots) == 1
+    g = gen(31)
+    ids = {"a": torch.randint(0, V, (41,), generator=g).tolist(), "b": torch.randint(0, V, (30,), generator=g).tolist()}
+    want = {k: plain(w64, v) for k, v in ids.items()}
+    # the window matters: with all keys the last logits are far off
+    t = (3e-5 if dtype == torch.float32 else 3e-2) * max(1.0, max(float(x.abs().max()) for x in want.values()))
+    h_all = attention(attention(P.embedding(w64["emb"], ids["a"]), w64, 0, 1, 0, True), w64, 1, 2, 0, False)
+    h_win = attention(attention(P.embedding(w64["emb"], ids["a"]), w64, 0, 1, 0, True), w64, 1, 2, W, False)
+    assert float((h_all - h_win).abs().max()) > 1e-2
+
+    eng.add_request("a")
+    got = eng.step([StepEntry("a", ids["a"], list(range(41)))]).double().cpu()
+    assert float((got - want["a"]).abs().max()) <= t
+    held = [[p for p in tb if p >= 0] for tb in eng.manager.get("a").tables]
+    assert len(held[0]) == 11 and len(held[1]) <= 4          # 41 tokens: all pages of group 0, the window's of group 1
+    eng.finish_request("a")
+    # portions beside each other: what a's window leaves behind, b takes, and the other way round
+    eng.add_request("a"); eng.add_request("b")
+    cuts = {"a": [9, 1, 13, 2, 8, 8], "b": [2, 7, 1, 11, 3, 6]}
+    at = {"a": 0, "b": 0}
+    out = {"a": [], "b": []}
+    for s in range(6):
+        entries = []
+        for k in ("a", "b"):
+            n = cuts[k][s]
+            entries.append(StepEntry(k, ids[k][at[k]:at[k] + n], list(range(n))))
+            at[k] += n
+        lg = eng.step(entries).double().cpu()
+        assert bool(torch.isfinite(lg).all()), s
+        o = 0
+        for e in entries:
+            out[e.rid].append(lg[o:o + len(e.tokens)])
+            o += len(e.tokens)
+        eng.manager.check()
+    for k in ids:
+        assert float((torch.cat(out[k]) - want[k][:at[k]]).abs().max()) <= t, k
+    assert at == {"a": 41, "b": 30}
+    # the recorded loop: 20 steps from the greedy choice, past several more pages of the window
+    first = [int(want["a"][-1].argmax()), int(want["b"][-1].argmax())]
+    chosen, bad = eng.decode(["a", "b"], first, 20)
+    assert not bad.any()
+    eng.manager.check()
+    for col, k in enumerate(("a", "b")):
+        seq = ids[k] + [first[col]] + [int(x) for x in chosen[:-1, col]]
+        ref = plain(w64, seq)[len(ids[k]):]
+        for s in range(20):
+            top = ref[s].topk(2).values
+            assert int(chosen[s, col]) == int(ref[s].argmax()) or float(top[0] - top[1]) < 2 * t, (k, s)
+        assert len([p for p in eng.manager.get(k).tables[1] if p >= 0]) <= 4
+    eng.finish_request("a"); eng.finish_request("b")
+    st = eng.manager.stats()
+    assert st["pages_free"] == [32, 32] and st["slots_free"] == 3
