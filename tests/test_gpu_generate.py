@@ -15,8 +15,8 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 # the benchmark description's workloads for the two tiny configurations
-PROMPTS = {"A": (5, 17, 32), "B": (1, 9, 40, 100)}
-NEW = {"A": 16, "B": 24}
+PROMPTS = {"A": (5, 17, 32), "B": (1, 9, 40, 100), "D": (3, 22, 45, 70)}
+NEW = {"A": 16, "B": 24, "D": 20}
 
 
 @pytest.fixture(scope="module")
@@ -57,12 +57,18 @@ def test_greedy_float32_equals_plain_greedy(plain, name):
     assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
-def test_greedy_bfloat16_picks_tokens_the_plain_logits_support(folders, name):
+@pytest.mark.parametrize("name,poison", [("A", False), ("B", False), ("A", True), ("B", True), ("D", True)])
+def test_greedy_bfloat16_picks_tokens_the_plain_logits_support(folders, name, poison):
+    """With ``poison``: pages of 4, two requests at a time, so that the later requests run on pages and slots that the
+    earlier ones gave back, filled with NaN in between: the recorded decode step with its fused kernels (D: heads of
+    64, where decode attention writes the step's key itself) must not meet what a page held before."""
     from gesso_amd import Session
     d = write_tiny(folders, name, torch.bfloat16)
     cfg, w = P.read_config(d), P.read_weights(d)
-    s = Session(d, dtype="bfloat16", context_length=160)
+    if poison:
+        s = Session(d, dtype="bfloat16", context_length=160, page_size=4, max_num_seqs=2, num_pages=64, poison=True)
+    else:
+        s = Session(d, dtype="bfloat16", context_length=160)
     prompts = prompts_of(name)
     got = s.generate(prompts, max_new_tokens=NEW[name], eos_ids=())
     for p, g in zip(prompts, got):
