@@ -179,7 +179,10 @@ def test_recorded_decode_at_the_real_layer_sizes(balanced, nreq, steps):
     from gesso_amd.engine.decode import _capacity
     m = balanced
     prompts = [random_ids(n, 65536, 7000 + 13 * i + n) for i, n in enumerate(([3, 18, 33] + [4 + (5 * i) % 17 for i in range(nreq)])[:nreq])]
-    eng = Engine.from_folder(m.dir, dtype="bfloat16", page_size=16, max_tokens=64 * nreq + 256, num_slots=nreq + 1)
+    # poisoned: free pages, the scratch page and the scratch slot hold NaN, so the rows beyond the live batch (the
+    # capacity is 4, 32 and 48) compute NaN throughout, and nothing of it may reach a live row
+    eng = Engine.from_folder(m.dir, dtype="bfloat16", page_size=16, max_tokens=64 * nreq + 256, num_slots=nreq + 1,
+                             poison=True)
     seqs, toks = [list(p) for p in prompts], []
     for i, p in enumerate(prompts):
         eng.add_request(i)
