@@ -332,6 +332,37 @@ def test_non_finite_logits_fail_their_request(folders):
     assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
 
 
+@pytest.mark.parametrize("bad_at", [4, 12])
+def test_a_request_that_turns_non_finite_fails_alone_and_what_it_leaves_behind_harms_nobody(tmp_path, bad_at):
+    """One request meets a token whose embedding row is NaN (in its first portion, or in a later one, after finite
+    portions); its rows are NaN from there through every kernel, in steps it shares with the others (prompt portions of
+    8 beside decoded tokens, bfloat16, heads of 64).  It fails alone; the others, of which two run later on the pages
+    and the slot it gave back with NaN in them, produce what they produce without it."""
+    import dataclasses
+    from gesso_amd import BatchRequest, Session, run_batch
+    from gesso_amd.errors import NumericalInstability
+    from gesso_amd.weights import write_model_folder
+    from tiny import TINY_D
+    cfg = dataclasses.replace(TINY_D, tie_word_embeddings=False)
+    d = write_model_folder(str(tmp_path / "m"), cfg, seed=4, dtype=torch.bfloat16, std=STD)
+    prompts = [random_ids(n, cfg.vocab_size, 300 + n) for n in (20, 19, 33, 14)]
+    kw = dict(dtype="bfloat16", context_length=96, page_size=4, max_num_seqs=2, num_pages=40, chunk_size=8,
+              max_num_batched_tokens=12)
+    clean = Session(d, **kw)
+    want = [r.ids for r in run_batch([BatchRequest(clean, p, max_new_tokens=12) for p in prompts])]
+    used = {t for g in want for t in g}
+    nan_id = next(t for t in range(cfg.vocab_size) if t not in used)
+    s = Session(d, **kw)
+    s.engine.model.embed[nan_id] = float("nan")
+    marred = prompts[1][:bad_at] + [nan_id] + prompts[1][bad_at + 1:]
+    res = run_batch([BatchRequest(s, p, max_new_tokens=12) for p in (prompts[0], marred, prompts[2], prompts[3])])
+    assert res[1].status == "failed" and isinstance(res[1].error, NumericalInstability)
+    for i in (0, 2, 3):
+        assert res[i].status != "failed" and res[i].ids == want[i], i
+    st = s.engine.manager.stats()
+    assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+
+
 def test_random_weights_session_and_cli(tmp_path):
     from gesso_amd import Session
     s = Session(TINY_B, random_weights_seed=4, random_weights_std=STD, dtype="bfloat16", context_length=64)
