@@ -363,6 +363,32 @@ def test_a_request_that_turns_non_finite_fails_alone_and_what_it_leaves_behind_h
     assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
+def test_nothing_reads_what_nobody_wrote(folders, monkeypatch, name, dtype):
+    """Every buffer that the engine asks for without a value (``torch.empty``: activations, partial results, tiled rows
+    with their padding) starts as NaN instead of whatever the allocator held: the tokens of five requests, in portions
+    beside decoded tokens and through the recorded loop, are the same as without."""
+    from gesso_amd import Session
+    d = write_tiny(folders, name, torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    cfg, seed = CONFIGS[name]
+    prompts = [random_ids(n, cfg.vocab_size, 10 * seed + n) for n in (3, 22, 45, 70, 17)]
+    kw = dict(dtype=dtype, context_length=160, page_size=4, max_num_seqs=3, num_pages=96, chunk_size=16,
+              max_num_batched_tokens=24)
+    want = Session(d, **kw).generate(prompts, max_new_tokens=20, eos_ids=())
+    real = torch.empty
+
+    def nan_empty(*a, **k):
+        t = real(*a, **k)
+        if t.is_floating_point() and t.is_cuda:
+            t.fill_(float("nan"))
+        return t
+
+    monkeypatch.setattr(torch, "empty", nan_empty)
+    got = Session(d, **kw).generate(prompts, max_new_tokens=20, eos_ids=())
+    assert got == want
+
+
 def test_random_weights_session_and_cli(tmp_path):
     from gesso_amd import Session
     s = Session(TINY_B, random_weights_seed=4, random_weights_std=STD, dtype="bfloat16", context_length=64)
