@@ -498,7 +498,7 @@ static int launch_decode(int G, dim3 grid, hipStream_t stream, const bf16* q, in
     g_decode_cus = n;
   }
   const long blocks = (long)grid.x * grid.y * grid.z;
-  if (D <= 64 && blocks >= 2L * g_decode_cus)
+  if (D <= 64 && blocks > 1L * g_decode_cus)
     return launch_decode_w<D, RAW, 4>(G, grid, stream, q, q_stride, kc, vc, positions, bt, max_blocks, page_size, page_magic,
                                       window, scale, out, part_o, part_ml, nh, nkv, out_tiles, raw);
   return launch_decode_w<D, RAW, DEC_WAVES>(G, grid, stream, q, q_stride, kc, vc, positions, bt, max_blocks, page_size,
