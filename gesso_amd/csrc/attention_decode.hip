@@ -458,8 +458,9 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
 #define DEC_WAVES 8
 
 // Wavefronts a block: eight, so that one block covers about a thousand keys in a pass or two; four where the grid
-// alone holds two blocks and more for every compute unit (many sequences): blocks of four leave a lane's registers
-// to two blocks a compute unit, whose chains of round trips then overlap.
+// holds more blocks than the chip has compute units (many sequences): blocks of four leave a lane's registers
+// to two blocks a compute unit, whose chains of round trips then overlap (measured at 48 and at 64 sequences of
+// 8 key heads: 18.5 against 23.8 us, 21 against 27).
 template <int D, int RAW, int WV>
 static int launch_decode_w(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, bf16* kc, bf16* vc,
                          const int* positions, const int* bt, int max_blocks, int page_size, unsigned page_magic,
