@@ -99,7 +99,7 @@ __global__ void short_conv8_kernel(const T* __restrict__ bcx, const float* __res
   }
 }
 
-// Prompt portions: a thread takes eight channels and a run of TT consecutive tokens, so every B and X row is read
+// Prompt portions: a thread takes eight channels and a run of TT consecutive tokens (4 or 2, see the launch), so every B and X row is read
 // once (plus W - 1 rows of run-in), all loads of the run are issued before anything is computed, and the products
 // u = B x stay in registers for the W tokens that use them.  Sums run over the taps in the same order as in the
 // kernels above.  The first W - 1 tokens of a sequence take what they miss from the history, read where needed.
@@ -201,18 +201,27 @@ extern "C" int gs_short_conv(const void* bcx, int dtype, const float* taps, cons
   const bool vec = H % 8 == 0 && ((uintptr_t)bcx & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
                    (dtype == GS_F32 || dtype == GS_BF16);
   if (vec && !all_single && W <= 4) {
-    constexpr int TT = 8;
-    dim3 gr(gs_ceil_div(H / 8, 64), gs_ceil_div(ntok, TT));
-    GS_REQUIRE(gr.y <= 65535, "short_conv: %d tokens in one call; at most %d", ntok, 65535 * TT);
-#define GS_RUN_CONV(TY, WW)                                                                                          \
+    // runs of 4 tokens a thread, of 2 where runs of 4 would leave the chip short of wavefronts (narrow models, short
+    // portions).  Measured, bfloat16, W = 3: 2,048 tokens of 2,048 channels 10.7 us with runs of 4, 11.1 with 2, 13.6
+    // with 8; some 900 tokens of 1,024 channels 7.7 us with runs of 2, 11.5 with 4, 18.0 with 8
+    const int cols = gs_ceil_div(H / 8, 64);
+    const int tt = (long)cols * gs_ceil_div(ntok, 4) >= 2048 ? 4 : 2;
+    dim3 gr(cols, gs_ceil_div(ntok, tt));
+    GS_REQUIRE(gr.y <= 65535, "short_conv: %d tokens in one call; at most %d", ntok, 65535 * tt);
+#define GS_RUN_CONV_T(TY, WW, TT)                                                                                    \
   short_conv_run_kernel<TY, WW, TT><<<gr, 64, 0, stream>>>((const TY*)bcx, taps, bias, state, seq_of_token, q_start, \
                                                            slots, (TY*)out, ntok, H)
+#define GS_RUN_CONV(TY, WW)                                                                                          \
+  do {                                                                                                               \
+    if (tt == 4) GS_RUN_CONV_T(TY, WW, 4); else GS_RUN_CONV_T(TY, WW, 2);                                           \
+  } while (0)
     if (dtype == GS_F32) {
       if (W == 2) GS_RUN_CONV(float, 2); else if (W == 3) GS_RUN_CONV(float, 3); else GS_RUN_CONV(float, 4);
     } else {
       if (W == 2) GS_RUN_CONV(bf16, 2); else if (W == 3) GS_RUN_CONV(bf16, 3); else GS_RUN_CONV(bf16, 4);
     }
 #undef GS_RUN_CONV
+#undef GS_RUN_CONV_T
   } else if (vec) {
     int th = H / 8 >= 256 ? 256 : 64;
     dim3 g8(gs_ceil_div(H / 8, th), grid.y);

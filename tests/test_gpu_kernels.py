@@ -156,14 +156,14 @@ def test_short_conv_segments_and_history(ops, H, W, bias, dtype):
     assert torch.equal(state[1].cpu(), torch.full((H, W - 1), 7.0)) and torch.equal(state[4].cpu(), torch.full((H, W - 1), 7.0))
 
 
+@pytest.mark.parametrize("H,n", [(136, [37, 1, 2, 19, 8, 3]), (4096, [500, 1, 2, 333, 3, 190])])
 @pytest.mark.parametrize("W", [2, 3, 4])
-def test_short_conv_long_portions_beside_short_ones(ops, W):
-    """Portions longer than a thread's run of tokens, beside ones of one and two tokens, each with its own history."""
-    H = 136
+def test_short_conv_long_portions_beside_short_ones(ops, W, H, n):
+    """Portions longer than a thread's run of tokens, beside ones of one and two tokens, each with its own history;
+    few tokens of few channels (runs of two tokens a thread) and enough of both for runs of four."""
     g = gen(W)
     taps = torch.randn(H, W, generator=g)
     b = torch.randn(H, generator=g)
-    n = [37, 1, 2, 19, 8, 3]
     state0 = torch.randn(len(n) + 1, H, W - 1, generator=g)
     slots = torch.tensor([4, 0, 6, 2, 1, 5], dtype=torch.int32)
     rows = [torch.randn(k, 3 * H, generator=g).bfloat16() for k in n]
