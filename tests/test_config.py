@@ -205,3 +205,15 @@ def test_schedule_is_checked():
         dataclasses.replace(spec, schedule=(LayerCall(0, cache=0),))
     ok = dataclasses.replace(spec, schedule=(LayerCall(2), LayerCall(2), LayerCall(5, cache=0)))
     assert len(ok.schedule) == 3
+
+
+def test_the_benchmark_says_so_and_exits_with_2_when_asked_for_more_than_one_gpu():
+    """The measurement's contract: one line and exit status 2 for N > 1, before anything touches a GPU."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert p.returncode == 2
+    assert len(p.stdout.strip().splitlines()) == 1 and "one GPU" in p.stdout
