@@ -167,64 +167,6 @@ __global__ void sample_temperature_kernel(const float* __restrict__ logits, int 
   row_sample(logits + (size_t)row * V, V, temperature[row], u[row], ids + row, bad + row);
 }
 
-// The decode loop's choice, made to be recorded into a HIP graph: everything that changes from step to
-// step is read from device memory.  Row r: temperature[r] <= 0 means greedy, else a draw with
-// u[step * rows + r], step = counter[r] (each row counts its own steps, so no block waits for another).
-// The chosen id goes to next_ids[r] (the token fed back) and, with the row's flag, to
-// ring[step * rows + r] and bad_ring[...], which the host reads once per run.  Then the row moves on:
-// its counter counts up and, if the row is live, so do its position and its number of keys.
-__global__ void decode_choose_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
-                                     const double* __restrict__ u, int* __restrict__ counter,
-                                     int* __restrict__ next_ids, int* __restrict__ ring, int* __restrict__ bad_ring,
-                                     int* __restrict__ positions, int* __restrict__ kv_len,
-                                     const int* __restrict__ live, int max_steps) {
-  __shared__ int sid, sbad;
-  int row = blockIdx.x, rows = gridDim.x;
-  int step = counter[row];
-  // a counter that the host forgot to reset must not write past the rings: such a step goes to the last ring row
-  // and marks itself bad, so the run fails loudly instead of overwriting a neighbour
-  bool over = step < 0 || step >= max_steps;
-  if (over) step = max_steps - 1;
-  double T = temperature[row];
-  const float* x = logits + (size_t)row * V;
-  if (T > 0.0)
-    row_sample(x, V, T, u[(size_t)step * rows + row], &sid, &sbad);
-  else
-    row_argmax(x, V, &sid, &sbad);
-  if (threadIdx.x == 0) {
-    next_ids[row] = sid;
-    ring[(size_t)step * rows + row] = sid;
-    bad_ring[(size_t)step * rows + row] = over ? 1 : sbad;
-    counter[row] = over ? max_steps : step + 1;
-    if (live[row]) {
-      positions[row] += 1;
-      kv_len[row] += 1;
-    }
-  }
-}
-
-extern "C" int gs_decode_choose(const float* logits, int rows, int V, const double* temperature, const double* u,
-                                int* counter, int* next_ids, int* ring, int* bad_ring, int* positions, int* kv_len,
-                                const int* live, int max_steps, hipStream_t stream) {
-  GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
-  GS_REQUIRE(max_steps > 0, "decode_choose: the rings hold %d steps", max_steps);
-  GS_REQUIRE(counter && positions && kv_len && live, "decode_choose: needs the rows' counters, positions, key counts and live flags");
-  decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, counter, next_ids, ring, bad_ring,
-                                                          positions, kv_len, live, max_steps);
-  GS_LAUNCH_CHECK("decode_choose");
-  return 0;
-}
-
-
-extern "C" int gs_sample_temperature(const float* logits, int rows, int V, const double* temperature,
-                                     const double* u, int* ids, int* bad, hipStream_t stream) {
-  GS_REQUIRE(rows >= 0 && V > 0, "sample: bad sizes rows=%d V=%d", rows, V);
-  if (rows == 0) return 0;
-  sample_temperature_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, ids, bad);
-  GS_LAUNCH_CHECK("sample_temperature");
-  return 0;
-}
-
 // ------------------------------------------------------------------ nucleus (top-p) sampling
 //
 // The reference orders ids by weight, descending and stable (ties keep id order), keeps the
@@ -266,13 +208,31 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
     // the largest weight this pass can meet: 1 (the row's maximum has weight exp(0)) or the largest pattern under the prefix
     const double wmax = pass == 0 ? 1.0 : __longlong_as_double((long long)(prefix | ((1ull << (shift + 8)) - 1ull)));
     const double scale = exp2((double)(62 - lv)) / wmax, unscale = 1.0 / scale;
+    // a thread adds up what falls into one bucket in a row before it goes to the histogram: in the first passes (sign,
+    // exponent) nearly every weight of the row shares a bucket, and one atomic add per weight on one address would
+    // queue up; the sums are integers, so neither this nor the order of the adds changes them
+    int run_b = -1, run_n = 0;
+    unsigned long long run_m = 0ull;
     for (int j = threadIdx.x; j < V; j += blockDim.x) {
       unsigned long long bits = (unsigned long long)__double_as_longlong(w[j]);
       if ((bits & himask) == prefix) {
         int b = (int)((bits >> shift) & 0xff);
-        atomicAdd(&hmass[b], (unsigned long long)__double2ll_rn(w[j] * scale));
-        atomicAdd(&hcount[b], 1);
+        if (b != run_b) {
+          if (run_n) {
+            atomicAdd(&hmass[run_b], run_m);
+            atomicAdd(&hcount[run_b], run_n);
+          }
+          run_b = b;
+          run_m = 0ull;
+          run_n = 0;
+        }
+        run_m += (unsigned long long)__double2ll_rn(w[j] * scale);
+        run_n += 1;
       }
+    }
+    if (run_n) {
+      atomicAdd(&hmass[run_b], run_m);
+      atomicAdd(&hcount[run_b], run_n);
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -306,9 +266,10 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
   return c;
 }
 
-__global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
-                                    const double* __restrict__ top_p, const double* __restrict__ u,
-                                    double* __restrict__ wbuf, int* __restrict__ ids, int* __restrict__ bad) {
+// One row by the whole block: T > 0, P in (0, 1), u in [0, 1); w: V float64 of scratch; thread 0 returns (id, bad)
+// through the pointers.
+__device__ void row_sample_top_p(const float* __restrict__ x, int V, double T, double P, double uu,
+                                 double* __restrict__ w, int* id_out, int* bad_out) {
   __shared__ unsigned long long hmass[256];
   __shared__ int hcount[256];
   __shared__ Crossing cross;
@@ -316,9 +277,6 @@ __global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, con
   __shared__ double redd[SAMP_THREADS / 64];
   __shared__ int bbad;
   __shared__ int tie_before[SAMP_THREADS];
-  int row = blockIdx.x;
-  const float* x = logits + (size_t)row * V;
-  double* w = wbuf + (size_t)row * V;
   int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
   if (tid == 0) bbad = 0;
   __syncthreads();
@@ -337,12 +295,12 @@ __global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, con
   for (int i = 1; i < nw; ++i) mx = fmaxf(mx, redf[i]);
   if (bbad) {
     if (tid == 0) {
-      ids[row] = 0;
-      bad[row] = 1;
+      *id_out = 0;
+      *bad_out = 1;
     }
     return;
   }
-  double hi = (double)mx, T = temperature[row];
+  double hi = (double)mx;
   double s = 0.0;
   for (int j = tid; j < V; j += blockDim.x) {
     double wj = exp(((double)x[j] - hi) / T);
@@ -357,7 +315,7 @@ __global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, con
   __syncthreads();
 
   // the nucleus' edge: weight tau at which the sorted running sum reaches top_p * total
-  double target = top_p[row] * total;
+  double target = P * total;
   Crossing edge = radix_descend(w, V, target, 0, hmass, hcount, &cross);
   double tau = __longlong_as_double((long long)edge.bits);
   // ties at tau that belong to the nucleus: added one by one until the sum reaches the target
@@ -367,7 +325,7 @@ __global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, con
   double cut = edge.above + (double)ties_kept * tau;
 
   // the draw: first running sum above r = u * cut, in the same order
-  double r = u[row] * cut;
+  double r = uu * cut;
   Crossing hit = radix_descend(w, V, r, 1, hmass, hcount, &cross);
   double wv = __longlong_as_double((long long)hit.bits);
   long long k = wv > 0.0 ? (long long)floor((r - hit.above) / wv) : 0;  // 0-based tie in id order
@@ -404,9 +362,83 @@ __global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, con
           ++seen;
         }
     }
-    ids[row] = pick >= 0 ? pick : (last >= 0 ? last : 0);
-    bad[row] = 0;
+    *id_out = pick >= 0 ? pick : (last >= 0 ? last : 0);
+    *bad_out = 0;
   }
+}
+
+__global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
+                                    const double* __restrict__ top_p, const double* __restrict__ u,
+                                    double* __restrict__ wbuf, int* __restrict__ ids, int* __restrict__ bad) {
+  int row = blockIdx.x;
+  row_sample_top_p(logits + (size_t)row * V, V, temperature[row], top_p[row], u[row], wbuf + (size_t)row * V, ids + row,
+                   bad + row);
+}
+
+
+// The decode loop's choice, made to be recorded into a HIP graph: everything that changes from step to
+// step is read from device memory.  Row r: temperature[r] <= 0 means greedy, else a draw with
+// u[step * rows + r], step = counter[r] (each row counts its own steps, so no block waits for another), from the
+// whole row or, with top_p[r] < 1, from its nucleus (wbuf: rows x V float64 of scratch for the weights).
+// The chosen id goes to next_ids[r] (the token fed back) and, with the row's flag, to
+// ring[step * rows + r] and bad_ring[...], which the host reads once per run.  Then the row moves on:
+// its counter counts up and, if the row is live, so do its position and its number of keys.
+__global__ void decode_choose_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
+                                     const double* __restrict__ top_p, double* __restrict__ wbuf,
+                                     const double* __restrict__ u, int* __restrict__ counter,
+                                     int* __restrict__ next_ids, int* __restrict__ ring, int* __restrict__ bad_ring,
+                                     int* __restrict__ positions, int* __restrict__ kv_len,
+                                     const int* __restrict__ live, int max_steps) {
+  __shared__ int sid, sbad;
+  int row = blockIdx.x, rows = gridDim.x;
+  int step = counter[row];
+  // a counter that the host forgot to reset must not write past the rings: such a step goes to the last ring row
+  // and marks itself bad, so the run fails loudly instead of overwriting a neighbour
+  bool over = step < 0 || step >= max_steps;
+  if (over) step = max_steps - 1;
+  double T = temperature[row];
+  const float* x = logits + (size_t)row * V;
+  const double P = top_p ? top_p[row] : 1.0;
+  if (T > 0.0 && P < 1.0)
+    row_sample_top_p(x, V, T, P, u[(size_t)step * rows + row], wbuf + (size_t)row * V, &sid, &sbad);
+  else if (T > 0.0)
+    row_sample(x, V, T, u[(size_t)step * rows + row], &sid, &sbad);
+  else
+    row_argmax(x, V, &sid, &sbad);
+  if (threadIdx.x == 0) {
+    next_ids[row] = sid;
+    ring[(size_t)step * rows + row] = sid;
+    bad_ring[(size_t)step * rows + row] = over ? 1 : sbad;
+    counter[row] = over ? max_steps : step + 1;
+    if (live[row]) {
+      positions[row] += 1;
+      kv_len[row] += 1;
+    }
+  }
+}
+
+// top_p (rows) and wbuf (rows x V float64) come together or not at all (then every draw is from the whole row).
+extern "C" int gs_decode_choose(const float* logits, int rows, int V, const double* temperature, const double* top_p,
+                                double* wbuf, const double* u, int* counter, int* next_ids, int* ring, int* bad_ring,
+                                int* positions, int* kv_len, const int* live, int max_steps, hipStream_t stream) {
+  GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
+  GS_REQUIRE(max_steps > 0, "decode_choose: the rings hold %d steps", max_steps);
+  GS_REQUIRE(counter && positions && kv_len && live, "decode_choose: needs the rows' counters, positions, key counts and live flags");
+  GS_REQUIRE((top_p == nullptr) == (wbuf == nullptr), "decode_choose: top_p and its scratch come together");
+  decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, wbuf, u, counter, next_ids, ring,
+                                                          bad_ring, positions, kv_len, live, max_steps);
+  GS_LAUNCH_CHECK("decode_choose");
+  return 0;
+}
+
+
+extern "C" int gs_sample_temperature(const float* logits, int rows, int V, const double* temperature,
+                                     const double* u, int* ids, int* bad, hipStream_t stream) {
+  GS_REQUIRE(rows >= 0 && V > 0, "sample: bad sizes rows=%d V=%d", rows, V);
+  if (rows == 0) return 0;
+  sample_temperature_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, ids, bad);
+  GS_LAUNCH_CHECK("sample_temperature");
+  return 0;
 }
 
 extern "C" int gs_sample_top_p(const float* logits, int rows, int V, const double* temperature, const double* top_p,

@@ -70,6 +70,8 @@ class DecodeRunner:
         self.q_start = torch.arange(cap + 1, **i32)
         self.block_tables = [torch.full((cap, self.max_blocks), n, **i32) for n in st.num_pages]
         self.temperature = torch.zeros(cap, dtype=torch.float64, device=dev)
+        self.top_p = torch.ones(cap, dtype=torch.float64, device=dev)
+        self.weights = engine.nucleus_scratch()      # float64, DECODE_MAX_BATCH x vocabulary: shared by all capacities
         self.u = torch.zeros((self.MAX_STEPS, cap), dtype=torch.float64, device=dev)
         self.counter = torch.zeros(cap, **i32)          # steps made since the host last looked, per row
         self.ring = torch.zeros((self.MAX_STEPS, cap), **i32)
@@ -90,7 +92,7 @@ class DecodeRunner:
         self.logits = logits
         with rt.stage("sample"):
             ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring,
-                              self.pos, self.kv_len, self.live)
+                              self.pos, self.kv_len, self.live, top_p=self.top_p, wbuf=self.weights)
 
     def _bound(self, longest: int) -> int:
         """The recording that serves contexts of up to ``longest`` tokens: 1024, 2048, 4096, ... tokens."""
@@ -106,6 +108,7 @@ class DecodeRunner:
         # leaves the counters at MAX_STEPS, one row past the rings): both start from zero here
         self.counter.zero_()
         self.temperature.zero_()
+        self.top_p.fill_(1.0)
         side = torch.cuda.Stream(device=self.engine.device)
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -187,21 +190,22 @@ class DecodeRunner:
                 row[row < 0] = st.num_pages[g]
                 tab[i, :len(row)] = row
             bt[:, :width].copy_(torch.from_numpy(tab).pin_memory().to(eng.device, non_blocking=True))
-        temp = np.zeros(cap, dtype=np.float64)
+        temp = np.zeros((2, cap), dtype=np.float64)          # temperatures, then top_p (1: the whole row)
+        temp[1] = 1.0
         before = {}               # row -> the sampler's state before each of its draws
         if samplers is not None and any(s is not None for s in samplers):
             u = np.zeros((n, cap), dtype=np.float64)
             for i, s in enumerate(samplers):
                 if s is not None:
-                    if s.top_p < 1:
-                        raise InvalidPlan("nucleus sampling does not run in the recorded decode loop")
-                    temp[i] = s.temperature
+                    temp[0, i] = s.temperature
+                    temp[1, i] = s.top_p
                     before[i] = []
                     for k in range(n):
                         before[i].append(s.state)
                         u[k, i] = s.unit()
             self.u[:n].copy_(torch.from_numpy(u).pin_memory().to(eng.device, non_blocking=True))
-        self.temperature.copy_(torch.from_numpy(temp).pin_memory().to(eng.device, non_blocking=True))
+        tp = torch.from_numpy(temp).pin_memory().to(eng.device, non_blocking=True)
+        self.temperature.copy_(tp[0]); self.top_p.copy_(tp[1])
         self.counter.zero_()
         profile = eng.rt.profile
         if profile is None:

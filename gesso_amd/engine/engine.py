@@ -173,16 +173,14 @@ class Engine:
 
         ``tokens``: each request's next input token; the tokens chosen are fed back on the device.
         ``samplers``: per request None (greedy) or a :class:`~gesso_amd.sampling.sampler.Sampler`
-        without nucleus.  Returns ``(ids, bad)`` as ``(n, batch)`` arrays; a row of ``bad`` marks a step
-        whose logits were not finite.  Raises :class:`~gesso_amd.errors.OutOfPages` before changing anything.
+        (temperature, with or without a nucleus).  Returns ``(ids, bad)`` as ``(n, batch)`` arrays; a row of
+        ``bad`` marks a step whose logits were not finite.  Raises :class:`~gesso_amd.errors.OutOfPages` before changing anything.
         """
         from .decode import DecodeRunner, _capacity
         if not 1 <= len(rids) <= self.DECODE_MAX_BATCH:
             raise InvalidPlan(f"the recorded decode loop takes 1 to {self.DECODE_MAX_BATCH} requests, not {len(rids)}")
         if len(set(rids)) != len(rids) or len(tokens) != len(rids):
             raise InvalidPlan("one token per request, each request once")
-        if samplers is not None and any(s is not None and s.top_p < 1 for s in samplers):
-            raise InvalidPlan("nucleus sampling does not run in the recorded decode loop")
         if not self.model.graph_safe:
             return self._decode_eager(rids, tokens, n, samplers)
         cap = _capacity(len(rids))
@@ -190,6 +188,14 @@ class Engine:
         if runner is None:
             runner = self._runners[cap] = DecodeRunner(self, cap)
         return runner.run(rids, tokens, n, samplers)
+
+    def nucleus_scratch(self) -> torch.Tensor:
+        """Float64 room for the weights of ``DECODE_MAX_BATCH`` rows of logits: what the recorded loop's choice needs
+        for draws from a nucleus; one per engine, made with the first recorded loop."""
+        if getattr(self, "_nucleus_scratch", None) is None:
+            self._nucleus_scratch = torch.empty(self.DECODE_MAX_BATCH * self.spec.vocab, dtype=torch.float64,
+                                                device=self.device)
+        return self._nucleus_scratch
 
     def _decode_eager(self, rids, tokens, n, samplers):
         """The same steps one by one through :meth:`step`, for models with parts that cannot be recorded."""

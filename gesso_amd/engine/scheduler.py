@@ -314,8 +314,6 @@ class Scheduler:
         if not all(s.count == 1 and s.samples for s in plan):
             return None
         reqs = [s.request for s in plan]
-        if any(r.sampler is not None and r.sampler.top_p < 1 for r in reqs):
-            return None
         n = min(self.decode_run_steps, min(r.max_new_tokens - len(r.output) for r in reqs))
         if self.waiting:
             n = 1                     # someone waits: look at admission again after every step

@@ -639,11 +639,13 @@ def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None, tiled: bool = F
     return out
 
 
-def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live) -> None:
-    """Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``; results into the loop's buffers;
-    then the row's counter counts up and a live row moves one position on.  A counter at or beyond the rings' step
-    count writes into their last row and marks the step bad."""
-    _dev(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live)
+def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p=None,
+                  wbuf=None) -> None:
+    """Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``, from the whole row or, where
+    ``top_p[row] < 1``, from its nucleus (``wbuf``: float64 scratch of at least ``rows * V``); results into the loop's
+    buffers; then the row's counter counts up and a live row moves one position on.  A counter at or beyond the rings'
+    step count writes into their last row and marks the step bad."""
+    _dev(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p, wbuf)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "decode_choose: logits are float32 (rows, V)")
     rows, V = logits.shape
     _need(temperature.dtype == torch.float64 and temperature.numel() == rows, "decode_choose: temperature float64 (rows,)")
@@ -653,7 +655,12 @@ def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, pos
     for t in (ring, bad_ring):
         _i32(t)
     _need(ring.shape == u.shape and bad_ring.shape == u.shape, "decode_choose: buffer shapes")
-    _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(u), _p(counter), _p(next_ids),
+    _need((top_p is None) == (wbuf is None), "decode_choose: top_p and its scratch come together")
+    if top_p is not None:
+        _need(top_p.dtype == torch.float64 and top_p.numel() == rows, "decode_choose: top_p float64 (rows,)")
+        _need(wbuf.dtype == torch.float64 and wbuf.numel() >= rows * V, "decode_choose: wbuf float64, rows * V at least")
+    _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(u),
+                                  _p(counter), _p(next_ids),
                                   _p(ring), _p(bad_ring), _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]),
                                   _stream()))
 

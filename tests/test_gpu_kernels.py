@@ -452,6 +452,44 @@ def test_sample_top_p_gives_the_same_id_every_time_and_at_the_models_vocabulary(
         assert first[r].item() == P.sample_id(logits[r].tolist(), 0.9, 0.73, 40 + r)[0], r
 
 
+def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_side(ops):
+    """The kernel that the recorded decode step ends with: rows that are greedy, rows that draw from the whole row and
+    rows that draw from a nucleus, each with its own draw per step; ids against the plain sampler's, the rows' steps,
+    positions and key counts advanced, a non-finite row marked."""
+    V, rows, steps = 777, 6, 3
+    logits = torch.randn(rows, V, generator=gen(5)) * 2
+    logits[5, 13] = float("inf")
+    temp = [0.0, 0.8, 0.8, 1.3, 0.0, 0.9]
+    top_p = [1.0, 1.0, 0.6, 0.2, 0.5, 0.7]              # a greedy row ignores its top_p
+    states = [[900 + r] for r in range(rows)]                # the plain sampler's generator, one step a draw
+    u = torch.zeros(steps, rows, dtype=torch.float64)
+    for r in range(rows):
+        for step in range(steps):
+            nxt_state, u[step, r] = P.splitmix64_unit(states[r][-1])
+            states[r].append(nxt_state)
+    dev = lambda t: t.to(DEV)
+    i32 = lambda *a: torch.tensor(*a, dtype=torch.int32, device=DEV)
+    counter, nxt = i32([0] * rows), i32([0] * rows)
+    ring, bad = torch.full((steps, rows), -1, dtype=torch.int32, device=DEV), torch.full((steps, rows), -1, dtype=torch.int32, device=DEV)
+    pos, kv, live = i32([10, 11, 12, 13, 14, 15]), i32([11, 12, 13, 14, 15, 16]), i32([1, 1, 1, 0, 1, 1])
+    wbuf = torch.full((rows * V,), float("nan"), dtype=torch.float64, device=DEV)
+    for step in range(steps):
+        ops.decode_choose(dev(logits), dev(torch.tensor(temp, dtype=torch.float64)), dev(u), counter, nxt, ring, bad, pos, kv,
+                          live, top_p=dev(torch.tensor(top_p, dtype=torch.float64)), wbuf=wbuf)
+    assert counter.tolist() == [steps] * rows
+    assert pos.tolist() == [13, 14, 15, 13, 17, 18] and kv.tolist() == [14, 15, 16, 14, 18, 19]     # row 3 is not live
+    assert bad[:, :5].sum().item() == 0 and bad[:, 5].tolist() == [1] * steps
+    got = ring.cpu()
+    for step in range(steps):
+        for r in range(5):
+            if temp[r] <= 0:
+                want = int(logits[r].argmax())
+            else:
+                want = P.sample_id(logits[r].tolist(), temp[r], top_p[r], states[r][step])[0]
+            assert int(got[step, r]) == want, (step, r)
+    assert nxt.tolist()[:5] == got[steps - 1].tolist()[:5]
+
+
 # ------------------------------------------------------------------ the weight-streaming product
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])

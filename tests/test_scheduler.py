@@ -305,7 +305,7 @@ def test_while_someone_waits_runs_are_single_steps():
     assert any(n > 1 for rids, n in eng.runs if rids == ["b"])
 
 
-def test_runs_shrink_to_the_pages_that_are_left_and_nucleus_requests_step_singly():
+def test_runs_shrink_to_the_pages_that_are_left_and_nucleus_requests_run_like_the_others():
     eng, s = make(FakeDecodeEngine(num_pages=3, page_size=4), decode_run_steps=8)
     a = s.add(Request("a", [1, 2, 3], max_new_tokens=8))
     s.run()
@@ -313,7 +313,7 @@ def test_runs_shrink_to_the_pages_that_are_left_and_nucleus_requests_step_singly
     eng2, s2 = make(FakeDecodeEngine(), decode_run_steps=8)
     c = s2.add(Request("c", [1, 2, 3], max_new_tokens=5, sampler=Sampler(0.9, 0.5, 3)))
     s2.run()
-    assert c.tokens == expected([1, 2, 3], 5) and eng2.runs == []
+    assert c.tokens == expected([1, 2, 3], 5) and eng2.runs and eng2.runs[0][1] > 1
 
 
 def test_a_request_that_outgrows_the_context_fails_alone_and_keeps_its_tokens():
