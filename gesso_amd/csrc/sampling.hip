@@ -191,12 +191,20 @@ struct Crossing {
 };
 
 // strict = 0: first running sum >= target; strict = 1: first running sum > target.
+//
+// The first passes read the whole row.  Once a pass has narrowed the candidates down to NUC_LIST or fewer (after its
+// second byte the weights left lie within a few percent of each other, a handful in a peaked row), their ids are
+// gathered into a list in LDS and the later passes read only those.
+#define NUC_LIST 2048
 __device__ Crossing radix_descend(const double* __restrict__ w, int V, double target, int strict,
                                   unsigned long long* hmass, int* hcount, Crossing* shared_out) {
+  __shared__ int clist[NUC_LIST];
+  __shared__ int cn, picked;
   unsigned long long prefix = 0;
   double above = 0.0;
   int lv = 1;                                   // V <= 2^lv
   while ((1 << lv) < V && lv < 30) ++lv;
+  int nlist = -1;                               // ids in the list, or -1: no list yet
   for (int pass = 0; pass < 8; ++pass) {
     int shift = 56 - 8 * pass;
     for (int b = threadIdx.x; b < 256; b += blockDim.x) {
@@ -213,7 +221,9 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
     // queue up; the sums are integers, so neither this nor the order of the adds changes them
     int run_b = -1, run_n = 0;
     unsigned long long run_m = 0ull;
-    for (int j = threadIdx.x; j < V; j += blockDim.x) {
+    const int n = nlist >= 0 ? nlist : V;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const int j = nlist >= 0 ? clist[i] : i;
       unsigned long long bits = (unsigned long long)__double_as_longlong(w[j]);
       if ((bits & himask) == prefix) {
         int b = (int)((bits >> shift) & 0xff);
@@ -254,11 +264,21 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
       }
       shared_out->bits = prefix | ((unsigned long long)pick << shift);
       shared_out->above = acc;
+      picked = hcount[pick];
+      cn = 0;
     }
     __syncthreads();
     prefix = shared_out->bits;
     above = shared_out->above;
+    const int left = picked;
     __syncthreads();
+    if (nlist < 0 && pass >= 1 && pass <= 5 && left <= NUC_LIST) {
+      const unsigned long long sofar = (~0ull) << shift;
+      for (int j = threadIdx.x; j < V; j += blockDim.x)
+        if (((unsigned long long)__double_as_longlong(w[j]) & sofar) == prefix) clist[atomicAdd(&cn, 1)] = j;
+      __syncthreads();
+      nlist = cn;
+    }
   }
   Crossing c;
   c.bits = prefix;
@@ -431,6 +451,161 @@ extern "C" int gs_decode_choose(const float* logits, int rows, int V, const doub
   return 0;
 }
 
+
+// ------------------------------------------------------------------ the decode loop's choice when rows draw
+//
+// One block a row weighs 65,536 logits in float64 in some 40 us (a compute unit's float64 rate), and a step of a few
+// rows leaves the rest of the chip idle meanwhile.  So when rows draw, the choice is three kernels: the rows' first
+// maxima (and whether they are finite); the weights exp((x - max) / T) by many blocks a row, each thread the sum of
+// four consecutive ids; then one block a row that finds where the running sum of those sums, in id order, crosses
+// u * total, and walks the four ids there.  Greedy rows take their maximum's id; rows that draw from a nucleus go on
+// from the same weights.  part: rows x nparts float64, nparts = gs_choice_parts(V).
+#define WIDE_CH 4
+#define WIDE_SPAN (SAMP_THREADS * WIDE_CH)
+
+extern "C" int gs_choice_parts(int V) { return ((V + WIDE_SPAN - 1) / WIDE_SPAN) * SAMP_THREADS; }
+
+__global__ __launch_bounds__(SAMP_THREADS) void choose_weights_kernel(
+    const float* __restrict__ logits, int V, const double* __restrict__ temperature, const double* __restrict__ top_p,
+    const int* __restrict__ amax, const int* __restrict__ bad0, double* __restrict__ wbuf, double* __restrict__ part,
+    int nparts) {
+  const int row = blockIdx.y;
+  const double T = temperature[row];
+  if (!(T > 0.0) || bad0[row]) return;
+  const float* x = logits + (size_t)row * V;
+  const double hi = (double)x[amax[row]];
+  const int j0 = blockIdx.x * WIDE_SPAN + threadIdx.x * WIDE_CH;
+  float xv[WIDE_CH];
+  if (j0 + WIDE_CH <= V && ((reinterpret_cast<uintptr_t>(x + j0) & 15) == 0)) {
+    const float4 v = *reinterpret_cast<const float4*>(x + j0);
+    xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+  } else {
+#pragma unroll
+    for (int k = 0; k < WIDE_CH; ++k) xv[k] = j0 + k < V ? x[j0 + k] : -INFINITY;
+  }
+  double w[WIDE_CH], p = 0.0;
+#pragma unroll
+  for (int k = 0; k < WIDE_CH; ++k) {
+    w[k] = j0 + k < V ? exp(((double)xv[k] - hi) / T) : 0.0;
+    p += w[k];
+  }
+  part[(size_t)row * nparts + blockIdx.x * SAMP_THREADS + threadIdx.x] = p;
+  if (wbuf && top_p && top_p[row] < 1.0) {
+#pragma unroll
+    for (int k = 0; k < WIDE_CH; ++k)
+      if (j0 + k < V) wbuf[(size_t)row * V + j0 + k] = w[k];
+  }
+}
+
+__global__ __launch_bounds__(SAMP_THREADS) void choose_pick_kernel(
+    const float* __restrict__ logits, int V, const double* __restrict__ temperature, const double* __restrict__ top_p,
+    double* __restrict__ wbuf, const double* __restrict__ part, int nparts, const int* __restrict__ amax,
+    const int* __restrict__ bad0, const double* __restrict__ u, int* __restrict__ counter, int* __restrict__ next_ids,
+    int* __restrict__ ring, int* __restrict__ bad_ring, int* __restrict__ positions, int* __restrict__ kv_len,
+    const int* __restrict__ live, int max_steps) {
+  __shared__ int sid, sbad, first_t;
+  __shared__ double scan[SAMP_THREADS];
+  const int row = blockIdx.x, rows = gridDim.x, tid = threadIdx.x;
+  int step = counter[row];
+  const bool over = step < 0 || step >= max_steps;
+  if (over) step = max_steps - 1;
+  const double T = temperature[row];
+  const float* x = logits + (size_t)row * V;
+  const double P = top_p ? top_p[row] : 1.0;
+  const double uu = u[(size_t)step * rows + row];
+  if (bad0[row] || !(T > 0.0)) {
+    if (tid == 0) {
+      sid = bad0[row] ? 0 : amax[row];
+      sbad = bad0[row];
+    }
+  } else if (P < 1.0) {
+    row_sample_top_p(x, V, T, P, uu, wbuf + (size_t)row * V, &sid, &sbad);
+  } else {
+    const double* pr = part + (size_t)row * nparts;
+    const int per = nparts / SAMP_THREADS;
+    double ls = 0.0;
+    for (int i = 0; i < per; ++i) ls += pr[tid * per + i];
+    scan[tid] = ls;
+    if (tid == 0) first_t = SAMP_THREADS;
+    __syncthreads();
+    for (int off = 1; off < SAMP_THREADS; off <<= 1) {     // running sums over the threads, in id order
+      const double v = tid >= off ? scan[tid - off] : 0.0;
+      __syncthreads();
+      scan[tid] += v;
+      __syncthreads();
+    }
+    const double r = uu * scan[SAMP_THREADS - 1];
+    if (r < scan[tid]) atomicMin(&first_t, tid);
+    __syncthreads();
+    const int ft = first_t;
+    if (ft == SAMP_THREADS) {
+      if (tid == 0) {
+        sid = V - 1;
+        sbad = 0;
+      }
+    } else if (tid == ft) {
+      const double hi = (double)x[amax[row]];
+      double acc = tid ? scan[tid - 1] : 0.0;
+      int pick = -1, last = V - 1;
+      for (int i = 0; i < per && pick < 0; ++i) {
+        const int q = tid * per + i;
+        const double pq = pr[q];
+        const int j0 = (q / SAMP_THREADS) * WIDE_SPAN + (q % SAMP_THREADS) * WIDE_CH;
+        if (j0 >= V) break;
+        if (r < acc + pq) {
+          double a2 = acc;
+          for (int k = 0; k < WIDE_CH && j0 + k < V; ++k) {
+            a2 += exp(((double)x[j0 + k] - hi) / T);
+            last = j0 + k;
+            if (r < a2) {
+              pick = j0 + k;
+              break;
+            }
+          }
+          if (pick < 0) pick = last;      // the sum of the four, added on its own, lay a rounding above their running sum
+        }
+        acc += pq;
+      }
+      sid = pick >= 0 ? pick : V - 1;
+      sbad = 0;
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    next_ids[row] = sid;
+    ring[(size_t)step * rows + row] = sid;
+    bad_ring[(size_t)step * rows + row] = over ? 1 : sbad;
+    counter[row] = over ? max_steps : step + 1;
+    if (live[row]) {
+      positions[row] += 1;
+      kv_len[row] += 1;
+    }
+  }
+}
+
+// The decode loop's choice in three kernels, for steps in which rows draw (what gs_decode_choose does in one).
+// amax, bad0: rows int32 each; part: rows x gs_choice_parts(V) float64; top_p and wbuf as in gs_decode_choose.
+extern "C" int gs_decode_choose_wide(const float* logits, int rows, int V, const double* temperature, const double* top_p,
+                                     double* wbuf, double* part, int* amax, int* bad0, const double* u, int* counter,
+                                     int* next_ids, int* ring, int* bad_ring, int* positions, int* kv_len, const int* live,
+                                     int max_steps, hipStream_t stream) {
+  GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
+  GS_REQUIRE(max_steps > 0, "decode_choose: the rings hold %d steps", max_steps);
+  GS_REQUIRE(counter && positions && kv_len && live && part && amax && bad0,
+             "decode_choose: needs the rows' counters, positions, key counts, live flags and scratch");
+  GS_REQUIRE((top_p == nullptr) == (wbuf == nullptr), "decode_choose: top_p and its scratch come together");
+  GS_REQUIRE(rows <= 65535, "decode_choose: %d rows in one call", rows);
+  const int nparts = gs_choice_parts(V);
+  argmax_rows_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, amax, bad0);
+  GS_LAUNCH_CHECK("decode_choose (maxima)");
+  choose_weights_kernel<<<dim3(nparts / SAMP_THREADS, rows), SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, amax,
+                                                                                        bad0, wbuf, part, nparts);
+  GS_LAUNCH_CHECK("decode_choose (weights)");
+  choose_pick_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, wbuf, part, nparts, amax, bad0, u,
+                                                        counter, next_ids, ring, bad_ring, positions, kv_len, live, max_steps);
+  GS_LAUNCH_CHECK("decode_choose (pick)");
+  return 0;
+}
 
 extern "C" int gs_sample_temperature(const float* logits, int rows, int V, const double* temperature,
                                      const double* u, int* ids, int* bad, hipStream_t stream) {

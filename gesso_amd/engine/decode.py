@@ -71,14 +71,16 @@ class DecodeRunner:
         self.block_tables = [torch.full((cap, self.max_blocks), n, **i32) for n in st.num_pages]
         self.temperature = torch.zeros(cap, dtype=torch.float64, device=dev)
         self.top_p = torch.ones(cap, dtype=torch.float64, device=dev)
-        self.weights = engine.nucleus_scratch()      # float64, DECODE_MAX_BATCH x vocabulary: shared by all capacities
+        self.weights, self.wide = engine.choice_scratch()      # shared by all capacities
         self.u = torch.zeros((self.MAX_STEPS, cap), dtype=torch.float64, device=dev)
         self.counter = torch.zeros(cap, **i32)          # steps made since the host last looked, per row
         self.ring = torch.zeros((self.MAX_STEPS, cap), **i32)
         self.bad_ring = torch.zeros((self.MAX_STEPS, cap), **i32)
         self.ctx = DecodeContext(self)
-        # one recording per bound on the context length: launch shapes (how attention splits its keys) depend on it
-        self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
+        # one recording per bound on the context length (launch shapes, how attention splits its keys, depend on it)
+        # and per kind of choice: all rows greedy (one kernel), or some rows draw (three, the weights by many blocks)
+        self.graphs: Dict[Tuple[int, bool], torch.cuda.CUDAGraph] = {}
+        self.draws = False
 
     def _body(self) -> None:
         ops = self.engine.rt.ops
@@ -92,7 +94,8 @@ class DecodeRunner:
         self.logits = logits
         with rt.stage("sample"):
             ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring,
-                              self.pos, self.kv_len, self.live, top_p=self.top_p, wbuf=self.weights)
+                              self.pos, self.kv_len, self.live, top_p=self.top_p, wbuf=self.weights,
+                              wide=self.wide if self.draws else None)
 
     def _bound(self, longest: int) -> int:
         """The recording that serves contexts of up to ``longest`` tokens: 1024, 2048, 4096, ... tokens."""
@@ -101,9 +104,10 @@ class DecodeRunner:
             b *= 2
         return b
 
-    def _record(self, bound: int) -> None:
+    def _record(self, bound: int, draws: bool) -> None:
         """One eager run on scratch rows (everything lazily initialised gets initialised), then the capture."""
         self.ctx.max_kv_len = bound
+        self.draws = draws
         # the eager run reads the rows' counters and temperatures as the last run left them (a run of MAX_STEPS steps
         # leaves the counters at MAX_STEPS, one row past the rings): both start from zero here
         self.counter.zero_()
@@ -127,7 +131,7 @@ class DecodeRunner:
         finally:
             if collecting:
                 gc.enable()
-        self.graphs[bound] = graph
+        self.graphs[(bound, draws)] = graph
 
     def run(self, rids: Sequence[Hashable], tokens: Sequence[int], n: int, samplers=None
             ) -> Tuple[np.ndarray, np.ndarray]:
@@ -142,7 +146,8 @@ class DecodeRunner:
         mgr, st = eng.manager, eng.storage
         rcs = [mgr.get(r) for r in rids]
         bound = self._bound(max(rc.length for rc in rcs) + n)
-        if bound not in self.graphs:
+        draws = samplers is not None and any(s is not None for s in samplers)
+        if (bound, draws) not in self.graphs:
             # before any live row is set: the eager run sees scratch rows only
             self.slots.fill_(st.scratch_slot)
             self.live.zero_()
@@ -150,8 +155,8 @@ class DecodeRunner:
             self.kv_len.fill_(1)
             for g, bt in enumerate(self.block_tables):
                 bt.fill_(st.num_pages[g])
-            self._record(bound)
-        graph = self.graphs[bound]
+            self._record(bound, draws)
+        graph = self.graphs[(bound, draws)]
         for t in tokens:
             if not 0 <= int(t) < eng.spec.vocab:
                 raise InvalidPlan(f"token id {int(t)} outside the vocabulary of {eng.spec.vocab}")
@@ -214,6 +219,7 @@ class DecodeRunner:
         else:
             # profiled: the same step, launched kernel by kernel, with a pair of events around every stage
             self.ctx.max_kv_len = self._bound(max(rc.length for rc in rcs) + n)
+            self.draws = samplers is not None and any(s is not None for s in samplers)
             profile.window = True
             try:
                 for _ in range(n):

@@ -189,13 +189,17 @@ class Engine:
             runner = self._runners[cap] = DecodeRunner(self, cap)
         return runner.run(rids, tokens, n, samplers)
 
-    def nucleus_scratch(self) -> torch.Tensor:
-        """Float64 room for the weights of ``DECODE_MAX_BATCH`` rows of logits: what the recorded loop's choice needs
-        for draws from a nucleus; one per engine, made with the first recorded loop."""
-        if getattr(self, "_nucleus_scratch", None) is None:
-            self._nucleus_scratch = torch.empty(self.DECODE_MAX_BATCH * self.spec.vocab, dtype=torch.float64,
-                                                device=self.device)
-        return self._nucleus_scratch
+    def choice_scratch(self):
+        """What the recorded loop's choice needs when rows draw: float64 room for the weights of ``DECODE_MAX_BATCH``
+        rows of logits (draws from a nucleus) and for their partial sums, and the rows' maxima and flags; one set per
+        engine, made with the first recorded loop.  Returns ``(weights, (part, amax, bad0))``."""
+        if getattr(self, "_choice_scratch", None) is None:
+            n, dev = self.DECODE_MAX_BATCH, self.device
+            self._choice_scratch = (
+                torch.empty(n * self.spec.vocab, dtype=torch.float64, device=dev),
+                (torch.empty(n * self.rt.ops.choice_parts(self.spec.vocab), dtype=torch.float64, device=dev),
+                 torch.zeros(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev)))
+        return self._choice_scratch
 
     def _decode_eager(self, rids, tokens, n, samplers):
         """The same steps one by one through :meth:`step`, for models with parts that cannot be recorded."""

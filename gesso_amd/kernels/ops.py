@@ -639,12 +639,21 @@ def gemm_skinny_conv(x, w_in, taps, bias, state, slots, wt=None, tiled: bool = F
     return out
 
 
+def choice_parts(V: int) -> int:
+    """Partial sums a row of ``V`` logits has in the many-block form of the decode loop's choice."""
+    return int(lib().gs_choice_parts(c_int(V)))
+
+
 def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p=None,
-                  wbuf=None) -> None:
+                  wbuf=None, wide=None) -> None:
     """Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``, from the whole row or, where
     ``top_p[row] < 1``, from its nucleus (``wbuf``: float64 scratch of at least ``rows * V``); results into the loop's
     buffers; then the row's counter counts up and a live row moves one position on.  A counter at or beyond the rings'
-    step count writes into their last row and marks the step bad."""
+    step count writes into their last row and marks the step bad.
+
+    ``wide``: ``(part, amax, bad0)``, float64 ``rows * choice_parts(V)`` and int32 ``rows`` twice: the same choice in
+    three kernels, the rows' weights by many blocks (for steps in which rows draw; one block weighs a row of 65,536
+    logits in some 40 us)."""
     _dev(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p, wbuf)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "decode_choose: logits are float32 (rows, V)")
     rows, V = logits.shape
@@ -659,6 +668,15 @@ def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, pos
     if top_p is not None:
         _need(top_p.dtype == torch.float64 and top_p.numel() == rows, "decode_choose: top_p float64 (rows,)")
         _need(wbuf.dtype == torch.float64 and wbuf.numel() >= rows * V, "decode_choose: wbuf float64, rows * V at least")
+    if wide is not None:
+        part, amax, bad0 = wide
+        _dev(part, amax, bad0)
+        _need(part.dtype == torch.float64 and part.numel() >= rows * choice_parts(V), "decode_choose: part float64, rows * choice_parts(V) at least")
+        _i32(amax, rows); _i32(bad0, rows)
+        _check(lib().gs_decode_choose_wide(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(part),
+                                           _p(amax), _p(bad0), _p(u), _p(counter), _p(next_ids), _p(ring), _p(bad_ring),
+                                           _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]), _stream()))
+        return
     _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(u),
                                   _p(counter), _p(next_ids),
                                   _p(ring), _p(bad_ring), _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]),

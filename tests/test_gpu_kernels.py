@@ -452,11 +452,14 @@ def test_sample_top_p_gives_the_same_id_every_time_and_at_the_models_vocabulary(
         assert first[r].item() == P.sample_id(logits[r].tolist(), 0.9, 0.73, 40 + r)[0], r
 
 
-def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_side(ops):
-    """The kernel that the recorded decode step ends with: rows that are greedy, rows that draw from the whole row and
-    rows that draw from a nucleus, each with its own draw per step; ids against the plain sampler's, the rows' steps,
-    positions and key counts advanced, a non-finite row marked."""
-    V, rows, steps = 777, 6, 3
+@pytest.mark.parametrize("wide", [False, True])
+@pytest.mark.parametrize("V", [777, 9000])
+def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_side(ops, V, wide):
+    """What the recorded decode step ends with, in one kernel and (``wide``) in three with the weights by many blocks:
+    rows that are greedy, rows that draw from the whole row and rows that draw from a nucleus, each with its own draw
+    per step; ids against the plain sampler's, the rows' steps, positions and key counts advanced, a non-finite row
+    marked."""
+    rows, steps = 6, 3
     logits = torch.randn(rows, V, generator=gen(5)) * 2
     logits[5, 13] = float("inf")
     temp = [0.0, 0.8, 0.8, 1.3, 0.0, 0.9]
@@ -473,9 +476,11 @@ def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_sid
     ring, bad = torch.full((steps, rows), -1, dtype=torch.int32, device=DEV), torch.full((steps, rows), -1, dtype=torch.int32, device=DEV)
     pos, kv, live = i32([10, 11, 12, 13, 14, 15]), i32([11, 12, 13, 14, 15, 16]), i32([1, 1, 1, 0, 1, 1])
     wbuf = torch.full((rows * V,), float("nan"), dtype=torch.float64, device=DEV)
+    scratch = (torch.full((rows * ops.choice_parts(V),), float("nan"), dtype=torch.float64, device=DEV), i32([7] * rows),
+               i32([7] * rows)) if wide else None
     for step in range(steps):
         ops.decode_choose(dev(logits), dev(torch.tensor(temp, dtype=torch.float64)), dev(u), counter, nxt, ring, bad, pos, kv,
-                          live, top_p=dev(torch.tensor(top_p, dtype=torch.float64)), wbuf=wbuf)
+                          live, top_p=dev(torch.tensor(top_p, dtype=torch.float64)), wbuf=wbuf, wide=scratch)
     assert counter.tolist() == [steps] * rows
     assert pos.tolist() == [13, 14, 15, 13, 17, 18] and kv.tolist() == [14, 15, 16, 14, 18, 19]     # row 3 is not live
     assert bad[:, :5].sum().item() == 0 and bad[:, 5].tolist() == [1] * steps
