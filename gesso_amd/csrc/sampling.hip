@@ -188,6 +188,7 @@ __global__ void sample_temperature_kernel(const float* __restrict__ logits, int 
 struct Crossing {
   unsigned long long bits;  // pattern of the weight at which the running sum crosses the target
   double above;             // mass of all weights greater than it
+  int nlist;                // ids gathered into the caller's list (all whose weight shares the pattern are among them), or -1
 };
 
 // strict = 0: first running sum >= target; strict = 1: first running sum > target.
@@ -196,9 +197,17 @@ struct Crossing {
 // second byte the weights left lie within a few percent of each other, a handful in a peaked row), their ids are
 // gathered into a list in LDS and the later passes read only those.
 #define NUC_LIST 2048
+//
+// ghist, when given: the histograms of the first two bytes, made ahead by many blocks (choose_weights_kernel) with the
+// scales that passes 0 and 1 use here: NUC_G0 sums for the first byte (0x3B, standing for everything below 2^-63, to
+// 0x3F: a weight is at most 1), then 256 for the second byte under each first byte from 0x3C on; after these
+// NUC_GHIST sums the counts, in the same order.  Where the first byte's crossing falls below 2^-63 the passes start
+// again and read the row themselves.
+#define NUC_G0 8
+#define NUC_GHIST (NUC_G0 + 4 * 256)
 __device__ Crossing radix_descend(const double* __restrict__ w, int V, double target, int strict,
-                                  unsigned long long* hmass, int* hcount, Crossing* shared_out) {
-  __shared__ int clist[NUC_LIST];
+                                  unsigned long long* hmass, int* hcount, Crossing* shared_out, int* clist,
+                                  const unsigned long long* __restrict__ ghist = nullptr) {
   __shared__ int cn, picked;
   unsigned long long prefix = 0;
   double above = 0.0;
@@ -221,7 +230,20 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
     // queue up; the sums are integers, so neither this nor the order of the adds changes them
     int run_b = -1, run_n = 0;
     unsigned long long run_m = 0ull;
-    const int n = nlist >= 0 ? nlist : V;
+    const bool ready = ghist != nullptr && pass < 2;
+    if (ready && pass == 0) {
+      for (int b = threadIdx.x; b < 5; b += blockDim.x) {
+        hmass[0x3B + b] = ghist[b];
+        hcount[0x3B + b] = (int)ghist[NUC_GHIST + b];
+      }
+    } else if (ready) {
+      const int under = (int)(prefix >> 56) - 0x3C;
+      for (int b = threadIdx.x; b < 256; b += blockDim.x) {
+        hmass[b] = ghist[NUC_G0 + under * 256 + b];
+        hcount[b] = (int)ghist[NUC_GHIST + NUC_G0 + under * 256 + b];
+      }
+    }
+    const int n = ready ? 0 : (nlist >= 0 ? nlist : V);
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
       const int j = nlist >= 0 ? clist[i] : i;
       unsigned long long bits = (unsigned long long)__double_as_longlong(w[j]);
@@ -245,33 +267,63 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
       atomicAdd(&hcount[run_b], run_n);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      double acc = above;
-      int pick = -1, lowest = -1;
-      for (int b = 255; b >= 0; --b) {
-        if (hcount[b] == 0) continue;
-        lowest = b;
-        double next = acc + (double)hmass[b] * unscale;
-        if (strict ? (target < next) : (next >= target)) {
-          pick = b;
-          break;
+    // the walk over the buckets, heaviest first, by one wavefront, four buckets a lane: running sums of the masses
+    // (integers, exact), each turned into a float64 once; the first bucket whose running sum crosses the target, or
+    // the last one that holds anything where rounding left the target just above the whole mass
+    if (threadIdx.x < 64) {
+      const int lane = threadIdx.x;
+      unsigned long long m[4], run[4];
+      int c[4];
+      unsigned long long mine = 0ull;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int b = 255 - (4 * lane + i);
+        m[i] = hmass[b];
+        c[i] = hcount[b];
+        mine += m[i];
+        run[i] = mine;
+      }
+      unsigned long long incl = mine;                      // running sum over the lanes, this lane included
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long v = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += v;
+      }
+      const unsigned long long before = incl - mine;
+      int hit = -1, full = -1;
+#pragma unroll
+      for (int i = 3; i >= 0; --i) {
+        if (c[i] > 0) {
+          const double next = above + (double)(before + run[i]) * unscale;
+          if (strict ? (target < next) : (next >= target)) hit = i;
+          if (full < 0) full = i;
         }
-        acc = next;
       }
-      if (pick < 0) {  // rounding left the target just above the whole mass: the last weight it is
-        pick = lowest;
-        acc -= (double)hmass[lowest] * unscale;
+      const unsigned long long hits = __ballot(hit >= 0), fulls = __ballot(full >= 0);
+      const int hl = hits ? __ffsll((long long)hits) - 1 : -1;
+      const int fl = fulls ? 63 - __clzll((long long)fulls) : -1;
+      const int owner = hl >= 0 ? hl : (fl >= 0 ? fl : 63);
+      if (lane == owner) {
+        const int i = hl >= 0 ? hit : (full >= 0 ? full : 3);
+        const int pick = 255 - (4 * lane + i);
+        shared_out->bits = prefix | ((unsigned long long)pick << shift);
+        shared_out->above = above + (double)(before + run[i] - m[i]) * unscale;
+        picked = c[i];
+        cn = 0;
       }
-      shared_out->bits = prefix | ((unsigned long long)pick << shift);
-      shared_out->above = acc;
-      picked = hcount[pick];
-      cn = 0;
     }
     __syncthreads();
     prefix = shared_out->bits;
     above = shared_out->above;
     const int left = picked;
     __syncthreads();
+    if (ghist != nullptr && pass == 0 && (prefix >> 56) < 0x3C) {   // below what the ready-made histograms resolve
+      ghist = nullptr;
+      prefix = 0;
+      above = 0.0;
+      pass = -1;
+      continue;
+    }
     if (nlist < 0 && pass >= 1 && pass <= 5 && left <= NUC_LIST) {
       const unsigned long long sofar = (~0ull) << shift;
       for (int j = threadIdx.x; j < V; j += blockDim.x)
@@ -283,20 +335,20 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
   Crossing c;
   c.bits = prefix;
   c.above = above;
+  c.nlist = nlist;
   return c;
 }
 
-// One row by the whole block: T > 0, P in (0, 1), u in [0, 1); w: V float64 of scratch; thread 0 returns (id, bad)
-// through the pointers.
+__device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, double uu, double total,
+                                 const unsigned long long* __restrict__ ghist, int* id_out, int* bad_out);
+
+// One row by the whole block: T > 0, P in (0, 1), u in [0, 1); w: V float64 of scratch; one thread returns (id, bad)
+// through the pointers (a barrier before another thread reads them).
 __device__ void row_sample_top_p(const float* __restrict__ x, int V, double T, double P, double uu,
                                  double* __restrict__ w, int* id_out, int* bad_out) {
-  __shared__ unsigned long long hmass[256];
-  __shared__ int hcount[256];
-  __shared__ Crossing cross;
   __shared__ float redf[SAMP_THREADS / 64];
   __shared__ double redd[SAMP_THREADS / 64];
   __shared__ int bbad;
-  __shared__ int tie_before[SAMP_THREADS];
   int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
   if (tid == 0) bbad = 0;
   __syncthreads();
@@ -333,10 +385,21 @@ __device__ void row_sample_top_p(const float* __restrict__ x, int V, double T, d
   double total = 0.0;
   for (int i = 0; i < nw; ++i) total += redd[i];
   __syncthreads();
+  row_nucleus_pick(w, V, P, uu, total, nullptr, id_out, bad_out);
+}
 
+// The draw from the nucleus of a row whose weights w (V float64) and their total are at hand; ghist as in radix_descend.
+__device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, double uu, double total,
+                                 const unsigned long long* __restrict__ ghist, int* id_out, int* bad_out) {
+  __shared__ unsigned long long hmass[256];
+  __shared__ int hcount[256];
+  __shared__ Crossing cross;
+  __shared__ int tie_before[SAMP_THREADS];
+  __shared__ int clist[NUC_LIST];
+  const int tid = threadIdx.x;
   // the nucleus' edge: weight tau at which the sorted running sum reaches top_p * total
   double target = P * total;
-  Crossing edge = radix_descend(w, V, target, 0, hmass, hcount, &cross);
+  Crossing edge = radix_descend(w, V, target, 0, hmass, hcount, &cross, clist, ghist);
   double tau = __longlong_as_double((long long)edge.bits);
   // ties at tau that belong to the nucleus: added one by one until the sum reaches the target
   double need = target - edge.above;
@@ -346,44 +409,68 @@ __device__ void row_sample_top_p(const float* __restrict__ x, int V, double T, d
 
   // the draw: first running sum above r = u * cut, in the same order
   double r = uu * cut;
-  Crossing hit = radix_descend(w, V, r, 1, hmass, hcount, &cross);
+  Crossing hit = radix_descend(w, V, r, 1, hmass, hcount, &cross, clist, ghist);
   double wv = __longlong_as_double((long long)hit.bits);
   long long k = wv > 0.0 ? (long long)floor((r - hit.above) / wv) : 0;  // 0-based tie in id order
   if (k < 0) k = 0;
   // the k-th id, in id order, whose weight has exactly this pattern (the last such, if k overshoots)
+  if (hit.nlist >= 0 && hit.nlist <= (int)blockDim.x) {
+    // they are all in the list, a thread to each: its place among them is the number of those with a lower id
+    const bool mine = tid < hit.nlist && (unsigned long long)__double_as_longlong(w[clist[tid]]) == hit.bits;
+    tie_before[tid] = mine ? 1 : 0;
+    const long long ties = __syncthreads_count(mine);
+    if (ties == 0) {
+      if (tid == 0) {
+        *id_out = 0;
+        *bad_out = 0;
+      }
+      return;
+    }
+    const long long kk = k < ties ? k : ties - 1;
+    if (mine) {
+      const int id = clist[tid];
+      long long lower = 0;
+      for (int i = 0; i < hit.nlist; ++i) lower += (tie_before[i] && clist[i] < id) ? 1 : 0;
+      if (lower == kk) {
+        *id_out = id;
+        *bad_out = 0;
+      }
+    }
+    return;
+  }
   int per = (V + blockDim.x - 1) / blockDim.x;
   int j0 = tid * per, j1 = j0 + per < V ? j0 + per : V;
   int cnt = 0;
   for (int j = j0; j < j1; ++j) cnt += ((unsigned long long)__double_as_longlong(w[j]) == hit.bits);
   tie_before[tid] = cnt;
   __syncthreads();
-  if (tid == 0) {
-    long long seen = 0;
-    int pick = -1, last = -1;
-    for (int i = 0; i < (int)blockDim.x && pick < 0; ++i) {
-      if (tie_before[i] == 0) continue;
-      int a = i * per, b = a + per < V ? a + per : V;
-      if (seen + tie_before[i] <= k) {
-        seen += tie_before[i];
-        for (int j = b - 1; j >= a; --j)
-          if ((unsigned long long)__double_as_longlong(w[j]) == hit.bits) {
-            last = j;
-            break;
-          }
-        continue;
-      }
-      for (int j = a; j < b; ++j)
-        if ((unsigned long long)__double_as_longlong(w[j]) == hit.bits) {
-          last = j;
-          if (seen == k) {
-            pick = j;
-            break;
-          }
-          ++seen;
-        }
+  for (int off = 1; off < (int)blockDim.x; off <<= 1) {    // running counts over the threads' ranges, in id order
+    const int v = tid >= off ? tie_before[tid - off] : 0;
+    __syncthreads();
+    tie_before[tid] += v;
+    __syncthreads();
+  }
+  const long long ties = tie_before[blockDim.x - 1];
+  if (ties == 0) {
+    if (tid == 0) {
+      *id_out = 0;
+      *bad_out = 0;
     }
-    *id_out = pick >= 0 ? pick : (last >= 0 ? last : 0);
-    *bad_out = 0;
+    return;
+  }
+  const long long kk = k < ties ? k : ties - 1;
+  const long long before = tie_before[tid] - cnt;
+  if (cnt > 0 && before <= kk && kk < before + cnt) {      // the thread whose range holds it walks there
+    long long seen = before;
+    for (int j = j0; j < j1; ++j)
+      if ((unsigned long long)__double_as_longlong(w[j]) == hit.bits) {
+        if (seen == kk) {
+          *id_out = j;
+          *bad_out = 0;
+          break;
+        }
+        ++seen;
+      }
   }
 }
 
@@ -425,6 +512,7 @@ __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, co
     row_sample(x, V, T, u[(size_t)step * rows + row], &sid, &sbad);
   else
     row_argmax(x, V, &sid, &sbad);
+  __syncthreads();      // a nucleus' id comes from the thread that found it
   if (threadIdx.x == 0) {
     next_ids[row] = sid;
     ring[(size_t)step * rows + row] = sid;
@@ -465,10 +553,20 @@ extern "C" int gs_decode_choose(const float* logits, int rows, int V, const doub
 
 extern "C" int gs_choice_parts(int V) { return ((V + WIDE_SPAN - 1) / WIDE_SPAN) * SAMP_THREADS; }
 
+__global__ void choose_max_kernel(const float* __restrict__ logits, int V, int* __restrict__ ids, int* __restrict__ bad,
+                                  unsigned long long* __restrict__ ghist) {
+  const int row = blockIdx.x;
+  if (ghist)   // sums that the next kernel's blocks add to: they start at zero in every step (a fill by a kernel)
+    for (int i = threadIdx.x; i < 2 * NUC_GHIST; i += blockDim.x) ghist[(size_t)row * 2 * NUC_GHIST + i] = 0ull;
+  row_argmax(logits + (size_t)row * V, V, ids + row, bad + row);
+}
+
 __global__ __launch_bounds__(SAMP_THREADS) void choose_weights_kernel(
     const float* __restrict__ logits, int V, const double* __restrict__ temperature, const double* __restrict__ top_p,
     const int* __restrict__ amax, const int* __restrict__ bad0, double* __restrict__ wbuf, double* __restrict__ part,
-    int nparts) {
+    int nparts, unsigned long long* __restrict__ ghist) {
+  __shared__ unsigned long long lm[NUC_GHIST];
+  __shared__ int lc[NUC_GHIST];
   const int row = blockIdx.y;
   const double T = temperature[row];
   if (!(T > 0.0) || bad0[row]) return;
@@ -494,6 +592,40 @@ __global__ __launch_bounds__(SAMP_THREADS) void choose_weights_kernel(
 #pragma unroll
     for (int k = 0; k < WIDE_CH; ++k)
       if (j0 + k < V) wbuf[(size_t)row * V + j0 + k] = w[k];
+    if (ghist) {
+      // the histograms of the weights' first two bytes, as passes 0 and 1 of radix_descend make them (same scales,
+      // integer sums): in LDS for this block's ids, then added to the row's
+      for (int i = threadIdx.x; i < NUC_GHIST; i += blockDim.x) {
+        lm[i] = 0ull;
+        lc[i] = 0;
+      }
+      __syncthreads();
+      int lv = 1;
+      while ((1 << lv) < V && lv < 30) ++lv;
+      const double scale0 = exp2((double)(62 - lv));
+#pragma unroll
+      for (int k = 0; k < WIDE_CH; ++k) {
+        if (j0 + k >= V) continue;
+        const unsigned long long bits = (unsigned long long)__double_as_longlong(w[k]);
+        const int b0 = (int)(bits >> 56);
+        const int i0 = b0 < 0x3C ? 0 : b0 - 0x3B;
+        atomicAdd(&lm[i0], (unsigned long long)__double2ll_rn(w[k] * scale0));
+        atomicAdd(&lc[i0], 1);
+        if (b0 >= 0x3C) {
+          const double wmax = __longlong_as_double((long long)(((unsigned long long)b0 << 56) | ((1ull << 56) - 1ull)));
+          const int i1 = NUC_G0 + (b0 - 0x3C) * 256 + (int)((bits >> 48) & 0xff);
+          atomicAdd(&lm[i1], (unsigned long long)__double2ll_rn(w[k] * (scale0 / wmax)));
+          atomicAdd(&lc[i1], 1);
+        }
+      }
+      __syncthreads();
+      unsigned long long* g = ghist + (size_t)row * 2 * NUC_GHIST;
+      for (int i = threadIdx.x; i < NUC_GHIST; i += blockDim.x)
+        if (lc[i]) {
+          atomicAdd(&g[i], lm[i]);
+          atomicAdd(&g[NUC_GHIST + i], (unsigned long long)lc[i]);
+        }
+    }
   }
 }
 
@@ -502,7 +634,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void choose_pick_kernel(
     double* __restrict__ wbuf, const double* __restrict__ part, int nparts, const int* __restrict__ amax,
     const int* __restrict__ bad0, const double* __restrict__ u, int* __restrict__ counter, int* __restrict__ next_ids,
     int* __restrict__ ring, int* __restrict__ bad_ring, int* __restrict__ positions, int* __restrict__ kv_len,
-    const int* __restrict__ live, int max_steps) {
+    const int* __restrict__ live, int max_steps, const unsigned long long* __restrict__ ghist) {
   __shared__ int sid, sbad, first_t;
   __shared__ double scan[SAMP_THREADS];
   const int row = blockIdx.x, rows = gridDim.x, tid = threadIdx.x;
@@ -518,8 +650,6 @@ __global__ __launch_bounds__(SAMP_THREADS) void choose_pick_kernel(
       sid = bad0[row] ? 0 : amax[row];
       sbad = bad0[row];
     }
-  } else if (P < 1.0) {
-    row_sample_top_p(x, V, T, P, uu, wbuf + (size_t)row * V, &sid, &sbad);
   } else {
     const double* pr = part + (size_t)row * nparts;
     const int per = nparts / SAMP_THREADS;
@@ -533,6 +663,13 @@ __global__ __launch_bounds__(SAMP_THREADS) void choose_pick_kernel(
       __syncthreads();
       scan[tid] += v;
       __syncthreads();
+    }
+    if (P < 1.0) {
+      const double total = scan[SAMP_THREADS - 1];
+      __syncthreads();
+      row_nucleus_pick(wbuf + (size_t)row * V, V, P, uu, total,
+                       ghist ? ghist + (size_t)row * 2 * NUC_GHIST : nullptr, &sid, &sbad);
+      goto chosen;
     }
     const double r = uu * scan[SAMP_THREADS - 1];
     if (r < scan[tid]) atomicMin(&first_t, tid);
@@ -570,6 +707,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void choose_pick_kernel(
       sbad = 0;
     }
   }
+chosen:
   __syncthreads();
   if (tid == 0) {
     next_ids[row] = sid;
@@ -585,8 +723,12 @@ __global__ __launch_bounds__(SAMP_THREADS) void choose_pick_kernel(
 
 // The decode loop's choice in three kernels, for steps in which rows draw (what gs_decode_choose does in one).
 // amax, bad0: rows int32 each; part: rows x gs_choice_parts(V) float64; top_p and wbuf as in gs_decode_choose.
+// hist: rows x gs_choice_hist() 64-bit integers (with top_p; cleared here in every call).
+extern "C" int gs_choice_hist() { return 2 * NUC_GHIST; }
+
 extern "C" int gs_decode_choose_wide(const float* logits, int rows, int V, const double* temperature, const double* top_p,
-                                     double* wbuf, double* part, int* amax, int* bad0, const double* u, int* counter,
+                                     double* wbuf, double* part, int* amax, int* bad0, unsigned long long* hist,
+                                     const double* u, int* counter,
                                      int* next_ids, int* ring, int* bad_ring, int* positions, int* kv_len, const int* live,
                                      int max_steps, hipStream_t stream) {
   GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
@@ -596,13 +738,15 @@ extern "C" int gs_decode_choose_wide(const float* logits, int rows, int V, const
   GS_REQUIRE((top_p == nullptr) == (wbuf == nullptr), "decode_choose: top_p and its scratch come together");
   GS_REQUIRE(rows <= 65535, "decode_choose: %d rows in one call", rows);
   const int nparts = gs_choice_parts(V);
-  argmax_rows_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, amax, bad0);
+  GS_REQUIRE(hist != nullptr || top_p == nullptr, "decode_choose: draws from a nucleus need the histograms' room");
+  choose_max_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, amax, bad0, top_p ? hist : nullptr);
   GS_LAUNCH_CHECK("decode_choose (maxima)");
-  choose_weights_kernel<<<dim3(nparts / SAMP_THREADS, rows), SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, amax,
-                                                                                        bad0, wbuf, part, nparts);
+  choose_weights_kernel<<<dim3(nparts / SAMP_THREADS, rows), SAMP_THREADS, 0, stream>>>(
+      logits, V, temperature, top_p, amax, bad0, wbuf, part, nparts, top_p ? hist : nullptr);
   GS_LAUNCH_CHECK("decode_choose (weights)");
   choose_pick_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, wbuf, part, nparts, amax, bad0, u,
-                                                        counter, next_ids, ring, bad_ring, positions, kv_len, live, max_steps);
+                                                        counter, next_ids, ring, bad_ring, positions, kv_len, live, max_steps,
+                                                        top_p ? hist : nullptr);
   GS_LAUNCH_CHECK("decode_choose (pick)");
   return 0;
 }

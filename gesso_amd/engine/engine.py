@@ -192,13 +192,14 @@ class Engine:
     def choice_scratch(self):
         """What the recorded loop's choice needs when rows draw: float64 room for the weights of ``DECODE_MAX_BATCH``
         rows of logits (draws from a nucleus) and for their partial sums, and the rows' maxima and flags; one set per
-        engine, made with the first recorded loop.  Returns ``(weights, (part, amax, bad0))``."""
+        engine, made with the first recorded loop.  Returns ``(weights, (part, amax, bad0, hist))``."""
         if getattr(self, "_choice_scratch", None) is None:
             n, dev = self.DECODE_MAX_BATCH, self.device
             self._choice_scratch = (
                 torch.empty(n * self.spec.vocab, dtype=torch.float64, device=dev),
                 (torch.empty(n * self.rt.ops.choice_parts(self.spec.vocab), dtype=torch.float64, device=dev),
-                 torch.zeros(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev)))
+                 torch.zeros(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev),
+                 torch.zeros(n * self.rt.ops.choice_hist(), dtype=torch.int64, device=dev)))
         return self._choice_scratch
 
     def _decode_eager(self, rids, tokens, n, samplers):

@@ -644,6 +644,11 @@ def choice_parts(V: int) -> int:
     return int(lib().gs_choice_parts(c_int(V)))
 
 
+def choice_hist() -> int:
+    """64-bit sums a row has in the ready-made histograms of the many-block choice."""
+    return int(lib().gs_choice_hist())
+
+
 def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p=None,
                   wbuf=None, wide=None) -> None:
     """Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``, from the whole row or, where
@@ -651,7 +656,8 @@ def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, pos
     buffers; then the row's counter counts up and a live row moves one position on.  A counter at or beyond the rings'
     step count writes into their last row and marks the step bad.
 
-    ``wide``: ``(part, amax, bad0)``, float64 ``rows * choice_parts(V)`` and int32 ``rows`` twice: the same choice in
+    ``wide``: ``(part, amax, bad0, hist)``, float64 ``rows * choice_parts(V)``, int32 ``rows`` twice and int64
+    ``rows * choice_hist()``: the same choice in
     three kernels, the rows' weights by many blocks (for steps in which rows draw; one block weighs a row of 65,536
     logits in some 40 us)."""
     _dev(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p, wbuf)
@@ -669,12 +675,13 @@ def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, pos
         _need(top_p.dtype == torch.float64 and top_p.numel() == rows, "decode_choose: top_p float64 (rows,)")
         _need(wbuf.dtype == torch.float64 and wbuf.numel() >= rows * V, "decode_choose: wbuf float64, rows * V at least")
     if wide is not None:
-        part, amax, bad0 = wide
-        _dev(part, amax, bad0)
+        part, amax, bad0, hist = wide
+        _dev(part, amax, bad0, hist)
         _need(part.dtype == torch.float64 and part.numel() >= rows * choice_parts(V), "decode_choose: part float64, rows * choice_parts(V) at least")
+        _need(hist.dtype == torch.int64 and hist.numel() >= rows * choice_hist(), "decode_choose: hist int64, rows * choice_hist() at least")
         _i32(amax, rows); _i32(bad0, rows)
         _check(lib().gs_decode_choose_wide(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(part),
-                                           _p(amax), _p(bad0), _p(u), _p(counter), _p(next_ids), _p(ring), _p(bad_ring),
+                                           _p(amax), _p(bad0), _p(hist), _p(u), _p(counter), _p(next_ids), _p(ring), _p(bad_ring),
                                            _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]), _stream()))
         return
     _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(u),

@@ -477,7 +477,7 @@ def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_sid
     pos, kv, live = i32([10, 11, 12, 13, 14, 15]), i32([11, 12, 13, 14, 15, 16]), i32([1, 1, 1, 0, 1, 1])
     wbuf = torch.full((rows * V,), float("nan"), dtype=torch.float64, device=DEV)
     scratch = (torch.full((rows * ops.choice_parts(V),), float("nan"), dtype=torch.float64, device=DEV), i32([7] * rows),
-               i32([7] * rows)) if wide else None
+               i32([7] * rows), torch.full((rows * ops.choice_hist(),), 12345, dtype=torch.int64, device=DEV)) if wide else None
     for step in range(steps):
         ops.decode_choose(dev(logits), dev(torch.tensor(temp, dtype=torch.float64)), dev(u), counter, nxt, ring, bad, pos, kv,
                           live, top_p=dev(torch.tensor(top_p, dtype=torch.float64)), wbuf=wbuf, wide=scratch)
