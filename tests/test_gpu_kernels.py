@@ -453,7 +453,7 @@ def test_sample_top_p_gives_the_same_id_every_time_and_at_the_models_vocabulary(
 
 
 @pytest.mark.parametrize("wide", [False, True])
-@pytest.mark.parametrize("V", [777, 9000])
+@pytest.mark.parametrize("V", [777, 9000, 65536])
 def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_side(ops, V, wide):
     """What the recorded decode step ends with, in one kernel and (``wide``) in three with the weights by many blocks:
     rows that are greedy, rows that draw from the whole row and rows that draw from a nucleus, each with its own draw
