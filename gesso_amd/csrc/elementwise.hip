@@ -19,7 +19,7 @@ void gs_set_error(const char* fmt, ...) {
 
 extern "C" const char* gs_last_error() { return g_err; }
 
-extern "C" int gs_abi_version() { return 8; }
+extern "C" int gs_abi_version() { return 9; }
 
 // ------------------------------------------------------------------ embedding
 

@@ -1,11 +1,11 @@
-// Choosing a token from a row of float32 logits: argmax, and temperature sampling by inverse CDF.
+// Choosing a token from a row of float32 logits: argmax, temperature sampling by inverse CDF, nucleus sampling.
 //
 // argmax: ties go to the lowest id; a NaN or infinity anywhere in the row sets the row's flag
 // (no token may be emitted from such a row).
 // temperature: weights exp((x - max) / T) and their total in float64; the uniform number u in
 // [0, 1) comes from the caller (one draw per token); the id returned is the first, in id order,
-// whose running sum exceeds u * total.  Each thread owns a contiguous range of ids, so the walk
-// is in id order: ranges are summed, scanned, and the range that holds the target is walked.
+// whose running sum exceeds u * total.  The weights are made by many blocks a row, each thread the sum of four
+// consecutive ids; one block a row then finds where the running sum of those sums crosses the target.
 #include "common.h"
 
 #define SAMP_THREADS 1024
@@ -92,79 +92,6 @@ extern "C" int gs_argmax_rows(const float* logits, int rows, int V, int* ids, in
   argmax_rows_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, ids, bad);
   GS_LAUNCH_CHECK("argmax_rows");
   return 0;
-}
-
-// One row by the whole block: T > 0, u in [0, 1); thread 0 returns (id, bad) through the pointers.
-__device__ void row_sample(const float* __restrict__ x, int V, double T, double uu, int* id_out, int* bad_out) {
-  __shared__ double part[SAMP_THREADS];
-  __shared__ float redf[SAMP_THREADS / 64];
-  __shared__ int bbad;
-  int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
-  if (tid == 0) bbad = 0;
-  __syncthreads();
-  // contiguous range of this thread
-  int per = (V + blockDim.x - 1) / blockDim.x;
-  int j0 = tid * per, j1 = j0 + per < V ? j0 + per : V;
-
-  float mx = -INFINITY;
-  int notfinite = 0;
-  for (int j = j0; j < j1; ++j) {
-    float v = x[j];
-    if (!(fabsf(v) <= 3.402823466e38f)) notfinite = 1;
-    mx = fmaxf(mx, v);
-  }
-  if (notfinite) atomicOr(&bbad, 1);
-  mx = wave_max(mx);
-  if (lane == 0) redf[wave] = mx;
-  __syncthreads();
-  mx = redf[0];
-  for (int w = 1; w < nw; ++w) mx = fmaxf(mx, redf[w]);
-  if (bbad) {
-    if (tid == 0) {
-      *id_out = 0;
-      *bad_out = 1;
-    }
-    return;
-  }
-  double hi = (double)mx;
-  double s = 0.0;
-  for (int j = j0; j < j1; ++j) s += exp(((double)x[j] - hi) / T);
-  part[tid] = s;
-  __syncthreads();
-  // total, then the walk in id order, by one thread: whole ranges are skipped by their sums and
-  // only the range that holds the target is walked id by id
-  if (tid == 0) {
-    double total = 0.0;
-    for (int i = 0; i < (int)blockDim.x; ++i) total += part[i];
-    double r = uu * total;
-    double acc = 0.0;
-    int pick = V - 1;
-    bool found = false;
-    for (int i = 0; i < (int)blockDim.x && !found; ++i) {
-      if (r < acc + part[i]) {
-        int a = i * per, b = a + per < V ? a + per : V;
-        for (int j = a; j < b; ++j) {
-          acc += exp(((double)x[j] - hi) / T);
-          if (r < acc) {
-            pick = j;
-            found = true;
-            break;
-          }
-        }
-      } else {
-        acc += part[i];
-      }
-    }
-    *id_out = pick;
-    *bad_out = 0;
-  }
-}
-
-__global__ void sample_temperature_kernel(const float* __restrict__ logits, int V,
-                                          const double* __restrict__ temperature, const double* __restrict__ u,
-                                          int* __restrict__ ids, int* __restrict__ bad) {
-  int row = blockIdx.x;
-  row_sample(logits + (size_t)row * V, V, temperature[row], u[row], ids + row, bad + row);
 }
 
 // ------------------------------------------------------------------ nucleus (top-p) sampling
@@ -339,56 +266,9 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
   return c;
 }
 
-__device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, double uu, double total,
-                                 const unsigned long long* __restrict__ ghist, int* id_out, int* bad_out);
-
-// One row by the whole block: T > 0, P in (0, 1), u in [0, 1); w: V float64 of scratch; one thread returns (id, bad)
-// through the pointers (a barrier before another thread reads them).
-__device__ void row_sample_top_p(const float* __restrict__ x, int V, double T, double P, double uu,
-                                 double* __restrict__ w, int* id_out, int* bad_out) {
-  __shared__ float redf[SAMP_THREADS / 64];
-  __shared__ double redd[SAMP_THREADS / 64];
-  __shared__ int bbad;
-  int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
-  if (tid == 0) bbad = 0;
-  __syncthreads();
-  float mx = -INFINITY;
-  int notfinite = 0;
-  for (int j = tid; j < V; j += blockDim.x) {
-    float v = x[j];
-    if (!(fabsf(v) <= 3.402823466e38f)) notfinite = 1;
-    mx = fmaxf(mx, v);
-  }
-  if (notfinite) atomicOr(&bbad, 1);
-  mx = wave_max(mx);
-  if (lane == 0) redf[wave] = mx;
-  __syncthreads();
-  mx = redf[0];
-  for (int i = 1; i < nw; ++i) mx = fmaxf(mx, redf[i]);
-  if (bbad) {
-    if (tid == 0) {
-      *id_out = 0;
-      *bad_out = 1;
-    }
-    return;
-  }
-  double hi = (double)mx;
-  double s = 0.0;
-  for (int j = tid; j < V; j += blockDim.x) {
-    double wj = exp(((double)x[j] - hi) / T);
-    w[j] = wj;
-    s += wj;
-  }
-  s = wave_sum_f64(s);
-  if (lane == 0) redd[wave] = s;
-  __syncthreads();
-  double total = 0.0;
-  for (int i = 0; i < nw; ++i) total += redd[i];
-  __syncthreads();
-  row_nucleus_pick(w, V, P, uu, total, nullptr, id_out, bad_out);
-}
-
-// The draw from the nucleus of a row whose weights w (V float64) and their total are at hand; ghist as in radix_descend.
+// The draw from the nucleus of a row whose weights w (V float64) and their total are at hand, by the whole block:
+// P in (0, 1), u in [0, 1); ghist as in radix_descend.  One thread returns (id, bad) through the pointers (a barrier
+// before another thread reads them).
 __device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, double uu, double total,
                                  const unsigned long long* __restrict__ ghist, int* id_out, int* bad_out) {
   __shared__ unsigned long long hmass[256];
@@ -474,25 +354,13 @@ __device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, 
   }
 }
 
-__global__ void sample_top_p_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
-                                    const double* __restrict__ top_p, const double* __restrict__ u,
-                                    double* __restrict__ wbuf, int* __restrict__ ids, int* __restrict__ bad) {
-  int row = blockIdx.x;
-  row_sample_top_p(logits + (size_t)row * V, V, temperature[row], top_p[row], u[row], wbuf + (size_t)row * V, ids + row,
-                   bad + row);
-}
-
-
 // The decode loop's choice, made to be recorded into a HIP graph: everything that changes from step to
-// step is read from device memory.  Row r: temperature[r] <= 0 means greedy, else a draw with
-// u[step * rows + r], step = counter[r] (each row counts its own steps, so no block waits for another), from the
-// whole row or, with top_p[r] < 1, from its nucleus (wbuf: rows x V float64 of scratch for the weights).
-// The chosen id goes to next_ids[r] (the token fed back) and, with the row's flag, to
+// step is read from device memory.  This is the form for steps in which every row is greedy, one kernel; rows that
+// draw take the three kernels below.  Row r's step is counter[r] (each row counts its own steps, so no block waits for
+// another).  The chosen id goes to next_ids[r] (the token fed back) and, with the row's flag, to
 // ring[step * rows + r] and bad_ring[...], which the host reads once per run.  Then the row moves on:
 // its counter counts up and, if the row is live, so do its position and its number of keys.
-__global__ void decode_choose_kernel(const float* __restrict__ logits, int V, const double* __restrict__ temperature,
-                                     const double* __restrict__ top_p, double* __restrict__ wbuf,
-                                     const double* __restrict__ u, int* __restrict__ counter,
+__global__ void decode_choose_kernel(const float* __restrict__ logits, int V, int* __restrict__ counter,
                                      int* __restrict__ next_ids, int* __restrict__ ring, int* __restrict__ bad_ring,
                                      int* __restrict__ positions, int* __restrict__ kv_len,
                                      const int* __restrict__ live, int max_steps) {
@@ -503,16 +371,7 @@ __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, co
   // and marks itself bad, so the run fails loudly instead of overwriting a neighbour
   bool over = step < 0 || step >= max_steps;
   if (over) step = max_steps - 1;
-  double T = temperature[row];
-  const float* x = logits + (size_t)row * V;
-  const double P = top_p ? top_p[row] : 1.0;
-  if (T > 0.0 && P < 1.0)
-    row_sample_top_p(x, V, T, P, u[(size_t)step * rows + row], wbuf + (size_t)row * V, &sid, &sbad);
-  else if (T > 0.0)
-    row_sample(x, V, T, u[(size_t)step * rows + row], &sid, &sbad);
-  else
-    row_argmax(x, V, &sid, &sbad);
-  __syncthreads();      // a nucleus' id comes from the thread that found it
+  row_argmax(logits + (size_t)row * V, V, &sid, &sbad);
   if (threadIdx.x == 0) {
     next_ids[row] = sid;
     ring[(size_t)step * rows + row] = sid;
@@ -525,20 +384,16 @@ __global__ void decode_choose_kernel(const float* __restrict__ logits, int V, co
   }
 }
 
-// top_p (rows) and wbuf (rows x V float64) come together or not at all (then every draw is from the whole row).
-extern "C" int gs_decode_choose(const float* logits, int rows, int V, const double* temperature, const double* top_p,
-                                double* wbuf, const double* u, int* counter, int* next_ids, int* ring, int* bad_ring,
+extern "C" int gs_decode_choose(const float* logits, int rows, int V, int* counter, int* next_ids, int* ring, int* bad_ring,
                                 int* positions, int* kv_len, const int* live, int max_steps, hipStream_t stream) {
   GS_REQUIRE(rows > 0 && V > 0, "decode_choose: bad sizes rows=%d V=%d", rows, V);
   GS_REQUIRE(max_steps > 0, "decode_choose: the rings hold %d steps", max_steps);
   GS_REQUIRE(counter && positions && kv_len && live, "decode_choose: needs the rows' counters, positions, key counts and live flags");
-  GS_REQUIRE((top_p == nullptr) == (wbuf == nullptr), "decode_choose: top_p and its scratch come together");
-  decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, wbuf, u, counter, next_ids, ring,
-                                                          bad_ring, positions, kv_len, live, max_steps);
+  decode_choose_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, counter, next_ids, ring, bad_ring, positions, kv_len, live,
+                                                          max_steps);
   GS_LAUNCH_CHECK("decode_choose");
   return 0;
 }
-
 
 // ------------------------------------------------------------------ the decode loop's choice when rows draw
 //
@@ -721,9 +576,11 @@ chosen:
   }
 }
 
-// The decode loop's choice in three kernels, for steps in which rows draw (what gs_decode_choose does in one).
-// amax, bad0: rows int32 each; part: rows x gs_choice_parts(V) float64; top_p and wbuf as in gs_decode_choose.
-// hist: rows x gs_choice_hist() 64-bit integers (with top_p; cleared here in every call).
+// The decode loop's choice in three kernels, for steps in which rows draw.  Row r: temperature[r] <= 0 greedy, else a
+// draw with u[step * rows + r] from the whole row or, with top_p[r] < 1, from its nucleus.  top_p (rows), wbuf
+// (rows x V float64, the weights) and hist (rows x gs_choice_hist() 64-bit integers, cleared here in every call) come
+// together or not at all (then every draw is from the whole row).  amax, bad0: rows int32 each; part: rows x
+// gs_choice_parts(V) float64.
 extern "C" int gs_choice_hist() { return 2 * NUC_GHIST; }
 
 extern "C" int gs_decode_choose_wide(const float* logits, int rows, int V, const double* temperature, const double* top_p,
@@ -748,23 +605,5 @@ extern "C" int gs_decode_choose_wide(const float* logits, int rows, int V, const
                                                         counter, next_ids, ring, bad_ring, positions, kv_len, live, max_steps,
                                                         top_p ? hist : nullptr);
   GS_LAUNCH_CHECK("decode_choose (pick)");
-  return 0;
-}
-
-extern "C" int gs_sample_temperature(const float* logits, int rows, int V, const double* temperature,
-                                     const double* u, int* ids, int* bad, hipStream_t stream) {
-  GS_REQUIRE(rows >= 0 && V > 0, "sample: bad sizes rows=%d V=%d", rows, V);
-  if (rows == 0) return 0;
-  sample_temperature_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, u, ids, bad);
-  GS_LAUNCH_CHECK("sample_temperature");
-  return 0;
-}
-
-extern "C" int gs_sample_top_p(const float* logits, int rows, int V, const double* temperature, const double* top_p,
-                               const double* u, double* wbuf, int* ids, int* bad, hipStream_t stream) {
-  GS_REQUIRE(rows >= 0 && V > 0, "sample_top_p: bad sizes rows=%d V=%d", rows, V);
-  if (rows == 0) return 0;
-  sample_top_p_kernel<<<rows, SAMP_THREADS, 0, stream>>>(logits, V, temperature, top_p, u, wbuf, ids, bad);
-  GS_LAUNCH_CHECK("sample_top_p");
   return 0;
 }

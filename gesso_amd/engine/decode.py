@@ -93,9 +93,12 @@ class DecodeRunner:
             rt.no_library = rt.fused = False
         self.logits = logits
         with rt.stage("sample"):
-            ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring,
-                              self.pos, self.kv_len, self.live, top_p=self.top_p, wbuf=self.weights,
-                              wide=self.wide if self.draws else None)
+            if self.draws:
+                ops.decode_choose(logits, self.temperature, self.u, self.counter, self.tok, self.ring, self.bad_ring,
+                                  self.pos, self.kv_len, self.live, self.wide, top_p=self.top_p, wbuf=self.weights)
+            else:
+                ops.decode_choose_greedy(logits, self.counter, self.tok, self.ring, self.bad_ring, self.pos, self.kv_len,
+                                         self.live)
 
     def _bound(self, longest: int) -> int:
         """The recording that serves contexts of up to ``longest`` tokens: 1024, 2048, 4096, ... tokens."""

@@ -156,6 +156,6 @@ def load() -> ctypes.CDLL:
         except OSError as err:
             raise KernelError(f"cannot load the HIP extension {path}: {err}") from err
         _lib.gs_last_error.restype = ctypes.c_char_p
-        if _lib.gs_abi_version() != 8:
+        if _lib.gs_abi_version() != 9:
             raise KernelError("the HIP extension has another interface version; build it again")
         return _lib

@@ -440,31 +440,33 @@ def argmax_rows(logits: torch.Tensor):
 
 def sample_temperature(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor):
     """One id per row from ``softmax(logits / temperature)`` by inverse CDF at ``u`` (float64 each)."""
-    _dev(logits, temperature, u)
-    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits are float32 (rows, V)")
-    rows, V = logits.shape
-    _need(temperature.dtype == torch.float64 and temperature.numel() == rows, "sample: temperature is float64 (rows,)")
-    _need(u.dtype == torch.float64 and u.numel() == rows, "sample: u is float64 (rows,)")
-    ids = torch.empty(rows, dtype=torch.int32, device=logits.device)
-    bad = torch.empty(rows, dtype=torch.int32, device=logits.device)
-    _check(lib().gs_sample_temperature(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(u), _p(ids), _p(bad),
-                                       _stream()))
-    return ids, bad
+    return choose_rows(logits, temperature, torch.ones_like(temperature), u)
 
 
 def sample_top_p(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, u: torch.Tensor):
     """Nucleus sampling: one id per row from the shortest descending-weight prefix whose mass reaches ``top_p``."""
+    return choose_rows(logits, temperature, top_p, u)
+
+
+def choose_rows(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, u: torch.Tensor):
+    """One id per row, each row in its own manner: ``temperature <= 0`` greedy, else a draw at ``u`` from the whole row
+    or (``top_p < 1``) from its nucleus; float64 ``(rows,)`` each.  ``(ids, bad)`` int32 as :func:`argmax_rows`.  The
+    weights are made by many blocks a row (the kernels of the decode loop's choice)."""
     _dev(logits, temperature, top_p, u)
-    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits are float32 (rows, V)")
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "choose: logits are float32 (rows, V)")
     rows, V = logits.shape
     for name, t in (("temperature", temperature), ("top_p", top_p), ("u", u)):
-        _need(t.dtype == torch.float64 and t.numel() == rows, f"sample: {name} is float64 (rows,)")
-    wbuf = torch.empty((rows, V), dtype=torch.float64, device=logits.device)
-    ids = torch.empty(rows, dtype=torch.int32, device=logits.device)
-    bad = torch.empty(rows, dtype=torch.int32, device=logits.device)
-    _check(lib().gs_sample_top_p(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(u), _p(wbuf),
-                                 _p(ids), _p(bad), _stream()))
-    return ids, bad
+        _need(t.dtype == torch.float64 and t.numel() == rows, f"choose: {name} is float64 (rows,)")
+    dev = logits.device
+    zeros = torch.zeros((5, rows), dtype=torch.int32, device=dev)      # counter, next id, position, key count, live
+    out = torch.empty((2, 1, rows), dtype=torch.int32, device=dev)
+    nucleus = bool((top_p < 1).any())
+    wide = (torch.empty(rows * choice_parts(V), dtype=torch.float64, device=dev), torch.empty(rows, dtype=torch.int32, device=dev),
+            torch.empty(rows, dtype=torch.int32, device=dev), torch.empty(rows * choice_hist(), dtype=torch.int64, device=dev))
+    decode_choose(logits, temperature, u.reshape(1, rows), zeros[0], zeros[1], out[0], out[1], zeros[2], zeros[3], zeros[4],
+                  wide, top_p=top_p if nucleus else None,
+                  wbuf=torch.empty(rows * V, dtype=torch.float64, device=dev) if nucleus else None)
+    return out[0, 0], out[1, 0]
 
 
 # ---------------------------------------------------------------------- decoding
@@ -649,45 +651,54 @@ def choice_hist() -> int:
     return int(lib().gs_choice_hist())
 
 
-def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p=None,
-                  wbuf=None, wide=None) -> None:
-    """Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``, from the whole row or, where
-    ``top_p[row] < 1``, from its nucleus (``wbuf``: float64 scratch of at least ``rows * V``); results into the loop's
-    buffers; then the row's counter counts up and a live row moves one position on.  A counter at or beyond the rings'
-    step count writes into their last row and marks the step bad.
-
-    ``wide``: ``(part, amax, bad0, hist)``, float64 ``rows * choice_parts(V)``, int32 ``rows`` twice and int64
-    ``rows * choice_hist()``: the same choice in
-    three kernels, the rows' weights by many blocks (for steps in which rows draw; one block weighs a row of 65,536
-    logits in some 40 us)."""
-    _dev(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, top_p, wbuf)
+def _choice_rows(logits, counter, next_ids, ring, bad_ring, positions, kv_len, live):
+    _dev(logits, counter, next_ids, ring, bad_ring, positions, kv_len, live)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.is_contiguous(), "decode_choose: logits are float32 (rows, V)")
     rows, V = logits.shape
-    _need(temperature.dtype == torch.float64 and temperature.numel() == rows, "decode_choose: temperature float64 (rows,)")
-    _need(u.dtype == torch.float64 and u.dim() == 2 and u.shape[1] == rows, "decode_choose: u is float64 (steps, rows)")
     for t in (counter, next_ids, positions, kv_len, live):
         _i32(t, rows)
     for t in (ring, bad_ring):
         _i32(t)
-    _need(ring.shape == u.shape and bad_ring.shape == u.shape, "decode_choose: buffer shapes")
+    _need(ring.dim() == 2 and ring.shape[1] == rows and bad_ring.shape == ring.shape, "decode_choose: rings are (steps, rows)")
+    return rows, V
+
+
+def decode_choose_greedy(logits, counter, next_ids, ring, bad_ring, positions, kv_len, live) -> None:
+    """The decode loop's choice while every row is greedy, one kernel: per row the first maximum into the loop's buffers
+    (``ring[counter[row], row]``, the flag of a non-finite row beside it, the id fed back); then the row's counter counts
+    up and a live row moves one position on.  A counter at or beyond the rings' step count writes into their last row
+    and marks the step bad."""
+    rows, V = _choice_rows(logits, counter, next_ids, ring, bad_ring, positions, kv_len, live)
+    _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(counter), _p(next_ids), _p(ring), _p(bad_ring),
+                                  _p(positions), _p(kv_len), _p(live), c_int(ring.shape[0]), _stream()))
+
+
+def decode_choose(logits, temperature, u, counter, next_ids, ring, bad_ring, positions, kv_len, live, wide, top_p=None,
+                  wbuf=None) -> None:
+    """The decode loop's choice when rows draw, three kernels (the rows' weights by many blocks: one block weighs a row
+    of 65,536 logits in some 40 us).  Per row: greedy (temperature <= 0) or a draw with ``u[counter[row], row]``, from
+    the whole row or, where ``top_p[row] < 1``, from its nucleus (``wbuf``: float64 scratch of at least ``rows * V``);
+    results and the rows' advance as in :func:`decode_choose_greedy`.
+
+    ``wide``: ``(part, amax, bad0, hist)``, float64 ``rows * choice_parts(V)``, int32 ``rows`` twice and int64
+    ``rows * choice_hist()``: scratch."""
+    rows, V = _choice_rows(logits, counter, next_ids, ring, bad_ring, positions, kv_len, live)
+    _dev(temperature, u, top_p, wbuf)
+    _need(temperature.dtype == torch.float64 and temperature.numel() == rows, "decode_choose: temperature float64 (rows,)")
+    _need(u.dtype == torch.float64 and u.shape == ring.shape, "decode_choose: u is float64 (steps, rows)")
     _need((top_p is None) == (wbuf is None), "decode_choose: top_p and its scratch come together")
     if top_p is not None:
         _need(top_p.dtype == torch.float64 and top_p.numel() == rows, "decode_choose: top_p float64 (rows,)")
         _need(wbuf.dtype == torch.float64 and wbuf.numel() >= rows * V, "decode_choose: wbuf float64, rows * V at least")
-    if wide is not None:
-        part, amax, bad0, hist = wide
-        _dev(part, amax, bad0, hist)
-        _need(part.dtype == torch.float64 and part.numel() >= rows * choice_parts(V), "decode_choose: part float64, rows * choice_parts(V) at least")
-        _need(hist.dtype == torch.int64 and hist.numel() >= rows * choice_hist(), "decode_choose: hist int64, rows * choice_hist() at least")
-        _i32(amax, rows); _i32(bad0, rows)
-        _check(lib().gs_decode_choose_wide(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(part),
-                                           _p(amax), _p(bad0), _p(hist), _p(u), _p(counter), _p(next_ids), _p(ring), _p(bad_ring),
-                                           _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]), _stream()))
-        return
-    _check(lib().gs_decode_choose(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(u),
-                                  _p(counter), _p(next_ids),
-                                  _p(ring), _p(bad_ring), _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]),
-                                  _stream()))
+    part, amax, bad0, hist = wide
+    _dev(part, amax, bad0, hist)
+    _need(part.dtype == torch.float64 and part.numel() >= rows * choice_parts(V), "decode_choose: part float64, rows * choice_parts(V) at least")
+    _need(hist.dtype == torch.int64 and hist.numel() >= rows * choice_hist(), "decode_choose: hist int64, rows * choice_hist() at least")
+    _i32(amax, rows)
+    _i32(bad0, rows)
+    _check(lib().gs_decode_choose_wide(_p(logits), c_int(rows), c_int(V), _p(temperature), _p(top_p), _p(wbuf), _p(part),
+                                       _p(amax), _p(bad0), _p(hist), _p(u), _p(counter), _p(next_ids), _p(ring), _p(bad_ring),
+                                       _p(positions), _p(kv_len), _p(live), c_int(u.shape[0]), _stream()))
 
 
 def attention_decode_supports(nh: int, nkv: int, d: int) -> bool:

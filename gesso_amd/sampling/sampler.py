@@ -58,35 +58,24 @@ def choose(ops, logits: torch.Tensor, samplers: Sequence[Optional[Sampler]]) -> 
     rows = logits.shape[0]
     if rows != len(samplers):
         raise InvalidPlan("one sampler entry per row of logits")
-    out: List[Union[int, Exception, None]] = [None] * rows
-    greedy = [i for i, s in enumerate(samplers) if s is None]
-    plain = [i for i, s in enumerate(samplers) if s is not None and s.top_p >= 1]
-    nucleus = [i for i, s in enumerate(samplers) if s is not None and s.top_p < 1]
     dev = logits.device
-
-    def run(idx, kind):
-        if not idx:
-            return
-        sub = logits if len(idx) == rows else logits[torch.tensor(idx, device=dev)].contiguous()
-        if kind == "greedy":
-            ids, bad = ops.argmax_rows(sub)
+    if all(s is None for s in samplers):
+        ids, bad = ops.argmax_rows(logits)
+    else:
+        # every row in one pass, each in its own manner.  The draws are made before the rows are known to be finite; a
+        # row that is not emits no token and makes no draw, so its sampler goes back to where it stood
+        before = [None if s is None else s.state for s in samplers]
+        facts = torch.tensor([[0.0 if s is None else s.temperature for s in samplers],
+                              [1.0 if s is None else s.top_p for s in samplers],
+                              [0.0 if s is None else s.unit() for s in samplers]], dtype=torch.float64).to(dev)
+        ids, bad = ops.choose_rows(logits, facts[0], facts[1], facts[2])
+    ids, bad = ids.tolist(), bad.tolist()
+    out: List[Union[int, Exception]] = []
+    for i, (tok, b) in enumerate(zip(ids, bad)):
+        if b:
+            if samplers[i] is not None:
+                samplers[i].state = before[i]
+            out.append(NumericalInstability("non-finite logits: no token is emitted", row=i))
         else:
-            # a draw is made only for rows that can emit a token: look for non-finite rows first
-            _, bad0 = ops.argmax_rows(sub)
-            bad0 = bad0.tolist()
-            t = torch.tensor([samplers[i].temperature for i in idx], dtype=torch.float64, device=dev)
-            u = torch.tensor([0.0 if b else samplers[i].unit() for i, b in zip(idx, bad0)],
-                             dtype=torch.float64, device=dev)
-            if kind == "plain":
-                ids, bad = ops.sample_temperature(sub, t, u)
-            else:
-                p = torch.tensor([samplers[i].top_p for i in idx], dtype=torch.float64, device=dev)
-                ids, bad = ops.sample_top_p(sub, t, p, u)
-        ids, bad = ids.tolist(), bad.tolist()
-        for i, tok, b in zip(idx, ids, bad):
-            out[i] = NumericalInstability("non-finite logits: no token is emitted", row=i) if b else int(tok)
-
-    run(greedy, "greedy")
-    run(plain, "plain")
-    run(nucleus, "nucleus")
+            out.append(int(tok))
     return out

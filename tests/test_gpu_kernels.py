@@ -452,13 +452,12 @@ def test_sample_top_p_gives_the_same_id_every_time_and_at_the_models_vocabulary(
         assert first[r].item() == P.sample_id(logits[r].tolist(), 0.9, 0.73, 40 + r)[0], r
 
 
-@pytest.mark.parametrize("wide", [False, True])
 @pytest.mark.parametrize("V", [777, 9000, 65536])
-def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_side(ops, V, wide):
-    """What the recorded decode step ends with, in one kernel and (``wide``) in three with the weights by many blocks:
-    rows that are greedy, rows that draw from the whole row and rows that draw from a nucleus, each with its own draw
-    per step; ids against the plain sampler's, the rows' steps, positions and key counts advanced, a non-finite row
-    marked."""
+def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_side(ops, V):
+    """What the recorded decode step ends with when rows draw (three kernels, the weights by many blocks): rows that are
+    greedy, rows that draw from the whole row and rows that draw from a nucleus, each with its own draw per step; ids
+    against the plain sampler's, the rows' steps, positions and key counts advanced, a non-finite row marked.  And the
+    one kernel for steps in which every row is greedy."""
     rows, steps = 6, 3
     logits = torch.randn(rows, V, generator=gen(5)) * 2
     logits[5, 13] = float("inf")
@@ -477,10 +476,10 @@ def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_sid
     pos, kv, live = i32([10, 11, 12, 13, 14, 15]), i32([11, 12, 13, 14, 15, 16]), i32([1, 1, 1, 0, 1, 1])
     wbuf = torch.full((rows * V,), float("nan"), dtype=torch.float64, device=DEV)
     scratch = (torch.full((rows * ops.choice_parts(V),), float("nan"), dtype=torch.float64, device=DEV), i32([7] * rows),
-               i32([7] * rows), torch.full((rows * ops.choice_hist(),), 12345, dtype=torch.int64, device=DEV)) if wide else None
+               i32([7] * rows), torch.full((rows * ops.choice_hist(),), 12345, dtype=torch.int64, device=DEV))
     for step in range(steps):
         ops.decode_choose(dev(logits), dev(torch.tensor(temp, dtype=torch.float64)), dev(u), counter, nxt, ring, bad, pos, kv,
-                          live, top_p=dev(torch.tensor(top_p, dtype=torch.float64)), wbuf=wbuf, wide=scratch)
+                          live, scratch, top_p=dev(torch.tensor(top_p, dtype=torch.float64)), wbuf=wbuf)
     assert counter.tolist() == [steps] * rows
     assert pos.tolist() == [13, 14, 15, 13, 17, 18] and kv.tolist() == [14, 15, 16, 14, 18, 19]     # row 3 is not live
     assert bad[:, :5].sum().item() == 0 and bad[:, 5].tolist() == [1] * steps
@@ -493,6 +492,16 @@ def test_the_decode_loops_choice_draws_greedy_plain_and_nucleus_rows_side_by_sid
                 want = P.sample_id(logits[r].tolist(), temp[r], top_p[r], states[r][step])[0]
             assert int(got[step, r]) == want, (step, r)
     assert nxt.tolist()[:5] == got[steps - 1].tolist()[:5]
+    # all greedy, in one kernel
+    counter, pos, kv = i32([0, 1, 2, 0, 1, 2]), i32([10] * rows), i32([11] * rows)
+    ring.fill_(-1); bad.fill_(-1)
+    ops.decode_choose_greedy(dev(logits), counter, nxt, ring, bad, pos, kv, live)
+    assert counter.tolist() == [1, 2, 3, 1, 2, 3] and pos.tolist() == [11, 11, 11, 10, 11, 11]
+    for r in range(rows):
+        step = [0, 1, 2, 0, 1, 2][r]
+        assert int(bad[step, r]) == (1 if r == 5 else 0)
+        if r < 5:
+            assert int(ring[step, r]) == int(logits[r].argmax()) == int(nxt[r])
 
 
 # ------------------------------------------------------------------ the weight-streaming product
