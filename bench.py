@@ -81,8 +81,10 @@ def kv_bytes(cfg, engine, lengths) -> int:
     return kv + conv
 
 
-def decode_run(engine, cfg, batch: int, prompt_len: int, steps: int, warmup: int, seed: int):
-    """Prefill `batch` random prompts, then time `steps` decode steps.  Returns (seconds, mean context)."""
+def decode_run(engine, cfg, batch: int, prompt_len: int, steps: int, warmup: int, seed: int, temperature: float = 0.0,
+               top_p: float = 1.0):
+    """Prefill `batch` random prompts, then time `steps` decode steps (greedy, or with `temperature` > 0 every row
+    drawing, from its nucleus with `top_p` < 1).  Returns (seconds, mean context)."""
     from gesso_amd.engine.decode import DecodeLoop
     g = torch.Generator().manual_seed(seed)
     rids = [("bench", seed, i) for i in range(batch)]
@@ -97,7 +99,11 @@ def decode_run(engine, cfg, batch: int, prompt_len: int, steps: int, warmup: int
         logits = engine.step([StepEntry(r, p, [prompt_len - 1]) for r, p in zip(rids[at:at + n], prompts[at:at + n])])
         first += logits.argmax(1).tolist()
         at += n
-    loop = DecodeLoop(engine, rids, first)
+    samplers = None
+    if temperature > 0:
+        from gesso_amd import Sampler
+        samplers = [Sampler(temperature, top_p, seed + i) for i in range(batch)]
+    loop = DecodeLoop(engine, rids, first, samplers)
     loop.run(warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -315,6 +321,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--temperature", type=float, default=0.0, help="the main decode run draws at this temperature (0: greedy)")
+    ap.add_argument("--top-p", type=float, default=1.0, help="with --temperature: draws from the nucleus of this mass")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     ap.add_argument("--only-prefill", action="store_true", help="measure the 2,048-token prefill alone (for profiling)")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the measurement of what the machine delivers")
@@ -356,7 +364,8 @@ def main() -> int:
         print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tok_s": round(2048 / sec, 1)}))
         return 0
 
-    dt, mean_ctx = decode_run(engine, cfg, args.batch, prompt_len, args.steps, args.warmup, seed=1)
+    dt, mean_ctx = decode_run(engine, cfg, args.batch, prompt_len, args.steps, args.warmup, seed=1,
+                              temperature=args.temperature, top_p=args.top_p)
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     bytes_step = wbytes + kv_bytes(cfg, engine, [mean_ctx] * args.batch)
@@ -385,6 +394,11 @@ def main() -> int:
             steps = min(args.steps, 128)
             dtb, _ = decode_run(engine, cfg, b, prompt_len, steps, min(args.warmup, 8), seed=10 + b)
             points[name] = round(b * steps / dtb, 1)
+        # the same batch as the headline with every row drawing: at a temperature, and from a nucleus
+        for name, tp in (("decode_b%d_temperature" % args.batch, 1.0), ("decode_b%d_top_p" % args.batch, 0.9)):
+            steps = min(args.steps, 128)
+            dtb, _ = decode_run(engine, cfg, args.batch, prompt_len, steps, min(args.warmup, 8), seed=30, temperature=0.8, top_p=tp)
+            points[name] = round(args.batch * steps / dtb, 1)
         out["points"] = points
         T = 2048
         sec = prefill_run(engine, cfg, T)

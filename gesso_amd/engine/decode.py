@@ -242,7 +242,8 @@ class DecodeRunner:
 
 
 class DecodeLoop:
-    """Continue requests whose prompts are in the cache: ``run(n)`` makes ``n`` greedy steps for all of them."""
+    """Continue requests whose prompts are in the cache: ``run(n)`` makes ``n`` steps for all of them (greedy, or each
+    row with its sampler)."""
 
     def __init__(self, engine, rids: Sequence[Hashable], first_tokens: Sequence[int], samplers=None):
         self.engine = engine
