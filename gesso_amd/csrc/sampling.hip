@@ -123,7 +123,7 @@ struct Crossing {
 // The first passes read the whole row.  Once a pass has narrowed the candidates down to NUC_LIST or fewer (after its
 // second byte the weights left lie within a few percent of each other, a handful in a peaked row), their ids are
 // gathered into a list in LDS and the later passes read only those.
-#define NUC_LIST 2048
+#define NUC_LIST 8192
 //
 // ghist, when given: the histograms of the first two bytes, made ahead by many blocks (choose_weights_kernel) with the
 // scales that passes 0 and 1 use here: NUC_G0 sums for the first byte (0x3B, standing for everything below 2^-63, to
