@@ -103,7 +103,7 @@ class Scheduled:
 
 class Scheduler:
     def __init__(self, executor, choose: Callable, max_num_seqs: int = 64, max_num_batched_tokens: int = 2048,
-                 chunk_size: int = 1024, decode_run_steps: int = 8, watermark: float = 0.01):
+                 chunk_size: int = 1024, decode_run_steps: int = 16, watermark: float = 0.01):
         """``executor``: ``add_request``, ``finish_request``, ``step(entries) -> logits`` and ``manager``.
 
         ``choose(logits, samplers) -> ids or exceptions``, one per row.
