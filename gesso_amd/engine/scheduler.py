@@ -27,7 +27,8 @@ Decisions, all tested without a GPU:
 * The token that ends a request (an id in ``eos_ids``/``stop_ids``) is returned and never fed.
 * When a step holds nothing but decoding requests and the executor has a recorded decode loop
   (``decode``), several steps run back to back on the device: as many as every request still has
-  tokens to generate, at most ``decode_run_steps``, and one only while requests wait for admission.
+  tokens to generate, at most ``decode_run_steps``, and one only while requests wait for admission
+  (more requests than the loop takes at once go through it in groups, one group after the other).
   Tokens come back together; a request that ends within the run (end token, callback) keeps its
   tokens up to there, what the device computed beyond is dropped with the request's cache.
 """
@@ -309,7 +310,8 @@ class Scheduler:
     def _decode_run(self, plan: List[Scheduled]) -> Optional[List[Tuple[Request, int]]]:
         """Several decode steps at once through the executor's recorded loop, when the plan allows it."""
         ex = self.executor
-        if not hasattr(ex, "decode") or len(plan) > getattr(ex, "DECODE_MAX_BATCH", 0):
+        most = getattr(ex, "DECODE_MAX_BATCH", 0)
+        if not hasattr(ex, "decode") or most < 1:
             return None
         if not all(s.count == 1 and s.samples for s in plan):
             return None
@@ -320,10 +322,16 @@ class Scheduler:
         n = min(n, min(self.manager.max_length - r.computed for r in reqs))    # schedule() left each room for one
         while n > 1 and self._pages_short([Scheduled(r, r.computed, n, True) for r in reqs]):
             n -= 1
-        ids, bad = ex.decode([r.rid for r in reqs], [r.last_token for r in reqs], n, [r.sampler for r in reqs])
+        # more requests than the recorded loop takes at once go through it in groups, one after the other (the pages
+        # of all of them were counted above, so no group finds the pool short)
+        runs = []
+        for a in range(0, len(reqs), most):
+            group = reqs[a:a + most]
+            runs.append(ex.decode([r.rid for r in group], [r.last_token for r in group], n, [r.sampler for r in group]))
         self.stats["steps"] += n
         emitted: List[Tuple[Request, int]] = []
-        for i, r in enumerate(reqs):
+        for j, r in enumerate(reqs):
+            (ids, bad), i = runs[j // most], j % most
             if r.computed < len(r.prompt):
                 self.stats["prompt_tokens"] += 1      # a prompt of one token decodes from its first step
             r.computed += n

@@ -79,6 +79,21 @@ def test_greedy_bfloat16_picks_tokens_the_plain_logits_support(folders, name, po
             assert float(row.max() - row[g[i]]) <= 1.5e-2 * max(1.0, float(row.abs().max())), (i, g[i])
 
 
+def test_seventy_requests_at_once_decode_through_the_recorded_loop_in_groups(plain):
+    """More requests than the recorded loop takes at once (64): a group of 64 and a group of 6 per run; every request's
+    tokens are the plain greedy ones."""
+    from gesso_amd import Session
+    d, cfg, w = plain["A"]
+    s = Session(d, dtype="float32", context_length=64, max_num_seqs=80, max_tokens=80 * 64)
+    prompts = [random_ids(2 + i % 7, cfg["V"], 700 + i) for i in range(70)]
+    got = s.generate(prompts, max_new_tokens=6, eos_ids=())
+    for i in (0, 13, 63, 64, 69):
+        assert got[i] == P.greedy(cfg, w, prompts[i], 6), i
+    assert sorted(s.engine._runners) == [8, 64]          # capacities of the groups: 64, and 6 rounded up
+    st = s.engine.manager.stats()
+    assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+
+
 def test_temperature_sampling_follows_the_plain_sampler(plain):
     from gesso_amd import Sampler, Session
     d, cfg, w = plain["B"]

@@ -282,6 +282,19 @@ def test_decode_runs_of_several_steps():
     assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
 
 
+def test_more_requests_than_the_recorded_loop_takes_run_through_it_in_groups():
+    """Six decoding requests, a loop that takes four at once: every run of steps goes through it as a group of four and
+    a group of two, and every request gets what it gets alone."""
+    eng, s = make(FakeDecodeEngine(), decode_run_steps=4, max_num_seqs=6)
+    reqs = [s.add(Request(chr(97 + i), [i + 1, i + 2], max_new_tokens=6 + i)) for i in range(6)]
+    s.run()
+    for i, r in enumerate(reqs):
+        assert r.tokens == expected([i + 1, i + 2], 6 + i), i
+    sizes = [len(rids) for rids, _ in eng.runs]
+    assert max(sizes) == 4 and [4, 2] == sizes[:2]
+    assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+
+
 def test_a_request_that_ends_inside_a_run_keeps_its_tokens_up_to_there():
     full = expected([4, 5], 10)
     eos = full[2 + 3]
