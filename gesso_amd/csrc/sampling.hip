@@ -122,8 +122,10 @@ struct Crossing {
 //
 // The first passes read the whole row.  Once a pass has narrowed the candidates down to NUC_LIST or fewer (after its
 // second byte the weights left lie within a few percent of each other, a handful in a peaked row), their ids are
-// gathered into a list in LDS and the later passes read only those.
+// gathered into a list in LDS and the later passes read only those; a list of NUC_DIRECT ids or fewer is
+// settled at once, a candidate to a thread.
 #define NUC_LIST 8192
+#define NUC_DIRECT 256
 //
 // ghist, when given: the histograms of the first two bytes, made ahead by many blocks (choose_weights_kernel) with the
 // scales that passes 0 and 1 use here: NUC_G0 sums for the first byte (0x3B, standing for everything below 2^-63, to
@@ -136,6 +138,7 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
                                   unsigned long long* hmass, int* hcount, Crossing* shared_out, int* clist,
                                   const unsigned long long* __restrict__ ghist = nullptr) {
   __shared__ int cn, picked;
+  __shared__ unsigned long long cbits[NUC_DIRECT], cmass[NUC_DIRECT];
   unsigned long long prefix = 0;
   double above = 0.0;
   int lv = 1;                                   // V <= 2^lv
@@ -257,6 +260,52 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
         if (((unsigned long long)__double_as_longlong(w[j]) & sofar) == prefix) clist[atomicAdd(&cn, 1)] = j;
       __syncthreads();
       nlist = cn;
+      if (nlist <= NUC_DIRECT) {
+        // a candidate to a thread: no more passes.  Each adds up the masses of the candidates heavier than its own
+        // and of those as heavy (integers, scaled to the largest weight under the prefix); the pattern at which the
+        // running sum crosses the target is the one whose candidates see the target between these two sums
+        const int t = threadIdx.x;
+        const double top = __longlong_as_double((long long)(prefix | ((1ull << shift) - 1ull)));
+        const double sc = exp2((double)(62 - lv)) / top, unsc = 1.0 / sc;
+        unsigned long long mybits = 0ull;
+        if (t < nlist) {
+          const double wt = w[clist[t]];
+          mybits = (unsigned long long)__double_as_longlong(wt);
+          cbits[t] = mybits;
+          cmass[t] = (unsigned long long)__double2ll_rn(wt * sc);
+        }
+        if (t == 0) {
+          cn = 0x7fffffff;      // the lowest thread at the crossing
+          picked = 0x7fffffff;  // the lowest thread with the lightest pattern, should nothing cross
+        }
+        __syncthreads();
+        unsigned long long heavier = 0ull, same = 0ull, lightest = ~0ull;
+        for (int j = 0; t < nlist && j < nlist; ++j) {
+          const unsigned long long b = cbits[j], m = cmass[j];
+          heavier += b > mybits ? m : 0ull;
+          same += b == mybits ? m : 0ull;
+          lightest = b < lightest ? b : lightest;
+        }
+        if (t < nlist) {
+          const double lo = above + (double)heavier * unsc, hi = above + (double)(heavier + same) * unsc;
+          const bool crossed = strict ? (target < hi && !(target < lo)) : (hi >= target && !(lo >= target));
+          if (crossed) atomicMin(&cn, t);
+          if (mybits == lightest) atomicMin(&picked, t);
+        }
+        __syncthreads();
+        const int owner = cn != 0x7fffffff ? cn : picked;
+        if (t == owner) {
+          shared_out->bits = mybits;
+          shared_out->above = above + (double)heavier * unsc;
+        }
+        __syncthreads();
+        Crossing c;
+        c.bits = shared_out->bits;
+        c.above = shared_out->above;
+        c.nlist = nlist;
+        __syncthreads();
+        return c;
+      }
     }
   }
   Crossing c;
