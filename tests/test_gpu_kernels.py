@@ -432,6 +432,25 @@ def test_sample_top_p_follows_the_plain_sampler(ops, V, temp, top_p):
     assert ids.tolist() == want and not any(bad.tolist())
 
 
+def test_sample_top_p_where_the_nucleus_edge_lies_among_weights_too_small_for_the_ready_histograms(ops):
+    """One id carries nearly all the mass, tens of thousands of others a weight of about 2^-64 each, and top_p is so
+    close to 1 that the nucleus' edge falls among those: the histograms that the many blocks make resolve weights from
+    2^-63 up only, so the descent starts again and reads the row itself.  The draws land where the plain sampler's do."""
+    V, rows, T = 65536, 4, 1.0
+    logits = torch.full((rows, V), -64.06 * math.log(2.0))
+    for r in range(rows):
+        logits[r, V - 1 - 7 * r] = 0.0                   # the heavy id late in the row: the small weights add up before it
+    top_p = 1.0 - 2.0 ** -50
+    want, us = [], []
+    for r in range(rows):
+        want.append(P.sample_id(logits[r].tolist(), T, top_p, 77 + r)[0])
+        us.append(P.splitmix64_unit(77 + r)[1])
+    ids, bad = ops.sample_top_p(logits.to(DEV), torch.full((rows,), T, dtype=torch.float64, device=DEV),
+                                torch.full((rows,), top_p, dtype=torch.float64, device=DEV),
+                                torch.tensor(us, dtype=torch.float64, device=DEV))
+    assert ids.tolist() == want and not any(bad.tolist())
+
+
 def test_sample_top_p_gives_the_same_id_every_time_and_at_the_models_vocabulary(ops):
     """The histogram's masses are integer sums, so no order of the threads' additions can move an edge; a row of
     65,536 logits with thousands of weights that differ in their last bits, drawn many times with the same draw."""
