@@ -1,9 +1,9 @@
 """Device memory of the cache: pages per group, state per slot.
 
-Pages of a group: one tensor ``(members, 2, num_pages + 1, n_kv_heads, page_size, head_dim)`` in the
-activation type; index 0/1 of the second axis is K/V, so that a page id addresses the same page
-in every layer of the group.  A head's rows of a page are contiguous (``page_size x head_dim``),
-which is what the attention kernels stream.  Slot state: per state-keeping layer and state
+Pages of a group: a key tensor ``(members, num_pages + 1, n_kv_heads, page_size, head_dim)`` and a value tensor
+of the same shape but for its last axis (the group's value width, which may differ from the key's or be zero),
+in the activation type; a page id addresses the same page in both and in every layer of the group.  A head's rows
+of a page are contiguous (``page_size x width``), which is what the attention kernels stream.  Slot state: per state-keeping layer and state
 name a tensor ``(num_slots + 1, *shape)`` of the type the layer asked for (float32 or bfloat16), with the value a
 fresh slot starts from in ``state_init``.  The extra page and the extra slot at the end
 belong to no request: padded entries of a fixed-size batch write there.
@@ -25,8 +25,8 @@ _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 class PagedView:
     """What an attention-like mixer sees of its cache in one step."""
 
-    k: torch.Tensor                  # (num_pages + 1, nkv, page_size, d)
-    v: torch.Tensor
+    k: torch.Tensor                  # (num_pages + 1, nkv, page_size, head_dim)
+    v: torch.Tensor                  # (num_pages + 1, nkv, page_size, value width)
     block_table: torch.Tensor        # int32 (nseq, max_blocks) of this step
     page_size: int
     write: bool                      # False: this call reads another call's cache
@@ -46,10 +46,11 @@ class CacheStorage:
             num_pages = [num_pages] * len(layout.paged)
         self.num_pages = list(num_pages)
         self.num_slots = num_slots
-        self.kv = []
+        self.keys, self.values = [], []
         for g, n in zip(layout.paged, num_pages):
-            self.kv.append(torch.zeros((len(g.members), 2, n + 1, g.need.n_kv_heads, page_size, g.need.head_dim),
-                                       dtype=dtype, device=device))
+            lead = (len(g.members), n + 1, g.need.n_kv_heads, page_size)
+            self.keys.append(torch.zeros(lead + (g.need.head_dim,), dtype=dtype, device=device))
+            self.values.append(torch.zeros(lead + (g.need.value_width,), dtype=dtype, device=device))
         self.member_index = {c: i for g in layout.paged for i, c in enumerate(g.members)}
         self.state: Dict[int, Dict[str, torch.Tensor]] = {}
         self.state_init: Dict[int, Dict[str, float]] = {}
@@ -76,8 +77,8 @@ class CacheStorage:
         write = src == call
         if src in self.layout.group_of_call:
             g = self.layout.group_of_call[src]
-            kv = self.kv[g][self.member_index[src]]
-            return PagedView(kv[0], kv[1], block_tables[g], self.page_size, write)
+            i = self.member_index[src]
+            return PagedView(self.keys[g][i], self.values[g][i], block_tables[g], self.page_size, write)
         if src in self.state:
             return SlotView(self.state[src], write)
         return None
@@ -96,19 +97,20 @@ class CacheStorage:
 
     def fill_pages(self, ops, group: int, pages, value: float) -> None:
         """Every layer's keys and values of the given pages of one group."""
-        kv = self.kv[group]
-        ids = torch.tensor(list(pages), dtype=torch.int32, device=kv.device)
-        ops.fill_rows(kv, ids, value, planes=3)          # (members, 2) planes of (pages + 1) rows
+        ids = torch.tensor(list(pages), dtype=torch.int32, device=self.keys[group].device)
+        for pool in (self.keys[group], self.values[group]):
+            if pool.numel():
+                ops.fill_rows(pool, ids, value, planes=2)          # a plane of (pages + 1) rows per member
 
     def poison_all(self) -> None:
         """NaN everywhere but in the spare page and slot (padded rows of a recorded batch compute on those)."""
-        for kv in self.kv:
-            kv[:, :, :-1].fill_(float("nan"))
+        for pool in self.keys + self.values:
+            pool[:, :-1].fill_(float("nan"))
         for states in self.state.values():
             for t in states.values():
                 t[:-1].fill_(float("nan"))
 
     def bytes(self) -> int:
-        n = sum(t.numel() * t.element_size() for t in self.kv)
+        n = sum(t.numel() * t.element_size() for t in self.keys + self.values)
         n += sum(t.numel() * t.element_size() for d in self.state.values() for t in d.values())
         return n

@@ -7,6 +7,15 @@ pattern and per-layer scalars are refused (``:66-86``), the short convolution's 
 length must exceed one (``src/Inference/architecture_spec.jl:175``).  The HF-style keys,
 ``layer_types`` / ``full_attn_idxs`` and the ``block_ff_dim`` adjustment have no reader in
 the reference and follow the architecture's published config.json.
+
+The feed-forward width.  The reference's metadata carries the width the SwiGLU really has
+(``feed_forward_length``, ``src/Inference/lfm2.jl:145``).  A config.json carries the width *before* the
+architecture's adjustment, under ``block_ff_dim`` or, in files serialised by newer writers, under
+``intermediate_size`` (one is an alias of the other); while ``block_auto_adjust_ff_dim`` is true, which
+it is when the file leaves it out, the SwiGLU has two thirds of it, scaled by
+``block_ffn_dim_multiplier`` and rounded up to ``block_multiple_of``.  A file that means its
+``intermediate_size`` as the SwiGLU's own width says ``block_auto_adjust_ff_dim: false``;
+:meth:`Lfm2Config.to_json` writes that for a configuration built with a direct width.
 """
 from __future__ import annotations
 
@@ -62,11 +71,13 @@ _KNOWN = frozenset({
 
 
 def adjusted_ff_dim(block_ff_dim: int, multiple_of: int, multiplier: Optional[float]) -> int:
-    """Width of the SwiGLU: two thirds of ``block_ff_dim``, scaled, rounded up to ``multiple_of``."""
+    """Width of the SwiGLU: two thirds of ``block_ff_dim``; with a multiplier, scaled by it and rounded up to
+    ``multiple_of`` (without one, two thirds and nothing more)."""
     ff = int(2 * block_ff_dim / 3)
     if multiplier is not None:
         ff = int(multiplier * ff)
-    return multiple_of * ((ff + multiple_of - 1) // multiple_of)
+        ff = multiple_of * ((ff + multiple_of - 1) // multiple_of)
+    return ff
 
 
 @dataclass(frozen=True)
@@ -196,22 +207,26 @@ class Lfm2Config:
                 raise ConfigError("layer_types and full_attn_idxs disagree")
             types = from_idxs
 
+        # the width before the adjustment, under either name (they must agree where a file has both; a file that
+        # holds the adjusted width beside block_ff_dim, as older writers left it, is taken too)
         block_ff = mult_of = mult = None
-        if "intermediate_size" in raw and "block_ff_dim" not in raw:
-            ff = need("intermediate_size", int)
+        if "block_ff_dim" not in raw and "intermediate_size" not in raw:
+            raise ConfigError("config.json lacks the feed-forward width: block_ff_dim or intermediate_size",
+                              key="block_ff_dim")
+        block_ff = need("block_ff_dim" if "block_ff_dim" in raw else "intermediate_size", int)
+        if need("block_auto_adjust_ff_dim", bool):
+            mult_of = need("block_multiple_of", int)
+            if mult_of <= 0:
+                raise ConfigError("block_multiple_of must be positive", block_multiple_of=mult_of)
+            mult = need("block_ffn_dim_multiplier", float) if raw.get("block_ffn_dim_multiplier", 1.0) is not None else None
+            ff = adjusted_ff_dim(block_ff, mult_of, mult)
         else:
-            block_ff = need("block_ff_dim", int)
-            if need("block_auto_adjust_ff_dim", bool):
-                mult_of = need("block_multiple_of", int)
-                if mult_of <= 0:
-                    raise ConfigError("block_multiple_of must be positive", block_multiple_of=mult_of)
-                mult = need("block_ffn_dim_multiplier", float) if raw.get("block_ffn_dim_multiplier") is not None else None
-                ff = adjusted_ff_dim(block_ff, mult_of, mult)
-            else:
-                ff = block_ff
-            if "intermediate_size" in raw and raw["intermediate_size"] != ff:
-                raise ConfigError("intermediate_size disagrees with the adjusted block_ff_dim",
-                                  intermediate_size=raw["intermediate_size"], adjusted=ff)
+            ff = block_ff
+        if "block_ff_dim" in raw and "intermediate_size" in raw:
+            given = need("intermediate_size", int)
+            if given not in (block_ff, ff):
+                raise ConfigError("intermediate_size is neither block_ff_dim nor the width adjusted from it",
+                                  intermediate_size=given, block_ff_dim=block_ff, adjusted=ff)
 
         tie = True
         for key in ("tie_word_embeddings", "tie_embedding"):
@@ -268,14 +283,15 @@ class Lfm2Config:
             "tie_word_embeddings": self.tie_word_embeddings,
             "max_position_embeddings": self.max_position_embeddings,
         }
-        if self.block_ff_dim is not None:
+        if self.block_ff_dim is not None and self.block_multiple_of is not None:
             out["block_ff_dim"] = self.block_ff_dim
-            out["block_auto_adjust_ff_dim"] = self.block_multiple_of is not None
-            if self.block_multiple_of is not None:
-                out["block_multiple_of"] = self.block_multiple_of
-                out["block_ffn_dim_multiplier"] = self.block_ffn_dim_multiplier
+            out["block_auto_adjust_ff_dim"] = True
+            out["block_multiple_of"] = self.block_multiple_of
+            out["block_ffn_dim_multiplier"] = self.block_ffn_dim_multiplier
         else:
+            # a direct width: said so, because a reader adjusts whatever width it finds unless told not to
             out["intermediate_size"] = self.intermediate_size
+            out["block_auto_adjust_ff_dim"] = False
         for name in ("eos_token_id", "bos_token_id", "pad_token_id"):
             if getattr(self, name) is not None:
                 out[name] = getattr(self, name)

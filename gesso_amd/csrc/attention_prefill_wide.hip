@@ -65,7 +65,7 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   static_assert(D == 64, "the swizzle of the transposed values is written for heads of 64");
   __shared__ __align__(16) uint16_t ks[2][PW_KS][KROW];
   __shared__ __align__(16) uint16_t vt[2][D][VROW];
-  __shared__ uint32_t rowoff[3][PW_KS];       // where a step's key rows start in the caches, in units of 16 bytes
+  __shared__ __align__(8) uint32_t rowoff[3][PW_KS];       // (read two at a time) where a step's key rows start in the caches, in units of 16 bytes
 
   // blocks in launch order: key head fastest, tiles from the last one back (late tiles walk the most keys)
   const int kvh = blockIdx.x % nkv, tile = (int)(gridDim.x / nkv) - 1 - (int)(blockIdx.x / nkv);

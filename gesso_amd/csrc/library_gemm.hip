@@ -4,7 +4,9 @@
 //
 // What is kept per shape is a plan: the operation's and the operands' descriptors and the algorithm.  The first
 // call of a shape asks the library for its candidate algorithms and, when tuning is asked for, runs each a few
-// times on the operands at hand and keeps the fastest (a few milliseconds a shape); every later call is one
+// times on the operands at hand and keeps the fastest (a few milliseconds a shape; which one wins can differ from
+// process to process, and with it the rounding of a bfloat16 result, so tuning is for measurements: without it the
+// library's first choice runs, the same in every process); every later call is one
 // hipblasLtMatmul with what the plan holds, a few microseconds of host time (torch.mm on the same library spends
 // 20 to 30 us a call on the host, which is what steps of a few hundred tokens were bound by).
 //
@@ -85,6 +87,32 @@ int run(hipblasLtHandle_t handle, const Plan& p, const void* X, const void* W, v
   return 0;
 }
 
+void destroy_plan(Plan& p) {
+  if (p.desc) (void)hipblasLtMatmulDescDestroy(p.desc);
+  if (p.a) (void)hipblasLtMatrixLayoutDestroy(p.a);
+  if (p.b) (void)hipblasLtMatrixLayoutDestroy(p.b);
+  if (p.c) (void)hipblasLtMatrixLayoutDestroy(p.c);
+  p.desc = nullptr;
+  p.a = p.b = p.c = nullptr;
+}
+
+// At most this many plans are kept.  A server sees a new row count in almost every step of mixed work; when the table is
+// full the plans that were not tuned go (making one again costs some tens of microseconds), the tuned ones stay.
+constexpr size_t MAX_PLANS = 512;
+
+void make_room() {
+  if (g_plans.size() < MAX_PLANS) return;
+  for (auto it = g_plans.begin(); it != g_plans.end();) {
+    if (std::get<7>(it->first) == 0) {
+      destroy_plan(it->second);
+      it = g_plans.erase(it);
+    } else {
+      ++it;
+    }
+  }
+}
+
+// Fills `p`; on failure whatever it has created so far is left in `p` for the caller to destroy.
 int make_plan(hipblasLtHandle_t handle, Plan& p, const void* X, int ldx, const void* W, void* Y, int ldy, int M, int N, int K,
               void* ws, size_t ws_bytes, int tune, hipStream_t stream) {
   LT_REQUIRE(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "operation descriptor");
@@ -97,8 +125,12 @@ int make_plan(hipblasLtHandle_t handle, Plan& p, const void* X, int ldx, const v
   hipblasLtMatmulPreference_t pref = nullptr;
   LT_REQUIRE(hipblasLtMatmulPreferenceCreate(&pref), "preference");
   const uint64_t max_ws = ws_bytes;
-  LT_REQUIRE(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws)),
-             "workspace limit");
+  {
+    const hipblasStatus_t sp = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws,
+                                                                     sizeof(max_ws));
+    if (sp != HIPBLAS_STATUS_SUCCESS) (void)hipblasLtMatmulPreferenceDestroy(pref);
+    LT_REQUIRE(sp, "workspace limit");
+  }
   constexpr int WANT = 24;
   std::vector<hipblasLtMatmulHeuristicResult_t> found(WANT);
   int n = 0;
@@ -114,8 +146,9 @@ int make_plan(hipblasLtHandle_t handle, Plan& p, const void* X, int ldx, const v
   float best_ms = 0.f;
   void* flush = tune && n > 1 ? flush_buffer() : nullptr;
   if (tune && n > 1) {
-    hipEvent_t e0, e1;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+      if (e0) (void)hipEventDestroy(e0);
       gs_set_error("library_gemm: no events for the tuning run");
       return -2;
     }
@@ -206,7 +239,11 @@ extern "C" int gs_library_gemm(const void* X, int ldx, const void* W, void* Y, i
   auto it = g_plans.find(key);
   if (it == g_plans.end()) {
     Plan p;
-    if (int rc = make_plan(handle, p, X, ldx, W, Y, ldy, M, N, K, workspace, (size_t)ws_bytes, tune, stream)) return rc;
+    if (int rc = make_plan(handle, p, X, ldx, W, Y, ldy, M, N, K, workspace, (size_t)ws_bytes, tune, stream)) {
+      destroy_plan(p);
+      return rc;
+    }
+    make_room();
     it = g_plans.emplace(key, p).first;
   }
   return run(handle, it->second, X, W, Y, workspace, stream);

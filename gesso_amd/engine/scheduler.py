@@ -31,6 +31,10 @@ Decisions, all tested without a GPU:
   (more requests than the loop takes at once go through it in groups, one group after the other).
   Tokens come back together; a request that ends within the run (end token, callback) keeps its
   tokens up to there, what the device computed beyond is dropped with the request's cache.
+* A pass that breaks off in the middle (the executor raises :class:`~gesso_amd.errors.StepFailed` and has
+  released the requests of that pass) ends those requests as ``failed`` with the tokens they had; every other
+  request goes on, a group of a decode run that ran before the failing group keeps its tokens
+  (the reference stops only the request whose pass failed, ``src/Runtime/Runtime.jl:175-178``).
 """
 from __future__ import annotations
 
@@ -39,7 +43,7 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Callable, Deque, Hashable, List, Optional, Sequence, Tuple
 
-from ..errors import GessoError, InvalidPlan, OutOfPages, OutOfSlots, ResourceLimit
+from ..errors import GessoError, InvalidPlan, NumericalInstability, OutOfPages, OutOfSlots, ResourceLimit, StepFailed
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
 
@@ -125,7 +129,7 @@ class Scheduler:
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []          # in admission order
         self.finished: List[Request] = []
-        self.stats = {"steps": 0, "preemptions": 0, "prompt_tokens": 0, "decode_tokens": 0}
+        self.stats = {"steps": 0, "preemptions": 0, "prompt_tokens": 0, "decode_tokens": 0, "failed_passes": 0}
 
     # ------------------------------------------------------------------ requests
 
@@ -152,6 +156,20 @@ class Scheduler:
             self.running.remove(r)
         r.status, r.finish_reason, r.error = FINISHED, reason, error
         self.finished.append(r)
+
+    def _fail_pass(self, reqs: Sequence[Request], err: StepFailed) -> None:
+        """The requests of a pass that broke off end as ``failed``.  The executor has released those it names in
+        ``err.detail["requests"]``; one it still holds is released here, its cache being of no use either."""
+        gone = set(err.detail.get("requests", ()))
+        holds = getattr(self.executor, "has_request", None)
+        for r in reqs:
+            if r.status != RUNNING:
+                continue
+            held = r.rid not in gone and (holds is None or holds(r.rid))
+            if not held:
+                self.running.remove(r)
+            self._finish(r, "failed", live=held, error=err)
+        self.stats["failed_passes"] += 1
 
     def _preempt(self, r: Request) -> None:
         self.executor.finish_request(r.rid)
@@ -289,6 +307,9 @@ class Scheduler:
             logits = self.executor.step(entries)
         except OutOfPages:
             raise AssertionError("the plan was checked against the pools and still ran out of pages")
+        except StepFailed as err:
+            self._fail_pass([s.request for s in plan], err)
+            return []
         self.stats["steps"] += 1
         emitted: List[Tuple[Request, int]] = []
         sampling = [s for s in plan if s.samples]
@@ -324,24 +345,26 @@ class Scheduler:
             n -= 1
         # more requests than the recorded loop takes at once go through it in groups, one after the other (the pages
         # of all of them were counted above, so no group finds the pool short)
-        runs = []
+        emitted: List[Tuple[Request, int]] = []
+        self.stats["steps"] += n
         for a in range(0, len(reqs), most):
             group = reqs[a:a + most]
-            runs.append(ex.decode([r.rid for r in group], [r.last_token for r in group], n, [r.sampler for r in group]))
-        self.stats["steps"] += n
-        emitted: List[Tuple[Request, int]] = []
-        for j, r in enumerate(reqs):
-            (ids, bad), i = runs[j // most], j % most
-            if r.computed < len(r.prompt):
-                self.stats["prompt_tokens"] += 1      # a prompt of one token decodes from its first step
-            r.computed += n
-            for s in range(n):
-                if bad[s][i]:
-                    from ..errors import NumericalInstability
-                    self._finish(r, "failed", error=NumericalInstability("non-finite logits: no token is emitted"))
-                    break
-                if self._emit(r, int(ids[s][i]), emitted):
-                    break
+            try:
+                ids, bad = ex.decode([r.rid for r in group], [r.last_token for r in group], n,
+                                     [r.sampler for r in group])
+            except StepFailed as err:
+                self._fail_pass(group, err)      # this group's requests end here; the other groups are untouched
+                continue
+            for i, r in enumerate(group):
+                if r.computed < len(r.prompt):
+                    self.stats["prompt_tokens"] += 1      # a prompt of one token decodes from its first step
+                r.computed += n
+                for s in range(n):
+                    if bad[s][i]:
+                        self._finish(r, "failed", error=NumericalInstability("non-finite logits: no token is emitted"))
+                        break
+                    if self._emit(r, int(ids[s][i]), emitted):
+                        break
         return emitted
 
     def _emit(self, r: Request, tok: int, emitted: List[Tuple[Request, int]]) -> bool:

@@ -65,13 +65,15 @@ class Session:
         kw = dict(page_size=page_size, num_slots=max_num_seqs, options=kernel_options, poison=poison)
         if isinstance(model, (str, os.PathLike)):
             from ..config.registry import load_config
-            _, cfg = load_config(os.fspath(model))
+            arch, cfg = load_config(os.fspath(model))
         else:
+            from ..config.registry import architecture_of
             cfg = model
             if random_weights_seed is None:
                 raise InvalidPlan("a configuration without a folder needs random_weights_seed")
-        max_pos = getattr(cfg, "max_position_embeddings", None) or 4096
-        self.context_length = int(context_length or min(max_pos, 4096))
+            arch = architecture_of(cfg.to_json())
+        # the longest context the model itself allows is a fact of its description, whatever its configuration calls it
+        self.context_length = int(context_length or min(arch.to_spec(cfg).max_position, 4096))
         if num_pages is None and max_tokens is None:
             max_tokens = 4 * self.context_length
         kw.update(num_pages=num_pages, max_tokens=max_tokens, max_context=self.context_length)
@@ -181,7 +183,8 @@ class Session:
                     raise InvalidPlan("the scheduler found nothing to run though requests are left")
         finally:
             for r in list(sched.running):       # an error above: give back what is still held
-                sched.executor.finish_request(r.rid)
+                if sched.executor.has_request(r.rid):
+                    sched.executor.finish_request(r.rid)
         torch.cuda.synchronize(dev)
         t1 = time.perf_counter()
         first = first or t1

@@ -239,6 +239,9 @@ def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
     return t
 
 
+FILL_MAX = 65535
+
+
 def fill_rows(pool: torch.Tensor, ids: torch.Tensor, value: float, planes: int = 1) -> None:
     """``pool[..., id, ...] = value`` for each id in ``ids`` (int32): ``pool`` is ``(planes..., rows, *row shape)`` with
     ``planes`` leading axes flattened into one (1: ``(rows, ...)``), float32 or bfloat16.  A fresh state slot gets its
@@ -251,8 +254,11 @@ def fill_rows(pool: torch.Tensor, ids: torch.Tensor, value: float, planes: int =
         outer *= n
     rows = pool.shape[len(lead)]
     row = pool[(0,) * (len(lead) + 1)].numel() if pool.numel() else 0
-    _check(lib().gs_fill_rows(_p(pool), c_int(_dt(pool)), _p(ids), c_int(ids.numel()), c_long(row), c_int(outer),
-                              c_long(rows), c_float(value), _stream()))
+    _need(outer <= FILL_MAX, f"fill_rows: {outer} planes are more than a launch takes ({FILL_MAX})")
+    for at in range(0, ids.numel(), FILL_MAX):            # a launch takes 65,535 ids: many freed pages go in turns
+        part = ids[at:at + FILL_MAX]
+        _check(lib().gs_fill_rows(_p(pool), c_int(_dt(pool)), _p(part), c_int(part.numel()), c_long(row), c_int(outer),
+                                  c_long(rows), c_float(value), _stream()))
 
 
 # ---------------------------------------------------------------------- short convolution

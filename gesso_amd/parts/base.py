@@ -42,7 +42,9 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class PagedKV:
-    """Per-token state: keys and values of ``n_kv_heads x head_dim`` per token, kept in pages.
+    """Per-token state kept in pages: per token and key head a key row of ``head_dim`` and a value row of
+    ``value_dim`` numbers (None: as wide as the key; 0: no value rows at all, for a mixer that caches one row per
+    token and derives both from it).
 
     ``window``: only the last ``window`` tokens are ever read again (None = all of them).
     """
@@ -50,6 +52,11 @@ class PagedKV:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else int(self.value_dim)
 
 
 @dataclass(frozen=True)

@@ -35,7 +35,9 @@ class RuntimeOptions:
     ``tune_library``: where the vendor library computes a product of 512, 1024, 2048, ... rows (whole prompt portions),
     the first product of a shape measures the library's two dozen best guesses on the operands at hand, cold, and
     keeps the library's first choice unless another is clearly faster (some ten milliseconds a shape).  Other row
-    counts, and all with this off, take the library's first choice.
+    counts, and all with this off, take the library's first choice.  Off unless asked for: which candidate a
+    measurement prefers can differ between two processes, and with it the rounding of prompt logits, so that one seed
+    would no longer give the same ids in every run; the benchmark switches it on.
     ``prompt_attention``: attention of prompt portions in bfloat16: ``"wide"`` = the kernel for long portions wherever it
     takes the sizes (heads of 64), ``"tiles"`` = the kernel with tiles of 16 or 32 queries always, ``"auto"`` = the
     first for steps with a portion of at least 64 tokens, else the second.
@@ -50,7 +52,7 @@ class RuntimeOptions:
     """
 
     many_rows: str = "auto"
-    tune_library: bool = True
+    tune_library: bool = False
     prompt_attention: str = "auto"
     tiled_rows: bool = True
     tile_weights: bool = True

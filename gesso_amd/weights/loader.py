@@ -127,7 +127,7 @@ def write_model_folder(out_dir: str, config, seed: int, dtype: torch.dtype = tor
     os.makedirs(out_dir, exist_ok=True)
     with open(os.path.join(out_dir, "config.json"), "w", encoding="utf-8") as f:
         json.dump(raw, f, indent=1)
-    tensors = random_tensors(tensor_table(spec), seed, dtype)
+    tensors = random_tensors(tensor_table(spec), seed, dtype, std=std)
     write_safetensors(os.path.join(out_dir, "model.safetensors"), tensors,
                       metadata={"format": "pt", "seed": str(seed)})
     return out_dir

@@ -15,11 +15,42 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TRACE_RUN = os.path.join(ROOT, "bin", "trace_run")
 
 
-def plain_logits(model_dir: str, ids) -> np.ndarray:
-    """(T, V) float64 logits of the whole sequence by the plain implementation."""
+def plain_logits(model_dir: str, ids, rounded: bool = False) -> np.ndarray:
+    """(T, V) float64 logits of the whole sequence by the plain implementation; ``rounded``: with its activations
+    rounded to bfloat16 wherever a pipeline with bfloat16 activations stores one."""
     cfg = P.read_config(model_dir)
     w = P.read_weights(model_dir, torch.float64)
-    return P.forward(cfg, w, list(ids)).numpy()
+    return P.forward(cfg, w, list(ids), **({"store": P.to_bfloat16} if rounded else {})).numpy()
+
+
+class Plain:
+    """The plain logits of some sequences (``ref``), the rounded model's for bfloat16 (``rounded``), and the
+    comparison of an engine's rows with them: float32 to ``1e-4 x max(1, max |ref|)`` at the worst logit (the
+    reference's own device bound, ``test/test_amdgpu_lfm2.jl:34``), bfloat16 to the rounded model's own distance
+    (``tests/noise.py``)."""
+
+    F32 = 1e-4
+
+    def __init__(self, model_dir: str, seqs: dict, dtype: str):
+        self.dtype = dtype
+        self.ref = {k: plain_logits(model_dir, ids) for k, ids in seqs.items()}
+        self.rounded = {k: plain_logits(model_dir, ids, rounded=True) for k, ids in seqs.items()} \
+            if dtype == "bfloat16" else None
+        self.scale = max(1.0, max(float(np.abs(r).max()) for r in self.ref.values()))
+
+    def check(self, got: dict, label: str) -> None:
+        """``got``: {sequence name: {position: logits row}}."""
+        if self.dtype == "float32":
+            w, where = worst(got, self.ref)
+            print(f"{label} float32: worst |diff| {w:.3e} at {where} (bound {self.F32 * self.scale:.3e})")
+            assert w <= self.F32 * self.scale, f"{label}: first look at {where}"
+            return
+        from noise import NoiseBound
+        b = NoiseBound()
+        for name, rows in got.items():
+            for pos, row in rows.items():
+                b.add(row, self.ref[name][pos], self.rounded[name][pos], (name, pos))
+        b.check(label)
 
 
 def round64(n: int) -> int:

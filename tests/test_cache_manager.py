@@ -189,3 +189,26 @@ def test_random_orders_of_requests(seed, page_size, num_pages, num_slots):
         m.release(rid)
     m.check()
     assert m.stats()["pages_free"] == [num_pages, max(2, num_pages // 2)] and m.stats()["slots_free"] == num_slots
+
+
+def test_keys_and_values_of_different_widths_get_pools_of_their_own():
+    """A mixer may keep values wider or narrower than its keys, or none at all (one cached row per token): its layers
+    form a group apart from layers with equal widths, and the storage gives the group a key pool and a value pool of
+    the widths asked for, addressed by the same page ids."""
+    import torch
+    from gesso_amd.cache.storage import CacheStorage
+    wide = PagedKV(2, 16, None, value_dim=40)
+    latent = PagedKV(1, 24, None, value_dim=0)
+    lay = CacheLayout.plan([FULL, wide, CONV, latent, wide, FULL], [None] * 6)
+    assert [g.need for g in lay.paged] == [FULL, wide, latent] and [g.members for g in lay.paged] == [(0, 5), (1, 4), (3,)]
+    st_ = CacheStorage(lay, page_size=4, num_pages=[5, 6, 7], num_slots=2, dtype=torch.float32, device="cpu")
+    assert st_.keys[0].shape == (2, 6, 2, 4, 16) and st_.values[0].shape == (2, 6, 2, 4, 16)
+    assert st_.keys[1].shape == (2, 7, 2, 4, 16) and st_.values[1].shape == (2, 7, 2, 4, 40)
+    assert st_.keys[2].shape == (1, 8, 1, 4, 24) and st_.values[2].shape == (1, 8, 1, 4, 0)
+    tables = [torch.zeros(1, 2, dtype=torch.int32)] * 3
+    v = st_.view(4, tables)
+    assert v.k.shape == (7, 2, 4, 16) and v.v.shape == (7, 2, 4, 40) and v.write
+    assert v.k.data_ptr() == st_.keys[1][1].data_ptr()
+    assert st_.view(3, tables).v.numel() == 0
+    assert st_.bytes() == 4 * sum(t.numel() for t in st_.keys + st_.values) + 4 * sum(
+        t.numel() for d in st_.state.values() for t in d.values())

@@ -63,16 +63,47 @@ def test_layer_types_and_idxs_agree():
         Lfm2Config.from_dict(raw)
 
 
-def test_direct_intermediate_size():
-    raw = {k: v for k, v in BASE.items() if not k.startswith("block_ff") and k not in
-           ("block_auto_adjust_ff_dim", "block_multiple_of")}
-    raw["intermediate_size"] = 1000
-    assert Lfm2Config.from_dict(raw).intermediate_size == 1000
-    raw = dict(BASE, intermediate_size=8000)
-    with pytest.raises(ConfigError, match="disagrees"):
-        Lfm2Config.from_dict(raw)
-    raw = dict(BASE, block_auto_adjust_ff_dim=False)
-    assert Lfm2Config.from_dict(raw).intermediate_size == 12288
+def test_the_feed_forward_width_under_either_name():
+    """``intermediate_size`` is another name of ``block_ff_dim``: the width before the adjustment, which applies while
+    ``block_auto_adjust_ff_dim`` is true or left out.  A direct width needs ``block_auto_adjust_ff_dim: false``."""
+    bare = {k: v for k, v in BASE.items() if not k.startswith("block_ff") and k not in
+            ("block_auto_adjust_ff_dim", "block_multiple_of")}
+    # a file as newer writers serialise LFM2-1.2B: the width before the adjustment under intermediate_size
+    for extra in ({}, {"block_auto_adjust_ff_dim": True}, {"block_auto_adjust_ff_dim": True, "block_multiple_of": 256,
+                                                           "block_ffn_dim_multiplier": 1.0}):
+        c = Lfm2Config.from_dict(dict(bare, intermediate_size=12288, **extra))
+        assert c.intermediate_size == 8192 and c.block_ff_dim == 12288, extra
+        assert Lfm2Config.from_dict(c.to_json()) == c
+    assert Lfm2Config.from_dict(dict(bare, intermediate_size=6656)).intermediate_size == 4608
+    assert Lfm2Config.from_dict(dict(bare, intermediate_size=10752)).intermediate_size == 7168
+    # a direct width, said to be one
+    c = Lfm2Config.from_dict(dict(bare, intermediate_size=1000, block_auto_adjust_ff_dim=False))
+    assert c.intermediate_size == 1000
+    assert Lfm2Config.from_dict(dict(BASE, block_auto_adjust_ff_dim=False)).intermediate_size == 12288
+    # both names in one file: equal (the alias), or the adjusted width beside block_ff_dim; anything else is refused
+    assert Lfm2Config.from_dict(dict(BASE, intermediate_size=12288)).intermediate_size == 8192
+    assert Lfm2Config.from_dict(dict(BASE, intermediate_size=8192)).intermediate_size == 8192
+    with pytest.raises(ConfigError, match="neither"):
+        Lfm2Config.from_dict(dict(BASE, intermediate_size=8000))
+    # the multiplier scales before the rounding; without one (null) two thirds stand as they are
+    assert Lfm2Config.from_dict(dict(bare, intermediate_size=1000, block_ffn_dim_multiplier=1.3,
+                                     block_multiple_of=7)).intermediate_size == 868
+    assert Lfm2Config.from_dict(dict(bare, intermediate_size=1000, block_ffn_dim_multiplier=None)).intermediate_size == 666
+    with pytest.raises(ConfigError, match="block_ff_dim or intermediate_size"):
+        Lfm2Config.from_dict(bare)
+
+
+def test_a_configuration_built_with_a_direct_width_is_written_so_that_any_reader_keeps_it():
+    """``Lfm2Config(intermediate_size=192)`` means a SwiGLU of 192; its config.json says so with
+    ``block_auto_adjust_ff_dim: false``, and reading it back gives 192 again (a reader that adjusted it would build a
+    model whose weights do not fit the file's)."""
+    c = Lfm2Config(vocab_size=256, hidden_size=64, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                   layer_types=("conv", "full_attention"), conv_L_cache=3, conv_bias=False, intermediate_size=192,
+                   norm_eps=1e-5, rope_theta=1e4, tie_word_embeddings=True, max_position_embeddings=256)
+    raw = c.to_json()
+    assert raw["intermediate_size"] == 192 and raw["block_auto_adjust_ff_dim"] is False and "block_ff_dim" not in raw
+    assert Lfm2Config.from_dict(raw).intermediate_size == 192
+    assert tensor_table(lfm2_spec(Lfm2Config.from_dict(raw)))["model.layers.0.feed_forward.w1.weight"].shape == (192, 64)
 
 
 @pytest.mark.parametrize("change,match", [
@@ -100,7 +131,7 @@ def test_malformed_fields_raise(change, match):
 
 
 @pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
-                                 "num_key_value_heads", "block_ff_dim"])
+                                 "num_key_value_heads"])
 def test_required_keys(key):
     raw = dict(BASE)
     del raw[key]

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import plain_lfm2 as P
+from noise import WORST, NoiseBound, supported
 from tiny import CONFIGS, STD, TINY_B, random_ids, write_tiny
 
 pytestmark = pytest.mark.gpu
@@ -73,10 +74,11 @@ def test_greedy_bfloat16_picks_tokens_the_plain_logits_support(folders, name, po
     got = s.generate(prompts, max_new_tokens=NEW[name], eos_ids=())
     for p, g in zip(prompts, got):
         ref = P.forward(cfg, w, g[:-1])
+        # the token chosen is the plain argmax, or as good as it within twice what bfloat16 logits may stand from the
+        # plain ones (the worst logit of the rounded plain model over this sequence, times the bound's factor)
+        slack = 2 * WORST * float((P.forward(cfg, w, g[:-1], store=P.to_bfloat16) - ref).abs().max())
         for i in range(len(p), len(g)):
-            row = ref[i - 1]
-            # the token chosen is the plain argmax, or as good as it within the bfloat16 tolerance of the logits
-            assert float(row.max() - row[g[i]]) <= 1.5e-2 * max(1.0, float(row.abs().max())), (i, g[i])
+            assert supported(ref[i - 1], g[i], slack), (i, g[i], slack)
 
 
 def test_seventy_requests_at_once_decode_through_the_recorded_loop_in_groups(plain):
@@ -195,8 +197,8 @@ def test_poison_fills_what_is_given_back_and_a_read_past_the_end_shows_it(plain)
     from gesso_amd import Engine, StepEntry
     d, cfg, w = plain["A"]
     eng = Engine.from_folder(d, dtype="float32", page_size=8, num_pages=6, num_slots=2, poison=True)
-    kv = eng.storage.kv[0]
-    assert bool(torch.isnan(kv[:, :, :-1]).all())                    # nothing holds a stale value from the start
+    look = lambda: torch.stack([eng.storage.keys[0], eng.storage.values[0]], dim=1)    # (members, K/V, pages + 1, ...)
+    assert bool(torch.isnan(look()[:, :, :-1]).all())                # nothing holds a stale value from the start
     ids = random_ids(13, cfg["V"], 31)
     eng.add_request("a")
     logits = eng.step([StepEntry("a", ids, [12])])
@@ -204,6 +206,7 @@ def test_poison_fills_what_is_given_back_and_a_read_past_the_end_shows_it(plain)
     assert float((logits[0].double().cpu() - ref).abs().max()) <= 1e-4 * max(1.0, float(ref.abs().max()))
     pages = list(eng.manager.get("a").tables[0])
     slot = eng.manager.get("a").slot
+    kv = look()
     assert len(pages) == 2 and not torch.isnan(kv[:, :, pages[0]]).any()
     # the second page holds rows 8..12; its last three rows belong to nobody yet
     assert not torch.isnan(kv[:, :, pages[1], :, :5]).any() and bool(torch.isnan(kv[:, :, pages[1], :, 5:]).all())
@@ -226,7 +229,7 @@ def test_poison_fills_what_is_given_back_and_a_read_past_the_end_shows_it(plain)
     held = eng.manager.get("b").tables[0]
     for p in pages:
         if p not in held:
-            assert bool(torch.isnan(kv[:, :, p]).all())
+            assert bool(torch.isnan(look()[:, :, p]).all())
     state = eng.storage.state[0]["history"]
     if eng.manager.get("b").slot != slot:
         assert bool(torch.isnan(state[slot]).all())
@@ -267,6 +270,43 @@ def test_a_step_that_fails_in_the_middle_releases_its_requests(plain):
     eng.add_request("a")
     got = eng.step([StepEntry("a", ids[:5], [4])])[0].double().cpu()
     assert float((got - ref[4]).abs().max()) <= 1e-4 * max(1.0, float(ref.abs().max()))
+
+
+def test_a_pass_that_breaks_off_inside_a_scheduled_run_fails_its_requests_only(plain):
+    """``run_batch`` with room for two requests at a time: the step that holds the first two prompts breaks off in the
+    middle of the model (a feed-forward that raises once).  Those two end as failed with nothing generated; the third,
+    admitted afterwards, generates what the plain model does; every page and slot is back (the reference stops only
+    the request whose pass failed, ``src/Runtime/Runtime.jl:175-178``)."""
+    from gesso_amd import BatchRequest, Session, run_batch
+    from gesso_amd.errors import KernelError, StepFailed
+    d, cfg, w = plain["A"]
+    s = Session(d, dtype="float32", context_length=64, max_tokens=256, max_num_seqs=2, page_size=8)
+    ffn = s.engine.model.blocks[1].ffn
+    real, calls = ffn.forward, []
+
+    def failing_once(x, ctx):
+        calls.append(1)
+        if len(calls) == 1:
+            raise KernelError("refused, for the test")
+        return real(x, ctx)
+
+    ffn.forward = failing_once
+    p = [random_ids(n, cfg["V"], 30 + n) for n in (6, 11, 9)]
+    try:
+        res = run_batch([BatchRequest(s, p[0], max_new_tokens=5), BatchRequest(s, p[1], max_new_tokens=5),
+                         BatchRequest(s, p[2], max_new_tokens=7)])
+    finally:
+        ffn.forward = real
+    assert [r.status for r in res] == ["failed", "failed", "complete"]
+    assert all(isinstance(r.error, StepFailed) and isinstance(r.error.__cause__, KernelError) for r in res[:2])
+    assert res[0].ids == p[0] and res[1].ids == p[1]
+    assert res[2].ids == P.greedy(cfg, w, p[2], 7)
+    st = s.engine.manager.stats()
+    assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+    s.engine.manager.check()
+    # and the session serves on: the two that failed come out right when asked again
+    got = s.generate(p[:2], max_new_tokens=5, eos_ids=())
+    assert got == [P.greedy(cfg, w, q, 5) for q in p[:2]]
 
 
 def test_one_requests_failure_leaves_the_others_their_results(plain):
@@ -475,9 +515,9 @@ def test_recorded_decode_loop_equals_single_steps(folders, name, dtype):
         for i, p in enumerate(prompts):
             seq = list(p) + [first[i]] + [row[i] for row in got]
             plain_rows = P.forward(cfgp, w, seq[:-1])
+            slack = 2 * WORST * float((P.forward(cfgp, w, seq[:-1], store=P.to_bfloat16) - plain_rows).abs().max())
             for at in range(len(p) + 1, len(seq)):
-                row = plain_rows[at - 1]
-                assert float(row.max() - row[seq[at]]) <= 1.5e-2 * max(1.0, float(row.abs().max())), (i, at)
+                assert supported(plain_rows[at - 1], seq[at], slack), (i, at, slack)
     assert [eng2.length(i) for i in range(3)] == [len(p) + 21 for p in prompts]
 
 
@@ -496,20 +536,21 @@ def test_recorded_decode_logits_follow_the_plain_model(folders, name, nreq, step
     for i, p in enumerate(prompts):
         eng.add_request(i)
         toks.append(int(eng.step([StepEntry(i, p, [len(p) - 1])]).argmax()))
-    worst = 0.0
+    kept = []
     for step in range(steps):
         for s, t in zip(seqs, toks):
             s.append(t)
         ids, bad = eng.decode(list(range(nreq)), toks, 1)
         assert not bad.any()
-        logits = eng._runners[_capacity(nreq)].logits[:nreq].double().cpu()
-        for i, s in enumerate(seqs):
-            ref = P.forward(cfg, w, s)[-1]
-            scale = max(1.0, float(ref.abs().max()))
-            worst = max(worst, float((logits[i] - ref).abs().max()) / scale)
+        kept.append(eng._runners[_capacity(nreq)].logits[:nreq].double().cpu())
         toks = ids[0].tolist()
-    print(f"{name}, {nreq} requests: worst relative difference of the recorded step's logits {worst:.3e}")
-    assert worst <= 1.5e-2
+    bound = NoiseBound()
+    for i, s in enumerate(seqs):          # a row of the whole sequence's logits is the last row of its prefix's
+        ref, rounded = P.forward(cfg, w, s), P.forward(cfg, w, s, store=P.to_bfloat16)
+        for step in range(steps):
+            at = len(s) - steps + step
+            bound.add(kept[step][i], ref[at], rounded[at], (step, i))
+    bound.check(f"{name}, recorded decode of {nreq} requests,")
 
 
 def test_recorded_decode_across_a_bound_on_the_context(tmp_path):
@@ -526,17 +567,17 @@ def test_recorded_decode_across_a_bound_on_the_context(tmp_path):
     eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, max_tokens=2048, num_slots=2)
     eng.add_request("r")
     tok = int(eng.step([StepEntry("r", seq, [len(seq) - 1])]).argmax())
-    checked = 0
+    checked, bound = 0, NoiseBound()
     for step in range(24):
         seq.append(tok)
         ids, bad = eng.decode(["r"], [tok], 1)
         assert not bad.any()
         if len(seq) in (1020, 1023, 1024, 1025, 1030):          # around the bound: the second recording takes over
             logits = eng._runners[1].logits[0].double().cpu()
-            ref = P.forward(cfg, w, seq)[-1]
-            assert float((logits - ref).abs().max()) <= 1.5e-2 * max(1.0, float(ref.abs().max()))
+            bound.add(logits, P.forward(cfg, w, seq)[-1], P.forward(cfg, w, seq, store=P.to_bfloat16)[-1], len(seq))
             checked += 1
         tok = int(ids[0][0])
+    bound.check("across a bound on the context,")
     assert checked == 5 and len(eng._runners[1].graphs) == 2
 
 
@@ -566,6 +607,7 @@ def test_a_full_run_before_a_new_recording_leaves_the_rings_alone(tmp_path):
         eng.add_request(i)
         toks.append(int(eng.step([StepEntry(i, s, [len(s) - 1])]).argmax()))
     rids = list(range(4))
+    bound = NoiseBound()
     for n in (steps, steps, 8):                             # 960 -> 992 -> 1024 (first recording), then beyond it
         ids, bad = eng.decode(rids, toks, n)
         assert not bad.any()
@@ -575,8 +617,8 @@ def test_a_full_run_before_a_new_recording_leaves_the_rings_alone(tmp_path):
             toks = ids[step].tolist()
         logits = runner.logits[:4].double().cpu()          # of the run's last step
         for i, s in enumerate(seqs):
-            ref = P.forward(cfg, w, s)[-1]
-            assert float((logits[i] - ref).abs().max()) <= 1.5e-2 * max(1.0, float(ref.abs().max()))
+            bound.add(logits[i], P.forward(cfg, w, s)[-1], P.forward(cfg, w, s, store=P.to_bfloat16)[-1], (n, i))
+    bound.check("full runs before a new recording,")
     assert len(runner.graphs) == 2
     for name, big in guard.items():
         assert bool((big[0] == -7).all()) and bool((big[-1] == -7).all()), f"a step wrote beside {name}"

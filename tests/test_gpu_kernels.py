@@ -817,7 +817,8 @@ def test_embed_leaves_rows_weighted_for_the_first_norm(ops, T, H, V):
 
 
 @pytest.mark.parametrize("weighted", [False, True])
-@pytest.mark.parametrize("M,H,W,bias", [(1, 64, 3, False), (8, 2048, 3, False), (20, 96, 4, True), (64, 48, 2, False)])
+@pytest.mark.parametrize("M,H,W,bias", [(1, 64, 3, False), (8, 2048, 3, False), (20, 96, 4, True), (64, 48, 2, False),
+                                        (64, 2048, 3, False), (40, 1024, 3, False)])
 def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias, weighted):
     res, nw, lazy = lazy_case(ops, M, H, M + H, weighted)
     g = gen(H + W)
@@ -835,6 +836,34 @@ def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias, weight
     assert float((s1 - s2).abs().max()) <= 1e-2 * max(1.0, float(s2.abs().max()))
     untouched = [i for i in range(M + 2) if i not in slots.tolist()]
     assert torch.equal(s1[untouched].cpu(), state0[untouched])
+
+
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("M,H,W", [(1, 2048, 3), (8, 2048, 3), (64, 2048, 3), (48, 1024, 3), (33, 96, 4)])
+def test_gemm_skinny_conv_against_the_plain_convolution(ops, M, H, W, weighted):
+    """The input product with the short convolution as its epilogue, at the widths and row counts of the benchmarked
+    decode steps (1, 8 and 64 rows of 2048; 48 of 1024), against the plain formulas: norm, product, ``B * x``, taps
+    over the slot's history and the new row, ``C * y``, and the history shifted by one."""
+    res, nw, lazy = lazy_case(ops, M, H, 3 * M + H, weighted)
+    g = gen(H + W + M)
+    w_in = (torch.randn(3 * H, H, generator=g) / math.sqrt(H)).bfloat16()
+    taps = torch.randn(H, W, generator=g)
+    state0 = torch.randn(M + 3, H, W - 1, generator=g)
+    slots = torch.randperm(M + 3, generator=g)[:M].to(torch.int32)
+    state = state0.clone().to(DEV)
+    got = ops.gemm_skinny_conv(lazy, w_in.to(DEV), taps.to(DEV), None, state, slots.to(DEV))
+    # plain: the product's inputs and its result rounded to bfloat16 as the kernel holds them, the rest in float64
+    normed = P.to_bfloat16(P.rmsnorm(res.double(), nw.double(), 1e-5))
+    bcx = normed @ w_in.double().T
+    want = torch.zeros(M, H, dtype=torch.float64)
+    hist = state0.double().clone()
+    for i in range(M):
+        out, h = P.short_conv(bcx[i:i + 1], taps.double(), None, state0[slots[i]].double())
+        want[i], hist[slots[i]] = out[0], h
+    close(got, want, torch.bfloat16)
+    assert float((state.double().cpu() - hist).abs().max()) <= 1e-2 * max(1.0, float(hist.abs().max()))
+    untouched = [i for i in range(M + 3) if i not in slots.tolist()]
+    assert torch.equal(state[untouched].cpu(), state0[untouched])
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 16384, 2048), (24, 96, 64), (64, 2048, 8192)])

@@ -119,7 +119,7 @@ def test_library_products_of_many_rows_are_planned_once_per_shape_and_stay_right
     x = torch.randn(512, 384, generator=g).bfloat16()
     w = (torch.randn(320, 384, generator=g) / math.sqrt(384)).bfloat16()
     want = x.double() @ w.double().T
-    rt = Runtime(DEV, torch.bfloat16)
+    rt = Runtime(DEV, torch.bfloat16, RuntimeOptions(tune_library=True))
     before = ops.library_gemm_plan(512, 320, 384)[0]
     for _ in range(3):
         got = rt.linear(x.to(DEV), w.to(DEV)).double().cpu()

@@ -5,10 +5,13 @@ most of it in one step and the last 32 tokens one by one; portions of changing s
 tokens; and a mix of up to four live requests with a pool so small that pages are used again.
 Every fed position's logits are compared with the plain implementation's whole-sequence logits.
 
-Tolerances, set before the first run and never widened: float32 ``1e-4 * max(1, max|ref|)``
-(the reference's own device bound, ``test/test_amdgpu_lfm2.jl:34``); bfloat16 ``1.5e-2 * max(1, max|ref|)``:
-the matrix products round their inputs and outputs to 8 bits of mantissa (2^-9 relative per
-rounding) over up to six blocks of about ten roundings each.
+Bounds: float32 ``1e-4 * max(1, max|ref|)`` at the worst logit (the reference's own device bound,
+``test/test_amdgpu_lfm2.jl:34``); bfloat16: the distance that the plain model itself takes when its activations are
+rounded to bfloat16, row by row, over all rows and at the worst logit (``tests/noise.py``; ``tests/test_sensitivity.py``
+shows without a GPU that a lost convolution history, reversed taps or a key past the causal edge break it at every
+configuration here).  The weights are drawn with a standard deviation of 0.1, at which any bfloat16 pipeline stands
+some 2 % of the logits' spread from the plain model: a fixed tolerance would be narrower than that noise or wider than
+a fault.
 """
 import numpy as np
 import pytest
@@ -19,7 +22,6 @@ from tiny import CONFIGS, random_ids, write_tiny
 
 pytestmark = pytest.mark.gpu
 
-TOL = {"float32": 1e-4, "bfloat16": 1.5e-2}
 
 # sequence lengths: the benchmark description's prompts plus generated tokens
 LENGTHS = {"A": (5 + 16, 17 + 16, 32 + 16, 70), "B": (1 + 24, 9 + 24, 40 + 24, 100 + 24), "C": (3, 50, 97),
@@ -42,9 +44,7 @@ def test_replay_four_ways(name, dtype, folders, tmp_path):
     cfg, _ = CONFIGS[name]
     model_dir = write_tiny(folders, name, torch.float32 if dtype == "float32" else torch.bfloat16)
     seqs = sequences(name)
-    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
-    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
-    tol = TOL[dtype] * scale
+    plain = R.Plain(model_dir, seqs, dtype)
 
     # the four ways in one process: names differ per way so that all requests are distinct
     ways = {"whole": R.trace_whole, "tail": R.trace_tail, "portions": R.trace_portions,
@@ -64,9 +64,7 @@ def test_replay_four_ways(name, dtype, folders, tmp_path):
     for way in ways:
         mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
         assert {k: len(v) for k, v in mine.items()} == {k: len(v) for k, v in seqs.items()}, way
-        w, where = R.worst(mine, ref)
-        print(f"{name} {dtype} {way}: worst |diff| {w:.3e} at {where} (tolerance {tol:.3e}, scale {scale:.2f})")
-        assert w <= tol, f"{way}: first look at {where}"
+        plain.check(mine, f"{name} {way}")
 
 
 def random_config(seed: int):
@@ -102,8 +100,7 @@ def test_replay_of_configurations_drawn_at_random(seed, dtype, tmp_path):
                                    std=STD)
     lens = [rng.randint(1, 6), rng.randint(20, 60), rng.randint(61, 110), rng.randint(111, 170)]
     seqs = {f"s{i}": random_ids(n, cfg.vocab_size, seed * 10 + i) for i, n in enumerate(lens)}
-    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
-    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    plain = R.Plain(model_dir, seqs, dtype)
     ways = {"whole": R.trace_whole, "tail": R.trace_tail, "portions": R.trace_portions,
             "mixed": lambda s: R.trace_mixed(s, seed=seed)}
     big = R.Trace()
@@ -117,10 +114,7 @@ def test_replay_of_configurations_drawn_at_random(seed, dtype, tmp_path):
     assert rc == 0
     for way in ways:
         mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
-        w, where = R.worst(mine, ref)
-        print(f"seed {seed} ({cfg.num_attention_heads}/{cfg.num_key_value_heads} heads of {cfg.head_dim}) {dtype} {way}: "
-              f"worst |diff| {w:.3e} at {where}")
-        assert w <= TOL[dtype] * scale, f"{way}: first look at {where}"
+        plain.check(mine, f"seed {seed} ({cfg.num_attention_heads}/{cfg.num_key_value_heads} heads of {cfg.head_dim}) {way}")
 
 
 @pytest.mark.parametrize("name", ["B", "D"])
@@ -130,15 +124,12 @@ def test_replay_with_the_hand_written_product_for_many_rows(name, folders, tmp_p
     cfg, _ = CONFIGS[name]
     model_dir = write_tiny(folders, name, torch.bfloat16)
     seqs = sequences(name)
-    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
-    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    plain = R.Plain(model_dir, seqs, "bfloat16")
     for way, make in (("whole", R.trace_whole), ("portions", lambda s: R.trace_portions(s, sizes=(70, 3, 66, 2, 90)))):
         got, rc = R.run_trace(model_dir, "bfloat16", str(tmp_path / way), make(seqs), cfg.vocab_size,
                               extra=["--gemm", "own"])
         assert rc == 0
-        w, where = R.worst(got, ref)
-        print(f"{name} own product, {way}: worst |diff| {w:.3e} at {where}")
-        assert w <= TOL["bfloat16"] * scale, f"{way}: first look at {where}"
+        plain.check(got, f"{name} own product, {way}")
 
 
 @pytest.mark.parametrize("poison", [False, True])
@@ -151,8 +142,7 @@ def test_replay_with_pages_of_eight_and_portions_of_thirteen(dtype, poison, fold
     cfg, _ = CONFIGS["B"]
     model_dir = write_tiny(folders, "B", torch.float32 if dtype == "float32" else torch.bfloat16)
     seqs = sequences("B")
-    ref = {k: R.plain_logits(model_dir, ids) for k, ids in seqs.items()}
-    scale = max(1.0, max(float(np.abs(r).max()) for r in ref.values()))
+    plain = R.Plain(model_dir, seqs, dtype)
     ways = {"whole": R.trace_whole, "tail": R.trace_tail, "portions": lambda s: R.trace_portions(s, sizes=(13,)),
             "mixed": lambda s: R.trace_mixed(s, seed=3)}
     big = R.Trace()
@@ -168,6 +158,4 @@ def test_replay_with_pages_of_eight_and_portions_of_thirteen(dtype, poison, fold
     for way in ways:
         mine = {k.split(".", 1)[1]: v for k, v in got.items() if k.startswith(way + ".")}
         assert {k: len(v) for k, v in mine.items()} == {k: len(v) for k, v in seqs.items()}, way
-        w, where = R.worst(mine, ref)
-        print(f"B, pages of 8, {dtype}, poison {poison}, {way}: worst |diff| {w:.3e} at {where}")
-        assert w <= TOL[dtype] * scale, f"{way}: first look at {where}"
+        plain.check(mine, f"B, pages of 8, poison {poison}, {way}")

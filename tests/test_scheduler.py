@@ -370,3 +370,73 @@ def test_admission_leaves_the_watermark_free_for_those_who_run():
     assert c.finish_reason == "complete" and c.tokens == expected(range(14), 2)
     with pytest.raises(InvalidPlan):
         make(watermark=1.0)
+
+
+class FailingEngine(FakeEngine):
+    """The stand-in with passes that break off as the engine's do: the requests of the pass are released, then
+    ``StepFailed`` names them (``Engine.fail_requests``)."""
+
+    def __init__(self, *a, fail_steps=(), fail_runs=(), **kw):
+        super().__init__(*a, **kw)
+        self.fail_steps, self.fail_runs = set(fail_steps), set(fail_runs)
+        self.n_steps = self.n_runs = 0
+
+    def has_request(self, rid):
+        return rid in self.manager.requests
+
+    def _break(self, rids):
+        from gesso_amd.errors import StepFailed
+        for r in rids:
+            self.finish_request(r)
+        return StepFailed("a kernel refused its sizes", requests=list(rids))
+
+    def step(self, entries):
+        self.n_steps += 1
+        if self.n_steps in self.fail_steps:
+            self.manager.reserve_many([(e.rid, len(e.tokens)) for e in entries])
+            raise self._break([e.rid for e in entries])
+        return super().step(entries)
+
+
+class FailingDecodeEngine(FailingEngine, FakeDecodeEngine):
+    def decode(self, rids, tokens, n, samplers=None):
+        self.n_runs += 1
+        if self.n_runs in self.fail_runs:
+            self.manager.reserve_many([(r, n) for r in rids])
+            raise self._break(rids)
+        return super().decode(rids, tokens, n, samplers)
+
+
+def test_a_step_that_breaks_off_fails_its_requests_and_nobody_else():
+    """The second step (a decoding beside b's second portion) breaks off: both end as failed with what they had; c,
+    which waited, comes out as it does alone; nothing is released twice, nothing is lost."""
+    from gesso_amd.errors import StepFailed
+    eng = FailingEngine(fail_steps={2})
+    s = Scheduler(eng, choose, chunk_size=4, max_num_batched_tokens=8, max_num_seqs=2)
+    a = s.add(Request("a", [1, 2, 3], max_new_tokens=5))
+    b = s.add(Request("b", list(range(9)), max_new_tokens=3))
+    c = s.add(Request("c", [7, 8], max_new_tokens=4))
+    s.run()
+    assert a.finish_reason == "failed" and isinstance(a.error, StepFailed) and a.tokens == expected([1, 2, 3], 1)
+    assert b.finish_reason == "failed" and isinstance(b.error, StepFailed) and b.output == []
+    assert c.finish_reason == "complete" and c.tokens == expected([7, 8], 4)
+    assert s.stats["failed_passes"] == 1 and not s.running and not s.waiting
+    assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+    eng.manager.check()
+
+
+def test_a_group_of_a_decode_run_that_breaks_off_leaves_the_other_groups_their_tokens():
+    """Six requests through a loop of four: the second group's first run breaks off.  Its two requests fail with the
+    token their prompts gave them; the four of the first group keep the run's tokens and finish as they do alone."""
+    from gesso_amd.errors import StepFailed
+    eng = FailingDecodeEngine(fail_runs={2})
+    s = Scheduler(eng, choose, decode_run_steps=4, max_num_seqs=6)
+    reqs = [s.add(Request(chr(97 + i), [i + 1, i + 2], max_new_tokens=6)) for i in range(6)]
+    s.run()
+    for i, r in enumerate(reqs[:4]):
+        assert r.finish_reason == "complete" and r.tokens == expected([i + 1, i + 2], 6), i
+    for i, r in enumerate(reqs[4:], start=4):
+        assert r.finish_reason == "failed" and isinstance(r.error, StepFailed), i
+        assert r.tokens == expected([i + 1, i + 2], 1), i
+    assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
+    eng.manager.check()
