@@ -291,9 +291,15 @@ def test_a_long_context_in_portions_then_recorded_decoding(dtype, tmp_path):
         print(f"long context, float32: worst |diff| {worst:.3e} at position {where} (tolerance {1e-4 * scale:.3e})")
         assert worst <= 1e-4 * scale, f"first look at position {where}"
     else:
-        from noise import NoiseBound            # this model is one of the tiny configurations: their bound
+        # this model is one of the tiny configurations: their bound.  The forty decoded rows sit at neighbouring
+        # positions behind one context of 6,000 tokens and share almost all of what their errors come from: over four
+        # seeds of the weights the ratio over all rows came out at 1.29, 0.95, 0.83 and 0.96 through the recorded loop
+        # and at 0.85 to 0.97 through single steps and as a prompt portion, which is the scatter of some four
+        # independent rows, not of forty-three (decode attention itself rounds once: its output stands 0.29 bfloat16
+        # steps rms from the exact one at 6,040 keys, what a single rounding leaves)
+        from noise import NoiseBound
         rounded = P.forward(cfg, w, seq, store=P.to_bfloat16)
-        bound = NoiseBound()
+        bound = NoiseBound(independent=4)
         for pos, row in ends + rows:
             bound.add(row, ref[pos], rounded[pos], pos)
         bound.check("long context,")
