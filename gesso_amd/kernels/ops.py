@@ -28,14 +28,18 @@ def lib():
 
 
 def _dt(t: torch.Tensor) -> int:
-    try:
-        return _DT[t.dtype]
-    except KeyError:
-        raise KernelError(f"kernels take float32 or bfloat16, got {t.dtype}") from None
+    d = t.dtype
+    if d is torch.bfloat16:
+        return BF16
+    if d is torch.float32:
+        return F32
+    raise KernelError(f"kernels take float32 or bfloat16, got {d}")
 
 
 def _p(t):
-    return None if t is None else c_void_p(t.data_ptr())
+    """A tensor's address as the library's entry points take it (their argument types are declared when the library is
+    loaded, so a plain integer or None is all a pointer argument needs)."""
+    return None if t is None else t.data_ptr()
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -44,8 +48,8 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 def _stream():
     """The current stream of the current device as a raw handle (a launch asks for it every time: the short way)."""
     if _raw_stream is not None:
-        return c_void_p(_raw_stream(torch.cuda.current_device()))
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(torch.cuda.current_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 def _check(rc: int):
@@ -59,16 +63,17 @@ def _need(cond: bool, msg: str):
 
 
 def _dev(*ts):
+    # (the messages are made only when a check fails: these run before every launch)
     for t in ts:
-        if t is not None:
-            _need(t.is_cuda, "kernel operands must live on the GPU")
-            _need(t.is_contiguous(), "kernel operands must be contiguous")
+        if t is not None and not (t.is_cuda and t.is_contiguous()):
+            raise KernelError("kernel operands must live on the GPU" if not t.is_cuda else "kernel operands must be contiguous")
 
 
 def _i32(t, n=None, what="index"):
-    _need(t.dtype == torch.int32, f"{what} must be int32, got {t.dtype}")
-    if n is not None:
-        _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} needed")
+    if t.dtype != torch.int32:
+        raise KernelError(f"{what} must be int32, got {t.dtype}")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{what} holds {t.numel()} entries, {n} needed")
 
 
 # ---------------------------------------------------------------------- tiled rows
@@ -158,21 +163,28 @@ def add_rmsnorm(res: torch.Tensor, delta, weight: torch.Tensor, eps: float, out_
 
     ``rows`` (int32) picks source rows; then ``res`` is not written.
     """
-    _dev(res, delta, weight, rows, out)
-    _need(res.dtype == torch.float32 and res.dim() == 2, "add_rmsnorm: the residual stream is float32 (T, H)")
+    f32 = torch.float32
+    if not (res.is_cuda and res.is_contiguous() and res.dtype is f32 and res.dim() == 2):
+        raise KernelError("add_rmsnorm: the residual stream is float32 (T, H), contiguous, on the GPU")
     T, H = res.shape
-    _need(weight.dtype == torch.float32 and weight.shape == (H,), "add_rmsnorm: weight must be float32 (H,)")
-    if delta is not None:
-        _need(delta.shape == res.shape, "add_rmsnorm: delta must have the stream's shape")
-    n_out = T if rows is None else rows.numel()
+    if not (weight.is_cuda and weight.dtype is f32 and weight.shape == (H,) and weight.is_contiguous()):
+        raise KernelError("add_rmsnorm: weight must be float32 (H,)")
+    if delta is not None and not (delta.is_cuda and delta.is_contiguous() and delta.shape == res.shape):
+        raise KernelError("add_rmsnorm: delta must have the stream's shape")
+    n_out = T
     if rows is not None:
+        _dev(rows)
         _i32(rows, what="rows")
+        n_out = rows.numel()
     if out is None:
         out = torch.empty((n_out, H), dtype=out_dtype, device=res.device)
-    _need(out.shape == (n_out, H) and out.dtype == out_dtype, "add_rmsnorm: out has the wrong shape or type")
-    _check(lib().gs_add_rmsnorm(_p(res), _p(delta), c_int(_dt(delta) if delta is not None else _dt(out)),
-                                _p(weight), c_float(eps), _p(out), c_int(_dt(out)), _p(rows), c_int(n_out),
-                                c_int(H), _stream()))
+    elif not (out.is_cuda and out.is_contiguous() and out.shape == (n_out, H) and out.dtype == out_dtype):
+        raise KernelError("add_rmsnorm: out has the wrong shape or type")
+    rc = lib().gs_add_rmsnorm(res.data_ptr(), None if delta is None else delta.data_ptr(),
+                              _dt(delta) if delta is not None else _dt(out), weight.data_ptr(), eps, out.data_ptr(),
+                              _dt(out), None if rows is None else rows.data_ptr(), n_out, H, _stream())
+    if rc != 0:
+        _check(rc)
     return out
 
 
@@ -185,14 +197,19 @@ def residual_add(res: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
 
 def swiglu(x: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     """``x (T, 2F)`` = gate | up  ->  ``silu(gate) * up (T, F)``."""
-    _dev(x, out)
+    if not (x.is_cuda and x.is_contiguous() and x.dim() == 2):
+        raise KernelError("swiglu: rows (T, 2F), contiguous, on the GPU")
     T, F2 = x.shape
-    _need(F2 % 2 == 0, "swiglu: the input holds gate and up side by side")
+    if F2 % 2:
+        raise KernelError("swiglu: the input holds gate and up side by side")
     F = F2 // 2
     if out is None:
         out = torch.empty((T, F), dtype=x.dtype, device=x.device)
-    _need(out.shape == (T, F) and out.dtype == x.dtype, "swiglu: out has the wrong shape or type")
-    _check(lib().gs_swiglu(_p(x), _p(out), c_int(_dt(x)), c_int(T), c_int(F), _stream()))
+    elif not (out.is_cuda and out.is_contiguous() and out.shape == (T, F) and out.dtype == x.dtype):
+        raise KernelError("swiglu: out has the wrong shape or type")
+    rc = lib().gs_swiglu(x.data_ptr(), out.data_ptr(), _dt(x), T, F, _stream())
+    if rc != 0:
+        _check(rc)
     return out
 
 
@@ -350,7 +367,8 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, bias=None, out_dtype=None, out:
     _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1, "gemm: x must be (M, K) with unit column stride")
     M, K = x.shape
     N = w.shape[0]
-    _need(w.shape == (N, K), f"gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    if w.shape != (N, K):
+        raise KernelError(f"gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
     _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (N,)), "gemm: bias must be float32 (N,)")
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype or x.dtype, device=x.device)
@@ -383,7 +401,8 @@ def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, out: torch.Tenso
     _need(mfma_ok(x, w), "gemm_mfma: operands must be bfloat16, K a multiple of 8, 16-byte aligned")
     M, K = x.shape
     N = w.shape[0]
-    _need(w.shape == (N, K), f"gemm_mfma: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    if w.shape != (N, K):
+        raise KernelError(f"gemm_mfma: weight is {tuple(w.shape)}, expected ({N}, {K})")
     _need(not swiglu or N % 2 == 0, "gemm_mfma: SwiGLU needs gate and up rows")
     cols = N // 2 if swiglu else N
     if out is None:
@@ -401,18 +420,23 @@ def library_gemm(x: torch.Tensor, w: torch.Tensor, workspace: torch.Tensor, out:
     first call of a shape makes its plan, with ``tune`` by measuring the library's two dozen best guesses on these
     operands (a few milliseconds), else by taking its first choice.
     ``workspace``: device bytes the library's kernels may use.  Not to be recorded into a graph."""
-    _dev(w, workspace, out if out is not None and out.is_contiguous() else None)
-    _need(x.is_cuda and x.dim() == 2 and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.stride(1) == 1,
-          "library_gemm: bfloat16 (M, K) rows and a bfloat16 weight")
+    bf = torch.bfloat16
+    if not (x.is_cuda and x.dim() == 2 and x.dtype is bf and w.dtype is bf and x.stride(1) == 1 and w.is_cuda
+            and w.is_contiguous() and workspace.is_cuda):
+        raise KernelError("library_gemm: bfloat16 (M, K) rows and a contiguous bfloat16 weight on the GPU")
     M, K = x.shape
     N = w.shape[0]
-    _need(w.shape == (N, K), f"library_gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    if w.shape != (N, K):
+        raise KernelError(f"library_gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
     if out is None:
-        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
-    _need(out.shape == (M, N) and out.dtype == torch.bfloat16 and out.stride(1) == 1, "library_gemm: out is bfloat16 (M, N)")
-    _check(lib().gs_library_gemm(_p(x), c_int(x.stride(0) if M > 1 else K), _p(w), _p(out),
-                                 c_int(out.stride(0) if M > 1 else N), c_int(M), c_int(N), c_int(K), _p(workspace),
-                                 c_long(workspace.numel() * workspace.element_size()), c_int(1 if tune else 0), _stream()))
+        out = torch.empty((M, N), dtype=bf, device=w.device)
+    elif not (out.is_cuda and out.shape == (M, N) and out.dtype is bf and out.stride(1) == 1):
+        raise KernelError("library_gemm: out is bfloat16 (M, N) on the GPU")
+    rc = lib().gs_library_gemm(x.data_ptr(), x.stride(0) if M > 1 else K, w.data_ptr(), out.data_ptr(),
+                               out.stride(0) if M > 1 else N, M, N, K, workspace.data_ptr(),
+                               workspace.numel() * workspace.element_size(), 1 if tune else 0, _stream())
+    if rc != 0:
+        _check(rc)
     return out
 
 
@@ -566,7 +590,8 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype=None, out=None, swiglu: bool = Fal
           "gemm_skinny: operands must be bfloat16, at most 64 rows, K a multiple of 8, aligned")
     M, K = x.shape
     N = w.shape[0]
-    _need(w.shape == (N, K), f"gemm_skinny: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    if w.shape != (N, K):
+        raise KernelError(f"gemm_skinny: weight is {tuple(w.shape)}, expected ({N}, {K})")
     cols = N // 2 if swiglu else N
     out, buf, tiled = _rows_out(out, M, cols, w.device, out_dtype or torch.bfloat16)
     _need(not tiled or swiglu, "gemm_skinny: only the SwiGLU epilogue writes tiled rows")
