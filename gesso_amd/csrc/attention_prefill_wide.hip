@@ -5,9 +5,13 @@
 // arithmetic runs and the other way round.  Here a block's wavefronts meet once per 64 keys, and two blocks
 // share a compute unit, so that one block's products run under the other's softmax:
 //
-//   * A block owns one key head and 32 WQ consecutive queries of one sequence; wavefront w takes query head
-//     w % G of the group and queries 32 (w / G) .. + 31.  (WQ = 8, 4, 2, 2, 1 for groups of 1, 2, 3, 4 and more
-//     heads: up to eight wavefronts share what is staged.)
+//   * A block owns one key head and WQ sub-tiles of up to 32 consecutive queries of one sequence; wavefront w takes
+//     query head w % G of the group and sub-tile w / G.  (WQ = 8, 4, 2, 2, 1 for groups of 1, 2, 3, 4 and more
+//     heads: up to eight wavefronts share what is staged.)  The sub-tiles of a block need not be neighbours: for a
+//     causal prompt the host gives a block late sub-tiles together with early ones (the first half of its entries
+//     the late ones, the second half their partners, so that the two wavefronts that share a SIMD are one of each),
+//     and every block then walks about as many steps, its wavefronts taken together; with consecutive sub-tiles the
+//     blocks of a prompt of 2,048 tokens walk 1 to 32 steps and the launch takes as long as the longest.
 //   * Keys are walked in steps of 64.  A step's key rows (as they lie in the pages) and value rows (transposed:
 //     features x keys) are staged in LDS, two buffers: the loads of step s + 1 are issued before step s is
 //     computed and written to the other buffer after it; one barrier a step.  Where each key's row starts in the
@@ -33,6 +37,7 @@
 
 typedef __attribute__((ext_vector_type(8))) __bf16 pw_bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float pw_f32x16_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t pw_u32x4_t;   // (a plain vector type: arrays of it stay in registers)
 
 #define PW_KS 64
 #define PW_SLACK 6.0f
@@ -72,27 +77,40 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hf = lane >> 5;
   const int h = kvh * G + wave % G, qsub = wave / G;
-  const int seq = tile_seq[tile], row0 = tile_row[tile], nq = tile_n[tile];
+  // A block's WQ sub-tiles of up to 32 queries each are entries tile * WQ .. + WQ - 1 of the three lists (sequence,
+  // first row, count; a count of 0: no such sub-tile).  They belong to one sequence and need not be neighbours: the
+  // host pairs a late sub-tile, which sees many keys, with an early one, which sees few, so that every block of a
+  // causal prompt walks about as many steps for its wavefronts taken together (a wavefront sits out the steps its
+  // queries see nothing of).  The block walks from the first key any of them sees to the last.
+  const int seq = tile_seq[tile * WQ];
   const int* bt = block_table + (size_t)seq * max_blocks;
-  const int pos0 = positions[row0];                       // positions of a tile are consecutive
-  const int last_key = pos0 + nq - 1;
-  const int first_key = window > 0 ? (pos0 - window + 1 > 0 ? pos0 - window + 1 : 0) : 0;
+  int last_key = 0, first_key = 0x7fffffff;
+#pragma unroll
+  for (int j = 0; j < WQ; ++j) {
+    const int n = tile_n[tile * WQ + j];
+    const int p0 = positions[tile_row[tile * WQ + j]];            // (an absent sub-tile names a valid row)
+    const int lo = window > 0 ? (p0 - window + 1 > 0 ? p0 - window + 1 : 0) : 0;
+    if (n > 0) {
+      last_key = p0 + n - 1 > last_key ? p0 + n - 1 : last_key;
+      first_key = lo < first_key ? lo : first_key;
+    }
+  }
+  if (first_key > last_key) first_key = last_key;                 // a block without queries: one masked step, nothing stored
   const int kbeg = (first_key / PW_KS) * PW_KS;
   const int nsteps = (last_key - kbeg) / PW_KS + 1;
-  const int blk_lo = (int)__umulhi((unsigned)first_key, page_magic), blk_hi = (int)__umulhi((unsigned)last_key, page_magic);
   const float sc = scale * PW_LOG2E;
 
   // this wavefront's queries
-  const int nqs = nq - qsub * 32 < 0 ? 0 : (nq - qsub * 32 > 32 ? 32 : nq - qsub * 32);
+  const int nqs = tile_n[tile * WQ + qsub];
   const bool has_rows = nqs > 0;
-  const int r0 = row0 + qsub * 32;
-  const int pfirst = pos0 + qsub * 32, plast = pfirst + (has_rows ? nqs : 1) - 1;
+  const int r0 = tile_row[tile * WQ + qsub];
+  const int pfirst = positions[r0], plast = pfirst + (has_rows ? nqs : 1) - 1;   // positions of a sub-tile are consecutive
   const bool live = l32 < nqs;
   const int my_pos = pfirst + (live ? l32 : (has_rows ? nqs - 1 : 0));
   const int my_lo = window > 0 ? (my_pos - window + 1 > 0 ? my_pos - window + 1 : 0) : 0;
   pw_bf16x8_t qf[KK];
   {
-    const bf16* qrow = q + (size_t)(has_rows ? r0 + (live ? l32 : nqs - 1) : row0) * q_stride + (size_t)h * D + hf * 8;
+    const bf16* qrow = q + (size_t)(has_rows ? r0 + (live ? l32 : nqs - 1) : r0) * q_stride + (size_t)h * D + hf * 8;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) qf[kk] = *reinterpret_cast<const pw_bf16x8_t*>(qrow + kk * 16);
   }
@@ -122,48 +140,47 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
       rowoff[s % 3][tid] = (((uint32_t)page * (uint32_t)nkv + (uint32_t)kvh) * (uint32_t)page_size + (uint32_t)offs) * DC;
     }
   };
-  const uint4* k16 = reinterpret_cast<const uint4*>(kcache);
-  const uint4* v16 = reinterpret_cast<const uint4*>(vcache);
-  uint4 kreg[CK], vreg[CV][2];
-  auto issue = [&](int s) {
-#pragma unroll
-    for (int x = 0; x < CK; ++x) {
-      const int i = tid + x * NT;
-      if (NKC % NT == 0 || i < NKC) kreg[x] = k16[(size_t)rowoff[s % 3][i / DC] + (i % DC)];
-    }
-#pragma unroll
-    for (int x = 0; x < CV; ++x) {
-      const int i = tid + x * NT;
-      if (NVU % NT == 0 || i < NVU) {
-        const int kp = i / DC, c = i % DC;
-        const uint2 two = *reinterpret_cast<const uint2*>(&rowoff[s % 3][2 * kp]);
-        vreg[x][0] = v16[(size_t)two.x + c];
-        vreg[x][1] = v16[(size_t)two.y + c];
-      }
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int x = 0; x < CK; ++x) {
-      const int i = tid + x * NT;
-      if (NKC % NT == 0 || i < NKC) *reinterpret_cast<uint4*>(&ks[buf][i / DC][(i % DC) * 8]) = kreg[x];
-    }
-#pragma unroll
-    for (int x = 0; x < CV; ++x) {
-      const int i = tid + x * NT;
-      if (NVU % NT == 0 || i < NVU) {
-        const int kp = i / DC, c = i % DC;
-        const int col = (2 * kp) ^ (8 * (c & 7));         // features 8 c .. 8 c + 7 share the swizzle
-        const uint32_t a[4] = {vreg[x][0].x, vreg[x][0].y, vreg[x][0].z, vreg[x][0].w};
-        const uint32_t b[4] = {vreg[x][1].x, vreg[x][1].y, vreg[x][1].z, vreg[x][1].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e][col]) = (a[e] & 0xffffu) | (b[e] << 16);
-          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e + 1][col]) = (a[e] >> 16) | (b[e] & 0xffff0000u);
-        }
-      }
-    }
-  };
+  const pw_u32x4_t* k16 = reinterpret_cast<const pw_u32x4_t*>(kcache);
+  const pw_u32x4_t* v16 = reinterpret_cast<const pw_u32x4_t*>(vcache);
+  // two sets of row registers: the rows of step s + 2 are asked for while step s is computed, so that a block
+  // alone on its compute unit (a prompt of a few thousand tokens: one block a unit, or two) does not wait a memory
+  // round trip in every step
+  pw_u32x4_t kreg[2][CK], vreg[2][CV][2];
+  // (as macros: arrays that closures take by reference are not always kept in registers)
+#define PW_ISSUE(s, S)                                                                                                  \
+  {                                                                                                                     \
+    _Pragma("unroll") for (int x = 0; x < CK; ++x) {                                                                    \
+      /* a thread past the step's last chunk loads the last one again: every register is written, none is stored */     \
+      const int i = (NKC % NT == 0 || tid + x * NT < NKC) ? tid + x * NT : NKC - 1;                                     \
+      kreg[S][x] = k16[(size_t)rowoff[(s) % 3][i / DC] + (i % DC)];                                                     \
+    }                                                                                                                   \
+    _Pragma("unroll") for (int x = 0; x < CV; ++x) {                                                                    \
+      const int i = (NVU % NT == 0 || tid + x * NT < NVU) ? tid + x * NT : NVU - 1;                                     \
+      const int kp = i / DC, c = i % DC;                                                                                \
+      const uint2 two = *reinterpret_cast<const uint2*>(&rowoff[(s) % 3][2 * kp]);                                      \
+      vreg[S][x][0] = v16[(size_t)two.x + c];                                                                           \
+      vreg[S][x][1] = v16[(size_t)two.y + c];                                                                           \
+    }                                                                                                                   \
+  }
+#define PW_STASH(buf, S)                                                                                                \
+  {                                                                                                                     \
+    _Pragma("unroll") for (int x = 0; x < CK; ++x) {                                                                    \
+      const int i = tid + x * NT;                                                                                       \
+      if (NKC % NT == 0 || i < NKC) *reinterpret_cast<pw_u32x4_t*>(&ks[buf][i / DC][(i % DC) * 8]) = kreg[S][x];             \
+    }                                                                                                                   \
+    _Pragma("unroll") for (int x = 0; x < CV; ++x) {                                                                    \
+      const int i = tid + x * NT;                                                                                       \
+      if (NVU % NT == 0 || i < NVU) {                                                                                   \
+        const int kp = i / DC, c = i % DC;                                                                              \
+        const int col = (2 * kp) ^ (8 * (c & 7));         /* features 8 c .. 8 c + 7 share the swizzle */               \
+        const pw_u32x4_t a = vreg[S][x][0], b = vreg[S][x][1];                                                          \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                                 \
+          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e][col]) = (a[e] & 0xffffu) | (b[e] << 16);                 \
+          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e + 1][col]) = (a[e] >> 16) | (b[e] & 0xffff0000u);         \
+        }                                                                                                               \
+      }                                                                                                                 \
+    }                                                                                                                   \
+  }
 
   // ---- one step of this wavefront's queries over the 64 keys in buffer `buf`
   auto compute = [&](int buf, int k0, auto masked) {
@@ -241,23 +258,34 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   if (nsteps > 1) put_rows(1, page_of(1));
   if (nsteps > 2) put_rows(2, page_of(2));
   __syncthreads();
-  issue(0);
-  stash(0);
+  PW_ISSUE(0, 0);
+  PW_STASH(0, 0);
+  if (nsteps > 1) PW_ISSUE(1, 1);
   __syncthreads();
-  for (int s = 0; s < nsteps; ++s) {
-    const int k0 = kbeg + s * PW_KS;
-    const int page_ahead = s + 3 < nsteps ? page_of(s + 3) : 0;
-    if (s + 1 < nsteps) issue(s + 1);
-    // the wavefront computes where its queries see any of the step's keys
-    if (has_rows && k0 <= plast && (window == 0 || k0 + PW_KS - 1 >= pfirst - window + 1)) {
-      const bool inner = k0 + PW_KS - 1 <= pfirst && (window == 0 || k0 >= plast - window + 1);
-      if (inner) compute(s & 1, k0, std::false_type{});
-      else compute(s & 1, k0, std::true_type{});
-    }
-    if (s + 1 < nsteps) stash((s + 1) & 1);
-    if (s + 3 < nsteps) put_rows(s + 3, page_ahead);     // rowoff[s % 3] was read for the last time when step s was issued
-    __syncthreads();
+  // step s: the rows of step s + 2 are asked for into the set that step s's rows have left, step s is computed, the
+  // rows of step s + 1 (asked for a step ago) go into the other buffer
+#define PW_STEP(s, MINE, NEXT)                                                                                        \
+  {                                                                                                                     \
+    const int k0 = kbeg + (s) * PW_KS;                                                                                  \
+    const int page_ahead = (s) + 3 < nsteps ? page_of((s) + 3) : 0;                                                     \
+    if ((s) + 2 < nsteps) PW_ISSUE((s) + 2, MINE);                                                                     \
+    /* the wavefront computes where its queries see any of the step's keys */                                           \
+    if (has_rows && k0 <= plast && (window == 0 || k0 + PW_KS - 1 >= pfirst - window + 1)) {                            \
+      const bool inner = k0 + PW_KS - 1 <= pfirst && (window == 0 || k0 >= plast - window + 1);                         \
+      if (inner) compute((s) & 1, k0, std::false_type{});                                                               \
+      else compute((s) & 1, k0, std::true_type{});                                                                      \
+    }                                                                                                                   \
+    if ((s) + 1 < nsteps) PW_STASH(((s) + 1) & 1, NEXT);                                                                 \
+    if ((s) + 3 < nsteps) put_rows((s) + 3, page_ahead);   /* rowoff[s % 3] was last read when step s was issued */     \
+    __syncthreads();                                                                                                    \
   }
+  for (int s = 0; s < nsteps; s += 2) {
+    PW_STEP(s, 0, 1);
+    if (s + 1 < nsteps) PW_STEP(s + 1, 1, 0);
+  }
+#undef PW_STEP
+#undef PW_ISSUE
+#undef PW_STASH
 
   if (!live) return;
   const float inv = 1.0f / l;
@@ -287,12 +315,13 @@ extern "C" int gs_attention_prefill_wide_supports(int nh, int nkv, int d) {
   return d == 64 && g >= 1 && g <= 8;
 }
 
-// The most queries a tile may hold (the host cuts each sequence's queries into tiles of at most this many).
+// The most queries a block may hold: 32 for each of its sub-tiles.
 extern "C" int gs_attention_prefill_wide_rows(int nh, int nkv, int full) { return nkv > 0 ? wide_rows(nh / nkv, full) : 0; }
 
 extern "C" int gs_attention_prefill_wide(const void* q, int q_stride, const void* kcache, const void* vcache,
                                          const int* positions, const int* tile_seq, const int* tile_row,
-                                         const int* tile_n, int ntiles, const int* block_table, int max_blocks,
+                                         const int* tile_n, int ntiles /* blocks: tile_rows / 32 entries of the three lists each */,
+                                         const int* block_table, int max_blocks,
                                          int page_size, long cache_pages, int window, float scale, void* out, int nh,
                                          int nkv, int d, int tile_rows, hipStream_t stream) {
   GS_REQUIRE(gs_attention_prefill_wide_supports(nh, nkv, d), "attention_prefill_wide: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);

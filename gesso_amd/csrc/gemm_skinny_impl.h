@@ -251,45 +251,62 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   // (4 x (width - 1) floats) are each one run of memory: moved sixteen bytes at a time, the width a compile-time
   // number in each of the three forms.  A block's channels past H read the last four (loaded, never used), a row
   // past M its row 0's slot.
-  auto conv_width = [&](auto&& body) {
-    switch (ex.conv_w) {
-      case 2: body(std::integral_constant<int, 2>{}); break;
-      case 3: body(std::integral_constant<int, 3>{}); break;
-      default: body(std::integral_constant<int, 4>{}); break;
-    }
-  };
-  auto preload_conv = [&]() {
-    if (EPI == 3 && wave == 0 && pre_conv) {
-      const int H = N / 3;
-      const int c0 = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4;
-      const int cc0 = c0 + 3 < H ? c0 : H - 4;
-      const f32x4_t bv = *reinterpret_cast<const f32x4_t*>((ex.conv_bias ? ex.conv_bias : ex.taps) + cc0);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) cbias[i] = bv[i];
-      conv_width([&](auto wc) {
-        constexpr int WD = decltype(wc)::value;
-        f32x4_t tq[WD];
-#pragma unroll
-        for (int q = 0; q < WD; ++q) tq[q] = *reinterpret_cast<const f32x4_t*>(ex.taps + (size_t)cc0 * WD + 4 * q);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int p = 0; p < WD; ++p) ctap[i][p] = tq[(i * WD + p) / 4][(i * WD + p) % 4];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          f32x4_t hq[WD - 1];
-          const float* hp = ex.state + ((size_t)cslot[mt] * H + cc0) * (WD - 1);
-#pragma unroll
-          for (int q = 0; q < WD - 1; ++q) hq[q] = *reinterpret_cast<const f32x4_t*>(hp + 4 * q);
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int p = 0; p < WD - 1; ++p) chist[mt][i][p] = hq[(i * (WD - 1) + p) / 4][(i * (WD - 1) + p) % 4];
+  // (macros, not closures: arrays that a closure takes by reference are not always kept in registers, and these
+  // were not: taps and history went through scratch memory, a store after each load's arrival and a load before use)
+#define GS_CONV_WIDTH(BODY)                                                                                            \
+  switch (ex.conv_w) {                                                                                                  \
+    case 2: { constexpr int WD = 2; BODY } break;                                                                       \
+    case 3: { constexpr int WD = 3; BODY } break;                                                                       \
+    default: { constexpr int WD = 4; BODY } break;                                                                      \
+  }
+#define GS_PRELOAD_CONV_BODY                                                                                           \
+  {                                                                                                                     \
+    f32x4_t tq[WD];                                                                                                     \
+    _Pragma("unroll") for (int q = 0; q < WD; ++q) tq[q] = *reinterpret_cast<const f32x4_t*>(ex.taps + (size_t)cc0_ * WD + 4 * q); \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                       \
+      _Pragma("unroll") for (int p = 0; p < WD; ++p) ctap[i][p] = tq[(i * WD + p) / 4][(i * WD + p) % 4];               \
+    _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                                                 \
+      f32x4_t hq[WD - 1];                                                                                               \
+      const float* hp = ex.state + ((size_t)cslot[mt] * H_ + cc0_) * (WD - 1);                                          \
+      _Pragma("unroll") for (int q = 0; q < WD - 1; ++q) hq[q] = *reinterpret_cast<const f32x4_t*>(hp + 4 * q);         \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                                     \
+        _Pragma("unroll") for (int p = 0; p < WD - 1; ++p)                                                              \
+          chist[mt][i][p] = hq[(i * (WD - 1) + p) / 4][(i * (WD - 1) + p) % 4];                                         \
+    }                                                                                                                   \
+  }
+#define GS_PRELOAD_CONV()                                                                                              \
+  if (EPI == 3 && wave == 0 && pre_conv) {                                                                              \
+    const int H_ = N / 3;                                                                                               \
+    const int c0_ = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4;                                                         \
+    const int cc0_ = c0_ + 3 < H_ ? c0_ : H_ - 4;                                                                       \
+    const f32x4_t bv_ = *reinterpret_cast<const f32x4_t*>((ex.conv_bias ? ex.conv_bias : ex.taps) + cc0_);              \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) cbias[i] = bv_[i];                                                    \
+    GS_CONV_WIDTH(GS_PRELOAD_CONV_BODY)                                                                                 \
+  }
+#define GS_CONV_EPI_BODY                                                                                                \
+        {                                                                                                              \
+          f32x4_t out, nh[WD - 1];                                                                                     \
+_Pragma("unroll")                                                                                                      \
+          for (int i = 0; i < 4; ++i) {                                                                                \
+            const float Bv = to_f32(f32_to_bf16(acc[0][mt][i])), Cv = to_f32(f32_to_bf16(acc[R > 1 ? 1 : 0][mt][i])),  \
+                        Xv = to_f32(f32_to_bf16(acc[R > 2 ? 2 : 0][mt][i]));                                           \
+            const float u = Bv * Xv;                                                                                   \
+            float y = 0.f;                                                                                             \
+_Pragma("unroll")                                                                                                      \
+            for (int p = 0; p < WD - 1; ++p) y += ctap[i][p] * chist[mt][i][p];                                        \
+            y += ctap[i][WD - 1] * u;                                                                                  \
+            if (ex.conv_bias) y += cbias[i];                                                                           \
+            out[i] = Cv * y;                                                                                           \
+_Pragma("unroll")                                                                                                      \
+            for (int p = 0; p < WD - 1; ++p)                                                                           \
+              nh[(i * (WD - 1) + p) / 4][(i * (WD - 1) + p) % 4] = p < WD - 2 ? chist[mt][i][p + 1] : u;               \
+          }                                                                                                            \
+          store4<TOut>(Y + (ex.y_tiled ? tiled_index(m, c0, MT) : (size_t)m * ldy + c0), out, 4);                      \
+          float* hp = ex.state + ((size_t)slot * H + c0) * (WD - 1);                                                   \
+_Pragma("unroll")                                                                                                      \
+          for (int q = 0; q < WD - 1; ++q) *reinterpret_cast<f32x4_t*>(hp + 4 * q) = nh[q];                            \
         }
-      });
-    }
-  };
-  if (EPI == 3 && MT >= 3) preload_conv();   // the loop of many row tiles keeps its order
+  if (EPI == 3 && MT >= 3) GS_PRELOAD_CONV()   // the loop of many row tiles keeps its order
   f32x4_t acc[R][MT];
 #pragma unroll
   for (int r = 0; r < R; ++r)
@@ -349,7 +366,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) b[u][mt] = xok[mt] ? load_x(mt, s + u) : zero8();
         }
-        preload_conv();
+        GS_PRELOAD_CONV()
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -359,7 +376,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
               acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r], b[u][mt], acc[r][mt], 0, 0, 0);
         s += U;
       } else if (EPI == 3) {
-        preload_conv();
+        GS_PRELOAD_CONV()
       }
       for (; s + U <= s1; s += U) {
         bf16x8_t a[U][R], b[U][MT];
@@ -379,7 +396,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
               acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][r], b[u][mt], acc[r][mt], 0, 0, 0);
       }
     } else if (EPI == 3) {
-      preload_conv();
+      GS_PRELOAD_CONV()
     }
   } else if (((K & 31) == 0 || SHUF) && s1 - s0 >= U) {
     // many rows: a ring of U steps in registers: a step is multiplied as soon as it has arrived and its place is
@@ -572,30 +589,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
       const int c0 = blockIdx.x * (SHUF == 2 ? 8 : 16) + kg * 4;
       if (pre_conv) {
         if (c0 >= H || !half_ok) continue;
-        conv_width([&](auto wc) {
-          constexpr int WD = decltype(wc)::value;
-          f32x4_t out, nh[WD - 1];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            // the products run on the values as the unfused path stores them: rounded to bfloat16
-            const float Bv = to_f32(f32_to_bf16(acc[0][mt][i])), Cv = to_f32(f32_to_bf16(acc[R > 1 ? 1 : 0][mt][i])),
-                        Xv = to_f32(f32_to_bf16(acc[R > 2 ? 2 : 0][mt][i]));
-            const float u = Bv * Xv;
-            float y = 0.f;
-#pragma unroll
-            for (int p = 0; p < WD - 1; ++p) y += ctap[i][p] * chist[mt][i][p];
-            y += ctap[i][WD - 1] * u;
-            if (ex.conv_bias) y += cbias[i];
-            out[i] = Cv * y;
-#pragma unroll
-            for (int p = 0; p < WD - 1; ++p)
-              nh[(i * (WD - 1) + p) / 4][(i * (WD - 1) + p) % 4] = p < WD - 2 ? chist[mt][i][p + 1] : u;
-          }
-          store4<TOut>(Y + (ex.y_tiled ? tiled_index(m, c0, MT) : (size_t)m * ldy + c0), out, 4);
-          float* hp = ex.state + ((size_t)slot * H + c0) * (WD - 1);
-#pragma unroll
-          for (int q = 0; q < WD - 1; ++q) *reinterpret_cast<f32x4_t*>(hp + 4 * q) = nh[q];
-        });
+        GS_CONV_WIDTH(GS_CONV_EPI_BODY)
         continue;
       }
 #pragma unroll

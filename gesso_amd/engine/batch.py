@@ -97,6 +97,51 @@ class BatchContext:
             self._tiles = ((rows, skip), t)
         return self._tiles[1]
 
+    def query_subtiles(self, wq: int, skip: int = 0, paired: bool = True) -> torch.Tensor:
+        """int32 ``(3, blocks * wq)`` on the device: :func:`subtile_lists` of this step's sequences from ``skip`` on."""
+        key = ("sub", wq, skip, paired)
+        if self._tiles is None or self._tiles[0] != key:
+            t = torch.tensor(subtile_lists(self.q_lens, wq, skip, paired), dtype=torch.int32)
+            self._tiles = (key, t.pin_memory().to(self.token_ids.device, non_blocking=True))
+        return self._tiles[1]
+
+
+def subtile_lists(q_lens: Sequence[int], wq: int, skip: int = 0, paired: bool = True):
+    """``[sequence], [first row], [row count]`` of sub-tiles of at most 32 consecutive queries of one sequence, ``wq`` of
+    them a block (a count of 0 fills a block up), for the sequences from ``skip`` on; rows count through all sequences.
+
+    ``paired`` (causal attention without a window): a block gets late sub-tiles, which see many keys, together with
+    early ones, which see few: the sub-tiles of a sequence are paired from both ends (last with first, ...), a block
+    takes ``wq / 2`` pairs, the late ones in the first half of its entries and their partners in the second, so that
+    every block has about the same number of (query, key) pairs to work through.  Otherwise blocks take neighbours."""
+    seq, row, cnt = [], [], []
+    at = 0
+    for i, n in enumerate(q_lens):
+        if i >= skip:
+            subs = [(at + a, min(32, n - a)) for a in range(0, n, 32)]
+            none = (at, 0)
+            if paired and wq >= 2:
+                pairs, lo, hi = [], 0, len(subs) - 1
+                while lo < hi:
+                    pairs.append((subs[hi], subs[lo]))
+                    lo, hi = lo + 1, hi - 1
+                if lo == hi:
+                    pairs.append((subs[lo], none))
+                half = wq // 2
+                blocks = []
+                for a in range(0, len(pairs), half):
+                    group = pairs[a:a + half] + [(none, none)] * (half - len(pairs[a:a + half]))
+                    blocks.append([p[0] for p in group] + [p[1] for p in group])
+            else:
+                blocks = [subs[a:a + wq] + [none] * (wq - len(subs[a:a + wq])) for a in range(0, len(subs), wq)]
+            for b in blocks:
+                for r, c in b:
+                    seq.append(i)
+                    row.append(r)
+                    cnt.append(c)
+        at += n
+    return [seq, row, cnt]
+
 
 class StepContext(BatchContext):
     """The flattened batch of one step on the device."""

@@ -851,8 +851,9 @@ def attention_prefill_wide_rows(nh: int, nkv: int, full: bool = True) -> int:
 def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv,
                            d, ntok, out: torch.Tensor = None, full: bool = True) -> torch.Tensor:
     """Causal GQA of long prompt portions (bfloat16, heads of 64): 32 queries a wavefront, keys and values shared by a
-    block through LDS.  ``tiles`` as for :func:`attention_prefill`, of at most ``attention_prefill_wide_rows(nh, nkv,
-    full)`` rows."""
+    block through LDS.  ``tiles``: int32 ``(3, blocks * wq)``, the sequence, first row and row count (at most 32; 0: none)
+    of every sub-tile, ``wq = attention_prefill_wide_rows(nh, nkv, full) // 32`` of them a block, all of one sequence,
+    neighbours or not (``BatchContext.query_subtiles`` pairs late ones with early ones)."""
     _dev(q, kcache, vcache, positions, tiles, block_table, out)
     _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
           "attention_prefill_wide takes bfloat16")
@@ -860,15 +861,17 @@ def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_
     _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
           "cache must be (pages, nkv, page_size, d)")
     _i32(positions, ntok, "positions")
-    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[0] == 3, "tiles must be int32 (3, ntiles)")
+    rows = attention_prefill_wide_rows(nh, nkv, full)
+    wq = rows // 32
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[0] == 3 and wq > 0 and tiles.shape[1] % wq == 0,
+          "tiles must be int32 (3, blocks * sub-tiles a block)")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (nseq, max_blocks)")
     if out is None:
         out = torch.empty((ntok, nh * d), dtype=q.dtype, device=q.device)
     _need(out.shape == (ntok, nh * d) and out.dtype == q.dtype, "attention_prefill_wide: out has the wrong shape or type")
-    nt = tiles.shape[1]
-    _check(lib().gs_attention_prefill_wide(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(tiles[0]),
-                                           _p(tiles[1]), _p(tiles[2]), c_int(nt), _p(block_table),
-                                           c_int(block_table.shape[1]), c_int(page_size), c_long(kcache.shape[0]),
-                                           c_int(window or 0), c_float(scale), _p(out), c_int(nh), c_int(nkv), c_int(d),
-                                           c_int(attention_prefill_wide_rows(nh, nkv, full)), _stream()))
+    nt = tiles.shape[1] // wq
+    _check(lib().gs_attention_prefill_wide(_p(q), q_stride, _p(kcache), _p(vcache), _p(positions), _p(tiles[0]),
+                                           _p(tiles[1]), _p(tiles[2]), nt, _p(block_table),
+                                           block_table.shape[1], page_size, kcache.shape[0],
+                                           window or 0, scale, _p(out), nh, nkv, d, rows, _stream()))
     return out

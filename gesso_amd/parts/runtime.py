@@ -110,6 +110,7 @@ class Runtime:
         self.tiled_rows = dtype == torch.bfloat16 and options.tiled_rows
         self.many_rows = options.many_rows
         self.tune_library = options.tune_library
+        self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         self._library_ws = None        # device bytes for the vendor library's kernels, made at the first such product
         self.profile = None            # a StageProfile while decode steps are profiled (engine/profile.py)
 

@@ -1007,11 +1007,13 @@ def paged(k, v, ps, g):
 
 
 @pytest.mark.parametrize("nh,nkv,ps", [(32, 8, 16), (3, 1, 16), (5, 5, 4), (4, 2, 8), (16, 2, 16), (6, 2, 6)])
-@pytest.mark.parametrize("window", [None, 37, 200])
-def test_attention_prefill_wide(ops, nh, nkv, ps, window):
+@pytest.mark.parametrize("window,paired", [(None, True), (None, False), (37, False), (200, False), (200, True)])
+def test_attention_prefill_wide(ops, nh, nkv, ps, window, paired):
     """The kernel for long portions, heads of 64: four sequences in one launch (a long chunk over a cached prefix that
     ends inside a page, a fresh prompt of some hundred tokens, a single token, a chunk that starts at a step's edge).
-    Rows of pages past a sequence's end hold NaN: a value read from there, even with weight zero, would show."""
+    Rows of pages past a sequence's end hold NaN: a value read from there, even with weight zero, would show.
+    A block's sub-tiles of 32 queries as neighbours, and paired from both ends of the sequence (late with early)."""
+    from gesso_amd.engine.batch import subtile_lists
     d = 64
     assert ops.attention_prefill_wide_supports(nh, nkv, d) and not ops.attention_prefill_wide_supports(nh, nkv, 128)
     rows = ops.attention_prefill_wide_rows(nh, nkv)
@@ -1039,12 +1041,8 @@ def test_attention_prefill_wide(ops, nh, nkv, ps, window):
         table[i, :t.numel()] = t
     qall, want = torch.cat(qs), torch.cat(want)
     positions = torch.tensor([p + j for p, n in zip(prefix, new) for j in range(n)], dtype=torch.int32)
-    tiles, row = [[], [], []], 0
-    for i, n in enumerate(new):
-        for a in range(0, n, rows):
-            tiles[0].append(i); tiles[1].append(row + a); tiles[2].append(min(rows, n - a))
-        row += n
-    tiles = torch.tensor(tiles, dtype=torch.int32)
+    tiles = torch.tensor(subtile_lists(new, rows // 32, 0, paired), dtype=torch.int32)
+    assert tiles.shape[1] % (rows // 32) == 0 and int(tiles[2].sum()) == sum(new)
     stride = (nh + 2 * nkv) * d
     wide = torch.zeros(sum(new), stride, dtype=torch.bfloat16)
     wide[:, :nh * d] = qall
@@ -1081,8 +1079,12 @@ def test_prompt_attention_never_sees_the_next_key_nor_the_one_before_its_window(
     kc, vc, tab = paged(k, v, ps, g)
     positions = torch.arange(prefix, K, dtype=torch.int32)
     rows = ops.attention_prefill_wide_rows(nh, nkv) if kernel == "wide" else int(kernel[5:])
-    tiles = torch.tensor([[0] * -(-new // rows), list(range(0, new, rows)), [min(rows, new - a) for a in range(0, new, rows)]],
-                         dtype=torch.int32)
+    if kernel == "wide":
+        from gesso_amd.engine.batch import subtile_lists
+        tiles = torch.tensor(subtile_lists([new], rows // 32, 0, paired=not window), dtype=torch.int32)
+    else:
+        tiles = torch.tensor([[0] * -(-new // rows), list(range(0, new, rows)), [min(rows, new - a) for a in range(0, new, rows)]],
+                             dtype=torch.int32)
     args = (q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV), positions.to(DEV), tiles.to(DEV), tab[None].to(DEV), ps,
             window, 1.0 / math.sqrt(d), nh, nkv, d, new)
     got = ops.attention_prefill_wide(*args) if kernel == "wide" else ops.attention_prefill(*args, tile_rows=rows)
@@ -1101,9 +1103,9 @@ def test_attention_prefill_wide_over_thousands_of_keys(ops):
         k[far, 0] = q[-1, 0] * 1.5
         q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
         kc, vc, tab = paged(k, v, ps, g)
+        from gesso_amd.engine.batch import subtile_lists
         rows = ops.attention_prefill_wide_rows(nh, nkv)
-        tiles = torch.tensor([[0] * -(-new // rows), list(range(0, new, rows)),
-                              [min(rows, new - a) for a in range(0, new, rows)]], dtype=torch.int32)
+        tiles = torch.tensor(subtile_lists([new], rows // 32, 0, paired=not window), dtype=torch.int32)
         got = ops.attention_prefill_wide(q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV),
                                          torch.arange(prefix, K, dtype=torch.int32, device=DEV), tiles.to(DEV),
                                          tab[None].contiguous().to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, new)

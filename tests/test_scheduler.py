@@ -440,3 +440,33 @@ def test_a_group_of_a_decode_run_that_breaks_off_leaves_the_other_groups_their_t
         assert r.tokens == expected([i + 1, i + 2], 1), i
     assert eng.manager.stats()["pages_free"] == [64] and eng.manager.stats()["slots_free"] == 8
     eng.manager.check()
+
+
+def test_sub_tiles_of_prompt_attention_pair_late_queries_with_early_ones():
+    """Every query row occurs once; a block's sub-tiles belong to one sequence; with pairing the (query, key) pairs
+    of the blocks of one causal prompt differ by at most one sub-tile's worth, without it by the whole prompt's."""
+    from gesso_amd.engine.batch import subtile_lists
+    lens = [1, 1, 300, 2048, 33]
+    for wq in (1, 2, 4, 8):
+        for paired in (False, True):
+            seq, row, cnt = subtile_lists(lens, wq, skip=2, paired=paired)
+            assert len(seq) % wq == 0
+            covered = sorted(r + j for r, c in zip(row, cnt) for j in range(c))
+            assert covered == list(range(2, sum(lens)))
+            for b in range(0, len(seq), wq):
+                assert len(set(seq[b:b + wq])) == 1 and all(0 <= c <= 32 for c in cnt[b:b + wq])
+    starts = [0, 1, 2, 302, 2350]
+
+    def work(wq, paired):
+        seq, row, cnt = subtile_lists(lens, wq, skip=2, paired=paired)
+        out = []
+        for b in range(0, len(seq), wq):
+            if seq[b] == 3:
+                out.append(sum((r - starts[3]) + c for r, c in zip(row[b:b + wq], cnt[b:b + wq]) if c))
+        return out
+    for wq in (2, 4, 8):
+        even, uneven = work(wq, True), work(wq, False)
+        assert max(even) - min(even) <= 32 * wq and max(uneven) - min(uneven) > 1500
+    # the late sub-tiles stand in the first half of a block's entries, their partners in the second
+    seq, row, cnt = subtile_lists([256], 4, 0, True)
+    assert row[:4] == [224, 192, 0, 32] and row[4:] == [160, 128, 64, 96]
