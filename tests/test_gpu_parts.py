@@ -241,6 +241,89 @@ def test_attention_mixer_whole_and_in_portions(fw, dtype, nh, nkv, d, window, qk
         assert len(held) <= 2
 
 
+@dataclasses.dataclass(frozen=True)
+class LatentSpec:
+    hidden: int
+    latent: int
+    value: int                      # 0: no value rows, values are the latent rows themselves
+    kind: str = "toy_latent"
+
+
+@pytest.mark.parametrize("value", [0, 40])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_toy_mixer_whose_cache_rows_are_not_keys_and_values_of_one_width(fw, dtype, value):
+    """A mixer defined here that caches one latent row of 24 numbers per token and either no value rows at all
+    (``value_dim=0``: it attends with the latent rows and sums them) or value rows of another width (40): the cache
+    manager gives its layer pages, the storage a key pool of the one width and a value pool of the other (or an empty
+    one), the block table addresses both; stepped whole and in portions against the arithmetic written out."""
+    from gesso_amd.parts import MATRIX, PagedKV, Part, TensorSpec, register, unregister
+
+    class LatentMixer(Part):
+        @staticmethod
+        def tensor_specs(spec):
+            out = {"down.weight": TensorSpec((spec.latent, spec.hidden), MATRIX),
+                   "query.weight": TensorSpec((spec.latent, spec.hidden), MATRIX),
+                   "out.weight": TensorSpec((spec.hidden, spec.value or spec.latent), MATRIX)}
+            if spec.value:
+                out["value.weight"] = TensorSpec((spec.value, spec.hidden), MATRIX)
+            return out
+
+        @staticmethod
+        def cache_need(spec):
+            return PagedKV(1, spec.latent, None, value_dim=spec.value)
+
+        def bind(self, tensors):
+            self.w = tensors
+
+        def forward(self, x, ctx, cache):
+            s = self.spec
+            assert cache.k.shape[1:] == (1, cache.page_size, s.latent) and cache.v.shape[1:] == (1, cache.page_size, s.value)
+            c = self.rt.linear(x, self.w["down.weight"])
+            q = self.rt.linear(x, self.w["query.weight"]).float()
+            v = self.rt.linear(x, self.w["value.weight"]) if s.value else None
+            pos, seq = ctx.positions.long(), ctx.seq_of_token.long()
+            page = cache.block_table.long()[seq, pos // cache.page_size]
+            cache.k[page, 0, pos % cache.page_size] = c
+            if s.value:
+                cache.v[page, 0, pos % cache.page_size] = v
+            rows = []
+            for t in range(x.shape[0]):
+                u = torch.arange(int(pos[t]) + 1, device=x.device)
+                pg = cache.block_table.long()[seq[t], u // cache.page_size]
+                keys = cache.k[pg, 0, u % cache.page_size].float()
+                vals = cache.v[pg, 0, u % cache.page_size].float() if s.value else keys
+                p = torch.softmax(keys @ q[t] / math.sqrt(s.latent), dim=0)
+                rows.append(p @ vals)
+            return self.rt.linear(torch.stack(rows).to(x.dtype), self.w["out.weight"])
+
+    register("mixer", "toy_latent", LatentMixer, replace=True)
+    try:
+        H, L = 48, 24
+        h = Harness("mixer", LatentSpec(H, L, value), dtype, seed=3 + value, std=0.3)
+        assert h.storage.keys[0].shape[-1] == L and h.storage.values[0].shape[-1] == value
+        T = 21
+        x = torch.randn(T, H, generator=gen(8)).to(dtype)
+        w = h.tensors
+        c = x.double() @ w["down.weight"].T
+        q = x.double() @ w["query.weight"].T
+        vals = x.double() @ w["value.weight"].T if value else c
+        want = torch.stack([torch.softmax(c[:t + 1] @ q[t] / math.sqrt(L), dim=0) @ vals[:t + 1] for t in range(T)])
+        want = want @ w["out.weight"].T
+        whole = h.mixer(x, [("a", T)])
+        assert float((whole - want).abs().max()) <= tol(dtype, want)
+        parts, at = [], 0
+        for n in (5, 1, 9, 2, 4):
+            parts.append(h.mixer(x[at:at + n], [("b", n)]))
+            at += n
+        assert float((torch.cat(parts) - want).abs().max()) <= tol(dtype, want)
+        h.manager.release("a")
+        h.manager.release("b")
+        h.manager.check()
+        assert h.manager.stats()["pages_free"] == [32]
+    finally:
+        unregister("mixer", "toy_latent")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_block_alone(fw, dtype):
     from gesso_amd.config import BlockSpec, RMSNormSpec, ShortConvSpec, SwiGLUSpec
