@@ -24,9 +24,11 @@ class StepEntry:
     want: Sequence[int] = field(default_factory=list)   # indices into ``tokens``
 
 
-def check_entries(entries: List[StepEntry], manager, vocab: int) -> None:
-    """Refuse a step that cannot run, before anything is reserved or written."""
+def check_entries(entries: List[StepEntry], manager, vocab: int) -> np.ndarray:
+    """Refuse a step that cannot run, before anything is reserved or written.  Returns the step's token ids, all
+    entries' in order, as one int64 array (the context takes them as they are)."""
     seen = set()
+    lens = []
     for e in entries:
         manager.get(e.rid)
         if e.rid in seen:
@@ -35,13 +37,17 @@ def check_entries(entries: List[StepEntry], manager, vocab: int) -> None:
         n = len(e.tokens)
         if n < 1:
             raise InvalidPlan(f"request {e.rid!r} brings no tokens to this step")
-        ids = np.asarray(e.tokens, dtype=np.int64)
-        if int(ids.min()) < 0 or int(ids.max()) >= vocab:
-            t = int(ids[(ids < 0) | (ids >= vocab)][0])
-            raise InvalidPlan(f"token id {t} outside the vocabulary of {vocab}", token=t, vocab=vocab)
+        lens.append(n)
         for w in e.want:
             if not 0 <= int(w) < n:
                 raise InvalidPlan(f"request {e.rid!r} wants logits at place {w} of {n} tokens")
+    # one array for all entries: the ids are checked at once (a bad one is then looked for entry by entry)
+    ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]) if len(entries) > 1 \
+        else np.asarray(entries[0].tokens, dtype=np.int64)
+    if ids.size and (int(ids.min()) < 0 or int(ids.max()) >= vocab):
+        t = int(ids[(ids < 0) | (ids >= vocab)][0])
+        raise InvalidPlan(f"token id {t} outside the vocabulary of {vocab}", token=t, vocab=vocab)
+    return ids
 
 
 # What parts may read of a step.  Host-side facts kernels are chosen by: T (tokens), nseq, n_want, q_lens, all_single,
@@ -146,40 +152,43 @@ def subtile_lists(q_lens: Sequence[int], wq: int, skip: int = 0, paired: bool = 
 class StepContext(BatchContext):
     """The flattened batch of one step on the device."""
 
-    def __init__(self, entries: List[StepEntry], manager, storage, vocab: int, device):
+    def __init__(self, entries: List[StepEntry], manager, storage, vocab: int, device, token_ids: np.ndarray = None):
+        """``token_ids``: the entries' tokens in order as one array, where the caller has it (``check_entries``)."""
         ps = manager.page_size
         nseq = len(entries)
-        lens = []
-        for e in entries:
-            lens.append(len(e.tokens))
+        lens = [len(e.tokens) for e in entries]
         T = sum(lens)
         rcs = [manager.get(e.rid) for e in entries]
+        lens_a = np.asarray(lens, dtype=np.int64)
         starts = np.zeros(nseq + 1, dtype=np.int32)
-        starts[1:] = np.cumsum(lens)
-        tokens = np.empty(T, dtype=np.int64)
-        positions = np.empty(T, dtype=np.int32)
-        seq_of = np.empty(T, dtype=np.int32)
+        starts[1:] = np.cumsum(lens_a)
+        if token_ids is None:
+            token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        tokens = token_ids
+        held = np.asarray([rc.length for rc in rcs], dtype=np.int64)
+        # token t of sequence i stands at position held[i] + (t - starts[i])
+        seq_of = np.repeat(np.arange(nseq, dtype=np.int32), lens_a)
+        positions = (np.arange(T, dtype=np.int64) + np.repeat(held - starts[:-1], lens_a)).astype(np.int32)
         want_rows: List[int] = []
-        for i, (e, rc) in enumerate(zip(entries, rcs)):
-            a, b = starts[i], starts[i + 1]
-            tokens[a:b] = np.asarray(e.tokens, dtype=np.int64)
-            positions[a:b] = np.arange(rc.length, rc.length + lens[i], dtype=np.int32)
-            seq_of[a:b] = i
-            want_rows.extend(int(a) + int(w) for w in e.want)
-        kv_len = np.asarray([rc.length + n for rc, n in zip(rcs, lens)], dtype=np.int32)
+        for i, e in enumerate(entries):
+            if e.want:
+                a = int(starts[i])
+                want_rows.extend(a + int(w) for w in e.want)
+        kv_len = (held + lens_a).astype(np.int32)
         max_kv_len = int(kv_len.max()) if nseq else 0
         slots = np.asarray([storage.scratch_slot if rc.slot is None else rc.slot for rc in rcs], dtype=np.int32)
         n_groups = len(manager.pools)
         max_blocks = max(1, -(-max_kv_len // ps))
         tables = np.empty((n_groups, nseq, max_blocks), dtype=np.int32)
         for g in range(n_groups):
-            tables[g, :, :] = storage.num_pages[g]            # the scratch page: never read
+            scratch = storage.num_pages[g]
+            tables[g, :, :] = scratch                         # the scratch page: never read
             for i, rc in enumerate(rcs):
                 t = rc.tables[g]
                 n = min(len(t), max_blocks)
-                row = np.asarray(t[:n], dtype=np.int32)
-                row[row < 0] = storage.num_pages[g]
-                tables[g, i, :n] = row
+                tables[g, i, :n] = t[:n]
+            tab = tables[g]
+            tab[tab < 0] = scratch                            # pages a window has passed and given back
         self.max_blocks = max_blocks
 
         parts = [tokens.astype(np.int32), positions, seq_of, starts, kv_len, slots,

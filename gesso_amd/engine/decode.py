@@ -31,7 +31,8 @@ from ..sampling.sampler import Sampler
 
 def _capacity(n: int) -> int:
     """The batch rounded up to a power of two, or to 48: the products take rows in tiles of 16, and a step of three
-    tiles is measurably shorter than one of four."""
+    tiles is measurably shorter than one of four.  (The most requests a step takes is the engine's
+    ``DECODE_MAX_BATCH``, which it has from the runtime's product kernels.)"""
     c = 1
     while c < n:
         c *= 2

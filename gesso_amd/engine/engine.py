@@ -69,6 +69,9 @@ class Engine:
             self.storage.poison_all()
         self.steps = 0
         self._runners = {}
+        # the most requests one recorded decode step takes: as many rows as the runtime's weight-streaming products do
+        # (the limit is the product kernels', asked of the runtime, not a number of the engine's own)
+        self.DECODE_MAX_BATCH = self.rt.streaming_rows_max
 
     # ------------------------------------------------------------------ construction
 
@@ -141,12 +144,12 @@ class Engine:
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if not entries:
             return None
-        check_entries(entries, self.manager, self.spec.vocab)
+        ids = check_entries(entries, self.manager, self.spec.vocab)
         self.manager.reserve_many([(e.rid, len(e.tokens)) for e in entries])
         # from here on the cache is written: an error leaves the requests of this step without a usable state
         try:
             self.prepare_cache()
-            ctx = StepContext(entries, self.manager, self.storage, self.spec.vocab, self.device)
+            ctx = StepContext(entries, self.manager, self.storage, self.spec.vocab, self.device, token_ids=ids)
             logits = self.model.forward(ctx)
         except Exception as err:
             raise self.fail_requests([e.rid for e in entries], err) from err
@@ -166,7 +169,6 @@ class Engine:
 
     # ------------------------------------------------------------------ decoding, recorded
 
-    DECODE_MAX_BATCH = 64
 
     def decode(self, rids: Sequence[Hashable], tokens: Sequence[int], n: int, samplers=None):
         """``n`` decode steps for requests that each bring one token, as replays of a recorded graph.

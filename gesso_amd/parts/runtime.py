@@ -111,6 +111,7 @@ class Runtime:
         self.many_rows = options.many_rows
         self.tune_library = options.tune_library
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
+        self.streaming_rows_max = ops.SKINNY_MAX_ROWS   # the most rows a weight-streaming product takes
         self._library_ws = None        # device bytes for the vendor library's kernels, made at the first such product
         self.profile = None            # a StageProfile while decode steps are profiled (engine/profile.py)
 
