@@ -26,6 +26,11 @@
 //     when the maximum has grown by more than 2^6 (see attention_prefill_impl.h).  Steps that every query of the
 //     wavefront sees whole carry no masks.
 //
+//   * Short prompts (fewer blocks than compute units): KS = 2 halves the longest walk.  The block's sub-tiles are
+//     then WQ / 2, each held by two wavefronts per head; the first walks the first half of the block's steps, the
+//     second the second half, both halves' keys and values staged side by side, and at the end the second hands its
+//     maximum, sum and accumulator to the first through LDS (the usual merge of two softmax parts).
+//
 // Bank conflicts: key rows are 16 bytes longer than the head; the transposed values put key k of feature f at
 // column k ^ 8 ((f / 8) % 8), which spreads the sixteen-byte chunks that one wavefront writes (eight features of two
 // keys a lane) over all banks and keeps every group of four keys that a product reads in one piece.
@@ -53,7 +58,7 @@ __device__ __forceinline__ float pair_sum(float x) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-template <int D, int G, int WQ>
+template <int D, int G, int WQ, int KS>
 __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int* __restrict__ positions, const int* __restrict__ tile_seq, const int* __restrict__ tile_row,
@@ -64,31 +69,33 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   constexpr int FT = D / 32;                  // feature tiles of the output
   constexpr int DC = D / 8;                   // 16-byte chunks of a row
   constexpr int KROW = D + 8, VROW = PW_KS + 4;
-  constexpr int NKC = PW_KS * DC;             // key chunks of a step
-  constexpr int NVU = (PW_KS / 2) * DC;       // value units of a step: two keys x one chunk
+  constexpr int SUBS = WQ / KS;               // sub-tiles of queries a block
+  constexpr int NKC1 = PW_KS * DC, NKC = KS * NKC1;             // key chunks of a step (of one half, of all)
+  constexpr int NVU1 = (PW_KS / 2) * DC, NVU = KS * NVU1;       // value units of a step: two keys x one chunk
   constexpr int CK = (NKC + NT - 1) / NT, CV = (NVU + NT - 1) / NT;
   static_assert(D == 64, "the swizzle of the transposed values is written for heads of 64");
-  __shared__ __align__(16) uint16_t ks[2][PW_KS][KROW];
-  __shared__ __align__(16) uint16_t vt[2][D][VROW];
-  __shared__ __align__(8) uint32_t rowoff[3][PW_KS];       // (read two at a time) where a step's key rows start in the caches, in units of 16 bytes
+  static_assert((KS == 1 || KS == 2) && WQ % KS == 0, "the keys of a block are walked whole or in two halves");
+  __shared__ __align__(16) uint16_t ks[KS][2][PW_KS][KROW];
+  __shared__ __align__(16) uint16_t vt[KS][2][D][VROW];
+  __shared__ __align__(8) uint32_t rowoff[KS][3][PW_KS];   // (read two at a time) where a step's key rows start in the caches, in units of 16 bytes
 
   // blocks in launch order: key head fastest, tiles from the last one back (late tiles walk the most keys)
   const int kvh = blockIdx.x % nkv, tile = (int)(gridDim.x / nkv) - 1 - (int)(blockIdx.x / nkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hf = lane >> 5;
-  const int h = kvh * G + wave % G, qsub = wave / G;
-  // A block's WQ sub-tiles of up to 32 queries each are entries tile * WQ .. + WQ - 1 of the three lists (sequence,
+  const int h = kvh * G + wave % G, qsub = (wave / G) / KS, kh = (wave / G) % KS;
+  // A block's SUBS sub-tiles of up to 32 queries each are entries tile * SUBS .. + SUBS - 1 of the three lists (sequence,
   // first row, count; a count of 0: no such sub-tile).  They belong to one sequence and need not be neighbours: the
   // host pairs a late sub-tile, which sees many keys, with an early one, which sees few, so that every block of a
   // causal prompt walks about as many steps for its wavefronts taken together (a wavefront sits out the steps its
   // queries see nothing of).  The block walks from the first key any of them sees to the last.
-  const int seq = tile_seq[tile * WQ];
+  const int seq = tile_seq[tile * SUBS];
   const int* bt = block_table + (size_t)seq * max_blocks;
   int last_key = 0, first_key = 0x7fffffff;
 #pragma unroll
-  for (int j = 0; j < WQ; ++j) {
-    const int n = tile_n[tile * WQ + j];
-    const int p0 = positions[tile_row[tile * WQ + j]];            // (an absent sub-tile names a valid row)
+  for (int j = 0; j < SUBS; ++j) {
+    const int n = tile_n[tile * SUBS + j];
+    const int p0 = positions[tile_row[tile * SUBS + j]];          // (an absent sub-tile names a valid row)
     const int lo = window > 0 ? (p0 - window + 1 > 0 ? p0 - window + 1 : 0) : 0;
     if (n > 0) {
       last_key = p0 + n - 1 > last_key ? p0 + n - 1 : last_key;
@@ -97,13 +104,14 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   }
   if (first_key > last_key) first_key = last_key;                 // a block without queries: one masked step, nothing stored
   const int kbeg = (first_key / PW_KS) * PW_KS;
-  const int nsteps = (last_key - kbeg) / PW_KS + 1;
+  const int nsteps_all = (last_key - kbeg) / PW_KS + 1;
+  const int nsteps = (nsteps_all + KS - 1) / KS;                  // steps of the walk: half h takes steps h nsteps .. of the keys
   const float sc = scale * PW_LOG2E;
 
   // this wavefront's queries
-  const int nqs = tile_n[tile * WQ + qsub];
+  const int nqs = tile_n[tile * SUBS + qsub];
   const bool has_rows = nqs > 0;
-  const int r0 = tile_row[tile * WQ + qsub];
+  const int r0 = tile_row[tile * SUBS + qsub];
   const int pfirst = positions[r0], plast = pfirst + (has_rows ? nqs : 1) - 1;   // positions of a sub-tile are consecutive
   const bool live = l32 < nqs;
   const int my_pos = pfirst + (live ? l32 : (has_rows ? nqs - 1 : 0));
@@ -125,19 +133,21 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   // Key u of step s is looked up by thread u - (first key of the step) of the first wavefront: its page is loaded
   // early (page_of), its row start put into LDS late (put_rows).  u is clamped to the keys of this tile: rows
   // beyond are masked, and every load is of a row the sequence holds.
+  // (thread t < 64 KS looks up key t % 64 of half t / 64)
   auto key_of = [&](int s) -> int {
-    const int u = kbeg + s * PW_KS + tid;
+    const int u = kbeg + ((tid / PW_KS) * nsteps + s) * PW_KS + tid % PW_KS;
     return u < first_key ? first_key : (u > last_key ? last_key : u);
   };
   auto page_of = [&](int s) -> int {
-    if (tid >= PW_KS) return 0;
+    if (tid >= KS * PW_KS) return 0;
     return bt[(int)__umulhi((unsigned)key_of(s), page_magic)];
   };
   auto put_rows = [&](int s, int page) {
-    if (tid < PW_KS) {
+    if (tid < KS * PW_KS) {
       const int u = key_of(s);
       const int offs = u - (int)__umulhi((unsigned)u, page_magic) * page_size;
-      rowoff[s % 3][tid] = (((uint32_t)page * (uint32_t)nkv + (uint32_t)kvh) * (uint32_t)page_size + (uint32_t)offs) * DC;
+      rowoff[tid / PW_KS][s % 3][tid % PW_KS] =
+          (((uint32_t)page * (uint32_t)nkv + (uint32_t)kvh) * (uint32_t)page_size + (uint32_t)offs) * DC;
     }
   };
   const pw_u32x4_t* k16 = reinterpret_cast<const pw_u32x4_t*>(kcache);
@@ -152,12 +162,12 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
     _Pragma("unroll") for (int x = 0; x < CK; ++x) {                                                                    \
       /* a thread past the step's last chunk loads the last one again: every register is written, none is stored */     \
       const int i = (NKC % NT == 0 || tid + x * NT < NKC) ? tid + x * NT : NKC - 1;                                     \
-      kreg[S][x] = k16[(size_t)rowoff[(s) % 3][i / DC] + (i % DC)];                                                     \
+      kreg[S][x] = k16[(size_t)rowoff[i / NKC1][(s) % 3][(i % NKC1) / DC] + (i % DC)];                                  \
     }                                                                                                                   \
     _Pragma("unroll") for (int x = 0; x < CV; ++x) {                                                                    \
       const int i = (NVU % NT == 0 || tid + x * NT < NVU) ? tid + x * NT : NVU - 1;                                     \
-      const int kp = i / DC, c = i % DC;                                                                                \
-      const uint2 two = *reinterpret_cast<const uint2*>(&rowoff[(s) % 3][2 * kp]);                                      \
+      const int kp = (i % NVU1) / DC, c = i % DC;                                                                       \
+      const uint2 two = *reinterpret_cast<const uint2*>(&rowoff[i / NVU1][(s) % 3][2 * kp]);                            \
       vreg[S][x][0] = v16[(size_t)two.x + c];                                                                           \
       vreg[S][x][1] = v16[(size_t)two.y + c];                                                                           \
     }                                                                                                                   \
@@ -166,23 +176,24 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   {                                                                                                                     \
     _Pragma("unroll") for (int x = 0; x < CK; ++x) {                                                                    \
       const int i = tid + x * NT;                                                                                       \
-      if (NKC % NT == 0 || i < NKC) *reinterpret_cast<pw_u32x4_t*>(&ks[buf][i / DC][(i % DC) * 8]) = kreg[S][x];             \
+      if (NKC % NT == 0 || i < NKC)                                                                                     \
+        *reinterpret_cast<pw_u32x4_t*>(&ks[i / NKC1][buf][(i % NKC1) / DC][(i % DC) * 8]) = kreg[S][x];                 \
     }                                                                                                                   \
     _Pragma("unroll") for (int x = 0; x < CV; ++x) {                                                                    \
       const int i = tid + x * NT;                                                                                       \
       if (NVU % NT == 0 || i < NVU) {                                                                                   \
-        const int kp = i / DC, c = i % DC;                                                                              \
+        const int kp = (i % NVU1) / DC, c = i % DC, hv = i / NVU1;                                                      \
         const int col = (2 * kp) ^ (8 * (c & 7));         /* features 8 c .. 8 c + 7 share the swizzle */               \
         const pw_u32x4_t a = vreg[S][x][0], b = vreg[S][x][1];                                                          \
         _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                                 \
-          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e][col]) = (a[e] & 0xffffu) | (b[e] << 16);                 \
-          *reinterpret_cast<uint32_t*>(&vt[buf][c * 8 + 2 * e + 1][col]) = (a[e] >> 16) | (b[e] & 0xffff0000u);         \
+          *reinterpret_cast<uint32_t*>(&vt[hv][buf][c * 8 + 2 * e][col]) = (a[e] & 0xffffu) | (b[e] << 16);             \
+          *reinterpret_cast<uint32_t*>(&vt[hv][buf][c * 8 + 2 * e + 1][col]) = (a[e] >> 16) | (b[e] & 0xffff0000u);     \
         }                                                                                                               \
       }                                                                                                                 \
     }                                                                                                                   \
   }
 
-  // ---- one step of this wavefront's queries over the 64 keys in buffer `buf`
+  // ---- one step of this wavefront's queries over the 64 keys of its half in buffer `buf`
   auto compute = [&](int buf, int k0, auto masked) {
     constexpr bool MASK = decltype(masked)::value;
     pw_f32x16_t st[2];
@@ -192,7 +203,7 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
       for (int e = 0; e < 16; ++e) st[kt][e] = 0.f;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
-        const pw_bf16x8_t a = *reinterpret_cast<const pw_bf16x8_t*>(&ks[buf][kt * 32 + l32][kk * 16 + hf * 8]);
+        const pw_bf16x8_t a = *reinterpret_cast<const pw_bf16x8_t*>(&ks[kh][buf][kt * 32 + l32][kk * 16 + hf * 8]);
         st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], st[kt], 0, 0, 0);
       }
     }
@@ -247,8 +258,8 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
           pw_bf16x8_t v;
           uint2 u2[2];
         } a;
-        a.u2[0] = *reinterpret_cast<const uint2*>(&vt[buf][f][kb ^ swz]);
-        a.u2[1] = *reinterpret_cast<const uint2*>(&vt[buf][f][(kb + 8) ^ swz]);
+        a.u2[0] = *reinterpret_cast<const uint2*>(&vt[kh][buf][f][kb ^ swz]);
+        a.u2[1] = *reinterpret_cast<const uint2*>(&vt[kh][buf][f][(kb + 8) ^ swz]);
         acc[ft] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[c], acc[ft], 0, 0, 0);
       }
     }
@@ -266,7 +277,7 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   // rows of step s + 1 (asked for a step ago) go into the other buffer
 #define PW_STEP(s, MINE, NEXT)                                                                                        \
   {                                                                                                                     \
-    const int k0 = kbeg + (s) * PW_KS;                                                                                  \
+    const int k0 = kbeg + (kh * nsteps + (s)) * PW_KS;                                                                  \
     const int page_ahead = (s) + 3 < nsteps ? page_of((s) + 3) : 0;                                                     \
     if ((s) + 2 < nsteps) PW_ISSUE((s) + 2, MINE);                                                                     \
     /* the wavefront computes where its queries see any of the step's keys */                                           \
@@ -287,6 +298,31 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
 #undef PW_ISSUE
 #undef PW_STASH
 
+  if (KS > 1) {
+    // the second half's wavefront hands over what it has; the first merges: both parts' weights are relative to a
+    // reference of their own, the common one is the larger
+    float* hand = reinterpret_cast<float*>(&ks[0][0][0][0]) + (size_t)(qsub * G + wave % G) * (FT * 16 + 2) * 64 + lane;
+    static_assert(KS == 1 || (size_t)G * SUBS * (FT * 16 + 2) * 64 * sizeof(float) <= sizeof(ks), "the hand-over fits where the keys were staged");
+    if (kh == 1) {
+#pragma unroll
+      for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) hand[(ft * 16 + e) * 64] = acc[ft][e];
+      hand[FT * 16 * 64] = m;
+      hand[(FT * 16 + 1) * 64] = l;
+    }
+    __syncthreads();
+    if (kh == 1) return;
+    const float m1 = hand[FT * 16 * 64], l1 = hand[(FT * 16 + 1) * 64];
+    const float mm = fmaxf(m, m1);
+    const float a0 = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mm);
+    const float a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - mm);
+    l = l * a0 + l1 * a1;
+#pragma unroll
+    for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[ft][e] = acc[ft][e] * a0 + hand[(ft * 16 + e) * 64] * a1;
+  }
   if (!live) return;
   const float inv = 1.0f / l;
   bf16* orow = out + (size_t)(r0 + l32) * nh * D + (size_t)h * D;
@@ -323,12 +359,15 @@ extern "C" int gs_attention_prefill_wide(const void* q, int q_stride, const void
                                          const int* tile_n, int ntiles /* blocks: tile_rows / 32 entries of the three lists each */,
                                          const int* block_table, int max_blocks,
                                          int page_size, long cache_pages, int window, float scale, void* out, int nh,
-                                         int nkv, int d, int tile_rows, hipStream_t stream) {
+                                         int nkv, int d, int tile_rows, int key_splits, hipStream_t stream) {
   GS_REQUIRE(gs_attention_prefill_wide_supports(nh, nkv, d), "attention_prefill_wide: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
   const int G = nh / nkv;
-  GS_REQUIRE(tile_rows == wide_rows(G, 1) || tile_rows == wide_rows(G, 0),
-             "attention_prefill_wide: tiles of a group of %d heads hold up to %d or %d queries, not %d", G, wide_rows(G, 1), wide_rows(G, 0), tile_rows);
-  const bool full = tile_rows == wide_rows(G, 1);
+  GS_REQUIRE(key_splits == 1 || (key_splits == 2 && wide_rows(G, 1) >= 64),
+             "attention_prefill_wide: the keys are walked whole or, for groups of up to 4 heads, in two halves, not in %d parts", key_splits);
+  GS_REQUIRE(tile_rows * key_splits == wide_rows(G, 1) || (key_splits == 1 && tile_rows == wide_rows(G, 0)),
+             "attention_prefill_wide: tiles of a group of %d heads hold up to %d or %d queries (%d with the keys in two halves), not %d",
+             G, wide_rows(G, 1), wide_rows(G, 0), wide_rows(G, 1) / 2, tile_rows);
+  const bool full = tile_rows * key_splits == wide_rows(G, 1);
   GS_REQUIRE(ntiles >= 0 && (long)ntiles * nkv < (1L << 31), "attention_prefill_wide: %d tiles x %d key heads are too many blocks", ntiles, nkv);
   GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill_wide: bad page_size/max_blocks/window");
   GS_REQUIRE(q_stride >= nh * d && q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_prefill_wide: q rows must be 16-byte aligned");
@@ -342,21 +381,23 @@ extern "C" int gs_attention_prefill_wide(const void* q, int q_stride, const void
   if (ntiles == 0) return 0;
   const unsigned page_magic = (unsigned)((1ull << 32) / (unsigned)page_size + 1);
   dim3 grid((unsigned)ntiles * (unsigned)nkv);
-#define GS_RUN(GG, WQ)                                                                                                \
-  attention_prefill_wide_kernel<64, GG, WQ><<<grid, GG * WQ * 64, 0, stream>>>(                                       \
+#define GS_RUN2(GG, WQ, KS)                                                                                           \
+  attention_prefill_wide_kernel<64, GG, WQ, KS><<<grid, GG * WQ * 64, 0, stream>>>(                                   \
       (const bf16*)q, q_stride, (const bf16*)kcache, (const bf16*)vcache, positions, tile_seq, tile_row, tile_n,       \
       block_table, max_blocks, page_size, page_magic, window, scale, (bf16*)out, nh, nkv)
+#define GS_RUN(GG, WQ) { if (key_splits == 2) GS_RUN2(GG, WQ, 2); else GS_RUN2(GG, WQ, 1); }
   switch (G) {
-    case 1: if (full) GS_RUN(1, 8); else GS_RUN(1, 4); break;
-    case 2: if (full) GS_RUN(2, 4); else GS_RUN(2, 2); break;
-    case 3: if (full) GS_RUN(3, 2); else GS_RUN(3, 1); break;
-    case 4: if (full) GS_RUN(4, 2); else GS_RUN(4, 1); break;
-    case 5: GS_RUN(5, 1); break;
-    case 6: GS_RUN(6, 1); break;
-    case 7: GS_RUN(7, 1); break;
-    default: GS_RUN(8, 1); break;
+    case 1: if (full) GS_RUN(1, 8) else GS_RUN2(1, 4, 1); break;
+    case 2: if (full) GS_RUN(2, 4) else GS_RUN2(2, 2, 1); break;
+    case 3: if (full) GS_RUN(3, 2) else GS_RUN2(3, 1, 1); break;
+    case 4: if (full) GS_RUN(4, 2) else GS_RUN2(4, 1, 1); break;
+    case 5: GS_RUN2(5, 1, 1); break;
+    case 6: GS_RUN2(6, 1, 1); break;
+    case 7: GS_RUN2(7, 1, 1); break;
+    default: GS_RUN2(8, 1, 1); break;
   }
 #undef GS_RUN
+#undef GS_RUN2
   GS_LAUNCH_CHECK("attention_prefill_wide");
   return 0;
 }

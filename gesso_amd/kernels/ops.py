@@ -849,11 +849,13 @@ def attention_prefill_wide_rows(nh: int, nkv: int, full: bool = True) -> int:
 
 
 def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv,
-                           d, ntok, out: torch.Tensor = None, full: bool = True) -> torch.Tensor:
+                           d, ntok, out: torch.Tensor = None, full: bool = True, key_splits: int = 1) -> torch.Tensor:
     """Causal GQA of long prompt portions (bfloat16, heads of 64): 32 queries a wavefront, keys and values shared by a
     block through LDS.  ``tiles``: int32 ``(3, blocks * wq)``, the sequence, first row and row count (at most 32; 0: none)
-    of every sub-tile, ``wq = attention_prefill_wide_rows(nh, nkv, full) // 32`` of them a block, all of one sequence,
-    neighbours or not (``BatchContext.query_subtiles`` pairs late ones with early ones)."""
+    of every sub-tile, ``wq = attention_prefill_wide_rows(nh, nkv, full) // 32 // key_splits`` of them a block, all of
+    one sequence, neighbours or not (``BatchContext.query_subtiles`` pairs late ones with early ones).  With
+    ``key_splits = 2`` (groups of up to four heads) a block holds half as many queries and two wavefronts walk half
+    of the keys each: twice the blocks, half the longest walk."""
     _dev(q, kcache, vcache, positions, tiles, block_table, out)
     _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
           "attention_prefill_wide takes bfloat16")
@@ -861,7 +863,9 @@ def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_
     _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
           "cache must be (pages, nkv, page_size, d)")
     _i32(positions, ntok, "positions")
-    rows = attention_prefill_wide_rows(nh, nkv, full)
+    _need(key_splits in (1, 2) and (key_splits == 1 or (full and attention_prefill_wide_rows(nh, nkv, True) >= 64)),
+          "attention_prefill_wide: the keys in two halves only for groups of up to four heads")
+    rows = attention_prefill_wide_rows(nh, nkv, full) // key_splits
     wq = rows // 32
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[0] == 3 and wq > 0 and tiles.shape[1] % wq == 0,
           "tiles must be int32 (3, blocks * sub-tiles a block)")
@@ -873,5 +877,5 @@ def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_
     _check(lib().gs_attention_prefill_wide(_p(q), q_stride, _p(kcache), _p(vcache), _p(positions), _p(tiles[0]),
                                            _p(tiles[1]), _p(tiles[2]), nt, _p(block_table),
                                            block_table.shape[1], page_size, kcache.shape[0],
-                                           window or 0, scale, _p(out), nh, nkv, d, rows, _stream()))
+                                           window or 0, scale, _p(out), nh, nkv, d, rows, key_splits, _stream()))
     return out

@@ -31,6 +31,7 @@ class RawQKV:
 class Attention(Part):
     graph_safe = True
     stage, out_stage = "attn_mixer", "attn_outproj"   # the decode profiler's names
+    HALVES_MAX_KEYS = 4096    # prompts whose sequences hold fewer keys may have their keys walked in two halves
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
@@ -151,12 +152,20 @@ class Attention(Part):
                 # heads on 8 key heads: 46.7 against 53.1 us; 2,048 over a prefix of 2,048: 97.8 against 104.7).  With
                 # more blocks than units the chip balances by itself and paired blocks, which all walk to their late
                 # queries' end, only add steps (4,096 tokens: 156 against 122 us); a window makes every walk as short.
+                # Short walks at most a block a unit: two wavefronts a head walk half of the keys each and merge at the end,
+                # so that the longest walk is half as long and twice the blocks spread evenly (the same prompt 40.4 us;
+                # 1,024 tokens 18.9 against 25.4; 512 over a prefix of 1,024: 24.5 against 37.4; over a prefix of 30,720,
+                # where every walk is long, staging two halves a step costs more than it saves: 897 against 834).
                 wq = ops.attention_prefill_wide_rows(nh, nkv) // 32
                 blocks = sum(-(-(-(-n // 32)) // wq) for n in ctx.q_lens[lead:]) * nkv
-                paired = not window and wq >= 2 and blocks <= rt.compute_units
+                few = blocks <= rt.compute_units
+                halves = 2 if few and wq >= 2 and ctx.max_kv_len is not None and ctx.max_kv_len < self.HALVES_MAX_KEYS else 1
+                wq //= halves
+                paired = not window and wq >= 2 and few
                 return ops.attention_prefill_wide(q, q_stride, cache.k, cache.v, ctx.positions,
                                                   ctx.query_subtiles(wq, lead, paired=paired), cache.block_table,
-                                                  cache.page_size, window, self.scale, nh, nkv, d, ctx.T, out=out)
+                                                  cache.page_size, window, self.scale, nh, nkv, d, ctx.T, out=out,
+                                                  key_splits=halves)
             # tiles of 32 share every key and value fragment between two products, which pays when portions are
             # long (groups of more than four heads have no registers for tiles of 32)
             rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16

@@ -1007,17 +1007,22 @@ def paged(k, v, ps, g):
 
 
 @pytest.mark.parametrize("nh,nkv,ps", [(32, 8, 16), (3, 1, 16), (5, 5, 4), (4, 2, 8), (16, 2, 16), (6, 2, 6)])
-@pytest.mark.parametrize("window,paired", [(None, True), (None, False), (37, False), (200, False), (200, True)])
-def test_attention_prefill_wide(ops, nh, nkv, ps, window, paired):
+@pytest.mark.parametrize("window,paired,halves", [(None, True, 1), (None, False, 1), (37, False, 1), (200, False, 1), (200, True, 1),
+                                                   (None, False, 2), (None, True, 2), (37, False, 2), (200, True, 2)])
+def test_attention_prefill_wide(ops, nh, nkv, ps, window, paired, halves):
     """The kernel for long portions, heads of 64: four sequences in one launch (a long chunk over a cached prefix that
     ends inside a page, a fresh prompt of some hundred tokens, a single token, a chunk that starts at a step's edge).
     Rows of pages past a sequence's end hold NaN: a value read from there, even with weight zero, would show.
-    A block's sub-tiles of 32 queries as neighbours, and paired from both ends of the sequence (late with early)."""
+    A block's sub-tiles of 32 queries as neighbours, and paired from both ends of the sequence (late with early); the
+    keys walked whole, and in two halves by two wavefronts that merge at the end."""
     from gesso_amd.engine.batch import subtile_lists
     d = 64
     assert ops.attention_prefill_wide_supports(nh, nkv, d) and not ops.attention_prefill_wide_supports(nh, nkv, 128)
     rows = ops.attention_prefill_wide_rows(nh, nkv)
     assert rows == {1: 256, 2: 128, 3: 64, 4: 64}.get(nh // nkv, 32)
+    if halves == 2 and rows < 64:
+        pytest.skip("groups of more than four heads hold one sub-tile a block: nothing to halve")
+    rows //= halves
     g = gen(nh + ps + (window or 0))
     prefix, new = [75, 0, 45, 128], [141, 333, 1, 70]
     kcs, vcs, tables, qs, want = [], [], [], [], []
@@ -1047,11 +1052,11 @@ def test_attention_prefill_wide(ops, nh, nkv, ps, window, paired):
     wide = torch.zeros(sum(new), stride, dtype=torch.bfloat16)
     wide[:, :nh * d] = qall
     got = ops.attention_prefill_wide(wide.to(DEV), stride, kc.to(DEV), vc.to(DEV), positions.to(DEV), tiles.to(DEV),
-                                     table.to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, sum(new))
+                                     table.to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, sum(new), key_splits=halves)
     close(got, want, torch.bfloat16)
 
 
-@pytest.mark.parametrize("kernel", ["wide", "tiles16", "tiles32"])
+@pytest.mark.parametrize("kernel", ["wide", "wide-halves", "tiles16", "tiles32"])
 @pytest.mark.parametrize("window", [None, 50])
 def test_prompt_attention_never_sees_the_next_key_nor_the_one_before_its_window(ops, kernel, window):
     """Every key stands out for the query one place before it (and, with a window, for the query `window` places after
@@ -1078,8 +1083,9 @@ def test_prompt_attention_never_sees_the_next_key_nor_the_one_before_its_window(
         assert float((loose - want).abs().max()) > 0.5
     kc, vc, tab = paged(k, v, ps, g)
     positions = torch.arange(prefix, K, dtype=torch.int32)
-    rows = ops.attention_prefill_wide_rows(nh, nkv) if kernel == "wide" else int(kernel[5:])
-    if kernel == "wide":
+    halves = 2 if kernel == "wide-halves" else 1
+    rows = ops.attention_prefill_wide_rows(nh, nkv) // halves if kernel.startswith("wide") else int(kernel[5:])
+    if kernel.startswith("wide"):
         from gesso_amd.engine.batch import subtile_lists
         tiles = torch.tensor(subtile_lists([new], rows // 32, 0, paired=not window), dtype=torch.int32)
     else:
@@ -1087,7 +1093,7 @@ def test_prompt_attention_never_sees_the_next_key_nor_the_one_before_its_window(
                              dtype=torch.int32)
     args = (q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV), positions.to(DEV), tiles.to(DEV), tab[None].to(DEV), ps,
             window, 1.0 / math.sqrt(d), nh, nkv, d, new)
-    got = ops.attention_prefill_wide(*args) if kernel == "wide" else ops.attention_prefill(*args, tile_rows=rows)
+    got = ops.attention_prefill_wide(*args, key_splits=halves) if kernel.startswith("wide") else ops.attention_prefill(*args, tile_rows=rows)
     close(got, want, torch.bfloat16)
 
 
@@ -1104,12 +1110,15 @@ def test_attention_prefill_wide_over_thousands_of_keys(ops):
         q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
         kc, vc, tab = paged(k, v, ps, g)
         from gesso_amd.engine.batch import subtile_lists
-        rows = ops.attention_prefill_wide_rows(nh, nkv)
-        tiles = torch.tensor(subtile_lists([new], rows // 32, 0, paired=not window), dtype=torch.int32)
-        got = ops.attention_prefill_wide(q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV),
-                                         torch.arange(prefix, K, dtype=torch.int32, device=DEV), tiles.to(DEV),
-                                         tab[None].contiguous().to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, new)
-        close(got, P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(new, -1), torch.bfloat16)
+        want = P.causal_attention(q.double(), k.double(), v.double(), window or 0).reshape(new, -1)
+        for halves in (1, 2):          # the far key lies in the first half of the walk, the queries' own keys in the second
+            rows = ops.attention_prefill_wide_rows(nh, nkv) // halves
+            tiles = torch.tensor(subtile_lists([new], rows // 32, 0, paired=not window), dtype=torch.int32)
+            got = ops.attention_prefill_wide(q.reshape(new, -1).to(DEV), nh * d, kc.to(DEV), vc.to(DEV),
+                                             torch.arange(prefix, K, dtype=torch.int32, device=DEV), tiles.to(DEV),
+                                             tab[None].contiguous().to(DEV), ps, window, 1.0 / math.sqrt(d), nh, nkv, d, new,
+                                             key_splits=halves)
+            close(got, want, torch.bfloat16)
 
 
 # ------------------------------------------------------------------ rows in the matrix cores' order (tiled rows)
