@@ -2,8 +2,8 @@
 //
 // The kernel of attention_prefill_impl.h gives a wavefront 16 or 32 queries, loads keys straight into registers
 // and meets at two barriers per 64 keys; its wavefronts move in step, so the matrix cores wait while the softmax's
-// arithmetic runs and the other way round.  Here a block's wavefronts meet once per 64 keys, and two blocks
-// share a compute unit, so that one block's products run under the other's softmax:
+// arithmetic runs and the other way round.  Here a block's wavefronts meet once per 64 keys, keys and values are
+// staged once for all of them, and their rows are asked for two steps before they are used:
 //
 //   * A block owns one key head and WQ sub-tiles of up to 32 consecutive queries of one sequence; wavefront w takes
 //     query head w % G of the group and sub-tile w / G.  (WQ = 8, 4, 2, 2, 1 for groups of 1, 2, 3, 4 and more
@@ -337,12 +337,12 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
     }
 }
 
-// Queries a tile of this kernel holds for a group of g query heads to a key head: 32 per wavefront, and as many
-// wavefronts per head as make eight to a block (`full`) or four (for steps with few tiles: twice the blocks, two to a
-// compute unit, which spreads a short prompt's uneven walks better).
-static int wide_rows(int g, int full) {
+// Queries a block of this kernel holds for a group of g query heads to a key head when it walks the keys whole: 32 per
+// wavefront, and as many wavefronts per head as make eight to a block.  (Blocks of four wavefronts, twice as many, were
+// measured too: 61.5 against 58.0 us at 2,048 tokens, 970 against 776 us over a prefix of 30,720.)
+static int wide_rows(int g) {
   const int wq = g == 1 ? 8 : (g == 2 ? 4 : (g <= 4 ? 2 : 1));
-  return 32 * (full || wq == 1 ? wq : wq / 2);
+  return 32 * wq;
 }
 
 extern "C" int gs_attention_prefill_wide_supports(int nh, int nkv, int d) {
@@ -352,7 +352,7 @@ extern "C" int gs_attention_prefill_wide_supports(int nh, int nkv, int d) {
 }
 
 // The most queries a block may hold: 32 for each of its sub-tiles.
-extern "C" int gs_attention_prefill_wide_rows(int nh, int nkv, int full) { return nkv > 0 ? wide_rows(nh / nkv, full) : 0; }
+extern "C" int gs_attention_prefill_wide_rows(int nh, int nkv) { return nkv > 0 ? wide_rows(nh / nkv) : 0; }
 
 extern "C" int gs_attention_prefill_wide(const void* q, int q_stride, const void* kcache, const void* vcache,
                                          const int* positions, const int* tile_seq, const int* tile_row,
@@ -362,12 +362,11 @@ extern "C" int gs_attention_prefill_wide(const void* q, int q_stride, const void
                                          int nkv, int d, int tile_rows, int key_splits, hipStream_t stream) {
   GS_REQUIRE(gs_attention_prefill_wide_supports(nh, nkv, d), "attention_prefill_wide: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
   const int G = nh / nkv;
-  GS_REQUIRE(key_splits == 1 || (key_splits == 2 && wide_rows(G, 1) >= 64),
+  GS_REQUIRE(key_splits == 1 || (key_splits == 2 && wide_rows(G) >= 64),
              "attention_prefill_wide: the keys are walked whole or, for groups of up to 4 heads, in two halves, not in %d parts", key_splits);
-  GS_REQUIRE(tile_rows * key_splits == wide_rows(G, 1) || (key_splits == 1 && tile_rows == wide_rows(G, 0)),
-             "attention_prefill_wide: tiles of a group of %d heads hold up to %d or %d queries (%d with the keys in two halves), not %d",
-             G, wide_rows(G, 1), wide_rows(G, 0), wide_rows(G, 1) / 2, tile_rows);
-  const bool full = tile_rows * key_splits == wide_rows(G, 1);
+  GS_REQUIRE(tile_rows * key_splits == wide_rows(G),
+             "attention_prefill_wide: blocks of a group of %d heads hold up to %d queries (%d with the keys in two halves), not %d",
+             G, wide_rows(G), wide_rows(G) / 2, tile_rows);
   GS_REQUIRE(ntiles >= 0 && (long)ntiles * nkv < (1L << 31), "attention_prefill_wide: %d tiles x %d key heads are too many blocks", ntiles, nkv);
   GS_REQUIRE(page_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill_wide: bad page_size/max_blocks/window");
   GS_REQUIRE(q_stride >= nh * d && q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attention_prefill_wide: q rows must be 16-byte aligned");
@@ -387,10 +386,10 @@ extern "C" int gs_attention_prefill_wide(const void* q, int q_stride, const void
       block_table, max_blocks, page_size, page_magic, window, scale, (bf16*)out, nh, nkv)
 #define GS_RUN(GG, WQ) { if (key_splits == 2) GS_RUN2(GG, WQ, 2); else GS_RUN2(GG, WQ, 1); }
   switch (G) {
-    case 1: if (full) GS_RUN(1, 8) else GS_RUN2(1, 4, 1); break;
-    case 2: if (full) GS_RUN(2, 4) else GS_RUN2(2, 2, 1); break;
-    case 3: if (full) GS_RUN(3, 2) else GS_RUN2(3, 1, 1); break;
-    case 4: if (full) GS_RUN(4, 2) else GS_RUN2(4, 1, 1); break;
+    case 1: GS_RUN(1, 8) break;
+    case 2: GS_RUN(2, 4) break;
+    case 3: GS_RUN(3, 2) break;
+    case 4: GS_RUN(4, 2) break;
     case 5: GS_RUN2(5, 1, 1); break;
     case 6: GS_RUN2(6, 1, 1); break;
     case 7: GS_RUN2(7, 1, 1); break;

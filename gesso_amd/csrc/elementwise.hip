@@ -531,20 +531,6 @@ extern "C" int gs_stream_read(const void* p, long bytes, unsigned* sink, int blo
   return 0;
 }
 
-__global__ void fill_f32_kernel(float* p, float v, long n) {
-  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = v;
-}
-
-// A fill that is an ordinary kernel, so that it may be recorded into a HIP graph.
-extern "C" int gs_fill_f32(float* p, float v, long n, hipStream_t stream) {
-  GS_REQUIRE(n >= 0, "fill: bad size");
-  if (n == 0) return 0;
-  fill_f32_kernel<<<gs_ceil_div(n, 256), 256, 0, stream>>>(p, v, n);
-  GS_LAUNCH_CHECK("fill_f32");
-  return 0;
-}
-
 // Fill chosen rows of a pool with one value: pool (outer, num_rows, row) of float32 or bfloat16, ids (n) rows to
 // fill in every one of the `outer` planes (a negative id is skipped).  A request's state slots are rows of a pool
 // with one plane, a cache page is a row in each layer's K and V plane.  Used to give a fresh slot its initial

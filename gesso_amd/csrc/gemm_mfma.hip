@@ -189,9 +189,6 @@ static void launch_mfma(const bf16* X, int ldx, const bf16* W, TOut* Y, int ldy,
   gemm_mfma_kernel<BM, BN, WM, WN, EPI, TOut><<<(unsigned)tiles, WM * WN * 64, lds, stream>>>(X, ldx, W, Y, ldy, M, N, K);
 }
 
-// Whether the kernel takes the product: any M, N; K a multiple of 8 (16-byte loads).
-extern "C" int gs_gemm_mfma_supports(int M, int N, int K) { return M > 0 && N > 0 && K > 0 && K % 8 == 0; }
-
 // epilogue 0: Y (M, N) = X W^T, bfloat16 or float32.  epilogue 1: Y (M, N / 2) = silu(X Wg^T) * (X Wu^T), bfloat16.
 extern "C" int gs_gemm_mfma(const void* X, int ldx, const void* W, void* Y, int y_dtype, int ldy, int M, int N, int K,
                             int epilogue, hipStream_t stream) {

@@ -249,13 +249,6 @@ def stream_read(buf: torch.Tensor, blocks: int = 2048, contiguous: bool = True, 
     _check(lib().gs_stream_read(_p(buf), c_long(nbytes), _p(sink), c_int(blocks), c_int(1 if contiguous else 0), _stream()))
 
 
-def fill_f32(t: torch.Tensor, value: float) -> torch.Tensor:
-    _dev(t)
-    _need(t.dtype == torch.float32, "fill_f32 takes float32")
-    _check(lib().gs_fill_f32(_p(t), c_float(value), c_long(t.numel()), _stream()))
-    return t
-
-
 FILL_MAX = 65535
 
 
@@ -842,17 +835,17 @@ def attention_prefill_wide_supports(nh: int, nkv: int, d: int) -> bool:
     return bool(lib().gs_attention_prefill_wide_supports(c_int(nh), c_int(nkv), c_int(d)))
 
 
-def attention_prefill_wide_rows(nh: int, nkv: int, full: bool = True) -> int:
-    """The most queries a tile of :func:`attention_prefill_wide` holds for these head counts: blocks of eight
-    wavefronts (``full``), or of four for steps with few tiles."""
-    return int(lib().gs_attention_prefill_wide_rows(c_int(nh), c_int(nkv), c_int(1 if full else 0)))
+def attention_prefill_wide_rows(nh: int, nkv: int) -> int:
+    """The most queries a block of :func:`attention_prefill_wide` holds for these head counts when it walks the keys
+    whole (half as many with the keys in two halves)."""
+    return int(lib().gs_attention_prefill_wide_rows(c_int(nh), c_int(nkv)))
 
 
 def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv,
-                           d, ntok, out: torch.Tensor = None, full: bool = True, key_splits: int = 1) -> torch.Tensor:
+                           d, ntok, out: torch.Tensor = None, key_splits: int = 1) -> torch.Tensor:
     """Causal GQA of long prompt portions (bfloat16, heads of 64): 32 queries a wavefront, keys and values shared by a
     block through LDS.  ``tiles``: int32 ``(3, blocks * wq)``, the sequence, first row and row count (at most 32; 0: none)
-    of every sub-tile, ``wq = attention_prefill_wide_rows(nh, nkv, full) // 32 // key_splits`` of them a block, all of
+    of every sub-tile, ``wq = attention_prefill_wide_rows(nh, nkv) // 32 // key_splits`` of them a block, all of
     one sequence, neighbours or not (``BatchContext.query_subtiles`` pairs late ones with early ones).  With
     ``key_splits = 2`` (groups of up to four heads) a block holds half as many queries and two wavefronts walk half
     of the keys each: twice the blocks, half the longest walk."""
@@ -863,9 +856,9 @@ def attention_prefill_wide(q, q_stride, kcache, vcache, positions, tiles, block_
     _need(kcache.dim() == 4 and kcache.shape[1:] == (nkv, page_size, d) and vcache.shape == kcache.shape,
           "cache must be (pages, nkv, page_size, d)")
     _i32(positions, ntok, "positions")
-    _need(key_splits in (1, 2) and (key_splits == 1 or (full and attention_prefill_wide_rows(nh, nkv, True) >= 64)),
+    _need(key_splits in (1, 2) and (key_splits == 1 or attention_prefill_wide_rows(nh, nkv) >= 64),
           "attention_prefill_wide: the keys in two halves only for groups of up to four heads")
-    rows = attention_prefill_wide_rows(nh, nkv, full) // key_splits
+    rows = attention_prefill_wide_rows(nh, nkv) // key_splits
     wq = rows // 32
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[0] == 3 and wq > 0 and tiles.shape[1] % wq == 0,
           "tiles must be int32 (3, blocks * sub-tiles a block)")
