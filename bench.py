@@ -322,6 +322,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--size", default="1.2b", choices=sorted(SIZES), help="the layer sizes (the default line: 1.2b)")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--temperature", type=float, default=0.0, help="the main decode run draws at this temperature (0: greedy)")
     ap.add_argument("--top-p", type=float, default=1.0, help="with --temperature: draws from the nucleus of this mass")
@@ -348,8 +349,9 @@ def main() -> int:
 
     from gesso_amd import Engine
 
-    cfg = model_config()
+    cfg = model_config(args.size)
     layers_full = cfg.num_hidden_layers
+    model_name = f"LFM2-{args.size.upper()} sizes"
     if args.layers is not None and args.layers < layers_full:
         import dataclasses
         cfg = dataclasses.replace(cfg, num_hidden_layers=args.layers, layer_types=cfg.layer_types[:args.layers])
@@ -373,11 +375,11 @@ def main() -> int:
     bytes_step = wbytes + kv_bytes(cfg, engine, [mean_ctx] * args.batch)
     achieved = bytes_step / (ms * 1e-3) / 1e9
     out = {
-        "metric": f"decode tok/s at batch {args.batch} (LFM2-1.2B sizes, 512-token prompts)", "value": round(value, 1),
+        "metric": f"decode tok/s at batch {args.batch} ({model_name}, 512-token prompts)", "value": round(value, 1),
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
-        "config": {"model": "LFM2-1.2B sizes", "layers": cfg.num_hidden_layers, "layers_full": layers_full,
+        "config": {"model": model_name, "layers": cfg.num_hidden_layers, "layers_full": layers_full,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "ff": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "conv_L_cache": cfg.conv_L_cache, "attn_layers": sum(t == "full_attention" for t in cfg.layer_types),
