@@ -839,6 +839,38 @@ def test_gemm_skinny_conv_equals_the_separate_kernels(ops, M, H, W, bias, weight
 
 
 @pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("W", [2, 3, 4])
+@pytest.mark.parametrize("H", [64, 96, 256, 1280])
+def test_gemm_skinny_conv_over_row_tiles_widths_and_shares_of_k(ops, H, W, bias, weighted):
+    """The fused input product + convolution at one to four row tiles (3, 20, 40 and 64 rows), every width the
+    epilogue holds in registers, with and without a bias, rows normed on the fly and pre-weighted, and hidden sizes that
+    give a wavefront less than a batch of steps, exactly one, and several with a remainder: the same as the product
+    followed by the convolution kernel, channel by channel (a value of one lane's four channels that went missing
+    would show in every fourth column)."""
+    for M in (3, 20, 40, 64):
+        res, nw, lazy = lazy_case(ops, M, H, M + H + W, weighted)
+        g = gen(H + W + M)
+        w_in = (torch.randn(3 * H, H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
+        taps = torch.randn(H, W, generator=g).to(DEV)
+        b = torch.randn(H, generator=g).to(DEV) if bias else None
+        state0 = torch.randn(M + 2, H, W - 1, generator=g)
+        slots = torch.randperm(M + 2, generator=g)[:M].to(torch.int32).to(DEV)
+        s1, s2 = state0.clone().to(DEV), state0.clone().to(DEV)
+        for wt in ([None] if H % 16 else [None, ops.tile_major(w_in)]):
+            s1.copy_(state0)
+            s2.copy_(state0)
+            got = ops.gemm_skinny_conv(lazy, w_in, taps, b, s1, slots, wt=wt)
+            bcx = ops.gemm_skinny(lazy, w_in, wt=wt)
+            ar = torch.arange(M, dtype=torch.int32, device=DEV)
+            want = ops.short_conv(bcx, taps, b, s2, ar, torch.arange(M + 1, dtype=torch.int32, device=DEV), slots, M, True)
+            d = (got.float() - want.float()).abs()
+            tol = 1e-2 * max(1.0, float(want.float().abs().max()))
+            assert float(d.max()) <= tol, f"M={M} tile-major={wt is not None}: columns {sorted(set((torch.nonzero(d > tol)[:, 1] % 4).tolist()))} (mod 4) differ"
+            assert float((s1 - s2).abs().max()) <= 1e-2 * max(1.0, float(s2.abs().max())), f"M={M}: history"
+
+
+@pytest.mark.parametrize("weighted", [False, True])
 @pytest.mark.parametrize("M,H,W", [(1, 2048, 3), (8, 2048, 3), (64, 2048, 3), (48, 1024, 3), (33, 96, 4)])
 def test_gemm_skinny_conv_against_the_plain_convolution(ops, M, H, W, weighted):
     """The input product with the short convolution as its epilogue, at the widths and row counts of the benchmarked
