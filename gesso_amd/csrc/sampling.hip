@@ -121,9 +121,11 @@ struct Crossing {
 // strict = 0: first running sum >= target; strict = 1: first running sum > target.
 //
 // The first passes read the whole row.  Once a pass has narrowed the candidates down to NUC_LIST or fewer (after its
-// second byte the weights left lie within a few percent of each other, a handful in a peaked row), their ids are
-// gathered into a list in LDS and the later passes read only those; a list of NUC_DIRECT ids or fewer is
-// settled at once, a candidate to a thread.
+// second byte the weights left lie within a few percent of each other, a handful in a peaked row), their ids and
+// their weights' patterns are gathered into lists in LDS (a wavefront takes its places in the lists with one atomic
+// add, a lane its place among the wavefront's by counting the lanes before it) and the later passes read only those,
+// from LDS; as soon as a pass leaves NUC_DIRECT candidates or fewer under its prefix they are settled at once, a
+// candidate to a thread.
 #define NUC_LIST 8192
 #define NUC_DIRECT 256
 //
@@ -136,7 +138,7 @@ struct Crossing {
 #define NUC_GHIST (NUC_G0 + 4 * 256)
 __device__ Crossing radix_descend(const double* __restrict__ w, int V, double target, int strict,
                                   unsigned long long* hmass, int* hcount, Crossing* shared_out, int* clist,
-                                  const unsigned long long* __restrict__ ghist = nullptr) {
+                                  unsigned long long* lbits, const unsigned long long* __restrict__ ghist = nullptr) {
   __shared__ int cn, picked;
   __shared__ unsigned long long cbits[NUC_DIRECT], cmass[NUC_DIRECT];
   unsigned long long prefix = 0;
@@ -175,8 +177,7 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
     }
     const int n = ready ? 0 : (nlist >= 0 ? nlist : V);
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
-      const int j = nlist >= 0 ? clist[i] : i;
-      unsigned long long bits = (unsigned long long)__double_as_longlong(w[j]);
+      const unsigned long long bits = nlist >= 0 ? lbits[i] : (unsigned long long)__double_as_longlong(w[i]);
       if ((bits & himask) == prefix) {
         int b = (int)((bits >> shift) & 0xff);
         if (b != run_b) {
@@ -188,7 +189,7 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
           run_m = 0ull;
           run_n = 0;
         }
-        run_m += (unsigned long long)__double2ll_rn(w[j] * scale);
+        run_m += (unsigned long long)__double2ll_rn(__longlong_as_double((long long)bits) * scale);
         run_n += 1;
       }
     }
@@ -256,56 +257,95 @@ __device__ Crossing radix_descend(const double* __restrict__ w, int V, double ta
     }
     if (nlist < 0 && pass >= 1 && pass <= 5 && left <= NUC_LIST) {
       const unsigned long long sofar = (~0ull) << shift;
-      for (int j = threadIdx.x; j < V; j += blockDim.x)
-        if (((unsigned long long)__double_as_longlong(w[j]) & sofar) == prefix) clist[atomicAdd(&cn, 1)] = j;
+      const int lane = threadIdx.x & 63;
+      // One compute unit pulls a row of 65,536 weights (512 KB) no faster than its loads in flight allow: eight loads
+      // a thread are asked for before the first is looked at (a turn of the loop is otherwise a round trip to memory,
+      // 64 of them a row; loads of two weights, and sixteen in flight, need more registers than 1,024 threads leave
+      // a lane and came out slower: 72 to 80 us against 64 for the step's three kernels on peaked rows).
+      constexpr int GATHER = 8;
+      for (int j0 = 0; j0 < V; j0 += GATHER * blockDim.x) {   // every thread makes every turn: the wavefront votes
+        unsigned long long got[GATHER];
+#pragma unroll
+        for (int g = 0; g < GATHER; ++g) {
+          const int j = j0 + g * blockDim.x + threadIdx.x;
+          got[g] = j < V ? (unsigned long long)__double_as_longlong(w[j]) : 0ull;
+        }
+#pragma unroll
+        for (int g = 0; g < GATHER; ++g) {
+          const int j = j0 + g * blockDim.x + threadIdx.x;
+          const bool take = j < V && (got[g] & sofar) == prefix;
+          const unsigned long long votes = __ballot(take);
+          if (votes) {
+            const int first = __ffsll((long long)votes) - 1;
+            int base = 0;
+            if (lane == first) base = atomicAdd(&cn, __popcll(votes));
+            base = __shfl(base, first, 64);
+            if (take) {
+              const int at = base + __popcll(votes & ((1ull << lane) - 1ull));
+              clist[at] = j;
+              lbits[at] = got[g];
+            }
+          }
+        }
+      }
       __syncthreads();
       nlist = cn;
-      if (nlist <= NUC_DIRECT) {
-        // a candidate to a thread: no more passes.  Each adds up the masses of the candidates heavier than its own
-        // and of those as heavy (integers, scaled to the largest weight under the prefix); the pattern at which the
-        // running sum crosses the target is the one whose candidates see the target between these two sums
-        const int t = threadIdx.x;
-        const double top = __longlong_as_double((long long)(prefix | ((1ull << shift) - 1ull)));
-        const double sc = exp2((double)(62 - lv)) / top, unsc = 1.0 / sc;
-        unsigned long long mybits = 0ull;
-        if (t < nlist) {
-          const double wt = w[clist[t]];
-          mybits = (unsigned long long)__double_as_longlong(wt);
-          cbits[t] = mybits;
-          cmass[t] = (unsigned long long)__double2ll_rn(wt * sc);
-        }
-        if (t == 0) {
-          cn = 0x7fffffff;      // the lowest thread at the crossing
-          picked = 0x7fffffff;  // the lowest thread with the lightest pattern, should nothing cross
-        }
-        __syncthreads();
-        unsigned long long heavier = 0ull, same = 0ull, lightest = ~0ull;
-        for (int j = 0; t < nlist && j < nlist; ++j) {
-          const unsigned long long b = cbits[j], m = cmass[j];
-          heavier += b > mybits ? m : 0ull;
-          same += b == mybits ? m : 0ull;
-          lightest = b < lightest ? b : lightest;
-        }
-        if (t < nlist) {
-          const double lo = above + (double)heavier * unsc, hi = above + (double)(heavier + same) * unsc;
-          const bool crossed = strict ? (target < hi && !(target < lo)) : (hi >= target && !(lo >= target));
-          if (crossed) atomicMin(&cn, t);
-          if (mybits == lightest) atomicMin(&picked, t);
-        }
-        __syncthreads();
-        const int owner = cn != 0x7fffffff ? cn : picked;
-        if (t == owner) {
-          shared_out->bits = mybits;
-          shared_out->above = above + (double)heavier * unsc;
-        }
-        __syncthreads();
-        Crossing c;
-        c.bits = shared_out->bits;
-        c.above = shared_out->above;
-        c.nlist = nlist;
-        __syncthreads();
-        return c;
+      __syncthreads();
+    }
+    if (nlist >= 0 && left <= NUC_DIRECT && pass < 7) {
+      // Few candidates are left under the prefix: no more passes.  They are picked out of the list, a thread to each;
+      // each adds up the masses of the candidates heavier than its own and of those as heavy (integers, scaled to the
+      // largest weight under the prefix); the pattern at which the running sum crosses the target is the one whose
+      // candidates see the target between these two sums.
+      const int t = threadIdx.x;
+      const unsigned long long sofar = (~0ull) << shift;
+      if (t == 0) cn = 0;
+      __syncthreads();
+      for (int i = t; i < nlist; i += blockDim.x) {
+        const unsigned long long bits = lbits[i];
+        if ((bits & sofar) == prefix) cbits[atomicAdd(&cn, 1)] = bits;       // as many as the pass counted: `left`
       }
+      __syncthreads();
+      const int m_ = cn;
+      __syncthreads();
+      const double top = __longlong_as_double((long long)(prefix | ((1ull << shift) - 1ull)));
+      const double sc = exp2((double)(62 - lv)) / top, unsc = 1.0 / sc;
+      unsigned long long mybits = 0ull;
+      if (t < m_) {
+        mybits = cbits[t];
+        cmass[t] = (unsigned long long)__double2ll_rn(__longlong_as_double((long long)mybits) * sc);
+      }
+      if (t == 0) {
+        cn = 0x7fffffff;      // the lowest thread at the crossing
+        picked = 0x7fffffff;  // the lowest thread with the lightest pattern, should nothing cross
+      }
+      __syncthreads();
+      unsigned long long heavier = 0ull, same = 0ull, lightest = ~0ull;
+      for (int j = 0; t < m_ && j < m_; ++j) {
+        const unsigned long long b = cbits[j], m = cmass[j];
+        heavier += b > mybits ? m : 0ull;
+        same += b == mybits ? m : 0ull;
+        lightest = b < lightest ? b : lightest;
+      }
+      if (t < m_) {
+        const double lo = above + (double)heavier * unsc, hi = above + (double)(heavier + same) * unsc;
+        const bool crossed = strict ? (target < hi && !(target < lo)) : (hi >= target && !(lo >= target));
+        if (crossed) atomicMin(&cn, t);
+        if (mybits == lightest) atomicMin(&picked, t);
+      }
+      __syncthreads();
+      const int owner = cn != 0x7fffffff ? cn : picked;
+      if (t == owner) {
+        shared_out->bits = mybits;
+        shared_out->above = above + (double)heavier * unsc;
+      }
+      __syncthreads();
+      Crossing c;
+      c.bits = shared_out->bits;
+      c.above = shared_out->above;
+      c.nlist = nlist;
+      __syncthreads();
+      return c;
     }
   }
   Crossing c;
@@ -325,10 +365,12 @@ __device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, 
   __shared__ Crossing cross;
   __shared__ int tie_before[SAMP_THREADS];
   __shared__ int clist[NUC_LIST];
+  __shared__ unsigned long long lbits[NUC_LIST];
+  __shared__ int ntie;
   const int tid = threadIdx.x;
   // the nucleus' edge: weight tau at which the sorted running sum reaches top_p * total
   double target = P * total;
-  Crossing edge = radix_descend(w, V, target, 0, hmass, hcount, &cross, clist, ghist);
+  Crossing edge = radix_descend(w, V, target, 0, hmass, hcount, &cross, clist, lbits, ghist);
   double tau = __longlong_as_double((long long)edge.bits);
   // ties at tau that belong to the nucleus: added one by one until the sum reaches the target
   double need = target - edge.above;
@@ -338,16 +380,24 @@ __device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, 
 
   // the draw: first running sum above r = u * cut, in the same order
   double r = uu * cut;
-  Crossing hit = radix_descend(w, V, r, 1, hmass, hcount, &cross, clist, ghist);
+  Crossing hit = radix_descend(w, V, r, 1, hmass, hcount, &cross, clist, lbits, ghist);
   double wv = __longlong_as_double((long long)hit.bits);
   long long k = wv > 0.0 ? (long long)floor((r - hit.above) / wv) : 0;  // 0-based tie in id order
   if (k < 0) k = 0;
   // the k-th id, in id order, whose weight has exactly this pattern (the last such, if k overshoots)
-  if (hit.nlist >= 0 && hit.nlist <= (int)blockDim.x) {
-    // they are all in the list, a thread to each: its place among them is the number of those with a lower id
-    const bool mine = tid < hit.nlist && (unsigned long long)__double_as_longlong(w[clist[tid]]) == hit.bits;
-    tie_before[tid] = mine ? 1 : 0;
-    const long long ties = __syncthreads_count(mine);
+  if (hit.nlist >= 0) {
+    // they are all in the list: their ids are picked out of it (as many as there are threads; more than that, a row of
+    // a thousand equal weights at the draw, goes the long way below), then a thread to each: its place among them is
+    // the number of those with a lower id
+    if (tid == 0) ntie = 0;
+    __syncthreads();
+    for (int i = tid; i < hit.nlist; i += blockDim.x)
+      if (lbits[i] == hit.bits) {
+        const int at = atomicAdd(&ntie, 1);
+        if (at < (int)blockDim.x) tie_before[at] = clist[i];
+      }
+    __syncthreads();
+    const int ties = ntie;
     if (ties == 0) {
       if (tid == 0) {
         *id_out = 0;
@@ -355,17 +405,20 @@ __device__ void row_nucleus_pick(const double* __restrict__ w, int V, double P, 
       }
       return;
     }
-    const long long kk = k < ties ? k : ties - 1;
-    if (mine) {
-      const int id = clist[tid];
-      long long lower = 0;
-      for (int i = 0; i < hit.nlist; ++i) lower += (tie_before[i] && clist[i] < id) ? 1 : 0;
-      if (lower == kk) {
-        *id_out = id;
-        *bad_out = 0;
+    if (ties <= (int)blockDim.x) {
+      const long long kk = k < ties ? k : ties - 1;
+      if (tid < ties) {
+        const int id = tie_before[tid];
+        long long lower = 0;
+        for (int i = 0; i < ties; ++i) lower += tie_before[i] < id ? 1 : 0;
+        if (lower == kk) {
+          *id_out = id;
+          *bad_out = 0;
+        }
       }
+      return;
     }
-    return;
+    __syncthreads();
   }
   int per = (V + blockDim.x - 1) / blockDim.x;
   int j0 = tid * per, j1 = j0 + per < V ? j0 + per : V;
