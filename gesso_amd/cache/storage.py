@@ -52,16 +52,26 @@ class CacheStorage:
             self.keys.append(torch.zeros(lead + (g.need.head_dim,), dtype=dtype, device=device))
             self.values.append(torch.zeros(lead + (g.need.value_width,), dtype=dtype, device=device))
         self.member_index = {c: i for g in layout.paged for i, c in enumerate(g.members)}
+        # States of one shape, type and initial value share a pool (members, slots + 1, *shape), as the layers of a page
+        # group share theirs: a step's fresh slots then take one fill a pool, not one a layer.  state[call][name] is
+        # the member's own (slots + 1, *shape).
         self.state: Dict[int, Dict[str, torch.Tensor]] = {}
         self.state_init: Dict[int, Dict[str, float]] = {}
+        alike: Dict[tuple, list] = {}
         for m in layout.slots:
             self.state[m.call], self.state_init[m.call] = {}, {}
             for name, shape, dt, init in m.need.entries():
                 if dt not in _DTYPES:
                     raise InvalidPlan(f"state {name!r} of schedule entry {m.call} asks for {dt!r}; slots hold "
                                       f"{sorted(_DTYPES)}")
-                self.state[m.call][name] = torch.full((num_slots + 1,) + shape, init, dtype=_DTYPES[dt], device=device)
+                alike.setdefault((tuple(shape), dt, float(init)), []).append((m.call, name))
                 self.state_init[m.call][name] = init
+        self.state_pools = []                      # (pool, initial value)
+        for (shape, dt, init), members in alike.items():
+            pool = torch.full((len(members), num_slots + 1) + shape, init, dtype=_DTYPES[dt], device=device)
+            self.state_pools.append((pool, init))
+            for i, (call, name) in enumerate(members):
+                self.state[call][name] = pool[i]
 
     @property
     def scratch_page(self):
@@ -88,12 +98,11 @@ class CacheStorage:
     def fill_slots(self, ops, slots, value) -> None:
         """``value``: a number, ``"initial"`` for each state's own initial value, or None for NaN."""
         ids = None
-        for call, states in self.state.items():
-            for name, t in states.items():
-                if ids is None:
-                    ids = torch.tensor(list(slots), dtype=torch.int32, device=t.device)
-                v = self.state_init[call][name] if value == "initial" else (float("nan") if value is None else value)
-                ops.fill_rows(t, ids, v)
+        for pool, init in self.state_pools:
+            if ids is None:
+                ids = torch.tensor(list(slots), dtype=torch.int32, device=pool.device)
+            v = init if value == "initial" else (float("nan") if value is None else value)
+            ops.fill_rows(pool, ids, v, planes=2)
 
     def fill_pages(self, ops, group: int, pages, value: float) -> None:
         """Every layer's keys and values of the given pages of one group."""
@@ -106,11 +115,10 @@ class CacheStorage:
         """NaN everywhere but in the spare page and slot (padded rows of a recorded batch compute on those)."""
         for pool in self.keys + self.values:
             pool[:, :-1].fill_(float("nan"))
-        for states in self.state.values():
-            for t in states.values():
-                t[:-1].fill_(float("nan"))
+        for pool, _ in self.state_pools:
+            pool[:, :-1].fill_(float("nan"))
 
     def bytes(self) -> int:
         n = sum(t.numel() * t.element_size() for t in self.keys + self.values)
-        n += sum(t.numel() * t.element_size() for d in self.state.values() for t in d.values())
+        n += sum(pool.numel() * pool.element_size() for pool, _ in self.state_pools)
         return n
