@@ -410,23 +410,28 @@ def gemm_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype=None, out: torch.Tenso
     return out
 
 
-def library_gemm(x: torch.Tensor, w: torch.Tensor, workspace: torch.Tensor, out: torch.Tensor = None, tune: bool = True):
+def library_gemm(x: torch.Tensor, w: torch.Tensor, workspace: torch.Tensor, out: torch.Tensor = None, tune: bool = True,
+                 checked: bool = False):
     """``x @ w.T`` for many rows by the vendor's library, called directly (bfloat16 in and out, float32 sums).  The
     first call of a shape makes its plan, with ``tune`` by measuring the library's two dozen best guesses on these
     operands (a few milliseconds), else by taking its first choice.
-    ``workspace``: device bytes the library's kernels may use.  Not to be recorded into a graph."""
+    ``workspace``: device bytes the library's kernels may use.  Not to be recorded into a graph.
+    ``checked``: the caller has asked :func:`library_gemm_ok` about ``x`` and ``w`` (and ``out`` is None or fits): the
+    operands are not looked at again here (a step of prompt portions makes 64 such calls; the entry point still
+    refuses misaligned or missing operands)."""
     bf = torch.bfloat16
-    if not (x.is_cuda and x.dim() == 2 and x.dtype is bf and w.dtype is bf and x.stride(1) == 1 and w.is_cuda
-            and w.is_contiguous() and workspace.is_cuda):
-        raise KernelError("library_gemm: bfloat16 (M, K) rows and a contiguous bfloat16 weight on the GPU")
     M, K = x.shape
     N = w.shape[0]
-    if w.shape != (N, K):
-        raise KernelError(f"library_gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
+    if not checked:
+        if not (x.is_cuda and x.dim() == 2 and x.dtype is bf and w.dtype is bf and x.stride(1) == 1 and w.is_cuda
+                and w.is_contiguous() and workspace.is_cuda):
+            raise KernelError("library_gemm: bfloat16 (M, K) rows and a contiguous bfloat16 weight on the GPU")
+        if w.shape != (N, K):
+            raise KernelError(f"library_gemm: weight is {tuple(w.shape)}, expected ({N}, {K})")
+        if out is not None and not (out.is_cuda and out.shape == (M, N) and out.dtype is bf and out.stride(1) == 1):
+            raise KernelError("library_gemm: out is bfloat16 (M, N) on the GPU")
     if out is None:
         out = torch.empty((M, N), dtype=bf, device=w.device)
-    elif not (out.is_cuda and out.shape == (M, N) and out.dtype is bf and out.stride(1) == 1):
-        raise KernelError("library_gemm: out is bfloat16 (M, N) on the GPU")
     rc = lib().gs_library_gemm(x.data_ptr(), x.stride(0) if M > 1 else K, w.data_ptr(), out.data_ptr(),
                                out.stride(0) if M > 1 else N, M, N, K, workspace.data_ptr(),
                                workspace.numel() * workspace.element_size(), 1 if tune else 0, _stream())
@@ -436,11 +441,15 @@ def library_gemm(x: torch.Tensor, w: torch.Tensor, workspace: torch.Tensor, out:
 
 
 def library_gemm_ok(x, w: torch.Tensor) -> bool:
-    """Whether :func:`library_gemm` takes these operands (bfloat16, K and the row stride multiples of 8, aligned)."""
-    return (isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
-            and x.shape[0] > 0 and x.shape[1] % 8 == 0 and x.stride(1) == 1
-            and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0 and w.is_contiguous()
-            and w.data_ptr() % 16 == 0 and w.shape[0] % 8 == 0)
+    """Whether :func:`library_gemm` takes these operands (bfloat16 on the GPU, a weight ``(N, K)`` for rows of K, K and
+    the row stride multiples of 8, aligned)."""
+    bf = torch.bfloat16
+    if not (isinstance(x, torch.Tensor) and x.dtype is bf and w.dtype is bf and x.dim() == 2 and w.dim() == 2):
+        return False
+    M, K = x.shape
+    return (M > 0 and K % 8 == 0 and w.shape[1] == K and w.shape[0] % 8 == 0 and x.stride(1) == 1
+            and (M <= 1 or x.stride(0) % 8 == 0) and x.is_cuda and w.is_cuda and w.is_contiguous()
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
 def library_gemm_plan(M: int, N: int, K: int):

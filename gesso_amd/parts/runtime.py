@@ -190,7 +190,8 @@ class Runtime:
         """``x @ w.T`` by the vendor library: called directly where it takes the operands (``ops.library_gemm``: a plan
         per shape, a few microseconds of host time a call), else through ``torch.mm``."""
         ops = self.ops
-        if ops.library_gemm_ok(x, w) and (out is None or (out.dtype == torch.bfloat16 and out.stride(1) == 1
+        if ops.library_gemm_ok(x, w) and (out is None or (out.dtype == torch.bfloat16 and out.is_cuda and out.stride(1) == 1
+                                                          and out.shape == (x.shape[0], w.shape[0])
                                                           and out.data_ptr() % 16 == 0
                                                           and (out.shape[0] <= 1 or out.stride(0) % 8 == 0))):
             if self._library_ws is None:
@@ -199,7 +200,7 @@ class Runtime:
             # 512 on): a measurement takes some ten milliseconds a shape, and a server's steps bring ever new row counts
             M = x.shape[0]
             return ops.library_gemm(x, w, self._library_ws, out=out,
-                                    tune=self.tune_library and M >= 512 and M & (M - 1) == 0)
+                                    tune=self.tune_library and M >= 512 and M & (M - 1) == 0, checked=True)
         return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
 
     def linear_swiglu(self, x, w13: torch.Tensor) -> torch.Tensor:
