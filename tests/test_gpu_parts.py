@@ -76,7 +76,8 @@ class Harness:
 
 
 def tol(dtype, ref):
-    return (2e-5 if dtype == torch.float32 else 2e-2) * max(1.0, float(ref.abs().max()))
+    # bfloat16: 1e-2 of the largest value (at 8e-3 the first sound part fails: a toy mixer with values 40 wide)
+    return (2e-5 if dtype == torch.float32 else 1e-2) * max(1.0, float(ref.abs().max()))
 
 
 # ------------------------------------------------------------------ norm, position, feed-forward
