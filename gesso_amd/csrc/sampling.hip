@@ -20,28 +20,32 @@ __device__ void row_argmax(const float* __restrict__ x, int V, int* id_out, int*
   float best = -INFINITY;
   int idx = 0x7fffffff;
   int notfinite = 0;
-  // 16-byte loads, four of them under way at a time; ids are visited in ascending order per thread, and a
-  // later equal value never replaces an earlier one
+  // 16-byte loads, eight of them under way at a time (a row of 65,536 logits is then two round trips for the block's
+  // 1,024 threads; sixteen need more registers than 1,024 threads leave a lane); ids are visited in ascending order per
+  // thread, and a later equal value never replaces an earlier one
+  constexpr int AHEAD = 8;
   const int V4 = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) ? (V >> 2) : 0;
-  const float4* x4 = reinterpret_cast<const float4*>(x);
-  for (int q0 = threadIdx.x; q0 < V4; q0 += 4 * blockDim.x) {
-    float4 v[4];
+  typedef float __attribute__((ext_vector_type(4))) row4_t;   // (a plain vector type: an array of it stays in registers)
+  const row4_t* x4 = reinterpret_cast<const row4_t*>(x);
+  for (int q0 = threadIdx.x; q0 < V4; q0 += AHEAD * blockDim.x) {
+    row4_t v[AHEAD];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < AHEAD; ++u) {
       int q = q0 + u * blockDim.x;
-      v[u] = q < V4 ? x4[q] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+      v[u] = q < V4 ? x4[q] : row4_t{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < AHEAD; ++u) {
       int q = q0 + u * blockDim.x;
-      if (q >= V4) break;
-      const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+      if (q < V4) {            // (no break: the loop must unroll whole, or the loads' array is indexed at run time)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (!(fabsf(e[i]) <= 3.402823466e38f)) notfinite = 1;
-        if (e[i] > best) {
-          best = e[i];
-          idx = 4 * q + i;
+        for (int i = 0; i < 4; ++i) {
+          const float e = v[u][i];
+          if (!(fabsf(e) <= 3.402823466e38f)) notfinite = 1;
+          if (e > best) {
+            best = e;
+            idx = 4 * q + i;
+          }
         }
       }
     }
