@@ -171,18 +171,20 @@ def measured_ceilings(reps: int = 5) -> dict:
     return {"read_gbps": round(read, 1), "mfma_tflops_vendor": round(vendor, 1), "mfma_tflops_ours": round(ours, 1)}
 
 
-def serve_workload(seed: int = 5) -> dict:
+def serve_workload(seed: int = 5, record: bool = True, tune: bool = True) -> dict:
     """LFM2-350M sizes: 64 requests at once, prompts of 64 to 2,048 tokens, 32 to 512 new tokens each, prompt
     portions of 512 tokens beside the decodes of the others; the scheduler's own loop, greedy."""
     from gesso_amd import Session
     from gesso_amd.engine.scheduler import Request
+    from gesso_amd.parts import RuntimeOptions
     cfg = model_config("350m")
     g = torch.Generator().manual_seed(seed)
     n = 64
     plen = torch.randint(64, 2049, (n,), generator=g).tolist()
     olen = torch.randint(32, 513, (n,), generator=g).tolist()
     sess = Session(cfg, random_weights_seed=0, context_length=4096, max_num_seqs=64, chunk_size=512,
-                   max_num_batched_tokens=1024, max_tokens=n * 2624)
+                   max_num_batched_tokens=1024, max_tokens=n * 2624,
+                   kernel_options=RuntimeOptions(record_portions=record, tune_library=tune))
     stamps = {}
 
     def run():
@@ -210,7 +212,7 @@ def serve_workload(seed: int = 5) -> dict:
             "prompt_tokens": sum(plen), "new_tokens": new, "prompt_tok_s": round(sum(plen) / (t1 - t0), 1),
             "mean_ttft_ms": round(1e3 * sum(ttft) / n, 2), "mean_tpot_ms": round(1e3 * sum(tpot) / len(tpot), 3),
             "steps": sched.stats["steps"], "preemptions": sched.stats["preemptions"], "chunk": 512,
-            "token_budget": 1024, "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
+            "token_budget": 1024, "recorded_steps": getattr(sess.engine.recorder, "replays", 0), "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
 
 
 def gemm_workload(reps: int = 10) -> dict:
@@ -331,6 +333,8 @@ def main() -> int:
     ap.add_argument("--no-ceilings", action="store_true", help="skip the measurement of what the machine delivers")
     ap.add_argument("--no-tune", action="store_true", help="the vendor library's first choice for every product of many "
                     "rows (for profiles: no tuning runs among the kernels)")
+    ap.add_argument("--launched-portions", action="store_true", help="--workload serve: launch the steps with prompt portions "
+                    "kernel by kernel instead of replaying recordings of them")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
@@ -343,7 +347,10 @@ def main() -> int:
         if args.workload == "stages":
             print(json.dumps(stages_workload(args.batch, min(args.steps, 32))))
             return 0
-        run = {"serve": serve_workload, "long": long_workload, "gemm": gemm_workload}[args.workload]
+        if args.workload == "serve":
+            print(json.dumps(serve_workload(record=not args.launched_portions, tune=not args.no_tune)))
+            return 0
+        run = {"long": long_workload, "gemm": gemm_workload}[args.workload]
         print(json.dumps(run()))
         return 0
 

@@ -41,6 +41,9 @@ def parse_launch(argv: List[str]) -> argparse.Namespace:
     ap.add_argument("--gemm", default="auto", choices=["auto", "own", "library"],
                     help="products of more than 64 rows: the vendor library where it is faster (auto), the hand-written "
                          "kernel everywhere (own), the library wherever it can go (library)")
+    ap.add_argument("--record-portions", action="store_true",
+                    help="steps with prompt portions whose kind recurs are recorded as HIP graphs and replayed (pays where "
+                         "the host's launches, not the kernels, bound such a step: small models, small portions)")
     ap.add_argument("--poison", action="store_true", help="debugging: fill pages and slots that are given back with NaN")
     ap.add_argument("--cpu", action="store_true", help="refused: there is no CPU path")
     ap.add_argument("--check", action="store_true", help="self-test on a tiny random model")
@@ -91,7 +94,8 @@ def main(argv=None) -> int:
     from .parts.runtime import RuntimeOptions
 
     kw = dict(dtype=args.dtype, page_size=args.page_size, context_length=args.n_ctx, chunk_size=args.prefill_chunk,
-              max_num_seqs=args.max_num_seqs, kernel_options=RuntimeOptions(many_rows=args.gemm), poison=args.poison)
+              max_num_seqs=args.max_num_seqs, kernel_options=RuntimeOptions(many_rows=args.gemm, record_portions=args.record_portions),
+              poison=args.poison)
     if args.model is not None:
         session = Session(args.model, **kw)
     else:

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
       first_key = lo < first_key ? lo : first_key;
     }
   }
-  if (first_key > last_key) first_key = last_key;                 // a block without queries: one masked step, nothing stored
+  if (first_key > last_key) return;                               // a block without queries (the same for all its threads)
   const int kbeg = (first_key / PW_KS) * PW_KS;
   const int nsteps_all = (last_key - kbeg) / PW_KS + 1;
   const int nsteps = (nsteps_all + KS - 1) / KS;                  // steps of the walk: half h takes steps h nsteps .. of the keys

@@ -227,9 +227,10 @@ extern "C" int gs_library_gemm(const void* X, int ldx, const void* W, void* Y, i
   GS_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)Y & 15) == 0 && ldx % 8 == 0 && ldy % 8 == 0 && K % 8 == 0,
              "library_gemm: operands must be 16-byte aligned, row strides and K multiples of 8");
   GS_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || workspace), "library_gemm: a workspace size without a workspace");
+  // While a stream records, a product whose plan exists is recorded like any launch; a plan is not made then (making
+  // one asks the library and, when tuning, measures: neither belongs into a recording).
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &cap) == hipSuccess)
-    GS_REQUIRE(cap == hipStreamCaptureStatusNone, "library_gemm: the vendor library's products are not recorded into graphs");
+  const bool recording = hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
   int dev = -1;
   GS_REQUIRE(hipGetDevice(&dev) == hipSuccess, "library_gemm: no current device");
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -238,6 +239,7 @@ extern "C" int gs_library_gemm(const void* X, int ldx, const void* W, void* Y, i
   const PlanKey key(dev, M, N, K, ldx, ldy, (size_t)ws_bytes, tune ? 1 : 0);
   auto it = g_plans.find(key);
   if (it == g_plans.end()) {
+    GS_REQUIRE(!recording, "library_gemm: no plan yet for %d x %d x %d rows: run the product once before it is recorded into a graph", M, N, K);
     Plan p;
     if (int rc = make_plan(handle, p, X, ldx, W, Y, ldy, M, N, K, workspace, (size_t)ws_bytes, tune, stream)) {
       destroy_plan(p);

@@ -65,6 +65,11 @@ class BatchContext:
     fields to :meth:`_set`, which refuses a missing or an unknown one: a field added to the list must be served
     by every builder before anything runs."""
 
+    # While a step of prompt portions is recorded for replay (engine/planned.py): the recorder.  A part whose launches
+    # depend on more than the token count and device buffers asks it for tile lists that every replay refills
+    # (``recording.subtiles``) and hands it what must run anew at every replay (``recording.eager``).
+    recording = None
+
     def _set(self, storage, **fields) -> None:
         if set(fields) != set(CONTEXT_FIELDS):
             missing, unknown = set(CONTEXT_FIELDS) - set(fields), set(fields) - set(CONTEXT_FIELDS)
@@ -102,6 +107,10 @@ class BatchContext:
             t = torch.tensor([seq, row, cnt], dtype=torch.int32).pin_memory().to(self.token_ids.device, non_blocking=True)
             self._tiles = ((rows, skip), t)
         return self._tiles[1]
+
+    def subtile_lists(self, wq: int, skip: int = 0, paired: bool = True):
+        """:func:`subtile_lists` of this step's sequences from ``skip`` on, on the host."""
+        return subtile_lists(self.q_lens, wq, skip, paired)
 
     def query_subtiles(self, wq: int, skip: int = 0, paired: bool = True) -> torch.Tensor:
         """int32 ``(3, blocks * wq)`` on the device: :func:`subtile_lists` of this step's sequences from ``skip`` on."""

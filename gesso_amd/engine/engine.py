@@ -69,6 +69,12 @@ class Engine:
             self.storage.poison_all()
         self.steps = 0
         self._runners = {}
+        # steps of prompt portions whose kind recurs are recorded and replayed, where the options ask for it and every
+        # part can be (bfloat16: the 32-bit path has no such parts' kernels)
+        self.recorder = None
+        if self.rt.options.record_portions and self.dtype == torch.bfloat16 and self.model.portions_recordable:
+            from .planned import StepRecorder
+            self.recorder = StepRecorder(self)
         # the most requests one recorded decode step takes: as many rows as the runtime's weight-streaming products do
         # (the limit is the product kernels', asked of the runtime, not a number of the engine's own)
         self.DECODE_MAX_BATCH = self.rt.streaming_rows_max
@@ -149,14 +155,27 @@ class Engine:
         # from here on the cache is written: an error leaves the requests of this step without a usable state
         try:
             self.prepare_cache()
-            ctx = StepContext(entries, self.manager, self.storage, self.spec.vocab, self.device, token_ids=ids)
-            logits = self.model.forward(ctx)
+            logits = self._step_recorded(entries, ids) if self.recorder is not None else False
+            if logits is False:
+                ctx = StepContext(entries, self.manager, self.storage, self.spec.vocab, self.device, token_ids=ids)
+                logits = self.model.forward(ctx)
         except Exception as err:
             raise self.fail_requests([e.rid for e in entries], err) from err
         for e in entries:
             self.manager.commit(e.rid, len(e.tokens))
         self.steps += 1
         return logits
+
+    def _step_recorded(self, entries, ids):
+        """The step through a recording of its kind (:mod:`gesso_amd.engine.planned`), or False where there is none."""
+        rec = self.recorder.recording_for(entries)
+        if rec is None:
+            return False
+        n_want = rec.fill(entries, ids)
+        if n_want is None:
+            return False
+        self.recorder.replays += 1
+        return rec.launch(n_want)
 
     # ------------------------------------------------------------------ profiling
 

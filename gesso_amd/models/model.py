@@ -81,22 +81,31 @@ class Model:
 
     def forward(self, ctx) -> Optional[torch.Tensor]:
         """Run the tokens of ``ctx`` through every scheduled block; float32 logits at ``ctx.want_rows``."""
-        ops, rt = self.rt.ops, self.rt
-        decode_only = ctx.decode_only
+        stream = self.run_blocks(ctx)
+        if ctx.n_want == 0:
+            return None
+        # every row wanted, in order (a decode step): no gather, and the norm may stay lazy
+        return self.logits(stream, None if ctx.decode_only else ctx.want_rows)
+
+    def run_blocks(self, ctx) -> ResidualStream:
+        """The embedding and every scheduled block: the residual stream as the last block leaves it (what is still
+        pending is added by the norm that follows)."""
+        rt = self.rt
         # the norm that reads the stream after the i-th scheduled block: the next block's first, then the final one
         # (``first_norm`` and ``row_weight`` are the optional hints of blocks and norms, see parts/base.py)
         order = [self.blocks[call.layer] for call in self.spec.schedule]
-        readers = [getattr(b, "first_norm", None) for b in order[1:]] + [self.final_norm if decode_only else None]
+        readers = [getattr(b, "first_norm", None) for b in order[1:]] + [self.final_norm if ctx.decode_only else None]
         scale = 1.0 if self.spec.embed_scale is None else float(self.spec.embed_scale)
         with rt.stage("embed"):
             stream = self._embed(ctx, order, scale)
         for i, call in enumerate(self.spec.schedule):
             stream.following = readers[i]
             order[i].forward(stream, ctx, ctx.cache_view(i))
-        if ctx.n_want == 0:
-            return None
-        # every row wanted, in order (a decode step): no gather, and the norm may stay lazy
-        rows = None if decode_only else ctx.want_rows
+        return stream
+
+    def logits(self, stream: ResidualStream, rows) -> torch.Tensor:
+        """The final norm of the stream's ``rows`` (int32 on the device; None: all, in order) and the head: float32."""
+        ops, rt = self.rt.ops, self.rt
         with rt.stage("norm"):
             normed = self.final_norm.add_norm(stream, rows=rows)
         with rt.stage("lm_head"):
@@ -104,6 +113,20 @@ class Model:
             if self.spec.logit_softcap is not None:
                 ops.softcap(logits, float(self.spec.logit_softcap))
         return logits
+
+    @property
+    def portions_recordable(self) -> bool:
+        """Whether steps of prompt portions through this model may be recorded for replay (every part says so: what it
+        launches then depends on the step's token count and on device buffers alone, or it tells the recorder)."""
+        return all(getattr(b, "portions_recordable", False) for b in self.blocks) and \
+            getattr(self.final_norm, "portions_recordable", False)
+
+    def replay_key(self, q_lens, max_kv_len):
+        """What a recording of a step of prompt portions must share with the step that replays it, beside the token
+        count: each block's own answer (None: nothing; False from any block: such a step is not to be recorded, and
+        the answer is None)."""
+        key = tuple(b.replay_key(q_lens, max_kv_len) if hasattr(b, "replay_key") else None for b in self.blocks)
+        return None if any(k is False for k in key) else key
 
     def _embed(self, ctx, order, scale):
         ops, rt = self.rt.ops, self.rt

@@ -13,6 +13,7 @@ import math
 
 import torch
 
+from ..errors import InvalidPlan
 from .base import MATRIX, VECTOR, PagedKV, Part, TensorSpec
 from .registry import build, register
 
@@ -30,6 +31,7 @@ class RawQKV:
 
 class Attention(Part):
     graph_safe = True
+    portions_recordable = True
     stage, out_stage = "attn_mixer", "attn_outproj"   # the decode profiler's names
     HALVES_MAX_KEYS = 4096    # prompts whose sequences hold fewer keys may have their keys walked in two halves
 
@@ -121,6 +123,63 @@ class Attention(Part):
         return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table,
                                     cache.page_size, window, self.scale, nh, nkv, d, nseq, nsplit, out=out)
 
+    def prompt_walk(self, q_lens, max_kv_len):
+        """How the kernel for long portions takes sequences that bring ``q_lens`` tokens: ``(sub-tiles a block, key
+        halves, late sub-tiles paired with early ones)``."""
+        s, rt, ops = self.spec, self.rt, self.rt.ops
+        nkv = s.n_kv_heads
+        wq = ops.attention_prefill_wide_rows(s.n_heads, nkv) // 32
+        blocks = sum(-(-(-(-n // 32)) // wq) for n in q_lens) * nkv
+        few = blocks <= rt.compute_units
+        halves = 2 if few and wq >= 2 and max_kv_len is not None and max_kv_len < self.HALVES_MAX_KEYS else 1
+        wq //= halves
+        return wq, halves, (not s.window and wq >= 2 and few)
+
+    def replay_key(self, q_lens, max_kv_len):
+        """A recorded step of prompt portions walks the keys as the step that replays it would: whole (1) or in halves
+        (2).  False: such a step does not go through the kernel for long portions, and is not to be recorded."""
+        s, rt, ops = self.spec, self.rt, self.rt.ops
+        nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
+        lead = 0
+        while lead < len(q_lens) and q_lens[lead] == 1:
+            lead += 1
+        choice = rt.options.prompt_attention
+        stride = (nh + 2 * nkv) * d
+        if not (rt.dtype == torch.bfloat16 and stride % 8 == 0 and lead < len(q_lens)
+                and ops.attention_prefill_supports(nh, nkv, d) and ops.attention_decode_supports(nh, nkv, d)
+                and choice != "tiles" and ops.attention_prefill_wide_supports(nh, nkv, d)
+                and (choice == "wide" or max(q_lens) >= 64)):
+            return False
+        return self.prompt_walk(q_lens[lead:], max_kv_len)[1]
+
+    def _attend_recorded(self, q, q_stride, ctx, cache) -> torch.Tensor:
+        """The prompt part of :meth:`attend` while a step is recorded for replay: the tile lists lie in a buffer that
+        every replay refills (as many blocks as the token count and the most sequences can make, the unused ones
+        without queries), and the decoded tokens at the batch's head, whose number changes from step to step, are left
+        to a call that every replay makes anew."""
+        s, rt, ops, rec = self.spec, self.rt, self.rt.ops, ctx.recording
+        nh, nkv, d, window = s.n_heads, s.n_kv_heads, s.head_dim, s.window
+        halves = rec.key_of(self)
+        if halves not in (1, 2) or isinstance(q, RawQKV) or q.dtype != torch.bfloat16 or cache.page_size < 2:
+            raise InvalidPlan("this step's attention cannot be recorded (see replay_key)")
+        wq = ops.attention_prefill_wide_rows(nh, nkv) // 32 // halves
+        out = torch.empty((ctx.T, nh * d), dtype=q.dtype, device=q.device)
+
+        def lists(c):
+            lead = c.lead_single
+            return c.subtile_lists(wq, lead, paired=self.prompt_walk(c.q_lens[lead:], c.max_kv_len)[2])
+
+        def decoded(c):
+            if c.lead_single:
+                self._single(q, q_stride, cache, c, c.lead_single, out[:c.lead_single])
+
+        # layers of one shape walk alike and share a list
+        tiles = rec.subtiles(("attention", nh, nkv, bool(window), halves), wq, lists)
+        rec.eager(decoded)
+        return ops.attention_prefill_wide(q, q_stride, cache.k, cache.v, ctx.positions, tiles, cache.block_table,
+                                          cache.page_size, window, self.scale, nh, nkv, d, ctx.T, out=out,
+                                          key_splits=halves)
+
     def attend(self, q, q_stride, ctx, cache) -> torch.Tensor:
         """Causal attention of this step's queries over the paged cache; ``(T, nh * d)``.
 
@@ -133,6 +192,8 @@ class Attention(Part):
         if isinstance(q, RawQKV):
             return self._single(q, q_stride, cache, ctx, ctx.nseq, out)
         fast = q.dtype == torch.bfloat16 and cache.page_size >= 2
+        if ctx.recording is not None:
+            return self._attend_recorded(q, q_stride, ctx, cache)
         if ctx.all_single and fast and ops.attention_decode_supports(nh, nkv, d):
             return self._single(q, q_stride, cache, ctx, ctx.nseq, out)
         if (not ctx.all_single and fast and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d)):
@@ -156,12 +217,8 @@ class Attention(Part):
                 # so that the longest walk is half as long and twice the blocks spread evenly (the same prompt 40.4 us;
                 # 1,024 tokens 18.9 against 25.4; 512 over a prefix of 1,024: 24.5 against 37.4; over a prefix of 30,720,
                 # where every walk is long, staging two halves a step costs more than it saves: 897 against 834).
-                wq = ops.attention_prefill_wide_rows(nh, nkv) // 32
-                blocks = sum(-(-(-(-n // 32)) // wq) for n in ctx.q_lens[lead:]) * nkv
-                few = blocks <= rt.compute_units
-                halves = 2 if few and wq >= 2 and ctx.max_kv_len is not None and ctx.max_kv_len < self.HALVES_MAX_KEYS else 1
-                wq //= halves
-                paired = not window and wq >= 2 and few
+                lens = ctx.q_lens[lead:]
+                wq, halves, paired = self.prompt_walk(lens, ctx.max_kv_len)
                 return ops.attention_prefill_wide(q, q_stride, cache.k, cache.v, ctx.positions,
                                                   ctx.query_subtiles(wq, lead, paired=paired), cache.block_table,
                                                   cache.page_size, window, self.scale, nh, nkv, d, ctx.T, out=out,

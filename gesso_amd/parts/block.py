@@ -69,6 +69,16 @@ class PreNormBlock(Part):
                     stream.push(out, rt, next_norm=after)
 
     @property
+    def portions_recordable(self) -> bool:
+        """Whether a step of prompt portions through this block may be recorded for replay (see ``Model``)."""
+        parts = [self.mixer_norm, self.mixer] + ([self.ffn_norm, self.ffn] if self.ffn is not None else [])
+        return all(getattr(p, "portions_recordable", False) for p in parts)
+
+    def replay_key(self, q_lens, max_kv_len):
+        f = getattr(self.mixer, "replay_key", None)
+        return f(q_lens, max_kv_len) if f is not None else None
+
+    @property
     def graph_safe(self) -> bool:
         """Whether a step through this block may be recorded into a HIP graph (no host round trips inside)."""
         parts = [self.mixer_norm, self.mixer] + ([self.ffn_norm, self.ffn] if self.ffn is not None else [])

@@ -77,6 +77,7 @@ def row_weight_of(norm, res, rt):
 
 class RMSNorm(Part):
     graph_safe = True
+    portions_recordable = True
 
     @staticmethod
     def tensor_specs(spec):

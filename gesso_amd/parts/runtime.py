@@ -49,9 +49,14 @@ class RuntimeOptions:
     ``weighted_rows_max``: up to this many rows a deferred product also leaves the rows weighted for the next norm,
     whose consumer then only scales its result; for more rows every block's reading of the partial sums costs
     more than one light norm pass.
+    ``record_portions``: steps that hold prompt portions are recorded as HIP graphs once their kind (token count,
+    room for keys, how attention walks) has come twice, and replayed from then on: a scheduler that fills its token
+    budget repeats one kind step after step, and launching such a step's kernels one by one takes the host longer than
+    the device needs for them on small models.  The logits are the same bit for bit.
     """
 
     many_rows: str = "auto"
+    record_portions: bool = False
     tune_library: bool = False
     prompt_attention: str = "auto"
     tiled_rows: bool = True

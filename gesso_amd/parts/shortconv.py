@@ -15,6 +15,7 @@ from .registry import register
 
 class ShortConv(Part):
     graph_safe = True
+    portions_recordable = True
     stage, out_stage = "conv_mixer", "conv_out"       # the decode profiler's names
 
     @staticmethod

@@ -14,6 +14,7 @@ from .registry import register
 
 class SwiGLU(Part):
     graph_safe = True
+    portions_recordable = True
     stage, out_stage = "dense_ffn", "ffn_down"        # the decode profiler's names
 
     @staticmethod

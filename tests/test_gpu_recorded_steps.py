@@ -1,0 +1,183 @@
+"""Steps of prompt portions through a recording (gesso_amd/engine/planned.py) give the logits of the same steps launched
+kernel by kernel, bit for bit: the same kernels run with the same arguments.  Two engines over one model folder take the
+same steps, one with ``record_portions``; the steps keep their token count while the sequences in them come, grow
+and go, and pages and slots are used again (poisoned in between)."""
+import random
+
+import pytest
+import torch
+
+from gesso_amd.config import Lfm2Config
+from gesso_amd.weights import write_model_folder
+from tiny import STD, random_ids
+
+pytestmark = pytest.mark.gpu
+
+# heads 64 wide (the kernel for long portions takes no others); E has four query heads to a key head, a bias on the
+# convolution and room for thousands of keys
+WIDE_D = Lfm2Config(
+    vocab_size=200, hidden_size=128, num_hidden_layers=3, num_attention_heads=2, num_key_value_heads=1,
+    layer_types=("full_attention", "conv", "full_attention"), conv_L_cache=3, conv_bias=False,
+    intermediate_size=136, norm_eps=1e-5, rope_theta=1e5, tie_word_embeddings=True, max_position_embeddings=1024)
+WIDE_E = Lfm2Config(
+    vocab_size=333, hidden_size=256, num_hidden_layers=4, num_attention_heads=4, num_key_value_heads=1,
+    layer_types=("conv", "full_attention", "conv", "full_attention"), conv_L_cache=4, conv_bias=True,
+    intermediate_size=344, norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False, max_position_embeddings=8192)
+
+
+def engines(folder, **kw):
+    from gesso_amd import Engine
+    from gesso_amd.parts import RuntimeOptions
+
+    plain = Engine.from_folder(folder, dtype="bfloat16", poison=True, **kw)
+    recorded = Engine.from_folder(folder, dtype="bfloat16", poison=True, options=RuntimeOptions(record_portions=True), **kw)
+    assert plain.recorder is None and recorded.recorder is not None
+    return plain, recorded
+
+
+class Workload:
+    """Requests with prompts of random lengths; every step holds ``T`` tokens: the decoded tokens of the requests whose
+    prompts are through (at the head), then portions of the prompts that are not, cut where the step is full."""
+
+    def __init__(self, vocab, T, seed, prompt_lens, new_tokens=(3, 9), live=6):
+        self.rng = random.Random(seed)
+        self.vocab, self.T, self.live_max = vocab, T, live
+        self.prompts = [random_ids(n, vocab, seed * 100 + i) for i, n in enumerate(prompt_lens)]
+        self.new_tokens = new_tokens
+        self.next_rid = 0
+        self.live = {}          # rid -> dict(prompt, done, left, token)
+
+    def admit(self, engines_):
+        while len(self.live) < self.live_max and self.next_rid < len(self.prompts):
+            rid = self.next_rid
+            self.next_rid += 1
+            self.live[rid] = dict(prompt=self.prompts[rid], done=0, left=self.rng.randint(*self.new_tokens), token=None)
+            for e in engines_:
+                e.add_request(rid)
+
+    def step_entries(self):
+        from gesso_amd import StepEntry
+        entries, room = [], self.T
+        for rid, r in self.live.items():
+            if r["token"] is not None and room > 2:
+                entries.append(StepEntry(rid, [r["token"]], [0]))
+                room -= 1
+        for rid, r in self.live.items():
+            rest = len(r["prompt"]) - r["done"]
+            if r["token"] is None and rest and room >= 2:
+                n = min(rest, room)
+                if rest - n == 1:          # (never leave a single token of a prompt over: it would look like a decoded one)
+                    n -= 1
+                if n < 2:
+                    continue
+                last = r["done"] + n == len(r["prompt"])
+                entries.append(StepEntry(rid, r["prompt"][r["done"]:r["done"] + n], [n - 1] if last else []))
+                room -= n
+        return entries
+
+    def advance(self, entries, logits, engines_):
+        row = 0
+        for e in entries:
+            r = self.live[e.rid]
+            if r["token"] is None:
+                r["done"] += len(e.tokens)
+            if e.want:
+                r["token"] = int(logits[row].argmax())
+                row += 1
+                r["left"] -= 1
+                if r["left"] == 0:
+                    del self.live[e.rid]
+                    for eng in engines_:
+                        eng.finish_request(e.rid)
+
+
+def run_both(plain, recorded, work, steps, kinds):
+    """``kinds``: how often each kind of step came (None: a step that is not to be recorded)."""
+    for s in range(steps):
+        work.admit((plain, recorded))
+        entries = work.step_entries()
+        if not entries:
+            break
+        kind = recorded.recorder.kind_of(entries)
+        kinds[kind] = kinds.get(kind, 0) + 1
+        a = plain.step(entries)
+        b = recorded.step(entries)
+        assert (a is None) == (b is None), s
+        if a is not None:
+            assert torch.isfinite(a).all(), s
+            assert torch.equal(a, b), (s, [(e.rid, len(e.tokens)) for e in entries], (a - b).abs().max().item())
+        work.advance(entries, a if a is not None else [], (plain, recorded))
+
+
+def replays_expected(kinds, recorder):
+    """Every step of a kind after the first few, for the kinds that were recorded (the first that came often enough)."""
+    assert not recorder.refused, recorder.refused
+    made = [k for k, r in recorder.recordings.items() if r is not None]
+    assert set(made) <= {k for k, n in kinds.items() if k is not None and n > recorder.SEEN_BEFORE}
+    assert len(made) == min(recorder.MAX_RECORDINGS, sum(1 for k, n in kinds.items() if k is not None and n > recorder.SEEN_BEFORE))
+    return sum(kinds[k] - recorder.SEEN_BEFORE for k in made)
+
+
+@pytest.mark.parametrize("name,T", [("D", 96), ("E", 160), ("E", 72)])
+def test_recorded_steps_of_portions_equal_the_launched_ones(tmp_path, name, T):
+    cfg = {"D": WIDE_D, "E": WIDE_E}[name]
+    folder = str(tmp_path / name)
+    write_model_folder(folder, cfg, 11, torch.bfloat16, std=STD)
+    # so few pages that they are used again: six live requests of up to 400 tokens
+    plain, recorded = engines(folder, page_size=16, max_tokens=6 * 448, num_slots=7)
+    rng = random.Random(T)
+    work = Workload(cfg.vocab_size, T, seed=T, prompt_lens=[rng.randint(20, 400) for _ in range(40)])
+    kinds = {}
+    run_both(plain, recorded, work, 60, kinds)
+    rec = recorded.recorder
+    assert rec.replays == replays_expected(kinds, rec) and rec.replays >= 20, (rec.replays, kinds)
+
+
+def test_recorded_steps_with_thousands_of_keys_walk_them_whole(tmp_path):
+    """A sequence with more keys than a walk in halves takes makes a kind of its own (another walk, a longer block table);
+    both kinds are recorded and both give the launched steps' logits."""
+    from gesso_amd import StepEntry
+
+    folder = str(tmp_path / "E")
+    write_model_folder(folder, WIDE_E, 12, torch.bfloat16, std=STD)
+    plain, recorded = engines(folder, page_size=16, max_tokens=4608 + 6 * 448, num_slots=8)
+    T = 128
+    rng = random.Random(5)
+    work = Workload(WIDE_E.vocab_size, T, seed=5, prompt_lens=[rng.randint(30, 300) for _ in range(30)], live=5)
+    kinds = {}
+    run_both(plain, recorded, work, 12, kinds)
+    # a long request beside them: most of its prompt in one step of its own, the rest in portions among the others
+    long_prompt = random_ids(4400, WIDE_E.vocab_size, 77)
+    for eng in (plain, recorded):
+        eng.add_request("long")
+        assert eng.step([StepEntry("long", long_prompt[:4000], [])]) is None
+    work.prompts.append(long_prompt)
+    work.live["long"] = dict(prompt=long_prompt, done=4000, left=6, token=None)
+    run_both(plain, recorded, work, 25, kinds)
+    rec = recorded.recorder
+    assert rec.replays == replays_expected(kinds, rec) and rec.replays >= 20, (rec.replays, kinds)
+    made = [k for k, r in rec.recordings.items() if r is not None]
+    assert {k[1] for k in made} == {4096, 8192}, made       # block tables for 4,096 and for 8,192 keys
+    assert {k[2] for k in made if k[1] == 8192} != {k[2] for k in made if k[1] == 4096}, made     # and another walk
+
+
+def test_the_scheduler_over_recorded_steps_generates_the_same_ids(tmp_path):
+    """Through the entry point: prompts cut into portions under a token budget, greedy; the ids are the same with
+    recording on and off, and most steps were replays."""
+    from gesso_amd import Session
+    from gesso_amd.parts import RuntimeOptions
+
+    folder = str(tmp_path / "E")
+    write_model_folder(folder, WIDE_E, 13, torch.bfloat16, std=STD)
+    rng = random.Random(3)
+    prompts = [random_ids(rng.randint(100, 700), WIDE_E.vocab_size, 300 + i) for i in range(24)]
+    out = []
+    for on in (False, True):
+        s = Session(folder, dtype="bfloat16", max_num_seqs=8, max_num_batched_tokens=256, chunk_size=256,
+                    kernel_options=RuntimeOptions(record_portions=on), max_tokens=8 * 1024)
+        out.append(s.generate(prompts, max_new_tokens=12))
+        if on:
+            rec = s.engine.recorder
+            assert not rec.refused and rec.replays >= 20, (rec.refused, rec.replays, rec.seen)
+        s.close()
+    assert out[0] == out[1]
