@@ -181,3 +181,54 @@ def test_the_scheduler_over_recorded_steps_generates_the_same_ids(tmp_path):
             assert not rec.refused and rec.replays >= 20, (rec.refused, rec.replays, rec.seen)
         s.close()
     assert out[0] == out[1]
+
+
+def test_recorded_steps_over_two_page_groups_one_of_them_windowed(tmp_path):
+    """A model of parts put together by hand: an attention layer that sees all keys, one that sees the last 40 (pages of
+    its own, given back as the window passes them and poisoned), a short convolution.  Recorded steps give the launched
+    steps' logits here too: block tables of both groups, entries of pages that are gone, the windowed walk."""
+    from gesso_amd import Engine
+    from gesso_amd.config import AttentionSpec, BlockSpec, LayerCall, ModelSpec, RMSNormSpec, RopeSpec, ShortConvSpec, SwiGLUSpec
+    from gesso_amd.models.model import tensor_table
+    from gesso_amd.parts import RuntimeOptions
+    from gesso_amd.weights import random_tensors
+    from gesso_amd.weights.loader import held_dtype
+
+    H, V, eps = 128, 90, 1e-5
+    norm = RMSNormSpec(H, eps)
+    rope = RopeSpec(head_dim=64, rotary_dim=64, theta=1e4, max_position=1024)
+    full = AttentionSpec(hidden=H, n_heads=2, n_kv_heads=1, head_dim=64, position=rope, qk_norm=RMSNormSpec(64, eps))
+    near = AttentionSpec(hidden=H, n_heads=2, n_kv_heads=2, head_dim=64, position=rope, qk_norm=None, window=40)
+
+    def names(i, mixer_names, ffn=True):
+        n = {f"mixer.{k}": f"L{i}.{k}" for k in mixer_names}
+        n["mixer_norm.weight"] = f"L{i}.n1"
+        if ffn:
+            n.update({"ffn_norm.weight": f"L{i}.n2", "ffn.w1.weight": f"L{i}.w1", "ffn.w3.weight": f"L{i}.w3", "ffn.w2.weight": f"L{i}.w2"})
+        return n
+
+    proj = ["q_proj.weight", "k_proj.weight", "v_proj.weight", "out_proj.weight"]
+    blocks = (BlockSpec(full, norm, SwiGLUSpec(H, 96), norm, names(0, proj + ["q_norm.weight", "k_norm.weight"])),
+              BlockSpec(near, norm, SwiGLUSpec(H, 64), norm, names(1, proj)),
+              BlockSpec(ShortConvSpec(H, 3), norm, None, None, names(2, ["in_proj.weight", "conv.weight", "out_proj.weight"], False)))
+    spec = ModelSpec(architecture="ToyTwoGroups", hidden=H, vocab=V, blocks=blocks,
+                     schedule=(LayerCall(0), LayerCall(1), LayerCall(2)), final_norm=norm, tie_embeddings=True,
+                     max_position=1024, names={"embed": "emb", "final_norm.weight": "fn"})
+    table = tensor_table(spec)
+    cpu = random_tensors(table, 29, torch.bfloat16, std=0.15)
+    dev = "cuda:0"
+    tensors = {k: v.to(dev, held_dtype(v.dtype, table[k].role, torch.bfloat16)) for k, v in cpu.items()}
+    made = []
+    for on in (False, True):
+        # the kernel for long portions at every length, so that steps whose longest portion is short are recorded too
+        made.append(Engine(spec, tensors, torch.bfloat16, dev, page_size=4, max_tokens=6 * 448, num_slots=7, poison=True,
+                           options=RuntimeOptions(record_portions=on, prompt_attention="wide")))
+    plain, recorded = made
+    assert [g.need.window for g in recorded.manager.layout.paged] == [None, 40]
+    rng = random.Random(9)
+    work = Workload(V, 80, seed=9, prompt_lens=[rng.randint(20, 400) for _ in range(30)])
+    kinds = {}
+    run_both(plain, recorded, work, 50, kinds)
+    rec = recorded.recorder
+    assert rec.replays == replays_expected(kinds, rec) and rec.replays >= 20, (rec.replays, kinds)
+    plain.manager.check(); recorded.manager.check()
