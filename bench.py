@@ -123,7 +123,8 @@ def prefill_run(engine, cfg, tokens: int, reps: int = 5):
     g = torch.Generator().manual_seed(99)
     ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
     times = []
-    for i in range(reps + 2):
+    warm = 4          # (a recorded step of portions is recorded at its fourth coming)
+    for i in range(reps + warm):
         rid = ("prefill", i)
         engine.add_request(rid)
         torch.cuda.synchronize()
@@ -132,7 +133,7 @@ def prefill_run(engine, cfg, tokens: int, reps: int = 5):
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         engine.finish_request(rid)
-    times = sorted(times[2:])
+    times = sorted(times[warm:])
     return times[len(times) // 2]
 
 
@@ -333,8 +334,8 @@ def main() -> int:
     ap.add_argument("--no-ceilings", action="store_true", help="skip the measurement of what the machine delivers")
     ap.add_argument("--no-tune", action="store_true", help="the vendor library's first choice for every product of many "
                     "rows (for profiles: no tuning runs among the kernels)")
-    ap.add_argument("--launched-portions", action="store_true", help="--workload serve: launch the steps with prompt portions "
-                    "kernel by kernel instead of replaying recordings of them")
+    ap.add_argument("--launched-portions", action="store_true", help="launch the steps with prompt portions kernel by kernel instead of "
+                    "replaying recordings of them (the prefill of the default line, --workload serve)")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
@@ -368,7 +369,8 @@ def main() -> int:
     from gesso_amd.parts import RuntimeOptions
     engine = Engine.from_config(cfg, seed=0, dtype=dtype, page_size=16, max_context=context,
                                 max_tokens=max_batch * (prompt_len + args.steps + args.warmup + 32) + 4096,
-                                num_slots=max_batch + 1, options=RuntimeOptions(tune_library=not args.no_tune))
+                                num_slots=max_batch + 1,
+                                options=RuntimeOptions(tune_library=not args.no_tune, record_portions=not args.launched_portions))
     wbytes = weight_bytes(engine)
     if args.only_prefill:
         sec = prefill_run(engine, cfg, 2048)
@@ -391,7 +393,8 @@ def main() -> int:
                    "head_dim": cfg.head_dim, "ff": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "conv_L_cache": cfg.conv_L_cache, "attn_layers": sum(t == "full_attention" for t in cfg.layer_types),
                    "global_batch": args.batch, "prompt_len": prompt_len, "seq_len": context, "page_size": 16,
-                   "parallelism": "single GPU", "weights_gb": round(wbytes / 1e9, 3)},
+                   "parallelism": "single GPU", "weights_gb": round(wbytes / 1e9, 3),
+                   "recorded_portions": engine.recorder is not None},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
     }
