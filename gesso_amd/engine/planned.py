@@ -198,10 +198,12 @@ class RecordedStep:
                 tg[i, :m] = t[:m]
             tg[tg < 0] = scratch                              # pages a window has passed and given back
         for at, cnt, (seq, row, num) in made:
+            # the step's tiles at the list's end, tiles of no rows before them (they name row 0 of sequence 0, which
+            # exist): the kernel starts its blocks from the end of the list, so the empty ones come last
             part = self.np[at:at + 3 * cnt].reshape(3, cnt)
             m = len(seq)
-            part[:, m:] = 0                                   # tiles of no rows (they name row 0 of sequence 0, which exist)
-            part[0, :m], part[1, :m], part[2, :m] = seq, row, num
+            part[:, :cnt - m] = 0
+            part[0, cnt - m:], part[1, cnt - m:], part[2, cnt - m:] = seq, row, num
         want = self._host("want")
         w = 0
         for i, e in enumerate(entries):
