@@ -9,7 +9,7 @@ one int32 buffer, one copy per step.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Sequence
+from typing import Hashable, List, Sequence
 
 import numpy as np
 import torch

@@ -19,14 +19,13 @@ from __future__ import annotations
 
 import gc
 
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Dict, Hashable, List, Sequence, Tuple
 
 import numpy as np
 import torch
 
 from ..errors import InvalidPlan
 from .batch import BatchContext
-from ..sampling.sampler import Sampler
 
 
 def _capacity(n: int) -> int:

@@ -11,7 +11,7 @@ before it has changed anything; the scheduler decides what to do then.
 """
 from __future__ import annotations
 
-from typing import Hashable, List, Optional, Sequence
+from typing import Hashable, Optional, Sequence
 
 import torch
 
@@ -19,7 +19,7 @@ from ..cache.manager import CacheLayout, CacheManager
 from ..cache.storage import CacheStorage
 from ..config.registry import load_config
 from ..config.spec import ModelSpec
-from ..errors import GessoError, InvalidPlan, StepFailed
+from ..errors import InvalidPlan, StepFailed
 from ..models.model import Model, tensor_table, tied_aliases
 from ..parts.runtime import Runtime, RuntimeOptions
 from ..weights.loader import load_tensors, random_tensors

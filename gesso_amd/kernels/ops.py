@@ -7,7 +7,7 @@ missing library or a refused size raises :class:`~gesso_amd.errors.KernelError`.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_double, c_float, c_int, c_long, c_void_p
+from ctypes import c_float, c_int, c_long
 
 import torch
 

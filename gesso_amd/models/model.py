@@ -13,7 +13,7 @@ import torch
 
 from ..config.spec import ModelSpec
 from ..errors import ConfigError
-from ..parts.base import MATRIX, TABLE, TensorSpec, sub_tensors
+from ..parts.base import MATRIX, TABLE, TensorSpec
 from ..parts.registry import build, part_class
 from ..parts.rmsnorm import ResidualStream, row_weight_of
 

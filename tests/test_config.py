@@ -226,7 +226,7 @@ def test_registry(tmp_path):
 
 
 def test_schedule_is_checked():
-    from gesso_amd.config import LayerCall, ModelSpec
+    from gesso_amd.config import LayerCall
     c = Lfm2Config.from_dict(BASE)
     spec = lfm2_spec(c)
     import dataclasses

@@ -13,7 +13,6 @@ configuration here).  The weights are drawn with a standard deviation of 0.1, at
 some 2 % of the logits' spread from the plain model: a fixed tolerance would be narrower than that noise or wider than
 a fault.
 """
-import numpy as np
 import pytest
 import torch
 

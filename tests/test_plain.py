@@ -6,7 +6,6 @@ the wrong place, a tap order reversed) fails it.
 """
 import math
 
-import numpy as np
 import pytest
 import torch
 import torch.nn.functional as F

@@ -8,7 +8,6 @@ The reference plants controls of this kind in its own model tests (``test/test_l
 """
 import math
 
-import numpy as np
 import pytest
 import torch
 
