@@ -191,6 +191,8 @@ class Session:
         st = dict(sched.stats)
         st.update(prefill_ms=(first - t0) * 1e3, decode_ms=(t1 - first) * 1e3,
                   new_tokens=sum(len(r.output) for r in requests), cache=self.engine.manager.stats())
+        if self.engine.recorder is not None:
+            st["replayed_steps"] = self.engine.recorder.replays       # since the session began
         profile = self.engine.rt.profile
         if profile is not None:
             st["decode_profile"] = profile.report()

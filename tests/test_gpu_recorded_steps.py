@@ -179,6 +179,7 @@ def test_the_scheduler_over_recorded_steps_generates_the_same_ids(tmp_path):
         if on:
             rec = s.engine.recorder
             assert not rec.refused and rec.replays >= 20, (rec.refused, rec.replays, rec.seen)
+            assert s.last_stats["replayed_steps"] == rec.replays
         s.close()
     assert out[0] == out[1]
 
