@@ -237,6 +237,7 @@ class StepRecorder:
 
     SEEN_BEFORE = 3
     MAX_RECORDINGS = 4           # each holds the activations of its token count
+    MAX_SEEN = 4096              # kinds whose comings are counted
     SEQ_CAP = 64
     MIN_KV_CAP = 4096
 
@@ -270,6 +271,8 @@ class StepRecorder:
             return None
         rec = self.recordings.get(kind)
         if rec is None and kind not in self.recordings:
+            if len(self.seen) >= self.MAX_SEEN and kind not in self.seen:
+                self.seen.clear()               # (a server sees a new token count in many of its steps: the tally starts over)
             n = self.seen[kind] = self.seen.get(kind, 0) + 1
             if n <= self.SEEN_BEFORE or sum(1 for r in self.recordings.values() if r is not None) >= self.MAX_RECORDINGS:
                 return None
