@@ -238,6 +238,7 @@ class StepRecorder:
     SEEN_BEFORE = 3
     MAX_RECORDINGS = 4           # each holds the activations of its token count
     MAX_SEEN = 4096              # kinds whose comings are counted
+    IDLE_STEPS = 256             # a recording unused for so many steps makes room when another kind wants it
     SEQ_CAP = 64
     MIN_KV_CAP = 4096
 
@@ -247,6 +248,8 @@ class StepRecorder:
         self.recordings: Dict = {}      # kind -> RecordedStep, or None where recording was refused
         self.refused: Dict = {}         # kind -> the error that refused it
         self.replays = 0
+        self.clock = 0                  # steps that could have been replayed, counted
+        self.used: Dict = {}            # kind -> the clock when its recording last served
 
     def kind_of(self, entries: Sequence[StepEntry]):
         eng = self.engine
@@ -269,13 +272,23 @@ class StepRecorder:
         kind = self.kind_of(entries)
         if kind is None:
             return None
+        self.clock += 1
         rec = self.recordings.get(kind)
         if rec is None and kind not in self.recordings:
             if len(self.seen) >= self.MAX_SEEN and kind not in self.seen:
                 self.seen.clear()               # (a server sees a new token count in many of its steps: the tally starts over)
             n = self.seen[kind] = self.seen.get(kind, 0) + 1
-            if n <= self.SEEN_BEFORE or sum(1 for r in self.recordings.values() if r is not None) >= self.MAX_RECORDINGS:
+            if n <= self.SEEN_BEFORE:
                 return None
+            held = [k for k, r in self.recordings.items() if r is not None]
+            if len(held) >= self.MAX_RECORDINGS:
+                # room for this kind only if a recording has lain idle for a while (sequences grow out of their block
+                # tables' room, a scheduler's budget changes): the one unused longest goes, with its graphs and buffers
+                oldest = min(held, key=lambda k: self.used[k])
+                if self.clock - self.used[oldest] < self.IDLE_STEPS:
+                    return None
+                del self.recordings[oldest], self.used[oldest]
+                self.seen.pop(oldest, None)
             T, kv_cap, key = kind
             rec = RecordedStep(self.engine, T, self.SEQ_CAP, kv_cap, key)
             try:
@@ -285,4 +298,6 @@ class StepRecorder:
                 self.refused[kind] = err
                 rec = None
             self.recordings[kind] = rec
+        if rec is not None:
+            self.used[kind] = self.clock
         return rec

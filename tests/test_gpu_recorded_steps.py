@@ -39,19 +39,19 @@ class Workload:
     """Requests with prompts of random lengths; every step holds ``T`` tokens: the decoded tokens of the requests whose
     prompts are through (at the head), then portions of the prompts that are not, cut where the step is full."""
 
-    def __init__(self, vocab, T, seed, prompt_lens, new_tokens=(3, 9), live=6):
+    def __init__(self, vocab, T, seed, prompt_lens, new_tokens=(3, 9), live=6, tag="w"):
         self.rng = random.Random(seed)
         self.vocab, self.T, self.live_max = vocab, T, live
         self.prompts = [random_ids(n, vocab, seed * 100 + i) for i, n in enumerate(prompt_lens)]
         self.new_tokens = new_tokens
-        self.next_rid = 0
+        self.next_rid, self.tag = 0, tag
         self.live = {}          # rid -> dict(prompt, done, left, token)
 
     def admit(self, engines_):
         while len(self.live) < self.live_max and self.next_rid < len(self.prompts):
-            rid = self.next_rid
+            rid = (self.tag, self.next_rid)
+            self.live[rid] = dict(prompt=self.prompts[self.next_rid], done=0, left=self.rng.randint(*self.new_tokens), token=None)
             self.next_rid += 1
-            self.live[rid] = dict(prompt=self.prompts[rid], done=0, left=self.rng.randint(*self.new_tokens), token=None)
             for e in engines_:
                 e.add_request(rid)
 
@@ -233,3 +233,27 @@ def test_recorded_steps_over_two_page_groups_one_of_them_windowed(tmp_path):
     rec = recorded.recorder
     assert rec.replays == replays_expected(kinds, rec) and rec.replays >= 20, (rec.replays, kinds)
     plain.manager.check(); recorded.manager.check()
+
+
+def test_a_recording_that_lies_idle_makes_room_for_another_kind(tmp_path):
+    """With room for one recording: steps of 96 tokens are recorded; when the steps turn to 80 tokens that recording is
+    given up after a few idle steps and the new kind recorded, and back again; the logits stay those of the launched steps."""
+    folder = str(tmp_path / "D")
+    write_model_folder(folder, WIDE_D, 14, torch.bfloat16, std=STD)
+    plain, recorded = engines(folder, page_size=16, max_tokens=12 * 448, num_slots=13)
+    rec = recorded.recorder
+    rec.MAX_RECORDINGS, rec.IDLE_STEPS = 1, 5
+    held = []
+    for round_, T in enumerate((96, 80, 96)):
+        rng = random.Random(T + round_)
+        work = Workload(WIDE_D.vocab_size, T, seed=T + round_, prompt_lens=[rng.randint(70, 400) for _ in range(12)], tag=round_)
+        before = rec.replays
+        run_both(plain, recorded, work, 16, {})
+        assert not rec.refused, rec.refused
+        made = [k for k, r in rec.recordings.items() if r is not None]
+        assert len(made) == 1 and made[0][0] == T, (T, made)
+        assert rec.replays - before >= 4, (T, rec.replays - before)
+        held.append(made[0])
+        for rid in list(work.live):             # what this round left unfinished
+            plain.finish_request(rid); recorded.finish_request(rid)
+    assert held[0] == held[2] != held[1]
