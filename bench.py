@@ -172,9 +172,10 @@ def measured_ceilings(reps: int = 5) -> dict:
     return {"read_gbps": round(read, 1), "mfma_tflops_vendor": round(vendor, 1), "mfma_tflops_ours": round(ours, 1)}
 
 
-def serve_workload(seed: int = 5, record: bool = True, tune: bool = True) -> dict:
+def serve_workload(seed: int = 5, record: bool = True, tune: bool = True, budget: int = 4096) -> dict:
     """LFM2-350M sizes: 64 requests at once, prompts of 64 to 2,048 tokens, 32 to 512 new tokens each, prompt
-    portions of 512 tokens beside the decodes of the others; the scheduler's own loop, greedy."""
+    portions of 512 tokens beside the decodes of the others, at most ``budget`` tokens a step; the scheduler's own loop,
+    greedy."""
     from gesso_amd import Session
     from gesso_amd.engine.scheduler import Request
     from gesso_amd.parts import RuntimeOptions
@@ -184,7 +185,7 @@ def serve_workload(seed: int = 5, record: bool = True, tune: bool = True) -> dic
     plen = torch.randint(64, 2049, (n,), generator=g).tolist()
     olen = torch.randint(32, 513, (n,), generator=g).tolist()
     sess = Session(cfg, random_weights_seed=0, context_length=4096, max_num_seqs=64, chunk_size=512,
-                   max_num_batched_tokens=1024, max_tokens=n * 2624,
+                   max_num_batched_tokens=budget, max_tokens=n * 2624,
                    kernel_options=RuntimeOptions(record_portions=record, tune_library=tune))
     stamps = {}
 
@@ -213,7 +214,7 @@ def serve_workload(seed: int = 5, record: bool = True, tune: bool = True) -> dic
             "prompt_tokens": sum(plen), "new_tokens": new, "prompt_tok_s": round(sum(plen) / (t1 - t0), 1),
             "mean_ttft_ms": round(1e3 * sum(ttft) / n, 2), "mean_tpot_ms": round(1e3 * sum(tpot) / len(tpot), 3),
             "steps": sched.stats["steps"], "preemptions": sched.stats["preemptions"], "chunk": 512,
-            "token_budget": 1024, "recorded_steps": getattr(sess.engine.recorder, "replays", 0), "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
+            "token_budget": budget, "recorded_steps": getattr(sess.engine.recorder, "replays", 0), "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights N(0, 0.02)"}
 
 
 def gemm_workload(reps: int = 10) -> dict:
@@ -336,6 +337,7 @@ def main() -> int:
                     "rows (for profiles: no tuning runs among the kernels)")
     ap.add_argument("--launched-portions", action="store_true", help="launch the steps with prompt portions kernel by kernel instead of "
                     "replaying recordings of them (the prefill of the default line, --workload serve)")
+    ap.add_argument("--token-budget", type=int, default=4096, help="--workload serve: the most tokens a step holds")
     ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
@@ -349,7 +351,7 @@ def main() -> int:
             print(json.dumps(stages_workload(args.batch, min(args.steps, 32))))
             return 0
         if args.workload == "serve":
-            print(json.dumps(serve_workload(record=not args.launched_portions, tune=not args.no_tune)))
+            print(json.dumps(serve_workload(record=not args.launched_portions, tune=not args.no_tune, budget=args.token_budget)))
             return 0
         run = {"long": long_workload, "gemm": gemm_workload}[args.workload]
         print(json.dumps(run()))
