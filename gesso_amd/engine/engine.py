@@ -39,10 +39,12 @@ def parse_dtype(dtype) -> torch.dtype:
 class Engine:
     def __init__(self, spec: ModelSpec, tensors, dtype, device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, num_slots: int = 8,
-                 max_context: Optional[int] = None, options: Optional[RuntimeOptions] = None, poison: bool = False):
+                 max_context: Optional[int] = None, options: Optional[RuntimeOptions] = None, poison: bool = False,
+                 memory_fraction: Optional[float] = None):
         """``tensors``: ``file name -> tensor`` on the device, in the widths the loader chose.
 
-        The page pool holds ``num_pages`` pages per group, or enough for ``max_tokens`` tokens.
+        The page pool holds ``num_pages`` pages per group, or enough for ``max_tokens`` tokens, or as many as fit into
+        ``memory_fraction`` of the device memory that is free once the weights are bound.
         ``options``: how kernels are chosen (:class:`~gesso_amd.parts.runtime.RuntimeOptions`).
         ``poison``: a debugging aid: every page and slot that is given back is filled with NaN before the next
         step runs, so that a kernel that reads a row it has no business with shows in the logits.
@@ -55,12 +57,15 @@ class Engine:
         self.model.bind(tensors)
         self.page_size = int(page_size)
         self.max_context = min(spec.max_position, max_context or spec.max_position)
-        if num_pages is None:
-            if max_tokens is None:
-                raise InvalidPlan("give the cache a size: num_pages or max_tokens")
-            num_pages = -(-int(max_tokens) // self.page_size)
         needs = self.model.cache_needs()
         layout = CacheLayout.plan(needs, [c.cache for c in spec.schedule])
+        if num_pages is None:
+            if max_tokens is not None:
+                num_pages = -(-int(max_tokens) // self.page_size)
+            elif memory_fraction is not None:
+                num_pages = self._pages_that_fit(layout, float(memory_fraction))
+            else:
+                raise InvalidPlan("give the cache a size: num_pages, max_tokens or memory_fraction")
         self.manager = CacheManager(layout, self.page_size, int(num_pages), int(num_slots), self.max_context)
         self.storage = CacheStorage(layout, self.page_size, int(num_pages), int(num_slots), self.dtype, self.device)
         self.poison = bool(poison)
@@ -78,6 +83,24 @@ class Engine:
         # the most requests one recorded decode step takes: as many rows as the runtime's weight-streaming products do
         # (the limit is the product kernels', asked of the runtime, not a number of the engine's own)
         self.DECODE_MAX_BATCH = self.rt.streaming_rows_max
+
+    def _pages_that_fit(self, layout: CacheLayout, fraction: float) -> int:
+        """Pages per group that ``fraction`` of the free device memory holds (every group gets as many)."""
+        if not 0.0 < fraction <= 1.0:
+            raise InvalidPlan(f"memory_fraction is a share of the free device memory in (0, 1], not {fraction}")
+        width = torch.empty((), dtype=self.dtype).element_size()
+        per_page = sum(len(g.members) * g.need.n_kv_heads * self.page_size * (g.need.head_dim + g.need.value_width) * width
+                       for g in layout.paged)
+        if per_page == 0:
+            return 1                               # no paged layers: a page is bookkeeping only
+        free, _ = torch.cuda.mem_get_info(self.device)
+        pages = int(free * fraction) // per_page - 1            # (one more page per group is scratch)
+        if pages < 1:
+            raise InvalidPlan(f"{fraction} of the {free} free bytes hold no page of {per_page} bytes")
+        # what the kernels' 32-bit offsets into one layer's pages reach (units of 16 bytes)
+        reach = min((1 << 32) // max(1, g.need.n_kv_heads * self.page_size * max(1, max(g.need.head_dim, g.need.value_width) * width // 16))
+                    for g in layout.paged)
+        return min(pages, reach - 2)
 
     # ------------------------------------------------------------------ construction
 

@@ -51,10 +51,11 @@ class Session:
                  chunk_size: Optional[int] = None, num_pages: Optional[int] = None,
                  max_tokens: Optional[int] = None, random_weights_seed: Optional[int] = None,
                  random_weights_std: float = 0.02, watermark: float = 0.01, kernel_options=None,
-                 poison: bool = False):
+                 poison: bool = False, memory_fraction: Optional[float] = None):
         """``model``: a folder with config.json and model.safetensors, or a typed configuration
         together with ``random_weights_seed``.  ``context_length``: most tokens one request may hold.
-        The cache holds ``num_pages`` pages, or ``max_tokens`` tokens (default: four contexts).
+        The cache holds ``num_pages`` pages, or ``max_tokens`` tokens, or what fits into ``memory_fraction`` of the
+        device memory left free by the weights (default: four contexts).
         ``watermark``: the fraction of the pages that an admission leaves free for those who run.
         ``kernel_options``: a :class:`~gesso_amd.parts.runtime.RuntimeOptions`; ``poison``: fill what is
         given back with NaN (a debugging aid, see :class:`Engine`)."""
@@ -74,9 +75,10 @@ class Session:
             arch = architecture_of(cfg.to_json())
         # the longest context the model itself allows is a fact of its description, whatever its configuration calls it
         self.context_length = int(context_length or min(arch.to_spec(cfg).max_position, 4096))
-        if num_pages is None and max_tokens is None:
+        if num_pages is None and max_tokens is None and memory_fraction is None:
             max_tokens = 4 * self.context_length
-        kw.update(num_pages=num_pages, max_tokens=max_tokens, max_context=self.context_length)
+        kw.update(num_pages=num_pages, max_tokens=max_tokens, max_context=self.context_length,
+                  memory_fraction=memory_fraction)
         if isinstance(model, (str, os.PathLike)):
             self.engine = Engine.from_folder(os.fspath(model), dtype=dtype, device=device, **kw)
         else:

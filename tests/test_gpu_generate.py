@@ -444,6 +444,30 @@ def test_nothing_reads_what_nobody_wrote(folders, monkeypatch, name, dtype):
     assert got == want
 
 
+def test_a_cache_sized_by_a_share_of_the_free_memory(folders):
+    """``memory_fraction``: as many pages as that share of the free device memory holds, and they serve."""
+    from gesso_amd import Engine, Session
+    from gesso_amd.errors import InvalidPlan
+
+    d = write_tiny(folders, "A", torch.bfloat16)
+    free, _ = torch.cuda.mem_get_info(0)
+    eng = Engine.from_folder(d, dtype="bfloat16", page_size=16, memory_fraction=1e-4)
+    cfg = CONFIGS["A"][0]
+    n_attn = sum(t == "full_attention" for t in cfg.layer_types)
+    per_page = n_attn * cfg.num_key_value_heads * 16 * 2 * cfg.head_dim * 2
+    pages = eng.manager.stats()["pages_total"][0]
+    assert 0.8 * (free * 1e-4 / per_page) <= pages <= free * 1e-4 / per_page, (pages, free, per_page)
+    assert eng.storage.keys[0].shape[1] == pages + 1
+    with pytest.raises(InvalidPlan, match="memory_fraction"):
+        Engine.from_folder(d, dtype="bfloat16", memory_fraction=1.5)
+    with pytest.raises(InvalidPlan, match="num_pages, max_tokens or memory_fraction"):
+        Engine.from_folder(d, dtype="bfloat16")
+    s = Session(d, dtype="bfloat16", memory_fraction=1e-4)
+    roomy = Session(d, dtype="bfloat16")
+    prompt = random_ids(40, cfg.vocab_size, 5)
+    assert s.generate(prompt, max_new_tokens=8) == roomy.generate(prompt, max_new_tokens=8)
+
+
 def test_random_weights_session_and_cli(tmp_path):
     from gesso_amd import Session
     s = Session(TINY_B, random_weights_seed=4, random_weights_std=STD, dtype="bfloat16", context_length=64)
