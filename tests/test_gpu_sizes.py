@@ -305,3 +305,46 @@ def test_a_long_context_in_portions_then_recorded_decoding(dtype, tmp_path):
         bound.check("long context,")
     if dtype == "bfloat16":
         assert len(eng._runners[1].graphs) == 1 and (8192, False) in eng._runners[1].graphs
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_pages_beyond_four_giga_elements_of_a_layers_cache(dtype, tmp_path):
+    """A cache sized for a machine of this kind holds more than 2^32 elements a layer.  An engine with a pool of 540,000
+    pages that hands out its highest pages first gives, bit for bit, the logits and the tokens of one with 256 pages: long
+    portions, short ones beside them, single tokens, the recorded decode loop (offsets into the pages are 64 bits wide,
+    or 32 bits in units of 16 bytes, in every kernel that reads or writes the cache)."""
+    from gesso_amd import Engine, StepEntry
+
+    d = write_real_size_folder(str(tmp_path / "m"), 25.0, "350M")
+    pages = 540_000
+    small = Engine.from_folder(d, dtype=dtype, page_size=16, num_pages=256, num_slots=5)
+    huge = Engine.from_folder(d, dtype=dtype, page_size=16, num_pages=pages, num_slots=5)
+    assert huge.storage.keys[0].numel() > 2 ** 32
+    for pool in huge.manager.pools:
+        pool._free.reverse()                       # the highest pages first
+    ids = {k: random_ids(n, 65536, 7 + n) for k, n in {"a": 700, "b": 300, "c": 90}.items()}
+
+    def run(eng):
+        out = []
+        for k in ids:
+            eng.add_request(k)
+        out.append(eng.step([StepEntry("a", ids["a"][:600], [599])]))
+        out.append(eng.step([StepEntry("a", ids["a"][600:640], [39]), StepEntry("b", ids["b"][:200], [0, 199])]))
+        out.append(eng.step([StepEntry("a", ids["a"][640:641], [0]), StepEntry("b", ids["b"][200:230], [29]),
+                             StepEntry("c", ids["c"][:90], [89])]))
+        out.append(eng.step([StepEntry("a", ids["a"][641:642], [0]), StepEntry("b", ids["b"][230:231], [0]),
+                             StepEntry("c", [5], [0])]))
+        chosen, bad = eng.decode(["a", "b", "c"], [1, 2, 3], 6)
+        assert not bad.any()
+        out.append(torch.from_numpy(chosen.copy()))
+        top = max(max(t for t in eng.manager.get(k).tables[0] if t >= 0) for k in ids)
+        for k in ids:
+            eng.finish_request(k)
+        return out, top
+
+    (a, top_a), (b, top_b) = run(small), run(huge)
+    assert top_a < 256 and top_b >= pages - 200
+    for i, (x, y) in enumerate(zip(a, b)):
+        assert torch.isfinite(x.float()).all(), i
+        assert torch.equal(x.cpu(), y.cpu()), (i, (x.float().cpu() - y.float().cpu()).abs().max().item())
