@@ -168,6 +168,8 @@ class RecordedStep:
         ctx.q_lens = lens
         ctx.max_kv_len = int((held + lens_a).max())
         ctx._tiles = None
+        if sum(len(e.want) for e in entries) > T:
+            return None                                       # (rows wanted more than once: more than the buffer holds)
         made = []
         for at, cnt, maker in self.tile_lists.values():
             lists = maker(ctx)
