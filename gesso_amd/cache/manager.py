@@ -145,21 +145,37 @@ class CacheManager:
             rc.tables[g].extend(self.pools[g].take(n))
 
     def reserve_many(self, asks: Sequence[Tuple[Hashable, int]]) -> None:
-        """:meth:`reserve` for several requests as one decision: all fit or nothing is taken."""
-        total = [0] * len(self.pools)
+        """:meth:`reserve` for several requests (each named once) as one decision: all fit or nothing is taken."""
+        groups = len(self.pools)
+        total = [0] * groups
+        needs = []
+        ps = self.page_size
         for rid, n_new in asks:
             rc = self.get(rid)
+            if n_new < 0:
+                raise InvalidPlan("cannot reserve a negative number of tokens")
             if rc.length + n_new > self.max_length:
                 raise ResourceLimit(f"request {rid!r} would hold {rc.length + n_new} tokens, the context holds {self.max_length}",
                                     length=rc.length + n_new, max_length=self.max_length)
-            for g, n in enumerate(self.pages_needed(rid, n_new)):
-                total[g] += n
+            blocks = -(-(rc.length + n_new) // ps)
+            need = None                                    # (most decoded tokens need no page)
+            for g, t in enumerate(rc.tables):
+                n = blocks - len(t)
+                if n > 0:
+                    if need is None:
+                        need = [0] * groups
+                    need[g] = n
+                    total[g] += n
+            if need is not None:
+                needs.append((rc, need))
         for g, n in enumerate(total):
             if n > self.pools[g].n_free:
                 raise self.pools[g].exhausted(f"group {g}: {n} pages asked for this step, {self.pools[g].n_free} free",
                                               group=g, asked=n, free=self.pools[g].n_free, total=self.pools[g].total)
-        for rid, n_new in asks:
-            self.reserve(rid, n_new)
+        for rc, need in needs:
+            for g, n in enumerate(need):
+                if n:
+                    rc.tables[g].extend(self.pools[g].take(n))
 
     def commit(self, rid: Hashable, n_new: int) -> None:
         """``n_new`` tokens were written: advance, and give back the pages a window has passed."""

@@ -35,8 +35,10 @@ class RecordedContext(BatchContext):
     hand (``q_lens``, ``max_kv_len``, ``lead_single``) are for the calls that a replay makes anew."""
 
     def __init__(self, rec: "RecordedStep"):
-        self._set(rec.engine.storage, T=rec.T, nseq=rec.seq_cap, n_want=0, q_lens=[rec.T], all_single=False,
-                  max_q_len=rec.T, max_kv_len=None, decode_only=False, token_ids=rec.field("tok"),
+        single = rec.single
+        self._set(rec.engine.storage, T=rec.T, nseq=rec.seq_cap, n_want=0, q_lens=[1] * rec.T if single else [rec.T],
+                  all_single=single, max_q_len=1 if single else rec.T, max_kv_len=None, decode_only=False,
+                  token_ids=rec.field("tok"),
                   positions=rec.field("pos"), seq_of_token=rec.field("seq_of"), q_start=rec.field("q_start"),
                   kv_len=rec.field("kv_len"), slots=rec.field("slots"), want_rows=rec.field("want"),
                   block_tables=rec.tables)
@@ -47,8 +49,9 @@ class RecordedStep:
 
     TILE_ROOM = 1 << 16          # int32 entries for the tile lists that parts ask for
 
-    def __init__(self, engine, T: int, seq_cap: int, kv_cap: int, key):
-        self.engine, self.T, self.seq_cap, self.kv_cap, self.key = engine, T, seq_cap, kv_cap, key
+    def __init__(self, engine, T: int, seq_cap: int, kv_cap: int, key, single: bool = False):
+        """``single``: a step of ``T`` sequences that bring one token each (then ``seq_cap`` is ``T``)."""
+        self.engine, self.T, self.seq_cap, self.kv_cap, self.key, self.single = engine, T, seq_cap, kv_cap, key, single
         storage = engine.storage
         self.max_blocks = -(-kv_cap // engine.page_size)
         self.groups = len(storage.num_pages)
@@ -241,7 +244,8 @@ class StepRecorder:
     MAX_RECORDINGS = 4           # each holds the activations of its token count
     MAX_SEEN = 4096              # kinds whose comings are counted
     IDLE_STEPS = 256             # a recording unused for so many steps makes room when another kind wants it
-    SEQ_CAP = 64
+    SEQ_CAP = 64                 # sequences in a recorded step with prompt portions
+    MAX_SINGLE = 1024            # sequences in a recorded step of single tokens
     MIN_KV_CAP = 4096
 
     def __init__(self, engine):
@@ -255,10 +259,13 @@ class StepRecorder:
 
     def kind_of(self, entries: Sequence[StepEntry]):
         eng = self.engine
-        if len(entries) > self.SEQ_CAP:
-            return None
         lens = [len(e.tokens) for e in entries]
         if max(lens) == 1:
+            # single tokens only: the recorded decode loop takes up to its own limit of them without the host; more
+            # than that are one step of library products, which is worth recording
+            if not getattr(eng, "DECODE_MAX_BATCH", 0) < len(entries) <= self.MAX_SINGLE:
+                return None
+        elif len(entries) > self.SEQ_CAP:
             return None
         longest = max(eng.manager.get(e.rid).length + n for e, n in zip(entries, lens))
         key = eng.model.replay_key(lens, longest)
@@ -292,7 +299,8 @@ class StepRecorder:
                 del self.recordings[oldest], self.used[oldest]
                 self.seen.pop(oldest, None)
             T, kv_cap, key = kind
-            rec = RecordedStep(self.engine, T, self.SEQ_CAP, kv_cap, key)
+            single = max(len(e.tokens) for e in entries) == 1
+            rec = RecordedStep(self.engine, T, T if single else self.SEQ_CAP, kv_cap, key, single)
             try:
                 rec.record()
             except GessoError as err:

@@ -137,15 +137,21 @@ class Attention(Part):
 
     def replay_key(self, q_lens, max_kv_len):
         """A recorded step of prompt portions walks the keys as the step that replays it would: whole (1) or in halves
-        (2).  False: such a step does not go through the kernel for long portions, and is not to be recorded."""
+        (2); a step of single tokens: "single".  False: such a step does not go through the kernel for long portions
+        (or, of single tokens, would split their keys over blocks by the longest sequence), and is not to be recorded."""
         s, rt, ops = self.spec, self.rt, self.rt.ops
         nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
         lead = 0
         while lead < len(q_lens) and q_lens[lead] == 1:
             lead += 1
+        if lead == len(q_lens):
+            # single tokens only: the kernel for single queries takes every sequence's keys in one block when the
+            # (sequence, key head) pairs fill the chip by themselves, and its launch then depends on their number alone
+            return "single" if (rt.dtype == torch.bfloat16 and ops.attention_decode_supports(nh, nkv, d)
+                                and 256 // (lead * nkv) <= 1) else False
         choice = rt.options.prompt_attention
         stride = (nh + 2 * nkv) * d
-        if not (rt.dtype == torch.bfloat16 and stride % 8 == 0 and lead < len(q_lens)
+        if not (rt.dtype == torch.bfloat16 and stride % 8 == 0
                 and ops.attention_prefill_supports(nh, nkv, d) and ops.attention_decode_supports(nh, nkv, d)
                 and choice != "tiles" and ops.attention_prefill_wide_supports(nh, nkv, d)
                 and (choice == "wide" or max(q_lens) >= 64)):
@@ -192,7 +198,7 @@ class Attention(Part):
         if isinstance(q, RawQKV):
             return self._single(q, q_stride, cache, ctx, ctx.nseq, out)
         fast = q.dtype == torch.bfloat16 and cache.page_size >= 2
-        if ctx.recording is not None:
+        if ctx.recording is not None and not ctx.all_single:
             return self._attend_recorded(q, q_stride, ctx, cache)
         if ctx.all_single and fast and ops.attention_decode_supports(nh, nkv, d):
             return self._single(q, q_stride, cache, ctx, ctx.nseq, out)

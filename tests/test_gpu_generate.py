@@ -96,6 +96,38 @@ def test_seventy_requests_at_once_decode_through_the_recorded_loop_in_groups(pla
     assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
 
 
+@pytest.mark.parametrize("record", [False, True])
+def test_a_hundred_and_fifty_requests_at_once_decode_in_steps_of_single_tokens(folders, record):
+    """In bfloat16, from 129 requests on, decoding leaves the recorded loop (groups of 64 that each read every weight) for
+    ordinary steps that hold one token of every request; with ``record_portions`` those steps are replayed from a
+    recording.  The tokens are ones the plain logits support, requests end at different lengths and their pages and slots
+    come back."""
+    from gesso_amd import Session
+    from gesso_amd.parts import RuntimeOptions
+    d = write_tiny(folders, "D", torch.bfloat16)
+    cfg, w = P.read_config(d), P.read_weights(d)
+    n = 150
+    s = Session(d, dtype="bfloat16", context_length=96, max_num_seqs=160, max_tokens=160 * 96,
+                kernel_options=RuntimeOptions(record_portions=record))
+    assert s.engine.WIDE_DECODE_FROM == 129
+    prompts = [random_ids(3 + i % 11, cfg["V"], 900 + i) for i in range(n)]
+    stops = {}                                          # some requests stop early, so that the steps shrink
+    got = s.generate(prompts, max_new_tokens=12, eos_ids=(),
+                     on_token=lambda i, tok: stops.setdefault(i, 0) is None or (stops.__setitem__(i, stops[i] + 1) or stops[i] < 6 + i % 7))
+    assert not s.engine._runners or max(s.engine._runners) <= 64
+    if record:
+        assert s.last_stats["replayed_steps"] >= 1 and not s.engine.recorder.refused
+    for i in (0, 7, 64, 128, 149):
+        p, g = prompts[i], got[i]
+        assert len(g) - len(p) == 6 + i % 7, (i, len(g) - len(p))
+        ref = P.forward(cfg, w, g[:-1])
+        slack = 2 * WORST * float((P.forward(cfg, w, g[:-1], store=P.to_bfloat16) - ref).abs().max())
+        for j in range(len(p), len(g)):
+            assert supported(ref[j - 1], g[j], slack), (i, j, g[j], slack)
+    st = s.engine.manager.stats()
+    assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+
+
 def test_temperature_sampling_follows_the_plain_sampler(plain):
     from gesso_amd import Sampler, Session
     d, cfg, w = plain["B"]

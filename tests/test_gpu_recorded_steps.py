@@ -257,3 +257,46 @@ def test_a_recording_that_lies_idle_makes_room_for_another_kind(tmp_path):
         for rid in list(work.live):             # what this round left unfinished
             plain.finish_request(rid); recorded.finish_request(rid)
     assert held[0] == held[2] != held[1]
+
+
+def test_recorded_steps_of_more_single_tokens_than_the_decode_loop_takes(tmp_path):
+    """140 sequences that bring one token each (the recorded decode loop takes 64): such steps run on the library's
+    products and are recorded like steps with portions; the same logits as launched, while sequences end and others
+    take their pages and slots."""
+    from gesso_amd import StepEntry
+
+    folder = str(tmp_path / "E")
+    write_model_folder(folder, WIDE_E, 15, torch.bfloat16, std=STD)
+    n = 140
+    plain, recorded = engines(folder, page_size=16, max_tokens=n * 96, num_slots=n + 1)
+    assert n > recorded.DECODE_MAX_BATCH
+    rng = random.Random(2)
+    tokens = {}
+    for a in range(0, n, 20):
+        entries = [StepEntry(i, random_ids(rng.randint(5, 60), WIDE_E.vocab_size, 40 + i), []) for i in range(a, a + 20)]
+        for eng in (plain, recorded):
+            for e in entries:
+                eng.add_request(e.rid)
+            assert eng.step(entries) is None
+    for i in range(n):
+        tokens[i] = rng.randrange(WIDE_E.vocab_size)
+    fresh = n
+    for s in range(14):
+        entries = [StepEntry(i, [t], [0]) for i, t in tokens.items()]
+        a, b = plain.step(entries), recorded.step(entries)
+        assert torch.isfinite(a).all() and torch.equal(a, b), (s, (a - b).abs().max().item())
+        picks = a.argmax(1).tolist()
+        tokens = {e.rid: p for e, p in zip(entries, picks)}
+        # three sequences end and three new ones of one token begin (their first token decodes from an empty cache)
+        for rid in list(tokens)[s % 5::50][:3]:
+            del tokens[rid]
+            for eng in (plain, recorded):
+                eng.finish_request(rid)
+                eng.add_request(fresh)
+            tokens[fresh] = rng.randrange(WIDE_E.vocab_size)
+            fresh += 1
+    rec = recorded.recorder
+    assert not rec.refused, rec.refused
+    (kind, step_), = [(k, r) for k, r in rec.recordings.items() if r is not None]
+    assert step_.single and kind[0] == n and rec.replays == 14 - rec.SEEN_BEFORE
+    plain.manager.check(); recorded.manager.check()

@@ -15,8 +15,8 @@ class Recording:
     made = []
     refuse = set()
 
-    def __init__(self, engine, T, seq_cap, kv_cap, key):
-        self.T, self.seq_cap, self.kv_cap, self.key = T, seq_cap, kv_cap, key
+    def __init__(self, engine, T, seq_cap, kv_cap, key, single=False):
+        self.T, self.seq_cap, self.kv_cap, self.key, self.single = T, seq_cap, kv_cap, key, single
 
     def record(self):
         if self.T in self.refuse:
@@ -31,8 +31,10 @@ def recorder(monkeypatch):
     held = {}
     manager = SimpleNamespace(get=lambda rid: SimpleNamespace(length=held.get(rid, 0)))
     # the model records steps whose longest portion has 64 tokens or more, and walks sequences of 4,096 keys another way
-    model = SimpleNamespace(replay_key=lambda lens, longest: (2 if longest < 4096 else 1,) if max(lens) >= 64 else None)
-    rec = planned.StepRecorder(SimpleNamespace(manager=manager, model=model))
+    # (steps of single tokens it walks in a way of their own)
+    model = SimpleNamespace(replay_key=lambda lens, longest: ("single",) if max(lens) == 1 else
+                            (2 if longest < 4096 else 1,) if max(lens) >= 64 else None)
+    rec = planned.StepRecorder(SimpleNamespace(manager=manager, model=model, DECODE_MAX_BATCH=64))
     rec.held = held
     return rec
 
@@ -55,6 +57,20 @@ def test_steps_that_are_never_recorded(recorder):
         assert recorder.recording_for(step(1, 30, 40)) is None                     # the model says no (short portions)
         assert recorder.recording_for(step(*([1] * recorder.SEQ_CAP + [80]))) is None      # more sequences than a recording holds
     assert Recording.made == [] and recorder.seen == {}
+
+
+def test_single_tokens_are_recorded_when_there_are_more_than_the_decode_loop_takes(recorder):
+    for _ in range(6):
+        assert recorder.recording_for(step(*[1] * 64)) is None           # the recorded decode loop's business
+        assert recorder.recording_for(step(*[1] * (recorder.MAX_SINGLE + 1))) is None
+    for _ in range(recorder.SEEN_BEFORE):
+        assert recorder.recording_for(step(*[1] * 200)) is None
+    rec = recorder.recording_for(step(*[1] * 200))
+    assert rec.single and rec.T == rec.seq_cap == 200 and rec.key == ("single",)
+    # 200 tokens with a portion among them are another kind, with room for the usual number of sequences
+    for _ in range(4):
+        other = recorder.recording_for(step(*[1] * 30, 170))
+    assert not other.single and other.seq_cap == recorder.SEQ_CAP and other.T == 200
 
 
 def test_room_for_keys_and_the_walk_make_kinds_of_their_own(recorder):
