@@ -71,7 +71,7 @@ class DecodeRunner:
         self.block_tables = [torch.full((cap, self.max_blocks), n, **i32) for n in st.num_pages]
         self.temperature = torch.zeros(cap, dtype=torch.float64, device=dev)
         self.top_p = torch.ones(cap, dtype=torch.float64, device=dev)
-        self.weights, self.wide = engine.choice_scratch()      # shared by all capacities
+        self.weights, self.wide = engine.choice_scratch(max(cap, engine.DECODE_MAX_BATCH))      # shared by all capacities
         self.u = torch.zeros((self.MAX_STEPS, cap), dtype=torch.float64, device=dev)
         self.counter = torch.zeros(cap, **i32)          # steps made since the host last looked, per row
         self.ring = torch.zeros((self.MAX_STEPS, cap), **i32)
@@ -85,8 +85,12 @@ class DecodeRunner:
     def _body(self) -> None:
         ops = self.engine.rt.ops
         rt = self.engine.rt
-        rt.no_library = True
-        rt.fused = rt.dtype == torch.bfloat16
+        # up to the weight-streaming products' limit of rows: their fused forms, no library call in the graph; beyond
+        # it the kernels of prompt steps, the library's products among them (their plans are made by the eager run
+        # that goes before every recording)
+        streaming = self.cap <= rt.streaming_rows_max
+        rt.no_library = streaming
+        rt.fused = streaming and rt.dtype == torch.bfloat16
         try:
             logits = self.engine.model.forward(self.ctx)
         finally:

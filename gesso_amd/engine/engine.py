@@ -83,11 +83,10 @@ class Engine:
         # the most requests one recorded decode step takes: as many rows as the runtime's weight-streaming products do
         # (the limit is the product kernels', asked of the runtime, not a number of the engine's own)
         self.DECODE_MAX_BATCH = self.rt.streaming_rows_max
-        # From so many requests on, decoding goes through ordinary steps of single tokens (the many-row products read
-        # every weight once for all of them) instead of through the recorded loop in groups that each read all weights.
-        # Measured at 1,000 keys a sequence, milliseconds a token for all: 128 requests 2.0 in groups against 2.2 to 2.6
-        # in one step at LFM2-350M sizes, 2.7 against 2.5 at 1.2B; 256 requests 4.0 against 3.1, and 5.5 against 3.7.
-        self.WIDE_DECODE_FROM = 2 * self.DECODE_MAX_BATCH + 1 if self.dtype == torch.bfloat16 else None
+        # More requests than that decode through a recording of the same loop in which the many-row products (the
+        # vendor's, each weight read once for all rows) and the kernels of prompt steps stand for the fused
+        # weight-streaming ones: up to this many at once (bfloat16; 0: no such loop).
+        self.DECODE_WIDE_MAX = 512 if self.dtype == torch.bfloat16 else 0
 
     def _pages_that_fit(self, layout: CacheLayout, fraction: float) -> int:
         """Pages per group that ``fraction`` of the free device memory holds (every group gets as many)."""
@@ -226,8 +225,9 @@ class Engine:
         ``bad`` marks a step whose logits were not finite.  Raises :class:`~gesso_amd.errors.OutOfPages` before changing anything.
         """
         from .decode import DecodeRunner, _capacity
-        if not 1 <= len(rids) <= self.DECODE_MAX_BATCH:
-            raise InvalidPlan(f"the recorded decode loop takes 1 to {self.DECODE_MAX_BATCH} requests, not {len(rids)}")
+        most = max(self.DECODE_MAX_BATCH, self.DECODE_WIDE_MAX)
+        if not 1 <= len(rids) <= most:
+            raise InvalidPlan(f"the recorded decode loop takes 1 to {most} requests, not {len(rids)}")
         if len(set(rids)) != len(rids) or len(tokens) != len(rids):
             raise InvalidPlan("one token per request, each request once")
         if not self.model.graph_safe:
@@ -238,18 +238,20 @@ class Engine:
             runner = self._runners[cap] = DecodeRunner(self, cap)
         return runner.run(rids, tokens, n, samplers)
 
-    def choice_scratch(self):
-        """What the recorded loop's choice needs when rows draw: float64 room for the weights of ``DECODE_MAX_BATCH``
-        rows of logits (draws from a nucleus) and for their partial sums, and the rows' maxima and flags; one set per
-        engine, made with the first recorded loop.  Returns ``(weights, (part, amax, bad0, hist))``."""
-        if getattr(self, "_choice_scratch", None) is None:
-            n, dev = self.DECODE_MAX_BATCH, self.device
-            self._choice_scratch = (
+    def choice_scratch(self, rows: int):
+        """What the recorded loop's choice needs when rows draw: float64 room for the weights of ``rows`` rows of logits
+        (draws from a nucleus) and for their partial sums, and the rows' maxima and flags; one set per engine, shared by
+        the loops of all capacities and made anew when a loop of more rows asks (the loops recorded before keep theirs).
+        Returns ``(weights, (part, amax, bad0, hist))``."""
+        held = getattr(self, "_choice_scratch", None)
+        if held is None or held[0] < rows:
+            n, dev = rows, self.device
+            self._choice_scratch = (rows, (
                 torch.empty(n * self.spec.vocab, dtype=torch.float64, device=dev),
                 (torch.empty(n * self.rt.ops.choice_parts(self.spec.vocab), dtype=torch.float64, device=dev),
                  torch.zeros(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev),
-                 torch.zeros(n * self.rt.ops.choice_hist(), dtype=torch.int64, device=dev)))
-        return self._choice_scratch
+                 torch.zeros(n * self.rt.ops.choice_hist(), dtype=torch.int64, device=dev))))
+        return self._choice_scratch[1]
 
     def _decode_eager(self, rids, tokens, n, samplers):
         """The same steps one by one through :meth:`step`, for models with parts that cannot be recorded."""

@@ -337,9 +337,8 @@ class Scheduler:
         if not all(s.count == 1 and s.samples for s in plan):
             return None
         reqs = [s.request for s in plan]
-        wide = getattr(ex, "WIDE_DECODE_FROM", None)
-        if wide is not None and len(reqs) >= wide:
-            return None               # so many that one step of single tokens beats the loop's groups one after the other
+        if len(reqs) > most:
+            most = max(most, getattr(ex, "DECODE_WIDE_MAX", 0))     # the loop for many rows, where the executor has one
         n = min(self.decode_run_steps, min(r.max_new_tokens - len(r.output) for r in reqs))
         if self.waiting:
             n = 1                     # someone waits: look at admission again after every step
