@@ -99,6 +99,53 @@ __global__ void short_conv8_kernel(const T* __restrict__ bcx, const float* __res
   }
 }
 
+// Every segment a single token, widths up to 4: a thread takes eight channels of one token; its history, its taps and
+// its B, C and X values are asked for together (the history and the taps of eight channels lie side by side), where the
+// kernel above walks them value by value behind one another.  Sums in the same order as there.
+template <typename T, int W>
+__global__ __launch_bounds__(64) void short_conv_single_kernel(const T* __restrict__ bcx, const float* __restrict__ taps,
+                                                               const float* __restrict__ bias,
+                                                               float* __restrict__ state,
+                                                               const int* __restrict__ seq_of_token,
+                                                               const int* __restrict__ slots, T* __restrict__ out,
+                                                               int ntok, int H) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (c >= H) return;
+  float tp[8 * W], bs[8];
+#pragma unroll
+  for (int q = 0; q < 2 * W; ++q)
+    *reinterpret_cast<float4*>(tp + 4 * q) = *reinterpret_cast<const float4*>(taps + (size_t)c * W + 4 * q);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) bs[i] = bias ? bias[c + i] : 0.f;
+  for (int t = blockIdx.y; t < ntok; t += gridDim.y) {
+    float* hist = state + ((size_t)slots[seq_of_token[t]] * H + c) * (W - 1);   // channel c + i at hist + i (W - 1)
+    float h[8 * (W - 1)], b8[8], x8[8], c8[8], y[8];
+#pragma unroll
+    for (int q = 0; q < 2 * (W - 1); ++q)
+      *reinterpret_cast<float4*>(h + 4 * q) = *reinterpret_cast<const float4*>(hist + 4 * q);
+    const T* row = bcx + (size_t)t * 3 * H + c;
+    load8f(row, b8);
+    load8f(row + 2 * H, x8);
+    load8f(row + H, c8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float u = b8[i] * x8[i];
+      float acc = 0.f;
+#pragma unroll
+      for (int p = 0; p < W - 1; ++p) acc += tp[i * W + p] * h[i * (W - 1) + p];
+      acc += tp[i * W + W - 1] * u;
+      y[i] = c8[i] * (bias ? acc + bs[i] : acc);
+#pragma unroll
+      for (int p = 0; p < W - 2; ++p) h[i * (W - 1) + p] = h[i * (W - 1) + p + 1];
+      h[i * (W - 1) + W - 2] = u;
+    }
+    store8f(out + (size_t)t * H + c, y);
+#pragma unroll
+    for (int q = 0; q < 2 * (W - 1); ++q)
+      *reinterpret_cast<float4*>(hist + 4 * q) = *reinterpret_cast<const float4*>(h + 4 * q);
+  }
+}
+
 // Prompt portions: a thread takes eight channels and a run of TT consecutive tokens (4 or 2, see the launch), so every B and X row is read
 // once (plus W - 1 rows of run-in), all loads of the run are issued before anything is computed, and the products
 // u = B x stay in registers for the W tokens that use them.  Sums run over the taps in the same order as in the
@@ -222,6 +269,17 @@ extern "C" int gs_short_conv(const void* bcx, int dtype, const float* taps, cons
     }
 #undef GS_RUN_CONV
 #undef GS_RUN_CONV_T
+  } else if (vec && all_single && W <= 4 && (((uintptr_t)taps | (uintptr_t)state) & 15) == 0) {
+    dim3 gs(gs_ceil_div(H / 8, 64), grid.y);
+#define GS_RUN_SINGLE(TY, WW)                                                                                          \
+  short_conv_single_kernel<TY, WW><<<gs, 64, 0, stream>>>((const TY*)bcx, taps, bias, state, seq_of_token, slots,      \
+                                                          (TY*)out, ntok, H)
+    if (dtype == GS_F32) {
+      if (W == 2) GS_RUN_SINGLE(float, 2); else if (W == 3) GS_RUN_SINGLE(float, 3); else GS_RUN_SINGLE(float, 4);
+    } else {
+      if (W == 2) GS_RUN_SINGLE(bf16, 2); else if (W == 3) GS_RUN_SINGLE(bf16, 3); else GS_RUN_SINGLE(bf16, 4);
+    }
+#undef GS_RUN_SINGLE
   } else if (vec) {
     int th = H / 8 >= 256 ? 256 : 64;
     dim3 g8(gs_ceil_div(H / 8, th), grid.y);

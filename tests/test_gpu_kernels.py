@@ -168,6 +168,37 @@ def test_short_conv_segments_and_history(ops, H, W, bias, dtype):
     assert torch.equal(state[1].cpu(), torch.full((H, W - 1), 7.0)) and torch.equal(state[4].cpu(), torch.full((H, W - 1), 7.0))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("W", [2, 3, 4, 5])
+@pytest.mark.parametrize("H", [8, 136, 2048])
+def test_short_conv_of_single_tokens_step_after_step(ops, H, W, bias, dtype):
+    """Every sequence brings one token a step (the kernel that asks for a thread's history, taps and values together, for
+    widths up to 4; width 5 goes the general way): 70 sequences in slots of their own order, six steps from an empty
+    history, against the convolution of the whole sequences; slots of no sequence stay as they were."""
+    g = gen(100 * H + 10 * W + bias)
+    nseq, steps = 70, 6
+    taps = torch.randn(H, W, generator=g)
+    b = torch.randn(H, generator=g) if bias else None
+    data = torch.randn(nseq, steps, 3 * H, generator=g).to(dtype)
+    want = [P.short_conv(data[i].double(), taps.double(), None if b is None else b.double()) for i in range(nseq)]
+    slots_h = torch.randperm(nseq + 3, generator=g)[:nseq].to(torch.int32)
+    state = torch.full((nseq + 3, H, W - 1), 7.0, device=DEV)
+    ops.fill_rows(state, slots_h.to(DEV), 0.0)
+    seq_of = torch.arange(nseq, dtype=torch.int32, device=DEV)
+    q_start = torch.arange(nseq + 1, dtype=torch.int32, device=DEV)
+    got = []
+    for s in range(steps):
+        got.append(ops.short_conv(data[:, s].contiguous().to(DEV), taps.to(DEV), None if b is None else b.to(DEV), state,
+                                  seq_of, q_start, slots_h.to(DEV), nseq, True).cpu())
+    got = torch.stack(got, 1)                                 # (nseq, steps, H)
+    for i in range(nseq):
+        close(got[i], want[i][0], dtype)
+        close(state[int(slots_h[i])], want[i][1], torch.float32)
+    idle = sorted(set(range(nseq + 3)) - set(slots_h.tolist()))
+    assert all(torch.equal(state[j].cpu(), torch.full((H, W - 1), 7.0)) for j in idle)
+
+
 @pytest.mark.parametrize("H,n", [(136, [37, 1, 2, 19, 8, 3]), (4096, [500, 1, 2, 333, 3, 190])])
 @pytest.mark.parametrize("W", [2, 3, 4])
 def test_short_conv_long_portions_beside_short_ones(ops, W, H, n):
