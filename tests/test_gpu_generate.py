@@ -126,6 +126,11 @@ def test_a_hundred_and_fifty_requests_at_once_decode_through_the_loop_for_many_r
             assert supported(ref[j - 1], g[j], slack), (i, j, g[j], slack)
     st = s.engine.manager.stats()
     assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+    # every row drawing from a nucleus, on the device: one seed gives the same ids again, other ids than the greedy ones
+    from gesso_amd import Sampler
+    drawn = [s.generate(prompts, max_new_tokens=5, eos_ids=(), sampler=Sampler(0.9, 0.8, seed=11)) for _ in range(2)]
+    assert drawn[0] == drawn[1]
+    assert sum(a[len(p):len(p) + 5] != b[len(p):len(p) + 5] for a, b, p in zip(drawn[0], got, prompts)) > n // 2
 
 
 def test_temperature_sampling_follows_the_plain_sampler(plain):
