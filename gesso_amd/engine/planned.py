@@ -236,7 +236,7 @@ class StepRecorder:
     """Which steps an engine records, and the recordings it holds.
 
     A step is recorded when it is the fourth of its kind: steps of one kind share the token count, the room their
-    longest sequence needs in a block table (a power of two of keys) and the blocks' key.  The first ones, run launch
+    longest sequence needs in a block table (a power of two of keys), the blocks' key and the room for sequences.  The first ones, run launch
     by launch, have made the plans of the library's products, which a recording cannot make, and a kind that comes
     once in a while (the last, shorter step of a wave of prompts) is not worth the four milliseconds of a recording."""
 
@@ -244,7 +244,8 @@ class StepRecorder:
     MAX_RECORDINGS = 4           # each holds the activations of its token count
     MAX_SEEN = 4096              # kinds whose comings are counted
     IDLE_STEPS = 256             # a recording unused for so many steps makes room when another kind wants it
-    SEQ_CAP = 64                 # sequences in a recorded step with prompt portions
+    SEQ_CAP = 64                 # sequences in a recorded step with prompt portions: room for so many, or twice, ...
+    MAX_SEQ_CAP = 512            # ... up to so many
     MAX_SINGLE = 1024            # sequences in a recorded step of single tokens
     MIN_KV_CAP = 4096
 
@@ -265,7 +266,7 @@ class StepRecorder:
             # than that are one step of library products, which is worth recording
             if not getattr(eng, "DECODE_MAX_BATCH", 0) < len(entries) <= self.MAX_SINGLE:
                 return None
-        elif len(entries) > self.SEQ_CAP:
+        elif len(entries) > self.MAX_SEQ_CAP:
             return None
         longest = max(eng.manager.get(e.rid).length + n for e, n in zip(entries, lens))
         key = eng.model.replay_key(lens, longest)
@@ -274,7 +275,13 @@ class StepRecorder:
         kv_cap = self.MIN_KV_CAP
         while kv_cap < longest:
             kv_cap *= 2
-        return sum(lens), kv_cap, key
+        # room for the step's sequences: as many as it has where every one brings a single token, else 64, 128, ...
+        seq_cap = len(entries)
+        if max(lens) > 1:
+            seq_cap = self.SEQ_CAP
+            while seq_cap < len(entries):
+                seq_cap *= 2
+        return sum(lens), kv_cap, key, seq_cap
 
     def recording_for(self, entries: Sequence[StepEntry]) -> Optional[RecordedStep]:
         """The recording that takes this step, made now if the step is the fourth of its kind; None: launch by launch."""
@@ -298,9 +305,8 @@ class StepRecorder:
                     return None
                 del self.recordings[oldest], self.used[oldest]
                 self.seen.pop(oldest, None)
-            T, kv_cap, key = kind
-            single = max(len(e.tokens) for e in entries) == 1
-            rec = RecordedStep(self.engine, T, T if single else self.SEQ_CAP, kv_cap, key, single)
+            T, kv_cap, key, seq_cap = kind
+            rec = RecordedStep(self.engine, T, seq_cap, kv_cap, key, single=max(len(e.tokens) for e in entries) == 1)
             try:
                 rec.record()
             except GessoError as err:

@@ -300,3 +300,21 @@ def test_recorded_steps_of_more_single_tokens_than_the_decode_loop_takes(tmp_pat
     (kind, step_), = [(k, r) for k, r in rec.recordings.items() if r is not None]
     assert step_.single and kind[0] == n and rec.replays == 14 - rec.SEEN_BEFORE
     plain.manager.check(); recorded.manager.check()
+
+
+def test_recorded_steps_with_more_sequences_than_sixty_four(tmp_path):
+    """A hundred live requests: steps of 230 tokens hold some eighty decoded tokens beside portions; their recording has
+    room for 128 sequences, and the logits are the launched steps'."""
+    folder = str(tmp_path / "E")
+    write_model_folder(folder, WIDE_E, 16, torch.bfloat16, std=STD)
+    live = 100
+    plain, recorded = engines(folder, page_size=16, max_tokens=live * 256, num_slots=live + 1)
+    rng = random.Random(4)
+    work = Workload(WIDE_E.vocab_size, 230, seed=4, prompt_lens=[rng.randint(20, 150) for _ in range(400)],
+                    new_tokens=(50, 80), live=live)
+    kinds = {}
+    run_both(plain, recorded, work, 80, kinds)
+    rec = recorded.recorder
+    made = [k for k, r in rec.recordings.items() if r is not None]
+    assert any(k[3] == 128 for k in made), (made, kinds)
+    assert rec.replays == replays_expected(kinds, rec) and rec.replays >= 10, (rec.replays, kinds)

@@ -55,7 +55,7 @@ def test_steps_that_are_never_recorded(recorder):
     for _ in range(6):
         assert recorder.recording_for(step(1, 1, 1)) is None                       # decoded tokens only
         assert recorder.recording_for(step(1, 30, 40)) is None                     # the model says no (short portions)
-        assert recorder.recording_for(step(*([1] * recorder.SEQ_CAP + [80]))) is None      # more sequences than a recording holds
+        assert recorder.recording_for(step(*([1] * recorder.MAX_SEQ_CAP + [80]))) is None  # more sequences than a recording holds
     assert Recording.made == [] and recorder.seen == {}
 
 
@@ -71,6 +71,10 @@ def test_single_tokens_are_recorded_when_there_are_more_than_the_decode_loop_tak
     for _ in range(4):
         other = recorder.recording_for(step(*[1] * 30, 170))
     assert not other.single and other.seq_cap == recorder.SEQ_CAP and other.T == 200
+    # more sequences than that beside a portion: room for twice as many, a kind of its own
+    for _ in range(4):
+        more = recorder.recording_for(step(*[1] * 100, 100))
+    assert more is not other and more.seq_cap == 128 and more.T == 200
 
 
 def test_room_for_keys_and_the_walk_make_kinds_of_their_own(recorder):
@@ -119,4 +123,4 @@ def test_the_tally_of_kinds_starts_over_when_it_is_full(recorder):
         recorder.recording_for(step(T))
     assert len(recorder.seen) == 5
     recorder.recording_for(step(105))
-    assert list(recorder.seen) == [(105, 4096, (2,))]
+    assert list(recorder.seen) == [(105, 4096, (2,), 64)]
