@@ -32,7 +32,7 @@ class RuntimeOptions:
     vendor's for bfloat16 results (measured on random data at 2,048 rows: 109 us against our 161 for gate|up, 124
     against 162 with the SwiGLU pass counted in; 50 against 75 for 6144 x 2048), ours where the result is float32 and
     inside a recorded graph.
-    ``tune_library``: where the vendor library computes a product of 512, 1024, 2048, ... rows (whole prompt portions),
+    ``tune_library``: where the vendor library computes a product of 128, 256, 512, 1024, ... rows (whole prompt portions, the decode loop for many rows),
     the first product of a shape measures the library's two dozen best guesses on the operands at hand, cold, and
     keeps the library's first choice unless another is clearly faster (some ten milliseconds a shape).  Other row
     counts, and all with this off, take the library's first choice.  Off unless asked for: which candidate a
@@ -205,7 +205,7 @@ class Runtime:
             # 512 on): a measurement takes some ten milliseconds a shape, and a server's steps bring ever new row counts
             M = x.shape[0]
             return ops.library_gemm(x, w, self._library_ws, out=out,
-                                    tune=self.tune_library and M >= 512 and M & (M - 1) == 0, checked=True)
+                                    tune=self.tune_library and M >= 128 and M & (M - 1) == 0, checked=True)
         return torch.mm(x, w.t(), out=out) if out is not None else torch.mm(x, w.t())
 
     def linear_swiglu(self, x, w13: torch.Tensor) -> torch.Tensor:
