@@ -31,7 +31,7 @@ class RuntimeOptions:
     everywhere (gate|up with SwiGLU in one kernel), ``"library"`` = the vendor's wherever it can go, ``"auto"`` = the
     vendor's for bfloat16 results (measured on random data at 2,048 rows: 109 us against our 161 for gate|up, 124
     against 162 with the SwiGLU pass counted in; 50 against 75 for 6144 x 2048), ours where the result is float32 and
-    inside a recorded graph.
+    inside the recording of the fused decode loop.
     ``tune_library``: where the vendor library computes a product of 128, 256, 512, 1024, ... rows (whole prompt portions, the decode loop for many rows),
     the first product of a shape measures the library's two dozen best guesses on the operands at hand, cold, and
     keeps the library's first choice unless another is clearly faster (some ten milliseconds a shape).  Other row
