@@ -552,8 +552,11 @@ def test_toy_parts_register_build_and_step(fw, dtype):
         table = tensor_table(spec)
         assert "L0.proj.weight" in table and "L2.w1" not in table and "L1.e2.down.weight" in table and "L1.w1" not in table
         cpu = random_tensors(table, 17, dtype, std=0.2)          # a seed whose routing choices are clear of ties
+        from gesso_amd.parts import RuntimeOptions
         eng = Engine(spec, {k: v.to(DEV, held_dtype(v.dtype, table[k].role, dtype)) for k, v in cpu.items()}, dtype,
-                     DEV, page_size=4, num_pages=24, num_slots=3)
+                     DEV, page_size=4, num_pages=24, num_slots=3, options=RuntimeOptions(record_portions=True))
+        # parts that say nothing about recorded steps are never recorded, whatever the options ask for
+        assert eng.recorder is None and not eng.model.portions_recordable
         lay = eng.manager.layout
         assert len(lay.paged) == 1 and lay.paged[0].members == (1,) and [m.call for m in lay.slots] == [0, 2]
         assert lay.source_of_call[3] == 1
