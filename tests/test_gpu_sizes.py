@@ -208,13 +208,15 @@ def test_replay_at_the_layer_sizes_of_the_other_benchmarked_models(others, size,
 
 
 @pytest.mark.parametrize("size,nreq,steps", [("1.2B", 3, 3), ("1.2B", 20, 2), ("1.2B", 40, 2), ("1.2B", 1, 3), ("1.2B", 8, 2),
-                                             ("1.2B", 64, 2), ("350M", 8, 2), ("350M", 64, 2), ("2.6B", 40, 2)])
+                                             ("1.2B", 64, 2), ("350M", 8, 2), ("350M", 64, 2), ("2.6B", 40, 2),
+                                             ("1.2B", 100, 2), ("350M", 130, 1)])
 def test_recorded_decode_at_the_real_layer_sizes(balanced, others, size, nreq, steps):
     """The fused kernels of the recorded decode step, each row's logits against the plain implementation: at 3, 20 and
     40 rows (pre-weighted rows; more than sixteen; products in parts of K) and at the batches the benchmark times, 1, 8
     and 64 rows (capacities 1, 8 and 64 of the recording: one row tile, and four with the register ring), at the layer
     sizes of LFM2-1.2B; at 8 and 64 rows with LFM2-350M's (groups of two in decode attention, products over 4,608), at
-    40 with LFM2-2.6B's (over 7,168)."""
+    40 with LFM2-2.6B's (over 7,168).  And the loop for more than 64 rows, whose products are the library's: 100 rows
+    (a capacity of 128) at LFM2-1.2B's sizes, 130 (of 256) at LFM2-350M's."""
     from gesso_amd import Engine, StepEntry
     from gesso_amd.engine.decode import _capacity
     m = balanced if size == "1.2B" else others(size)
