@@ -79,7 +79,9 @@ __global__ __launch_bounds__(G * WQ * 64) void attention_prefill_wide_kernel(
   __shared__ __align__(16) uint16_t vt[KS][2][D][VROW];
   __shared__ __align__(8) uint32_t rowoff[KS][3][PW_KS];   // (read two at a time) where a step's key rows start in the caches, in units of 16 bytes
 
-  // blocks in launch order: key head fastest, tiles from the last one back (late tiles walk the most keys)
+  // blocks in launch order: key head fastest, tiles from the last one back (late tiles walk the most keys).  Blocks go to
+  // the eight XCDs in turn, so with 1, 2, 4 or 8 key heads all blocks of one key head run on the same XCDs and meet their
+  // keys and values in those XCDs' L2 (block b: key head b % nkv, XCD b % 8)
   const int kvh = blockIdx.x % nkv, tile = (int)(gridDim.x / nkv) - 1 - (int)(blockIdx.x / nkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hf = lane >> 5;

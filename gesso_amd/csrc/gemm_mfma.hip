@@ -40,9 +40,22 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mfma_kernel(const bf16* __r
   const int wm = wave / WN, wn = wave % WN;
   const int l32 = lane & 31, kh = lane >> 5;
   const int F = N >> 1;                                    // EPI 1: output width
-  // consecutive blocks walk down M first: they share their rows of W through L2
+  // Blocks are handed to the eight XCDs in turn (block b runs on XCD b % 8), each with an L2 of its own.  A run of
+  // consecutive tile numbers goes to one XCD, and tile numbers walk the output in bands of four row tiles, column by
+  // column: the tiles in an XCD's L2 at one time then share few rows of X and few rows of W.
   const int tiles_m = (M + BM - 1) / BM;
-  const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+  int bm, bn;
+  {
+    const int nb = (int)gridDim.x, per = nb / 8, rem = nb % 8;
+    const int xcd = (int)blockIdx.x % 8, turn = (int)blockIdx.x / 8;
+    const int t = xcd * per + (xcd < rem ? xcd : rem) + turn;        // XCD x owns per (+ 1) consecutive numbers
+    const int tiles_n = nb / tiles_m;
+    constexpr int BAND = 4;
+    const int band = t / (BAND * tiles_n), in_band = t - band * BAND * tiles_n;
+    const int rows = tiles_m - band * BAND < BAND ? tiles_m - band * BAND : BAND;   // the last band may be narrower
+    bm = band * BAND + in_band % rows;
+    bn = in_band / rows;
+  }
   const int m0 = bm * BM;
   const int n0 = EPI == 1 ? bn * (BN / 2) : bn * BN;       // first output column of the block
 
