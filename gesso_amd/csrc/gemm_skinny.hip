@@ -100,6 +100,7 @@ extern "C" int gs_gemm_skinny_parts(const void* X, int ldx, int x_tiled, const v
                                     int M, int N, int K, hipStream_t stream) {
   if (check_common(W, M, N, K) || check_tiles(Wt, N, K, 16) || check_rows(X, ldx, x_tiled, K)) return -1;
   GS_REQUIRE(part && parts >= 1 && parts <= 64 && ((uintptr_t)part & 15) == 0, "gemm_skinny_parts: 1 to 64 parts and an aligned buffer");
+  GS_REQUIRE(N <= 65535 * 32, "gemm_skinny_parts: %d weight rows are more than a launch takes", N);
   if (M == 0) return 0;
   gs_skinny_run_parts(X, ldx, x_tiled, W, Wt, part, parts, M, N, K, stream);
   GS_LAUNCH_CHECK("gemm_skinny_parts");

@@ -36,7 +36,7 @@
 // What is done with Y (EPI):
 //   0  stored (bfloat16 or float32).
 //   1  SwiGLU: W holds gate rows [0, N/2) then up rows; stores silu(gate) * up, N/2 wide.
-//   5  partial sums: K is shared out over gridDim.y blocks as well, each writes its float32 (M, N) sheet; a second
+//   5  partial sums: K is shared out over gridDim.x blocks as well (the weight tiles over gridDim.y), each writes its float32 (M, N) sheet; a second
 //      kernel adds the sheets.  For many rows: every block reads all rows of X for its part of K, so the fewer
 //      weight rows and the more of K a block takes, the more X traffic; sharing K over blocks caps it.
 //   2  added to the residual stream in place (float32), and the sums of squares of the new rows over this
@@ -129,7 +129,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16* __r
   } else if (SHUF == 2) {
     rowbase[0] = blockIdx.x * 8;  // half a tile: twice the blocks for a weight of few rows
   } else {
-    const int n0 = blockIdx.x * 16 * R;
+    // (EPI 5: the grid is (parts of K, weight tiles), see below)
+    const int n0 = (EPI == 5 ? blockIdx.y : blockIdx.x) * 16 * R;
 #pragma unroll
     for (int r = 0; r < R; ++r) rowbase[r] = n0 + r * 16;
   }
@@ -337,12 +338,14 @@ _Pragma("unroll")                                                               
   };
 
   // this wavefront's share of K, in steps of 32
-  // (EPI 5: the blocks of one column of the grid share K among themselves first, blockIdx.y taking its part)
+  // (EPI 5: the blocks that own the same weight rows share K among themselves first, blockIdx.x taking its part.  The part
+  // runs fastest in launch order and blocks go to the eight XCDs in turn, so with eight parts every XCD works on one
+  // part of K and holds that part of X alone in its L2; with four, two XCDs a part.)
   const int ksteps_all = (K + 31) >> 5;
   int kbeg = 0, kend = ksteps_all;
   if (EPI == 5) {
-    const int part = (ksteps_all + (int)gridDim.y - 1) / (int)gridDim.y;
-    kbeg = blockIdx.y * part;
+    const int part = (ksteps_all + (int)gridDim.x - 1) / (int)gridDim.x;
+    kbeg = blockIdx.x * part;
     kend = kbeg + part < ksteps_all ? kbeg + part : ksteps_all;
     if (kend < kbeg) kend = kbeg;
   }
@@ -540,7 +543,7 @@ _Pragma("unroll")                                                               
     const bool live = m < M;
     if (EPI == 0 || EPI == 5) {
       if (!live) continue;
-      TOut* Yp = EPI == 5 ? Y + (size_t)blockIdx.y * M * ldy : Y;   // partial sums: one (M, N) sheet per part of K
+      TOut* Yp = EPI == 5 ? Y + (size_t)blockIdx.x * M * ldy : Y;   // partial sums: one (M, N) sheet per part of K
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int n = rowbase[r] + kg * 4;
@@ -633,7 +636,7 @@ static void launch_skinny_parts(int blocks, int parts, const bf16* X, int ldx, c
                                 int K, const SkinnyExtra& ex, hipStream_t stream) {
   const size_t lds = (size_t)(WAVES - 1) * R * MT * 256 * sizeof(float);
   gemm_skinny_kernel<R, MT, WAVES, 0, 5, SHUF, float>
-      <<<dim3(blocks, parts), WAVES * 64, lds, stream>>>(X, ldx, W, Y, N, M, N, K, ex);
+      <<<dim3(parts, blocks), WAVES * 64, lds, stream>>>(X, ldx, W, Y, N, M, N, K, ex);
 }
 
 // MT from M; the wavefronts per block are given per MT so that the LDS for the partial tiles,
