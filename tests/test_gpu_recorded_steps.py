@@ -244,9 +244,9 @@ def test_a_recording_that_lies_idle_makes_room_for_another_kind(tmp_path):
     rec = recorded.recorder
     rec.MAX_RECORDINGS, rec.IDLE_STEPS = 1, 5
     held = []
-    for round_, T in enumerate((96, 80, 96)):
-        rng = random.Random(T + round_)
-        work = Workload(WIDE_D.vocab_size, T, seed=T + round_, prompt_lens=[rng.randint(70, 400) for _ in range(12)], tag=round_)
+    for turn, T in enumerate((96, 80, 96)):
+        rng = random.Random(T + turn)
+        work = Workload(WIDE_D.vocab_size, T, seed=T + turn, prompt_lens=[rng.randint(70, 400) for _ in range(12)], tag=turn)
         before = rec.replays
         run_both(plain, recorded, work, 16, {})
         assert not rec.refused, rec.refused
@@ -254,7 +254,7 @@ def test_a_recording_that_lies_idle_makes_room_for_another_kind(tmp_path):
         assert len(made) == 1 and made[0][0] == T, (T, made)
         assert rec.replays - before >= 4, (T, rec.replays - before)
         held.append(made[0])
-        for rid in list(work.live):             # what this round left unfinished
+        for rid in list(work.live):             # what this turn left unfinished
             plain.finish_request(rid); recorded.finish_request(rid)
     assert held[0] == held[2] != held[1]
 
