@@ -48,6 +48,7 @@ class RecordedStep:
     """One recording: ``T`` tokens in up to ``seq_cap`` sequences of up to ``kv_cap`` keys, the blocks' ``key``."""
 
     TILE_ROOM = 1 << 16          # int32 entries for the tile lists that parts ask for
+    HOST_COPIES = 4              # pinned buffers the steps are filled into in turn
 
     def __init__(self, engine, T: int, seq_cap: int, kv_cap: int, key, single: bool = False):
         """``single``: a step of ``T`` sequences that bring one token each (then ``seq_cap`` is ``T``)."""
@@ -63,9 +64,16 @@ class RecordedStep:
             self.layout[name] = (at, n)
             at += n
         self._used = at
-        self.host = torch.zeros(at + self.TILE_ROOM, dtype=torch.int32).pin_memory()
+        # The host's side in several copies taken in turn: a step's copy to the device runs when the device gets to it,
+        # which may be after the host has filled in the next step (a step that wants no logits makes the host wait for
+        # nothing), so a buffer is written again only when the copy it was last the source of has been made.
+        self.hosts = [torch.zeros(at + self.TILE_ROOM, dtype=torch.int32).pin_memory() for _ in range(self.HOST_COPIES)]
+        self.copied = [None] * self.HOST_COPIES          # the event after each buffer's last copy
+        self.turn = 0
+        self.nps = [h.numpy() for h in self.hosts]
+        self.host = self.hosts[0]
         self.dev = torch.zeros(at + self.TILE_ROOM, dtype=torch.int32, device=engine.device)
-        self.np = self.host.numpy()
+        self.np = self.nps[0]
         t = self.field("tables").view(self.groups, seq_cap, self.max_blocks)
         self.tables = [t[g] for g in range(self.groups)]
         self.tile_lists: Dict = {}           # what parts asked for: kind -> (offset, entries, maker)
@@ -173,6 +181,10 @@ class RecordedStep:
         ctx._tiles = None
         if sum(len(e.want) for e in entries) > T:
             return None                                       # (rows wanted more than once: more than the buffer holds)
+        self.turn = (self.turn + 1) % self.HOST_COPIES
+        if self.copied[self.turn] is not None:
+            self.copied[self.turn].synchronize()              # (the copy of HOST_COPIES steps ago: long done, as a rule)
+        self.host, self.np = self.hosts[self.turn], self.nps[self.turn]
         made = []
         for at, cnt, maker in self.tile_lists.values():
             lists = maker(ctx)
@@ -220,6 +232,8 @@ class RecordedStep:
     def launch(self, n_want: int) -> Optional[torch.Tensor]:
         """The filled step: one copy, the graphs and calls in order, then the final norm and the head of the wanted rows."""
         self.dev.copy_(self.host, non_blocking=True)
+        done = self.copied[self.turn] = self.copied[self.turn] or torch.cuda.Event()
+        done.record()
         ctx = self.ctx
         for item in self.items:
             if isinstance(item, torch.cuda.CUDAGraph):

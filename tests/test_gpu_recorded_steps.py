@@ -318,3 +318,35 @@ def test_recorded_steps_with_more_sequences_than_sixty_four(tmp_path):
     made = [k for k, r in rec.recordings.items() if r is not None]
     assert any(k[3] == 128 for k in made), (made, kinds)
     assert rec.replays == replays_expected(kinds, rec) and rec.replays >= 10, (rec.replays, kinds)
+
+
+def test_steps_that_want_nothing_follow_each_other_while_the_device_lags(tmp_path):
+    """Portions in the middle of a prompt want no logits, so the host waits for nothing and fills in the next step while the
+    device has not begun the last one: each step's indices must still be its own when the device copies them.  A long
+    product keeps the device busy; twelve steps of 192 tokens are queued behind it without a wait, the last wants its
+    logits; they are the launched steps' (with the pages of earlier requests poisoned in between)."""
+    from gesso_amd import StepEntry
+
+    folder = str(tmp_path / "E")
+    write_model_folder(folder, WIDE_E, 17, torch.bfloat16, std=STD)
+    plain, recorded = engines(folder, page_size=16, max_tokens=3 * 1280, num_slots=4)
+    busy = torch.randn(8192, 8192, device="cuda:0")
+    for turn in range(3):
+        prompts = {(turn, i): random_ids(12 * 64, WIDE_E.vocab_size, 50 * turn + i) for i in range(3)}
+        got = []
+        for eng in (plain, recorded):
+            for rid in prompts:
+                eng.add_request(rid)
+            torch.cuda.synchronize()
+            if eng is recorded:
+                for _ in range(40):
+                    busy @ busy                           # some tens of milliseconds of work before the steps' first kernel
+            for s in range(12):
+                last = s == 11
+                out = eng.step([StepEntry(rid, p[64 * s:64 * s + 64], [63] if last else []) for rid, p in prompts.items()])
+                assert (out is not None) == last
+            got.append(out)
+            for rid in prompts:
+                eng.finish_request(rid)
+        assert torch.isfinite(got[0]).all() and torch.equal(got[0], got[1]), (turn, (got[0] - got[1]).abs().max().item())
+    assert recorded.recorder.replays >= 3 * 12 - recorded.recorder.SEEN_BEFORE and not recorded.recorder.refused
