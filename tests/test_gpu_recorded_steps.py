@@ -350,3 +350,29 @@ def test_steps_that_want_nothing_follow_each_other_while_the_device_lags(tmp_pat
                 eng.finish_request(rid)
         assert torch.isfinite(got[0]).all() and torch.equal(got[0], got[1]), (turn, (got[0] - got[1]).abs().max().item())
     assert recorded.recorder.replays >= 3 * 12 - recorded.recorder.SEEN_BEFORE and not recorded.recorder.refused
+
+
+def test_the_scheduler_short_of_pages_over_recorded_steps(tmp_path):
+    """Six long prompts in portions of 64 under a budget of 128 tokens, with so few pages that requests are preempted
+    dozens of times and their pages poisoned: many steps hold portions only and want no logits.  The ids are the
+    launched steps' ids (this is the case that showed a step's indices overwritten before the device had copied them)."""
+    from gesso_amd import Session
+    from gesso_amd.parts import RuntimeOptions
+
+    folder = str(tmp_path / "E")
+    write_model_folder(folder, WIDE_E, 5, torch.bfloat16, std=STD)
+    lens = [462, 477, 464, 365, 499, 214]
+    prompts = [random_ids(n, WIDE_E.vocab_size, 12900 + i) for i, n in enumerate(lens)]
+    out = []
+    for on in (False, True):
+        s = Session(folder, dtype="bfloat16", context_length=640, num_pages=66, page_size=16, chunk_size=64, max_num_seqs=7,
+                    max_num_batched_tokens=128, watermark=0.0, poison=True,
+                    kernel_options=RuntimeOptions(record_portions=on, prompt_attention="wide"))
+        out.append(s.generate(prompts, max_new_tokens=18, eos_ids=()))
+        assert s.last_stats["preemptions"] >= 10
+        if on:
+            assert s.last_stats["replayed_steps"] >= 30 and not s.engine.recorder.refused
+        st = s.engine.manager.stats()
+        assert st["pages_free"] == st["pages_total"] and st["slots_free"] == st["slots_total"]
+        s.close()
+    assert out[0] == out[1]
