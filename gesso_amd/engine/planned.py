@@ -317,6 +317,9 @@ class StepRecorder:
                 oldest = min(held, key=lambda k: self.used[k])
                 if self.clock - self.used[oldest] < self.IDLE_STEPS:
                     return None
+                device = getattr(self.engine, "device", None)
+                if device is not None and device.type == "cuda":
+                    torch.cuda.synchronize(device)             # (its last replay may still be running: graphs go when idle)
                 del self.recordings[oldest], self.used[oldest]
                 self.seen.pop(oldest, None)
             T, kv_cap, key, seq_cap = kind
