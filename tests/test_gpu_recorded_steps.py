@@ -233,6 +233,33 @@ def test_recorded_steps_over_two_page_groups_one_of_them_windowed(tmp_path):
     rec = recorded.recorder
     assert rec.replays == replays_expected(kinds, rec) and rec.replays >= 20, (rec.replays, kinds)
     plain.manager.check(); recorded.manager.check()
+    # Seventy requests of this model through the decode loop for many rows (a capacity of 128; the windowed group gives
+    # pages back on the way, poisoned) against the same tokens as ordinary steps of seventy single tokens: the same
+    # kernels but for the final norm's laziness, so the logits agree to the last bits and the tokens are the same.
+    from gesso_amd import StepEntry
+    from gesso_amd.engine.decode import _capacity
+    for eng in made:
+        for rid in list(eng.manager.requests):
+            eng.finish_request(rid)
+    n = 70
+    wide = Engine(spec, tensors, torch.bfloat16, dev, page_size=4, max_tokens=n * 96, num_slots=n + 1, poison=True)
+    steps = Engine(spec, tensors, torch.bfloat16, dev, page_size=4, max_tokens=n * 96, num_slots=n + 1, poison=True)
+    toks = []
+    for i in range(n):
+        prompt = random_ids(3 + (7 * i) % 50, V, 600 + i)
+        for eng in (wide, steps):
+            eng.add_request(i)
+            first = eng.step([StepEntry(i, prompt, [len(prompt) - 1])])
+        toks.append(int(first.argmax()))
+    for s in range(12):
+        a = steps.step([StepEntry(i, [t], [0]) for i, t in enumerate(toks)])
+        ids, bad = wide.decode(list(range(n)), toks, 1)
+        b = wide._runners[_capacity(n)].logits[:n]
+        assert not bad.any() and torch.isfinite(a).all()
+        assert float((a - b).abs().max()) <= 2e-2 * float(a.abs().max()), (s, float((a - b).abs().max()), float(a.abs().max()))
+        toks = ids[0].tolist()
+        assert sum(int(x) != y for x, y in zip(a.argmax(1).tolist(), toks)) <= 1, s
+    assert _capacity(n) == 128 and len(wide.manager.get(0).tables) == 2
 
 
 def test_a_recording_that_lies_idle_makes_room_for_another_kind(tmp_path):
