@@ -350,3 +350,38 @@ def test_pages_beyond_four_giga_elements_of_a_layers_cache(dtype, tmp_path):
     for i, (x, y) in enumerate(zip(a, b)):
         assert torch.isfinite(x.float()).all(), i
         assert torch.equal(x.cpu(), y.cpu()), (i, (x.float().cpu() - y.float().cpu()).abs().max().item())
+
+
+@pytest.mark.gpu
+def test_recorded_steps_at_the_real_layer_sizes_replay_what_was_launched(tmp_path):
+    """At LFM2-1.2B's layer sizes the library takes other kernels for its products than at tiny sizes (work shared out
+    over K among them).  A prompt of 2,048 tokens and steps of 1,024 tokens in portions, recorded and replayed eight times
+    each with launched steps of other shapes between the replays: every replay's logits are, bit for bit, those of an
+    engine that launches the same steps."""
+    from gesso_amd import Engine, StepEntry
+    from gesso_amd.parts import RuntimeOptions
+
+    d = write_real_size_folder(str(tmp_path / "m"), 25.0, "1.2B")
+    kw = dict(dtype="bfloat16", page_size=16, max_tokens=6 * 2304, num_slots=7, poison=True)
+    launched = Engine.from_folder(d, **kw)
+    replayed = Engine.from_folder(d, options=RuntimeOptions(record_portions=True), **kw)
+    whole = [random_ids(2048, 65536, 30 + i) for i in range(12)]
+    parts = [random_ids(1500, 65536, 60 + i) for i in range(4)]
+    for turn in range(12):
+        outs = []
+        for eng in (launched, replayed):
+            eng.add_request(("w", turn))
+            a = eng.step([StepEntry(("w", turn), whole[turn], [2047, 5])])
+            # steps of 1,024 tokens: two portions of 500 and one of 24; then a launched step of another shape
+            for i in range(3):
+                eng.add_request(("p", turn, i))
+            b = eng.step([StepEntry(("p", turn, 0), parts[turn % 4][:500], [499]), StepEntry(("p", turn, 1), parts[(turn + 1) % 4][:500], []),
+                          StepEntry(("p", turn, 2), parts[(turn + 2) % 4][:24], [23])])
+            c = eng.step([StepEntry(("p", turn, 0), parts[turn % 4][500:500 + 70 + turn], [69 + turn])])
+            outs.append((a, b, c))
+            for rid in [("w", turn)] + [("p", turn, i) for i in range(3)]:
+                eng.finish_request(rid)
+        for x, y in zip(*outs):
+            assert torch.isfinite(x).all() and torch.equal(x, y), (turn, (x - y).abs().max().item())
+    rec = replayed.recorder
+    assert not rec.refused and rec.replays == 2 * (12 - rec.SEEN_BEFORE), (rec.replays, rec.refused)
