@@ -11,6 +11,9 @@ whose number changes), made anew at every replay.  The final norm and the head, 
 are wanted, follow as ordinary launches.  The reference has no counterpart: it runs one sequence per pass
 (``src/Inference/Inference.jl:2272-2530``).
 
+A step of many sequences that bring one token each (more than the recorded decode loop takes) is recorded the same
+way: its kind is the number of sequences, and nothing in it is left to a call.
+
 Sequences beyond the step's own (the buffers hold ``seq_cap``) are empty: they start at the token count and own
 the scratch slot and the scratch page.  Nothing in a graph clears memory with a memset node.  The kernels of a
 replay are those of the same step run launch by launch, with the same arguments but for the addresses of the
